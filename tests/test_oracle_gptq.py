@@ -1,0 +1,137 @@
+"""Pins the oracle's Hessian / quantize_weight restatement by what the mathematics fixes."""
+import pytest
+import torch
+
+from oracle import gptq as G
+from oracle import observers as O
+from oracle import qformat as F
+
+
+def _obs(w, args, name="memoryless_minmax"):
+    o = O.Observer(name, "weight", args)
+    o(w)
+    return o
+
+
+def _rtn(w, args):
+    qp = _obs(w, args).get_qparams()
+    return F.fake_quantize(w, qp["scale"], qp["zero_point"], args, global_scale=qp["global_scale"])
+
+
+def test_hessian_closed_form_fp64():
+    torch.manual_seed(0)
+    K = 96
+    H = G.make_empty_hessian(K)
+    n = torch.zeros(())
+    xs = [torch.randn(2, 40, K).bfloat16(), torch.randn(33, K).bfloat16(), torch.randn(1, 2, 5, K).bfloat16()]
+    for x in xs:
+        H, n = G.accumulate_hessian(x, H, n)
+    ref = sum(2 * x.double().reshape(-1, K).t() @ x.double().reshape(-1, K) for x in xs)
+    assert n.item() == 2 + 1 + 1  # batch entries, not tokens (gptq_quantize.py:40)
+    assert (H.double() - ref).norm() / ref.norm() < 1e-6
+    assert torch.equal(H, H.t())
+
+
+@pytest.mark.parametrize("actorder", [None, "weight", "group"])
+def test_reference_fixture_shapes_group(actorder):
+    # tests/llmcompressor/modifiers/gptq/test_gptq_quantize.py:21-60
+    torch.manual_seed(1)
+    w = torch.nn.Linear(8, 6, bias=False).weight.data
+    args = F.QArgs(num_bits=4, strategy="group", group_size=2, actorder=actorder)
+    H = G.make_empty_hessian(8) + torch.diag(torch.arange(1, 9, dtype=torch.float32))
+    loss, out, _ = G.quantize_weight(w, _obs(w, args), args, H)
+    assert loss >= 0
+    assert out["weight"].shape == w.shape
+    assert out["weight_scale"].shape == (6, 4) and out["weight_zero_point"].shape == (6, 4)
+    assert ("weight_g_idx" in out) == (actorder == "group")
+    if actorder == "group":
+        assert out["weight_g_idx"].shape == (8,)
+    if actorder != "group":
+        # diagonal Hessian => no error propagation => GPTQ == round-to-nearest
+        assert torch.equal(out["weight"], _rtn(w, args))
+
+
+def test_reference_fixture_shapes_block_and_channel():
+    torch.manual_seed(2)
+    w = torch.nn.Linear(7, 5, bias=False).weight.data
+    args = F.QArgs(num_bits=8, strategy="block", block_structure=[2, 4])
+    loss, out, _ = G.quantize_weight(w, _obs(w, args), args, torch.eye(7), blocksize=3)
+    assert loss >= 0 and out["weight_scale"].shape == (3, 2) and "weight_g_idx" not in out
+    assert torch.allclose(out["weight"], _rtn(w, args))
+    w = torch.nn.Linear(8, 4, bias=False).weight.data
+    args = F.QArgs(num_bits=4, strategy="channel", actorder="weight")
+    H = torch.diag(torch.arange(1, 9, dtype=torch.float32))
+    loss, out, _ = G.quantize_weight(w, _obs(w, args), args, H, blocksize=4)
+    assert out["weight_scale"].shape[0] == 4 and "weight_g_idx" not in out
+    assert torch.equal(out["weight"], _rtn(w, args))
+
+
+def _problem(R=12, K=32, seed=0, dtype=torch.bfloat16):
+    torch.manual_seed(seed)
+    w = (torch.randn(R, K) * 0.05).to(dtype)
+    x = torch.randn(4 * K, K)
+    x[:, 3] *= 8
+    H = 2 * x.t() @ x / 4
+    return w, H
+
+
+@pytest.mark.parametrize("bs", [1, 3, 8, 32])
+def test_blocksize_independence(bs):
+    w, H = _problem()
+    args = F.QArgs(num_bits=4, strategy="group", group_size=8)
+    _, ref, _ = G.quantize_weight(w, _obs(w, args), args, H.clone(), blocksize=128)
+    _, out, _ = G.quantize_weight(w, _obs(w, args), args, H.clone(), blocksize=bs)
+    agree = (out["weight"] == ref["weight"]).float().mean().item()
+    assert agree >= 0.99
+
+
+def test_matches_textbook_gptq_fp64():
+    w, H = _problem(R=16, K=24, seed=3, dtype=torch.float32)
+    args = F.QArgs(num_bits=4, strategy="group", group_size=8)
+    obs = _obs(w, args)
+    scale, zp = F.calculate_qparams(obs.min_vals, obs.max_vals, args)
+
+    def qcol(j, col):
+        g = j // 8
+        return F.fake_quantize(col.float(), scale[:, g], zp[:, g], args.copy(strategy="channel")).double()
+
+    Q = G.textbook_gptq_fp64(w, H, qcol)
+    loss, out, info = G.quantize_weight(w, obs, args, H.clone())
+    assert info["ok"]
+    assert (out["weight"].double() == Q).float().mean().item() >= 0.98
+    # loss recomputed independently: 1/2 sum (w-q)^2/d^2 is >= 0 and finite
+    assert loss >= 0 and torch.isfinite(torch.tensor(loss))
+
+
+def test_grid_membership_and_scale_invariance():
+    w, H = _problem(seed=5)
+    args = F.QArgs(num_bits=4, strategy="group", group_size=8)
+    _, a, _ = G.quantize_weight(w, _obs(w, args), args, H.clone())
+    _, b, _ = G.quantize_weight(w, _obs(w, args), args, (H * 1024.0).clone())
+    assert (a["weight"] == b["weight"]).float().mean() >= 0.99
+    s = a["weight_scale"].float().repeat_interleave(8, dim=1)
+    codes = a["weight"].float() / s
+    assert torch.all((codes - codes.round()).abs() <= 8 * 2.0**-8)  # bf16 rounding of q*s
+    assert codes.round().min() >= -8 and codes.round().max() <= 7
+
+
+def test_non_pd_hessian_falls_back_to_rtn_and_dead_columns_zeroed():
+    w, _ = _problem(seed=6)
+    args = F.QArgs(num_bits=4, strategy="group", group_size=8)
+    _, out, info = G.quantize_weight(w, _obs(w, args), args, -torch.eye(32))
+    assert not info["ok"]
+    assert torch.equal(out["weight"], _rtn(w, args))
+    _, out, _ = G.quantize_weight(w, _obs(w, args), args, torch.zeros(32, 32))
+    assert torch.count_nonzero(out["weight"]) == 0
+
+
+def test_upper_factor_identity():
+    # U^T U = H^-1 with U upper, positive diagonal; also equals inverse of the reverse Cholesky factor
+    _, H = _problem(K=24, seed=7)
+    Hd = H.double() + 0.01 * H.double().diag().mean() * torch.eye(24, dtype=torch.float64)
+    U, ok = G.hessian_inverse_factor(H.clone(), 0.01)
+    assert ok
+    assert torch.allclose(U.double().t() @ U.double() @ Hd, torch.eye(24, dtype=torch.float64), atol=1e-3)
+    J = torch.eye(24, dtype=torch.float64).flip(0)
+    Rr = J @ torch.linalg.cholesky(J @ Hd @ J) @ J
+    assert torch.allclose(torch.linalg.inv(Rr), U.double(), atol=1e-4, rtol=1e-3)
