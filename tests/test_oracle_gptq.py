@@ -14,8 +14,11 @@ def _obs(w, args, name="memoryless_minmax"):
 
 
 def _rtn(w, args):
+    # quantize_weight divides the fp32 work copy by the (weight-dtype) scale, so the
+    # round-to-nearest it degenerates to is the one taken on fp32 weights
     qp = _obs(w, args).get_qparams()
-    return F.fake_quantize(w, qp["scale"], qp["zero_point"], args, global_scale=qp["global_scale"])
+    out = F.fake_quantize(w.float(), qp["scale"], qp["zero_point"], args, global_scale=qp["global_scale"])
+    return out.to(w.dtype)
 
 
 def test_hessian_closed_form_fp64():
