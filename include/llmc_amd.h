@@ -61,6 +61,79 @@ int llmc_hessian_accumulate(float* H, int64_t ldh, const void* X, int64_t ldx,
                             int64_t T, int64_t K, int32_t x_dtype, float alpha,
                             int32_t flags, void* stream);
 
+/* ---- a10/a11: min-max observers --------------------------------------------
+ * Replace _get_min_max() = torch.amin/amax(observed, dim=(0,-1)) on the
+ * flattened weight (src/llmcompressor/observers/min_max.py:70-74 with
+ * observers/helpers.py:28-157).  Outputs are in the observed dtype.
+ *   llmc_minmax_groups : weight [R,K], groups of `group` consecutive columns
+ *                        (group = K: per channel; R=1, group=K=numel: per tensor)
+ *                        -> [R, K/group]
+ *   llmc_minmax_blocks : block strategy, zero-padded edges -> [ceil(R/bh), ceil(K/bw)]
+ *   llmc_minmax_strided: generic (num_observations, n1, group) view with element
+ *                        strides (stride0, stride1, 1) -> [n1]  (activations)
+ */
+int64_t llmc_minmax_workspace_bytes(void);
+int llmc_minmax_groups(const void* x, int32_t dtype, int64_t R, int64_t K, int64_t ldw,
+                       int64_t group, void* min_out, void* max_out, void* workspace,
+                       int64_t workspace_bytes, void* stream);
+int llmc_minmax_blocks(const void* x, int32_t dtype, int64_t R, int64_t K, int64_t ldw,
+                       int32_t block_h, int32_t block_w, void* min_out, void* max_out,
+                       void* stream);
+int llmc_minmax_strided(const void* x, int32_t dtype, int64_t n0, int64_t n1, int64_t group,
+                        int64_t stride0, int64_t stride1, void* min_out, void* max_out,
+                        void* stream);
+
+/* ---- a12/a16: qparams ------------------------------------------------------
+ * llmc_absmax_accumulate + llmc_generate_gparam replace Observer.get_global_scale()
+ * (src/llmcompressor/observers/base.py:78-96; CT generate_gparam): absmax_inout
+ * (fp32, caller zero-initialised) takes max(absmax, -min, max) over the arrays of
+ * every observer of a fused group, one call each; gparam = 448*6/absmax divided in
+ * the statistics' dtype, returned as fp32 [1].
+ * llmc_calculate_qparams replaces CT calculate_qparams as called from
+ * observers/base.py:114-119: n (min,max) pairs -> scale (scale_out_dtype; fp32
+ * e4m3-grid values for LLMC_SCALE_NVFP4), int8 zero points (NULL when symmetric),
+ * and optionally the stored scale code (e4m3 byte for NVFP4, E8M0 byte for MXFP4).
+ */
+int llmc_absmax_accumulate(const void* min_vals, const void* max_vals, int64_t n, int32_t dtype,
+                           float* absmax_inout, void* stream);
+int llmc_generate_gparam(const float* absmax, int32_t stats_dtype, float* global_scale_out,
+                         void* stream);
+int llmc_calculate_qparams(const void* min_vals, const void* max_vals, int64_t n,
+                           int32_t stats_dtype, int32_t fmt, int32_t num_bits, int32_t symmetric,
+                           int32_t scale_mode, const float* global_scale, void* scale_out,
+                           int32_t scale_out_dtype, int8_t* zero_point_out,
+                           uint8_t* scale_code_out, void* stream);
+
+/* ---- a17/a18: quantise, fake-quantise, pack --------------------------------
+ * Replaces CT fake_quantize / quantize (call sites gptq_quantize.py:184-225,
+ * observers/mse_quant.py:275-280, modifiers/quantization/calibration.py:178-183)
+ * and the compressors' pack step (pack_to_int32, pack_fp4_to_uint8, fp8 storage;
+ * call site transformers/compression/compressed_tensors_utils.py:134-138).
+ * The scale of element (r,c) is scale[(r/row_div)*scale_row_stride +
+ * (g_idx ? g_idx[c] : c/col_div)]; with global_scale the effective scale is
+ * float(scale)/global_scale[0].
+ *   LLMC_OUT_FAKEQUANT: dequantised values, out_dtype, ldo in elements
+ *   LLMC_OUT_CODES    : one byte per element (int8 code | e4m3 byte | e2m1 nibble)
+ *   LLMC_OUT_PACKED   : int -> int32 words, 32/num_bits offset-binary fields per
+ *                       word, field j at bit j*num_bits (ldo in words);
+ *                       fp4 -> uint8, even column in the low nibble (ldo in bytes);
+ *                       fp8 -> e4m3 bytes (ldo in bytes)
+ */
+enum { LLMC_OUT_FAKEQUANT = 0, LLMC_OUT_CODES = 1, LLMC_OUT_PACKED = 2 };
+int llmc_quantize(const void* x, int32_t x_dtype, int64_t R, int64_t K, int64_t ldx,
+                  const void* scale, int32_t scale_dtype, const int8_t* zero_point,
+                  const int32_t* g_idx, const float* global_scale, int32_t fmt, int32_t num_bits,
+                  int64_t row_div, int64_t scale_row_stride, int64_t col_div, int32_t out_mode,
+                  void* out, int32_t out_dtype, int64_t ldo, void* stream);
+
+/* Dynamic per-token quantisation (CT compute_dynamic_scales_and_zp + fake_quantize,
+ * strategy "token", reached through forward_quantize, calibration.py:178-183):
+ * per row absmax -> scale = absmax/(range/2) in the row dtype -> quantise.
+ * out_mode FAKEQUANT (row dtype) or CODES (bytes). scale_out: [N] in the row dtype. */
+int llmc_dynamic_per_token_quantize(const void* x, int32_t x_dtype, int64_t N, int64_t K,
+                                    int64_t ldx, int32_t fmt, int32_t num_bits, int32_t out_mode,
+                                    void* out, int64_t ldo, void* scale_out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

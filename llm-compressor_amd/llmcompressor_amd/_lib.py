@@ -51,14 +51,26 @@ _F32 = ctypes.c_float
 SIGNATURES = {
     "llmc_version": [],
     "llmc_hessian_accumulate": [_P, _I64, _P, _I64, _I64, _I64, _I32, _F32, _I32, _P],
+    "llmc_minmax_groups": [_P, _I32, _I64, _I64, _I64, _I64, _P, _P, _P, _I64, _P],
+    "llmc_minmax_blocks": [_P, _I32, _I64, _I64, _I64, _I32, _I32, _P, _P, _P],
+    "llmc_minmax_strided": [_P, _I32, _I64, _I64, _I64, _I64, _I64, _P, _P, _P],
+    "llmc_absmax_accumulate": [_P, _P, _I64, _I32, _P, _P],
+    "llmc_generate_gparam": [_P, _I32, _P, _P],
+    "llmc_calculate_qparams": [_P, _P, _I64, _I32, _I32, _I32, _I32, _I32, _P, _P, _I32, _P, _P, _P],
+    "llmc_quantize": [_P, _I32, _I64, _I64, _I64, _P, _I32, _P, _P, _P, _I32, _I32, _I64, _I64, _I64,
+                      _I32, _P, _I32, _I64, _P],
+    "llmc_dynamic_per_token_quantize": [_P, _I32, _I64, _I64, _I64, _I32, _I32, _I32, _P, _I64, _P, _P],
 }
+# functions whose return type is not int
+RESTYPES = {"llmc_minmax_workspace_bytes": ctypes.c_int64}
+SIGNATURES["llmc_minmax_workspace_bytes"] = []
 
 
 def _declare(l: ctypes.CDLL) -> None:
     for name, argtypes in SIGNATURES.items():
         fn = getattr(l, name)
         fn.argtypes = argtypes
-        fn.restype = ctypes.c_int
+        fn.restype = RESTYPES.get(name, ctypes.c_int)
 
 
 def check(rc: int, what: str) -> None:

@@ -41,3 +41,166 @@ def hessian_accumulate_(H: torch.Tensor, x: torch.Tensor, alpha: float = 2.0, as
         )
     _lib.check(rc, "llmc_hessian_accumulate")
     return H
+
+
+FMT_INT, FMT_FP8, FMT_FP4 = 0, 1, 2
+SCALE_PLAIN, SCALE_NVFP4, SCALE_MXFP4 = 0, 1, 2
+OUT_FAKEQUANT, OUT_CODES, OUT_PACKED = 0, 1, 2
+_TD = {BF16: torch.bfloat16, F16: torch.float16, F32: torch.float32}
+
+_ws_cache = {}
+
+
+def _workspace(device, nbytes: int) -> torch.Tensor:
+    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    ws = _ws_cache.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1 << 16), dtype=torch.uint8, device=device)
+        _ws_cache[key] = ws
+    return ws
+
+
+def _ptr(t):
+    return 0 if t is None else t.data_ptr()
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise TypeError(f"unsupported dtype {t.dtype}; expected bf16/f16/f32") from None
+
+
+def minmax_groups(w: torch.Tensor, group: int):
+    """min/max of each run of `group` consecutive columns of w [R,K] -> two [R, K/group] tensors."""
+    _require_gpu(w)
+    assert w.ndim == 2 and w.stride(1) == 1
+    R, K = w.shape
+    mn = torch.empty((R, K // group), dtype=w.dtype, device=w.device)
+    mx = torch.empty_like(mn)
+    ws = _workspace(w.device, 1 << 16)
+    with torch.cuda.device(w.device):
+        rc = _lib.lib().llmc_minmax_groups(w.data_ptr(), _dt(w), R, K, w.stride(0), group, mn.data_ptr(),
+                                           mx.data_ptr(), ws.data_ptr(), ws.numel(), _stream(w))
+    _lib.check(rc, "llmc_minmax_groups")
+    return mn, mx
+
+
+def minmax_blocks(w: torch.Tensor, bh: int, bw: int):
+    _require_gpu(w)
+    assert w.ndim == 2 and w.stride(1) == 1
+    R, K = w.shape
+    shape = ((R + bh - 1) // bh, (K + bw - 1) // bw)
+    mn = torch.empty(shape, dtype=w.dtype, device=w.device)
+    mx = torch.empty_like(mn)
+    with torch.cuda.device(w.device):
+        rc = _lib.lib().llmc_minmax_blocks(w.data_ptr(), _dt(w), R, K, w.stride(0), bh, bw, mn.data_ptr(),
+                                           mx.data_ptr(), _stream(w))
+    _lib.check(rc, "llmc_minmax_blocks")
+    return mn, mx
+
+
+def minmax_strided(x: torch.Tensor, n0: int, n1: int, group: int, s0: int, s1: int):
+    """x viewed as (n0, n1, group) with element strides (s0, s1, 1): reduce dims (0,-1) -> [n1]."""
+    _require_gpu(x)
+    mn = torch.empty((n1,), dtype=x.dtype, device=x.device)
+    mx = torch.empty_like(mn)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().llmc_minmax_strided(x.data_ptr(), _dt(x), n0, n1, group, s0, s1, mn.data_ptr(),
+                                            mx.data_ptr(), _stream(x))
+    _lib.check(rc, "llmc_minmax_strided")
+    return mn, mx
+
+
+def global_scale_from_stats(stats):
+    """NVFP4 global scale from the (min, max) arrays of every observer of a fused group -> fp32 [1]."""
+    mn0 = stats[0][0]
+    _require_gpu(mn0)
+    absmax = torch.zeros(1, dtype=torch.float32, device=mn0.device)
+    out = torch.empty(1, dtype=torch.float32, device=mn0.device)
+    with torch.cuda.device(mn0.device):
+        for mn, mx in stats:
+            mn, mx = mn.contiguous(), mx.contiguous()
+            rc = _lib.lib().llmc_absmax_accumulate(mn.data_ptr(), mx.data_ptr(), mn.numel(), _dt(mn),
+                                                   absmax.data_ptr(), _stream(mn0))
+            _lib.check(rc, "llmc_absmax_accumulate")
+        rc = _lib.lib().llmc_generate_gparam(absmax.data_ptr(), _dt(mn0), out.data_ptr(), _stream(mn0))
+    _lib.check(rc, "llmc_generate_gparam")
+    return out
+
+
+def calculate_qparams(mn, mx, fmt: int, bits: int, symmetric: bool, scale_mode: int = SCALE_PLAIN,
+                      global_scale=None, want_codes: bool = False):
+    """(min,max) -> (scale, zero_point int8, scale_code uint8|None); shapes follow `mn`."""
+    _require_gpu(mn, mx)
+    mn, mx = mn.contiguous(), mx.contiguous()
+    sdt = torch.float32 if scale_mode == SCALE_NVFP4 else mn.dtype
+    scale = torch.empty(mn.shape, dtype=sdt, device=mn.device)
+    zp = torch.zeros(mn.shape, dtype=torch.int8, device=mn.device)
+    codes = torch.empty(mn.shape, dtype=torch.uint8, device=mn.device) if want_codes else None
+    with torch.cuda.device(mn.device):
+        rc = _lib.lib().llmc_calculate_qparams(
+            mn.data_ptr(), mx.data_ptr(), mn.numel(), _dt(mn), fmt, bits, 1 if symmetric else 0, scale_mode,
+            _ptr(global_scale), scale.data_ptr(), _DT[sdt], 0 if symmetric else zp.data_ptr(), _ptr(codes),
+            _stream(mn))
+    _lib.check(rc, "llmc_calculate_qparams")
+    return scale, zp, codes
+
+
+def quantize(x, scale, zero_point, fmt: int, bits: int, row_div: int, scale_row_stride: int, col_div: int,
+             out_mode: int = OUT_FAKEQUANT, g_idx=None, global_scale=None, out_dtype=None):
+    """Element-wise quantise of x [R,K]; see llmc_quantize in include/llmc_amd.h for the scale indexing."""
+    _require_gpu(x, scale)
+    assert x.ndim == 2 and x.stride(1) == 1
+    R, K = x.shape
+    scale = scale.contiguous()
+    if zero_point is not None:
+        zero_point = zero_point.contiguous()
+        assert zero_point.dtype == torch.int8
+    if g_idx is not None:
+        g_idx = g_idx.to(torch.int32).contiguous()
+    if out_mode == OUT_FAKEQUANT:
+        out_dtype = out_dtype or x.dtype
+        out = torch.empty((R, K), dtype=out_dtype, device=x.device)
+        odt, ldo = _DT[out_dtype], K
+    elif out_mode == OUT_CODES:
+        tdt = torch.int8 if fmt == FMT_INT else (torch.float8_e4m3fn if fmt == FMT_FP8 else torch.uint8)
+        out = torch.empty((R, K), dtype=tdt, device=x.device)
+        odt, ldo = 0, K
+    else:
+        if fmt == FMT_INT:
+            pf = 32 // bits
+            ldo = (K + pf - 1) // pf
+            out = torch.empty((R, ldo), dtype=torch.int32, device=x.device)
+        elif fmt == FMT_FP4:
+            ldo = (K + 1) // 2
+            out = torch.empty((R, ldo), dtype=torch.uint8, device=x.device)
+        else:
+            ldo = K
+            out = torch.empty((R, K), dtype=torch.float8_e4m3fn, device=x.device)
+        odt = 0
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().llmc_quantize(
+            x.data_ptr(), _dt(x), R, K, x.stride(0), scale.data_ptr(), _dt(scale), _ptr(zero_point),
+            _ptr(g_idx), _ptr(global_scale), fmt, bits, row_div, scale_row_stride, col_div, out_mode,
+            out.data_ptr(), odt, ldo, _stream(x))
+    _lib.check(rc, "llmc_quantize")
+    return out
+
+
+def dynamic_per_token_quantize(x, fmt: int = FMT_FP8, bits: int = 8, out_mode: int = OUT_FAKEQUANT):
+    """x [N,K] bf16/f16 -> (fake-quantised x | code bytes, per-row scale [N,1])."""
+    _require_gpu(x)
+    assert x.ndim == 2 and x.stride(1) == 1
+    N, K = x.shape
+    scale = torch.empty((N, 1), dtype=x.dtype, device=x.device)
+    if out_mode == OUT_FAKEQUANT:
+        out = torch.empty((N, K), dtype=x.dtype, device=x.device)
+    else:
+        out = torch.empty((N, K), dtype=torch.float8_e4m3fn if fmt == FMT_FP8 else torch.int8, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().llmc_dynamic_per_token_quantize(x.data_ptr(), _dt(x), N, K, x.stride(0), fmt, bits,
+                                                        out_mode, out.data_ptr(), K, scale.data_ptr(),
+                                                        _stream(x))
+    _lib.check(rc, "llmc_dynamic_per_token_quantize")
+    return out, scale

@@ -1,0 +1,234 @@
+"""GPU parity (bit-exact): min-max observers, qparams, fake-quant and packed storage vs the CPU oracle."""
+import pytest
+import torch
+
+from oracle import observers as O
+from oracle import pack as P
+from oracle import qformat as F
+
+pytestmark = pytest.mark.gpu
+
+E4M3 = torch.float8_e4m3fn
+
+
+def _w(R, K, dtype=torch.bfloat16, seed=0, std=0.02):
+    g = torch.Generator().manual_seed(seed)
+    w = torch.randn(R, K, generator=g) * std
+    w[0, 0] = 0.0
+    if R > 1:
+        w[1, :] = 0.0  # an all-zero row: zero scale -> epsilon substitution
+    return w.to(dtype)
+
+
+def _bits(t):
+    if t.dtype == torch.float32:
+        return t.view(torch.int32)
+    if t.dtype in (torch.bfloat16, torch.float16):
+        return t.view(torch.int16)
+    return t
+
+
+def _same(a, b):
+    """bit-exact up to the sign of zero"""
+    a, b = a.cpu(), b.cpu()
+    assert a.shape == b.shape and a.dtype == b.dtype, (a.shape, b.shape, a.dtype, b.dtype)
+    return torch.equal(a, b)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("R,K,g", [(64, 512, 16), (64, 512, 32), (64, 512, 128), (64, 512, 512), (8, 56, 7),
+                                   (3, 8200, 8200), (1, 64 * 512, 64 * 512), (5, 24, 3), (16, 4096, 4096)])
+def test_minmax_groups(dtype, R, K, g):
+    from llmcompressor_amd import ops
+
+    w = _w(R, K, dtype, seed=R + K + g)
+    mn, mx = ops.minmax_groups(w.cuda(), g)
+    flat = w.unflatten(-1, (-1, g)).unsqueeze(0)
+    emn, emx = O.get_min_max(flat)
+    assert _same(mn, emn) and _same(mx, emx)
+
+
+def test_minmax_tensor_large_and_blocks_and_strided():
+    from llmcompressor_amd import ops
+
+    w = _w(1024, 4096, seed=3)
+    mn, mx = ops.minmax_groups(w.cuda().view(1, -1), w.numel())
+    assert mn.item() == w.min().item() and mx.item() == w.max().item()
+    for (R, K, bh, bw) in [(10, 8, 3, 3), (10, 8, 5, 4), (256, 512, 128, 128), (4, 6, 2, 3)]:
+        w = _w(R, K, seed=R)
+        args = F.QArgs(strategy="block", block_structure=[bh, bw])
+        emn, emx = O.get_min_max(O.flatten_for_calibration(w, "weight", args))
+        mn, mx = ops.minmax_blocks(w.cuda(), bh, bw)
+        assert _same(mn, emn) and _same(mx, emx)
+    x = _w(6 * 10, 64, seed=9, std=1.0).reshape(6, 10, 64)
+    args = F.QArgs(strategy="group", group_size=16)
+    emn, emx = O.get_min_max(O.flatten_for_calibration(x, "input", args))
+    mn, mx = ops.minmax_strided(x.cuda(), 60, 4, 16, 64, 16)
+    assert _same(mn, emn) and _same(mx, emx)
+
+
+SCHEMES = {
+    "int4_sym_g128": dict(num_bits=4, strategy="group", group_size=128),
+    "int4_asym_g32": dict(num_bits=4, strategy="group", group_size=32, symmetric=False),
+    "int8_sym_channel": dict(num_bits=8, strategy="channel"),
+    "int8_asym_tensor": dict(num_bits=8, strategy="tensor", symmetric=False),
+    "fp8_channel": dict(num_bits=8, type="float", strategy="channel"),
+    "nvfp4": dict(num_bits=4, type="float", strategy="tensor_group", group_size=16, scale_dtype=E4M3),
+    "mxfp4": dict(num_bits=4, type="float", strategy="group", group_size=32, scale_dtype=torch.uint8),
+    "int4_block": dict(num_bits=4, strategy="block", block_structure=[128, 128]),
+    "int3_g64": dict(num_bits=3, strategy="group", group_size=64),
+}
+
+
+def _fmt(args):
+    from llmcompressor_amd import ops
+
+    if args.type == "int":
+        return ops.FMT_INT, args.num_bits
+    return (ops.FMT_FP8, 8) if args.num_bits == 8 else (ops.FMT_FP4, 4)
+
+
+def _gpu_pipeline(w, args, dtype):
+    """observe -> qparams -> fake-quant / codes / packed, all through the C ABI."""
+    from llmcompressor_amd import ops
+
+    wg = w.cuda()
+    R, K = w.shape
+    s = args.strategy
+    if s == "tensor":
+        mn, mx = ops.minmax_groups(wg.view(1, -1), R * K)
+        mn, mx = mn.view(1), mx.view(1)
+        idx = (1 << 40, 0, 1 << 40)
+    elif s == "channel":
+        mn, mx = ops.minmax_groups(wg, K)
+        idx = (1, 1, 1 << 40)
+    elif s in ("group", "tensor_group"):
+        mn, mx = ops.minmax_groups(wg, args.group_size)
+        idx = (1, K // args.group_size, args.group_size)
+    else:
+        bh, bw = args.block_structure
+        mn, mx = ops.minmax_blocks(wg, bh, bw)
+        idx = (bh, (K + bw - 1) // bw, bw)
+    fmt, bits = _fmt(args)
+    mode = ops.SCALE_MXFP4 if args.is_mx else (ops.SCALE_NVFP4 if s == "tensor_group" and args.scale_dtype else ops.SCALE_PLAIN)
+    gs = ops.global_scale_from_stats([(mn, mx)]) if s == "tensor_group" else None
+    scale, zp, codes = ops.calculate_qparams(mn, mx, fmt, bits, args.symmetric, mode, gs, want_codes=mode != ops.SCALE_PLAIN)
+    zpa = None if args.symmetric else zp
+    fq = ops.quantize(wg, scale, zpa, fmt, bits, *idx, out_mode=ops.OUT_FAKEQUANT, global_scale=gs)
+    cd = ops.quantize(wg, scale, zpa, fmt, bits, *idx, out_mode=ops.OUT_CODES, global_scale=gs)
+    pk = ops.quantize(wg, scale, zpa, fmt, bits, *idx, out_mode=ops.OUT_PACKED, global_scale=gs)
+    return dict(min=mn, max=mx, scale=scale, zp=zp, scale_codes=codes, gs=gs, fq=fq, codes=cd, packed=pk)
+
+
+@pytest.mark.parametrize("name", list(SCHEMES))
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_rtn_pipeline_bit_exact(name, dtype):
+    args = F.QArgs(**SCHEMES[name])
+    if args.is_mx and dtype != torch.bfloat16:
+        pytest.skip("MXFP4 scale generation is defined on bf16 statistics")
+    w = _w(256, 512, dtype, seed=len(name), std=0.05)
+    w[7, 100] = 3.0  # outlier
+    got = _gpu_pipeline(w, args, dtype)
+
+    obs = O.Observer("memoryless_minmax", "weight", args)
+    obs(w)
+    assert _same(got["min"], obs.min_vals) and _same(got["max"], obs.max_vals)
+    qp = obs.get_qparams()
+    scale, zp, gs = qp["scale"], qp["zero_point"], qp["global_scale"]
+    assert _same(got["scale"], scale), name
+    if not args.symmetric:
+        assert _same(got["zp"], zp.to(torch.int8))
+    if gs is not None:
+        assert _same(got["gs"], gs)
+    exp_fq = F.fake_quantize(w, scale, zp, args, global_scale=gs)
+    assert _same(got["fq"], exp_fq.to(dtype)), name
+
+    if args.type == "int":
+        codes = F.quantize(w, scale, zp, args, dtype=torch.int8)
+        assert _same(got["codes"], codes)
+        assert _same(got["packed"], P.pack_to_int32(codes, args.num_bits))
+        assert torch.equal(P.unpack_from_int32(got["packed"].cpu(), args.num_bits, w.shape), codes)
+    elif args.num_bits == 8:
+        q8 = F.quantize(w, scale, zp, args, dtype=E4M3)
+        assert torch.equal(got["codes"].cpu().view(torch.uint8), q8.view(torch.uint8))
+        assert torch.equal(got["packed"].cpu().view(torch.uint8), q8.view(torch.uint8))
+    else:
+        q4 = F.quantize(w, scale, zp, args, global_scale=gs)
+        exp_pk = P.pack_fp4_to_uint8(q4)
+        assert _same(got["packed"], exp_pk), name
+        if args.is_mx:
+            exp_codes = (torch.log2(scale.float()) + 127).to(torch.uint8)
+        else:
+            exp_codes = scale.to(E4M3).view(torch.uint8)
+        assert _same(got["scale_codes"], exp_codes)
+
+
+def test_quantize_with_g_idx_and_fp32_input():
+    """GPTQ-style call: fp32 weights, bf16 scales, column -> group map through g_idx."""
+    from llmcompressor_amd import ops
+
+    torch.manual_seed(0)
+    R, K, g = 32, 256, 64
+    w = _w(R, K, torch.bfloat16, seed=11, std=0.05)
+    args = F.QArgs(num_bits=4, strategy="group", group_size=g)
+    obs = O.Observer("memoryless_minmax", "weight", args)
+    obs(w)
+    qp = obs.get_qparams()
+    perm = torch.randperm(K)
+    g_idx = (torch.arange(K, dtype=torch.int32) // g)[perm]
+    wp = w[:, perm].float().contiguous()
+    got = ops.quantize(wp.cuda(), qp["scale"].cuda(), None, ops.FMT_INT, 4, 1, K // g, 1, g_idx=g_idx.cuda(),
+                       out_dtype=torch.bfloat16)
+    chan = args.copy(strategy="channel")
+    exp = torch.stack([F.fake_quantize(wp[:, j], qp["scale"][:, g_idx[j]], qp["zero_point"][:, g_idx[j]], chan)
+                       for j in range(K)], dim=1)
+    assert exp.dtype == torch.bfloat16
+    assert _same(got, exp)
+
+
+@pytest.mark.parametrize("N,K", [(64, 4096), (7, 100), (3, 12288)])
+def test_dynamic_per_token_fp8(N, K):
+    from llmcompressor_amd import ops
+
+    torch.manual_seed(N)
+    x = torch.randn(N, K)
+    mask = torch.rand(N, K) < 0.02
+    x[mask] = torch.distributions.StudentT(3.0).sample((int(mask.sum()),))
+    x[0] = 0
+    x = x.bfloat16()
+    args = F.QArgs(num_bits=8, type="float", strategy="token", dynamic=True)
+    exp_fq, exp_scale = F.forward_quantize_dynamic(x.unsqueeze(0), args)
+    fq, scale = ops.dynamic_per_token_quantize(x.cuda())
+    assert _same(scale, exp_scale[0])
+    assert _same(fq, exp_fq[0])
+    codes, _ = ops.dynamic_per_token_quantize(x.cuda(), out_mode=ops.OUT_CODES)
+    exp_codes = F.quantize(x.unsqueeze(0), exp_scale, None, args, dtype=E4M3)[0]
+    assert torch.equal(codes.cpu().view(torch.uint8), exp_codes.view(torch.uint8))
+
+
+def test_full_size_properties():
+    """Config-2/3 shapes: properties that do not need the (slow) oracle at full size."""
+    from llmcompressor_amd import ops
+
+    torch.manual_seed(0)
+    w = (torch.randn(14336, 4096, device="cuda") * 0.02).bfloat16()
+    # idempotence: fake-quantising a fake-quantised weight with the same qparams is a fixed point
+    mn, mx = ops.minmax_groups(w, 128)
+    scale, _, _ = ops.calculate_qparams(mn, mx, ops.FMT_INT, 4, True)
+    fq = ops.quantize(w, scale, None, ops.FMT_INT, 4, 1, 4096 // 128, 128)
+    fq2 = ops.quantize(fq, scale, None, ops.FMT_INT, 4, 1, 4096 // 128, 128)
+    assert torch.equal(fq, fq2)
+    # pack -> unpack -> dequantise reproduces the fake-quantised weight
+    pk = ops.quantize(w, scale, None, ops.FMT_INT, 4, 1, 4096 // 128, 128, out_mode=ops.OUT_PACKED)
+    shifts = torch.arange(8, device="cuda", dtype=torch.int32) * 4
+    codes = (((pk.unsqueeze(-1) >> shifts) & 15) - 8).reshape(14336, 4096)
+    deq = (codes.to(torch.bfloat16).unflatten(-1, (-1, 128)) * scale.unsqueeze(-1)).flatten(-2)
+    assert torch.equal(deq, fq)
+    # min/max against torch on the same device
+    assert torch.equal(mn, w.unflatten(-1, (-1, 128)).amin(-1)) and torch.equal(mx, w.unflatten(-1, (-1, 128)).amax(-1))
+    # fp8 per-channel: codes decode to the fake-quantised weight
+    mn, mx = ops.minmax_groups(w, 4096)
+    s8, _, _ = ops.calculate_qparams(mn, mx, ops.FMT_FP8, 8, True)
+    fq8 = ops.quantize(w, s8, None, ops.FMT_FP8, 8, 1, 1, 1 << 40)
+    c8 = ops.quantize(w, s8, None, ops.FMT_FP8, 8, 1, 1, 1 << 40, out_mode=ops.OUT_PACKED)
+    assert torch.equal((c8.to(torch.bfloat16) * s8), fq8)
