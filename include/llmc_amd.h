@@ -134,6 +134,46 @@ int llmc_dynamic_per_token_quantize(const void* x, int32_t x_dtype, int64_t N, i
                                     int64_t ldx, int32_t fmt, int32_t num_bits, int32_t out_mode,
                                     void* out, int64_t ldo, void* scale_out, void* stream);
 
+/* ---- a4-a7: damped Cholesky chain --------------------------------------------
+ * Replaces, in quantize_weight (gptq_quantize.py:107-108,144-164, with the
+ * H/num_samples of modifiers/gptq/base.py:336 folded in):
+ *     H = H / divisor; [H = H[perm][:,perm]]; dead = diag(H)==0; H[dead,dead] = 1;
+ *     H += percdamp*mean(diag H) * I; H = cholesky(H); H = cholesky_inverse(H);
+ *     Hinv = cholesky(H, upper=True)
+ * H is overwritten by the upper factor U (U^T U = H^-1, zeros below the diagonal).
+ * dead_out[K] (may be NULL) flags the zero-diagonal columns in permuted order.
+ * *info_out (device int, may be NULL) = 0, or the 1-based index of the first
+ * non-positive pivot; in that case H becomes the identity, which is the
+ * reference's round-to-nearest fallback on _LinAlgError (gptq_quantize.py:157-164).
+ * perm may be NULL.  workspace must be 256-byte aligned.
+ */
+int64_t llmc_gptq_hinv_workspace_bytes(int64_t K);
+int llmc_gptq_hinv(float* H, int64_t ldh, int64_t K, const int32_t* perm, float divisor,
+                   float percdamp, uint8_t* dead_out, void* workspace, int64_t workspace_bytes,
+                   int32_t* info_out, void* stream);
+
+/* ---- a8/a9: GPTQ block column loop ---------------------------------------------
+ * Replaces the loop of quantize_weight (gptq_quantize.py:88-92,144-146,167-250):
+ * W = float(weight)[:, perm], dead columns zeroed; per block of `blocksize`
+ * columns, per column: q = fake_quantize(w), err = (w-q)/U[i,i],
+ * W1[:, i:] -= err (x) U[i, i:]; per block W[:, i2:] -= Err1 @ U[i1:i2, i2:];
+ * finally out_weight[:, perm[c]] = W[:, c] cast to w_dtype and
+ * *loss_out = sum over rows and columns of (w-q)^2 / U[i,i]^2 / 2.
+ * The scale of (row r, permuted column c) is
+ *   scale[(r/row_div)*scale_row_stride + (g_idx ? g_idx[c] : 0)]
+ * (per tensor: row_div >= R; per channel: row_div 1, stride 1; per group: stride K/g and
+ * g_idx[c] = group of permuted column c; block strategy: row_div = block height).
+ * blocksize above 128 runs as 128-wide blocks (same result up to fp32 summation order).
+ */
+int64_t llmc_gptq_quantize_workspace_bytes(int64_t R, int64_t K);
+int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R, int64_t K, int64_t ldw,
+                       const float* U, int64_t ldu, const int32_t* perm, const uint8_t* dead,
+                       const void* scale, int32_t scale_dtype, const int8_t* zero_point,
+                       const float* global_scale, const int32_t* g_idx, int64_t row_div,
+                       int64_t scale_row_stride, int32_t fmt, int32_t num_bits, int32_t blocksize,
+                       void* out_weight, int64_t ldo, float* loss_out, void* workspace,
+                       int64_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,29 @@
+// Internal fp32 GEMM on the matrix cores (v_mfma_f32_32x32x2_f32), used for the
+// trailing-matrix updates of the Cholesky chain and of the GPTQ block loop.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+struct GemmF32 {
+  // C[M,N] = alpha * A[M,Kc] * B' + beta * C,   all row-major
+  //   trans_b = 0: B' = B,  B stored [Kc,N];   trans_b = 1: B' = B^T, B stored [N,Kc]
+  const float* A;
+  int64_t lda;
+  const float* B;
+  int64_t ldb;
+  float* C;
+  int64_t ldc;
+  int M, N, Kc;
+  float alpha, beta;
+  int trans_b;
+  // structure hints (tile-granular; operands must hold exact zeros where the structure says so)
+  int c_lower;      // only tiles that touch the lower triangle of C are computed
+  int a_lower_tri;  // A[m,k] = 0 for k > m : contraction stops at the tile's last row
+  int b_lower_tri;  // B'[k,n] = 0 for k < n : contraction starts at the tile's first column
+  // batching over blockIdx.z
+  int batch;
+  int64_t stride_a, stride_b, stride_c;
+};
+
+// enqueue on `st`; returns 0 or 1000 + hipError_t
+int llmc_gemm_f32(const GemmF32& g, hipStream_t st);

@@ -61,8 +61,19 @@ SIGNATURES = {
                       _I32, _P, _I32, _I64, _P],
     "llmc_dynamic_per_token_quantize": [_P, _I32, _I64, _I64, _I64, _I32, _I32, _I32, _P, _I64, _P, _P],
 }
+SIGNATURES.update({
+    "llmc_gptq_hinv_workspace_bytes": [_I64],
+    "llmc_gptq_hinv": [_P, _I64, _I64, _P, _F32, _F32, _P, _P, _I64, _P, _P],
+    "llmc_gptq_quantize_workspace_bytes": [_I64, _I64],
+    "llmc_gptq_quantize": [_P, _I32, _I64, _I64, _I64, _P, _I64, _P, _P, _P, _I32, _P, _P, _P, _I64, _I64,
+                           _I32, _I32, _I32, _P, _I64, _P, _P, _I64, _P],
+})
 # functions whose return type is not int
-RESTYPES = {"llmc_minmax_workspace_bytes": ctypes.c_int64}
+RESTYPES = {
+    "llmc_minmax_workspace_bytes": ctypes.c_int64,
+    "llmc_gptq_hinv_workspace_bytes": ctypes.c_int64,
+    "llmc_gptq_quantize_workspace_bytes": ctypes.c_int64,
+}
 SIGNATURES["llmc_minmax_workspace_bytes"] = []
 
 

@@ -204,3 +204,51 @@ def dynamic_per_token_quantize(x, fmt: int = FMT_FP8, bits: int = 8, out_mode: i
                                                         _stream(x))
     _lib.check(rc, "llmc_dynamic_per_token_quantize")
     return out, scale
+
+
+def gptq_hinv_(H: torch.Tensor, perm=None, divisor: float = 1.0, percdamp: float = 0.01):
+    """In place: H -> upper factor U of (H/divisor [permuted] + damping)^-1.
+
+    Returns (U (= H), dead uint8 [K], info int32 [1] on device)."""
+    _require_gpu(H)
+    assert H.dtype == torch.float32 and H.ndim == 2 and H.shape[0] == H.shape[1] and H.stride(1) == 1
+    K = H.shape[0]
+    dead = torch.empty(K, dtype=torch.uint8, device=H.device)
+    info = torch.zeros(1, dtype=torch.int32, device=H.device)
+    if perm is not None:
+        perm = perm.to(torch.int32).contiguous()
+    nbytes = _lib.lib().llmc_gptq_hinv_workspace_bytes(K)
+    ws = _workspace(H.device, nbytes)
+    with torch.cuda.device(H.device):
+        rc = _lib.lib().llmc_gptq_hinv(H.data_ptr(), H.stride(0), K, _ptr(perm), float(divisor), float(percdamp),
+                                       dead.data_ptr(), ws.data_ptr(), ws.numel(), info.data_ptr(), _stream(H))
+    _lib.check(rc, "llmc_gptq_hinv")
+    return H, dead, info
+
+
+def gptq_quantize(weight, U, scale, zero_point, fmt: int, bits: int, row_div: int, scale_row_stride: int,
+                  g_idx=None, perm=None, dead=None, global_scale=None, blocksize: int = 128):
+    """The GPTQ column loop.  Returns (quantised-dequantised weight in weight.dtype, loss fp32 [1])."""
+    _require_gpu(weight, U, scale)
+    assert weight.ndim == 2 and weight.stride(1) == 1 and U.stride(1) == 1
+    R, K = weight.shape
+    scale = scale.contiguous()
+    if zero_point is not None:
+        zero_point = zero_point.contiguous()
+        assert zero_point.dtype == torch.int8
+    if g_idx is not None:
+        g_idx = g_idx.to(torch.int32).contiguous()
+    if perm is not None:
+        perm = perm.to(torch.int32).contiguous()
+    out = torch.empty((R, K), dtype=weight.dtype, device=weight.device)
+    loss = torch.empty(1, dtype=torch.float32, device=weight.device)
+    nbytes = _lib.lib().llmc_gptq_quantize_workspace_bytes(R, K)
+    ws = _workspace(weight.device, nbytes)
+    with torch.cuda.device(weight.device):
+        rc = _lib.lib().llmc_gptq_quantize(
+            weight.data_ptr(), _dt(weight), R, K, weight.stride(0), U.data_ptr(), U.stride(0), _ptr(perm),
+            _ptr(dead), scale.data_ptr(), _dt(scale), _ptr(zero_point), _ptr(global_scale), _ptr(g_idx), row_div,
+            scale_row_stride, fmt, bits, blocksize, out.data_ptr(), K, loss.data_ptr(), ws.data_ptr(), ws.numel(),
+            _stream(weight))
+    _lib.check(rc, "llmc_gptq_quantize")
+    return out, loss
