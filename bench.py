@@ -1,0 +1,210 @@
+#!/usr/bin/env python3
+"""Benchmark of the calibration-time quantization hot path on one MI355X.
+
+Workload (BASELINE.json configs[3], one decoder layer per step): GPTQ W4A16 g128,
+activation ordering "static", of the seven Linears of a random-init
+Llama-3-8B-shaped decoder layer.  A step is
+
+  Hessian phase : 256 calibration batches x 2048 tokens; per batch one
+                  H += 2 X^T X launch per Linear (q/k/v/o/gate/up on the 4096-wide
+                  input, down on the 14336-wide one) -- 3.21e14 algorithmic FLOP
+  quantize phase: per Linear  min-max observer -> scales -> diag argsort ->
+                  damped Cholesky chain -> GPTQ column loop -> int4 packing
+
+All inputs are resident in HBM before the timed region.  `value` is the Hessian
+phase's algorithmic TFLOP/s (2*T*K^2 per launch); `quantize_weight_ms_per_linear`
+is the second half of the metric.  Prints ONE JSON line.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "llm-compressor_amd"))
+
+HIDDEN, INTER, KV = 4096, 14336, 1024
+LINEARS = [  # name, out_features, in_features
+    ("q_proj", HIDDEN, HIDDEN),
+    ("k_proj", KV, HIDDEN),
+    ("v_proj", KV, HIDDEN),
+    ("o_proj", HIDDEN, HIDDEN),
+    ("gate_proj", INTER, HIDDEN),
+    ("up_proj", INTER, HIDDEN),
+    ("down_proj", HIDDEN, INTER),
+]
+GROUP = 128
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+
+
+def cpu_baseline(tokens: int):
+    """The oracle (a port of the reference's torch CPU path) on a bounded sample of the same workload."""
+    import torch
+
+    from oracle import gptq as G
+    from oracle import observers as O
+    from oracle import qformat as F
+
+    cores = os.cpu_count() or 1
+    cores = min(cores, 16)
+    torch.set_num_threads(cores)
+    torch.manual_seed(0)
+    K = HIDDEN
+    calls = 8
+    x = torch.randn(calls, 1, tokens, K).bfloat16()
+    H = G.make_empty_hessian(K)
+    n = torch.zeros(())
+    G.accumulate_hessian(x[0], H, n)  # warm-up
+    t0 = time.perf_counter()
+    for i in range(calls):
+        G.accumulate_hessian(x[i], H, n)
+    t_h = (time.perf_counter() - t0) / calls
+    w = (torch.randn(HIDDEN, K) * 0.02).bfloat16()
+    args = F.QArgs(num_bits=4, strategy="group", group_size=GROUP, actorder="weight")
+    obs = O.Observer("memoryless_minmax", "weight", args)
+    t0 = time.perf_counter()
+    obs(w)
+    G.quantize_weight(w, obs, args, H / n)
+    t_q = time.perf_counter() - t0
+    return {
+        "value": round(2.0 * tokens * K * K / t_h / 1e12, 4),
+        "unit": "TFLOP/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"{calls} accumulate_hessian calls of [1,{tokens},{K}] bf16 (fp32 GEMM) + 1 quantize_weight of a "
+        f"{HIDDEN}x{K} Linear (W4A16 g128, actorder static)",
+        "quantize_weight_ms_per_linear": round(t_q * 1e3, 1),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--batches", type=int, default=256, help="calibration batches per step (config: 256)")
+    ap.add_argument("--tokens", type=int, default=2048, help="tokens per batch (config: 2048)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU figure is produced)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from llmcompressor_amd import ops
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    B, T = a.batches, a.tokens
+    gen = torch.Generator(device=dev).manual_seed(0)
+    weights = {
+        name: (torch.randn(r, k, device=dev, generator=gen) * 0.02).bfloat16() for name, r, k in LINEARS
+    }
+    # calibration activations, resident in HBM: one stream per distinct Linear input
+    x_hidden = torch.empty(B, T, HIDDEN, dtype=torch.bfloat16, device=dev)
+    x_inter = torch.empty(B, T, INTER, dtype=torch.bfloat16, device=dev)
+    for b in range(B):
+        x_hidden[b] = torch.randn(T, HIDDEN, device=dev, generator=gen).bfloat16()
+        x_inter[b] = torch.randn(T, INTER, device=dev, generator=gen).bfloat16()
+    hess = {name: torch.zeros(k, k, device=dev) for name, r, k in LINEARS}
+    g_idx_base = {k: (torch.arange(k, dtype=torch.int32, device=dev) // GROUP) for k in (HIDDEN, INTER)}
+
+    dom_events = []
+
+    def step(record: bool):
+        for h in hess.values():
+            h.zero_()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for b in range(B):
+            for name, r, k in LINEARS:
+                x = x_hidden[b] if k == HIDDEN else x_inter[b]
+                if record and k == INTER:
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    ops.hessian_accumulate_(hess[name], x)
+                    e1.record()
+                    dom_events.append((e0, e1))
+                else:
+                    ops.hessian_accumulate_(hess[name], x)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        out = {}
+        for name, r, k in LINEARS:
+            w = weights[name]
+            mn, mx = ops.minmax_groups(w, GROUP)
+            scale, _, _ = ops.calculate_qparams(mn, mx, ops.FMT_INT, 4, True)
+            perm = torch.argsort(torch.diagonal(hess[name]), descending=True).to(torch.int32)
+            g_idx = g_idx_base[k][perm.long()]
+            U, dead, info = ops.gptq_hinv_(hess[name], perm, divisor=float(B), percdamp=0.01)
+            wq, loss = ops.gptq_quantize(w, U, scale, None, ops.FMT_INT, 4, 1, k // GROUP, g_idx=g_idx, perm=perm,
+                                         dead=dead, blocksize=128)
+            packed = ops.quantize(wq, scale, None, ops.FMT_INT, 4, 1, k // GROUP, GROUP, out_mode=ops.OUT_PACKED)
+            out[name] = (packed, scale, loss)
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        return t1 - t0, t2 - t1, out
+
+    for _ in range(a.warmup):
+        step(False)
+    th = tq = 0.0
+    torch.cuda.synchronize()
+    wall0 = time.perf_counter()
+    for _ in range(a.steps):
+        h, q, out = step(True)
+        th += h
+        tq += q
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - wall0
+
+    flop_step = sum(2.0 * T * k * k for _, _, k in LINEARS) * B
+    value = flop_step * a.steps / th / 1e12
+    dom_ms = sum(e0.elapsed_time(e1) for e0, e1 in dom_events) / max(1, len(dom_events))
+    dom_flop = 2.0 * T * INTER * INTER
+    achieved = dom_flop / (dom_ms * 1e-3) / 1e12
+    rec = {
+        "metric": "GPTQ quantize_weight ms/Linear + Hessian TFLOP/s, Llama-3-8B shapes, W4A16 g128",
+        "value": round(value, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": a.steps,
+        "warmup": a.warmup,
+        "ms_per_step": round(wall / a.steps * 1e3, 2),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": "configs[3]: sequential GPTQ W4A16 g128 actorder=static, one Llama-3-8B-shaped decoder layer "
+            f"per step ({B} batches x {T} tokens, 7 Linears: Hessians 6x4096^2 + 14336^2, then quantize_weight + pack)",
+            "batches": B,
+            "tokens": T,
+        },
+        "quantize_weight_ms_per_linear": round(tq / a.steps / len(LINEARS) * 1e3, 3),
+        "hessian_phase_ms_per_step": round(th / a.steps * 1e3, 2),
+        "hessian_algorithmic_flop_per_step": flop_step,
+        "roofline": {
+            "kernel": "hessian_syrk_kernel<256> (down_proj Hessian, T=%d, K=%d)" % (T, INTER),
+            "bound": "mfma",
+            "achieved": round(achieved, 2),
+            "peak": MFMA_BF16_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
+            "traffic": None,
+            "avg_launch_ms": round(dom_ms, 4),
+            "launches_timed": len(dom_events),
+        },
+    }
+    if not a.no_cpu_baseline:
+        rec["cpu_baseline"] = cpu_baseline(T)
+    print(json.dumps(rec))
+
+
+if __name__ == "__main__":
+    main()
