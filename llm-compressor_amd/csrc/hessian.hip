@@ -9,12 +9,14 @@
 // the operand shape of v_mfma_f32_32x32x16_{bf16,f16}.  bf16 x bf16 products
 // are exact in fp32 and the accumulation is fp32, so the result differs from
 // an fp32 GEMM on the upcast inputs only by summation order.
+#include <type_traits>
+
 #include "common.h"
 
 namespace {
 
-constexpr int BK = 64;                  // tokens per slab
-constexpr int ROW_BYTES = BK * 2 + 16;  // LDS bytes per feature row (padded: 36 dwords)
+constexpr int BK = 64;          // tokens per slab
+constexpr int ROW_BYTES = BK * 2;  // LDS bytes per feature row: 8 chunks of 8 tokens, XOR-swizzled
 
 template <int DT>
 struct Mfma;
@@ -33,23 +35,27 @@ struct Mfma<LLMC_F16> {
   }
 };
 
-// 8 consecutive 16-bit features of token row t starting at feature c (zero outside [T,K))
+// 8 consecutive 16-bit features of token row t starting at feature c (zero outside [T,K)).
+// The aligned form is branch-free (clamped address) so the main loop stays one basic block.
 template <bool ALIGNED>
 __device__ __forceinline__ uint4 load8(const uint16_t* X, int64_t ldx, int t, int c, int T, int K) {
+  if (ALIGNED) {
+    const int tt = t < T ? t : T - 1;
+    const int cc = c < K ? c : K - 8;
+    // rows past T are zeroed by the caller before use (last slab only); columns past K only
+    // feed outputs that are never stored, so their (in-bounds) garbage is harmless
+    return *(const uint4*)(X + (int64_t)tt * ldx + cc);
+  }
   uint4 v = make_uint4(0, 0, 0, 0);
   if (t >= T || c >= K) return v;
   const uint16_t* p = X + (int64_t)t * ldx + c;
-  if (ALIGNED) {
-    v = *(const uint4*)p;
-  } else {
-    uint16_t e[8];
+  uint16_t e[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) e[j] = (c + j < K) ? p[j] : (uint16_t)0;
-    v.x = e[0] | ((uint32_t)e[1] << 16);
-    v.y = e[2] | ((uint32_t)e[3] << 16);
-    v.z = e[4] | ((uint32_t)e[5] << 16);
-    v.w = e[6] | ((uint32_t)e[7] << 16);
-  }
+  for (int j = 0; j < 8; ++j) e[j] = (c + j < K) ? p[j] : (uint16_t)0;
+  v.x = e[0] | ((uint32_t)e[1] << 16);
+  v.y = e[2] | ((uint32_t)e[3] << 16);
+  v.z = e[4] | ((uint32_t)e[5] << 16);
+  v.w = e[6] | ((uint32_t)e[7] << 16);
   return v;
 }
 
@@ -57,31 +63,48 @@ __device__ __forceinline__ uint32_t dword_of(const uint4& v, int j) {
   return j == 0 ? v.x : j == 1 ? v.y : j == 2 ? v.z : v.w;
 }
 
-// BT x BT output tile, 256 threads = 2x2 waves, each wave (BT/2)x(BT/2) = MI x MI MFMA tiles
-template <int BT, int DT, bool ALIGNED>
+// byte offset of 16-byte chunk q (tokens 8q..8q+7) of feature row i.  The XOR keeps both access
+// patterns conflict-free: MFMA operand reads touch 8+ consecutive rows at one q, the transposing
+// writes touch rows 8 apart at one q.
+__device__ __forceinline__ int chunk_off(int i, int q) {
+  return i * ROW_BYTES + ((q ^ (i & 7) ^ ((i >> 3) & 7)) << 4);
+}
+
+// BT x BT output tile, 256 threads = 2x2 waves, each wave (BT/2)x(BT/2) = MI x MI MFMA tiles.
+// LDS holds two stages of the two feature-major panels; global loads for slab s+2 are in
+// flight while slab s is multiplied and slab s+1 is transposed into the other stage.
+template <int BT, int DT, bool ALIGNED, bool FAST_EPI>
 __global__ __launch_bounds__(256) void hessian_syrk_kernel(float* __restrict__ H, int64_t ldh,
                                                             const uint16_t* __restrict__ X, int64_t ldx,
                                                             int T, int K, float alpha, int assume_sym,
-                                                            int vec_ok, int nb, int ntiles) {
+                                                            int vec_ok, int nb, int nslots) {
   constexpr int RT = BT / 32;  // token rows per thread per panel
   constexpr int GI = BT / 8;   // 8-feature groups per panel
   constexpr int MI = BT / 64;
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  unsigned char* sA = smem;
-  unsigned char* sB = smem + BT * ROW_BYTES;
+  constexpr int PANEL = BT * ROW_BYTES;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];  // [2 stages][A,B][BT][128 B]
 
-  // consecutive tile ids land on the same XCD (workgroups are dealt round-robin to the 8 XCDs)
-  const int per_xcd = (ntiles + 7) / 8;
+  // Tile order.  Workgroups are dealt round-robin to the 8 XCDs (each with a private L2), so
+  // block b runs on XCD b%8; p makes every XCD walk a contiguous range of tile slots.  Slots are
+  // grouped into SH x SW super-tiles (as many tiles as run concurrently on one XCD), so the
+  // workgroups sharing an L2 touch only SH + SW feature panels of X per slab instead of one each.
+  constexpr int SH = BT == 256 ? 4 : 8, SW = 8;
+  const int per_xcd = (nslots + 7) / 8;
   const int p = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-  if (p >= ntiles) return;
-  // p -> (I, J), J >= I, row-major over the upper triangle
-  int I = 0, rem = p;
-  while (rem >= nb - I) {
-    rem -= nb - I;
-    ++I;
+  if (p >= nslots) return;
+  const int nsj = (nb + SW - 1) / SW;
+  int su = p / (SH * SW), SI = 0;
+  // super-row SI holds super-columns (SH*SI)/SW .. nsj-1 (those that reach the upper triangle)
+  while (su >= nsj - (SH * SI) / SW) {
+    su -= nsj - (SH * SI) / SW;
+    ++SI;
   }
-  const int J = I + rem;
+  const int SJ = (SH * SI) / SW + su;
+  const int I = SI * SH + (p % (SH * SW)) / SW;
+  const int J = SJ * SW + p % SW;
+  if (I >= nb || J >= nb || J < I) return;
   const int i0 = I * BT, j0 = J * BT;
+  const bool diag = (I == J);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -106,10 +129,12 @@ __global__ __launch_bounds__(256) void hessian_syrk_kernel(float* __restrict__ H
       rb[r] = load8<ALIGNED>(X, ldx, t, j0 + g_i * 8, T, K);
     }
   };
-  // registers hold RT token rows x 8 features; LDS wants, per feature, RT consecutive tokens
-  auto store_slab = [&]() {
+  // registers hold RT token rows x 8 features; LDS wants, per feature, RT consecutive tokens.
+  // Feature columns [c_lo, c_hi) of this thread's 8 are written.
+  auto store_cols = [&](unsigned char* stA, unsigned char* stB, int c_lo, int c_hi) {
 #pragma unroll
     for (int c = 0; c < 8; ++c) {
+      if (c < c_lo || c >= c_hi) continue;
       uint32_t oa[RT / 2], ob[RT / 2];
       const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
 #pragma unroll
@@ -117,83 +142,133 @@ __global__ __launch_bounds__(256) void hessian_syrk_kernel(float* __restrict__ H
         oa[q] = __builtin_amdgcn_perm(dword_of(ra[2 * q + 1], c >> 1), dword_of(ra[2 * q], c >> 1), sel);
         ob[q] = __builtin_amdgcn_perm(dword_of(rb[2 * q + 1], c >> 1), dword_of(rb[2 * q], c >> 1), sel);
       }
-      const int off = (g_i * 8 + c) * ROW_BYTES + g_t * RT * 2;
-      if (RT == 8) {
-        *(uint4*)(sA + off) = make_uint4(oa[0], oa[1], oa[2 % (RT / 2)], oa[3 % (RT / 2)]);
-        *(uint4*)(sB + off) = make_uint4(ob[0], ob[1], ob[2 % (RT / 2)], ob[3 % (RT / 2)]);
+      const int row = g_i * 8 + c;
+      if constexpr (RT == 8) {
+        const int off = chunk_off(row, g_t);
+        *(uint4*)(stA + off) = make_uint4(oa[0], oa[1], oa[2], oa[3]);
+        *(uint4*)(stB + off) = make_uint4(ob[0], ob[1], ob[2], ob[3]);
       } else {
-        *(uint2*)(sA + off) = make_uint2(oa[0], oa[1 % (RT / 2)]);
-        *(uint2*)(sB + off) = make_uint2(ob[0], ob[1 % (RT / 2)]);
+        const int off = chunk_off(row, g_t >> 1) + (g_t & 1) * 8;
+        *(uint2*)(stA + off) = make_uint2(oa[0], oa[1]);
+        *(uint2*)(stB + off) = make_uint2(ob[0], ob[1]);
       }
     }
   };
-
-  const int nslab = (T + BK - 1) / BK;
-  load_slab(0);
-  store_slab();
-  __syncthreads();
-  for (int s = 0; s < nslab; ++s) {
-    if (s + 1 < nslab) load_slab((s + 1) * BK);
+  // one slab of MFMAs from stage `cur`; when STORE, the second half also transposes the
+  // register-held next slab into stage `nxt` so the LDS writes hide under the matrix ops
+  // zero the token rows of the register-held slab that lie past T (only the last slab has any)
+  auto mask_tail = [&](int t0) {
+    if (!ALIGNED) return;  // the element-wise loader already zero-fills
+#pragma unroll
+    for (int r = 0; r < RT; ++r) {
+      const bool ok = t0 + g_t * RT + r < T;
+      ra[r].x = ok ? ra[r].x : 0u; ra[r].y = ok ? ra[r].y : 0u; ra[r].z = ok ? ra[r].z : 0u; ra[r].w = ok ? ra[r].w : 0u;
+      rb[r].x = ok ? rb[r].x : 0u; rb[r].y = ok ? rb[r].y : 0u; rb[r].z = ok ? rb[r].z : 0u; rb[r].w = ok ? rb[r].w : 0u;
+    }
+  };
+  auto compute = [&](unsigned char* curA, unsigned char* nxtA, auto store_tag) {
+    constexpr bool STORE = decltype(store_tag)::value;
+    unsigned char* curB = curA + PANEL;
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
       uint4 fa[MI], fb[MI];
-      const int koff = ks * 32 + (lane >> 5) * 16;
+      const int q = ks * 2 + (lane >> 5);
 #pragma unroll
-      for (int a = 0; a < MI; ++a)
-        fa[a] = *(const uint4*)(sA + (wm * (BT / 2) + a * 32 + (lane & 31)) * ROW_BYTES + koff);
+      for (int a = 0; a < MI; ++a) fa[a] = *(const uint4*)(curA + chunk_off(wm * (BT / 2) + a * 32 + (lane & 31), q));
 #pragma unroll
-      for (int b = 0; b < MI; ++b)
-        fb[b] = *(const uint4*)(sB + (wn * (BT / 2) + b * 32 + (lane & 31)) * ROW_BYTES + koff);
+      for (int b = 0; b < MI; ++b) fb[b] = *(const uint4*)(curB + chunk_off(wn * (BT / 2) + b * 32 + (lane & 31), q));
+      if (STORE && ks >= 2) store_cols(nxtA, nxtA + PANEL, (ks - 2) * 4, (ks - 2) * 4 + 4);
 #pragma unroll
       for (int a = 0; a < MI; ++a)
 #pragma unroll
         for (int b = 0; b < MI; ++b) acc[a][b] = Mfma<DT>::run(fa[a], fb[b], acc[a][b]);
     }
-    __syncthreads();
-    if (s + 1 < nslab) {
-      store_slab();
-      __syncthreads();
-    }
-  }
+  };
 
-  // 32x32 accumulator layout: lane holds column (lane&31); register v holds row
-  // (v/4)*8 + (lane>>5)*4 + (v&3)
-  const bool diag = (I == J);
+  const int nslab = (T + BK - 1) / BK;
+  load_slab(0);
+  mask_tail(0);
+  store_cols(smem, smem + PANEL, 0, 8);
+  load_slab(nslab > 1 ? BK : 0);
+  __syncthreads();
+  // steady state: slab s multiplied, slab s+1 (full) transposed into the other stage, slab s+2 in flight
+  for (int s = 0; s + 2 < nslab; ++s) {
+    compute(smem + (s & 1) * 2 * PANEL, smem + ((s + 1) & 1) * 2 * PANEL, std::true_type{});
+    load_slab((s + 2) * BK);
+    __syncthreads();
+  }
+  if (nslab >= 2) {
+    const int s = nslab - 2;
+    mask_tail((s + 1) * BK);
+    compute(smem + (s & 1) * 2 * PANEL, smem + ((s + 1) & 1) * 2 * PANEL, std::true_type{});
+    __syncthreads();
+  }
+  compute(smem + ((nslab - 1) & 1) * 2 * PANEL, smem, std::false_type{});
+
+  // 32x32 accumulator layout: lane holds column n = lane&31; register v holds row
+  // (v/4)*8 + (lane>>5)*4 + (v&3), i.e. 4 consecutive rows per register quad.  Seen from the
+  // mirrored tile H[j][i] a quad is 4 consecutive floats of one row, so the read-modify-write
+  // runs there with 16-byte accesses (4x fewer, 4x larger requests in flight); the tile
+  // H[i][j] itself then only needs stores, which are row-contiguous across lanes.
+  if (FAST_EPI && i0 + BT <= K && j0 + BT <= K) {
+    // interior tile: no bounds checks, so the 16-byte loads of a whole row of MFMA tiles are
+    // issued back to back before the first use
+#pragma unroll
+    for (int a = 0; a < MI; ++a) {
+      float4 old[MI][4];
+#pragma unroll
+      for (int b = 0; b < MI; ++b) {
+        const int col = j0 + wn * (BT / 2) + b * 32 + (lane & 31);
+        const int rbase = i0 + wm * (BT / 2) + a * 32 + (lane >> 5) * 4;
+#pragma unroll
+        for (int vq = 0; vq < 4; ++vq) old[b][vq] = *(const float4*)(H + (int64_t)col * ldh + rbase + vq * 8);
+      }
+#pragma unroll
+      for (int b = 0; b < MI; ++b) {
+        const int col = j0 + wn * (BT / 2) + b * 32 + (lane & 31);
+        const int rbase = i0 + wm * (BT / 2) + a * 32 + (lane >> 5) * 4;
+#pragma unroll
+        for (int vq = 0; vq < 4; ++vq) {
+          const int r0 = rbase + vq * 8;
+          float4 o;
+          o.x = old[b][vq].x + alpha * acc[a][b][vq * 4 + 0];
+          o.y = old[b][vq].y + alpha * acc[a][b][vq * 4 + 1];
+          o.z = old[b][vq].z + alpha * acc[a][b][vq * 4 + 2];
+          o.w = old[b][vq].w + alpha * acc[a][b][vq * 4 + 3];
+          *(float4*)(H + (int64_t)col * ldh + r0) = o;
+          if (!diag) {
+            H[(int64_t)(r0 + 0) * ldh + col] = o.x;
+            H[(int64_t)(r0 + 1) * ldh + col] = o.y;
+            H[(int64_t)(r0 + 2) * ldh + col] = o.z;
+            H[(int64_t)(r0 + 3) * ldh + col] = o.w;
+          }
+        }
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int a = 0; a < MI; ++a) {
 #pragma unroll
     for (int b = 0; b < MI; ++b) {
       const int col = j0 + wn * (BT / 2) + b * 32 + (lane & 31);
       const int rbase = i0 + wm * (BT / 2) + a * 32 + (lane >> 5) * 4;
-      if (col >= K) continue;
+      if (col < K) {
 #pragma unroll
-      for (int vq = 0; vq < 4; ++vq) {
-        float out[4];
-        const int r0 = rbase + vq * 8;
+        for (int vq = 0; vq < 4; ++vq) {
+          const int r0 = rbase + vq * 8;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int row = r0 + e;
-          out[e] = 0.f;
-          if (row < K) {
-            float* hp = H + (int64_t)row * ldh + col;
-            out[e] = *hp + alpha * acc[a][b][vq * 4 + e];
-            *hp = out[e];
-          }
-        }
-        if (!diag) {
-          float* mp = H + (int64_t)col * ldh + r0;
-          if (assume_sym) {
-            if (r0 + 3 < K && vec_ok) {
-              *(float4*)mp = make_float4(out[0], out[1], out[2], out[3]);
-            } else {
-#pragma unroll
-              for (int e = 0; e < 4; ++e)
-                if (r0 + e < K) mp[e] = out[e];
+          for (int e = 0; e < 4; ++e) {
+            const int row = r0 + e;
+            if (row < K) {
+              float* hp = H + (int64_t)row * ldh + col;
+              const float out = *hp + alpha * acc[a][b][vq * 4 + e];
+              *hp = out;
+              if (!diag) {
+                float* mp = H + (int64_t)col * ldh + row;
+                *mp = assume_sym ? out : *mp + alpha * acc[a][b][vq * 4 + e];
+              }
             }
-          } else {
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-              if (r0 + e < K) mp[e] += alpha * acc[a][b][vq * 4 + e];
           }
         }
       }
@@ -205,19 +280,26 @@ template <int BT, int DT>
 int launch(float* H, int64_t ldh, const void* X, int64_t ldx, int64_t T, int64_t K, float alpha,
            int flags, hipStream_t st) {
   const int nb = (int)((K + BT - 1) / BT);
-  const int ntiles = nb * (nb + 1) / 2;
-  const int grid = ((ntiles + 7) / 8) * 8;
+  constexpr int SH = BT == 256 ? 4 : 8, SW = 8;  // must match the kernel
+  const int nsi = (nb + SH - 1) / SH, nsj = (nb + SW - 1) / SW;
+  int nsuper = 0;
+  for (int si = 0; si < nsi; ++si) nsuper += nsj - (SH * si) / SW;
+  const int nslots = nsuper * SH * SW;
+  const int grid = ((nslots + 7) / 8) * 8;
   const bool aligned = (K % 8 == 0) && (ldx % 8 == 0) && (((uintptr_t)X & 15) == 0);
   const int sym = (flags & LLMC_HESSIAN_ASSUME_SYMMETRIC) ? 1 : 0;
   const int vec_ok = ((ldh & 3) == 0 && ((uintptr_t)H & 15) == 0) ? 1 : 0;
-  constexpr int smem = 2 * BT * ROW_BYTES;
-  auto kern = aligned ? hessian_syrk_kernel<BT, DT, true> : hessian_syrk_kernel<BT, DT, false>;
+  constexpr int smem = 4 * BT * ROW_BYTES;
+  // 16-byte read-modify-write epilogue needs a symmetric H and 16-byte aligned rows
+  const bool fast = sym && vec_ok;
+  auto kern = aligned ? (fast ? hessian_syrk_kernel<BT, DT, true, true> : hessian_syrk_kernel<BT, DT, true, false>)
+                      : (fast ? hessian_syrk_kernel<BT, DT, false, true> : hessian_syrk_kernel<BT, DT, false, false>);
   if (smem > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return 1000 + (int)e;
   }
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), smem, st, H, ldh, (const uint16_t*)X, ldx, (int)T,
-                     (int)K, alpha, sym, vec_ok, nb, ntiles);
+                     (int)K, alpha, sym, vec_ok, nb, nslots);
   LLMC_LAUNCH_STATUS();
   return 0;
 }
