@@ -83,6 +83,34 @@ int llmc_minmax_strided(const void* x, int32_t dtype, int64_t n0, int64_t n1, in
                         int64_t stride0, int64_t stride1, void* min_out, void* max_out,
                         void* stream);
 
+/* ---- a13: MSE observers ------------------------------------------------------
+ * Replace _grid_search_mse (eager path, src/llmcompressor/observers/mse_quant.py:19-141,
+ * 255-285) for memoryless_mse / mse / nvfp4_expanded_mse: for i in range(steps):
+ * p = 1 - i/grid; qparams from (p*min, p*max); err = sum |fq(x) - x|^norm over the
+ * group; keep the first strict minimum per group; stop globally after `patience`
+ * consecutive steps without any improvement.  steps = int(maxshrink*grid) <= 256.
+ * All intermediates are rounded to the observed dtype as the eager ops do.
+ * Outputs (min, max) in the observed dtype with the same shapes as the min-max calls.
+ * scale_mode is LLMC_SCALE_PLAIN (the reference searches TENSOR_GROUP with
+ * scale_dtype=None) or LLMC_SCALE_MXFP4.  workspace: llmc_mse_workspace_bytes(#groups).
+ */
+int64_t llmc_mse_workspace_bytes(int64_t n_groups);
+int llmc_mse_observe_groups(const void* x, int32_t dtype, int64_t R, int64_t K, int64_t ldw,
+                            int64_t group, int32_t fmt, int32_t num_bits, int32_t symmetric,
+                            int32_t scale_mode, int32_t steps, double grid, int32_t patience,
+                            float norm, float expand, void* min_out, void* max_out, void* workspace,
+                            int64_t workspace_bytes, void* stream);
+int llmc_mse_observe_strided(const void* x, int32_t dtype, int64_t n0, int64_t n1, int64_t group,
+                             int64_t stride0, int64_t stride1, int32_t fmt, int32_t num_bits,
+                             int32_t symmetric, int32_t scale_mode, int32_t steps, double grid,
+                             int32_t patience, float norm, float expand, void* min_out, void* max_out,
+                             void* workspace, int64_t workspace_bytes, void* stream);
+int llmc_mse_observe_blocks(const void* x, int32_t dtype, int64_t R, int64_t K, int64_t ldw,
+                            int32_t block_h, int32_t block_w, int32_t fmt, int32_t num_bits,
+                            int32_t symmetric, int32_t scale_mode, int32_t steps, double grid,
+                            int32_t patience, float norm, float expand, void* min_out, void* max_out,
+                            void* workspace, int64_t workspace_bytes, void* stream);
+
 /* ---- a12/a16: qparams ------------------------------------------------------
  * llmc_absmax_accumulate + llmc_generate_gparam replace Observer.get_global_scale()
  * (src/llmcompressor/observers/base.py:78-96; CT generate_gparam): absmax_inout

@@ -1,0 +1,424 @@
+// MSE observer: grid search over shrink factors p_i = 1 - i/grid of each group's (min,max).
+//
+// The reference walks the steps on the host and stops GLOBALLY after `patience`
+// consecutive steps in which no group improved.  Here every group walks all steps in
+// one launch with its running best in registers and records the steps at which it
+// improved in a bit mask; the masks are OR-ed into a global per-step flag word.  A
+// one-thread kernel replays the patience rule on the flags to get the stop step, and
+// a last kernel picks, per group, its latest improvement at or before that step --
+// the same selection as the host loop, without a host round trip per step.
+// The inner loop is VALU/transcendental bound (powf per element per step); the
+// weight is read from HBM once.
+#include <string.h>
+
+#include "qformat.h"
+
+namespace {
+
+constexpr int MAX_STEPS = 256;
+constexpr int MASK_WORDS = MAX_STEPS / 64;
+
+struct MseParams {
+  const void* x;
+  int dt;            // dtype of the observed values (and of every intermediate)
+  int fmt, bits, symmetric, scale_mode;
+  int steps;
+  double grid;       // step i shrinks the range by p_i = (float)(1.0 - i/grid), as the host loop does
+  float norm;
+  float expand;
+  void* min0;        // [N] expanded observed min (dtype dt)
+  void* max0;        // [N]
+  uint64_t* masks;   // [N][MASK_WORDS]
+  uint64_t* flags;   // [MASK_WORDS] zero-initialised
+};
+
+__device__ __forceinline__ float step_factor(int i, double grid) { return (float)(1.0 - (double)i / grid); }
+
+// |fq(x) - x|^norm with every intermediate rounded to dt
+__device__ __forceinline__ float elem_error(float x, float s, float zp, bool has_zp, int dt, const QFormat& f,
+                                            float norm) {
+  const float q = quantize_value(x, s, zp, has_zp, dt, f);
+  const float dq = dequantize_value(q, s, zp, has_zp, dt);
+  const float a = fabsf(round_rt(dq - x, dt));
+  // `norm` arrives already rounded to dt: the eager pow converts its scalar exponent to the tensor dtype
+  const float pw = norm == 2.0f ? a * a : powf(a, norm);
+  return round_rt(pw, dt);
+}
+
+__device__ __forceinline__ void unpack8(uint4 v, int dt, float* o) {
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    if (dt == LLMC_BF16) {
+      o[2 * j] = __uint_as_float(w[j] << 16);
+      o[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+    } else {
+      o[2 * j] = f16_bits_to_f32((uint16_t)(w[j] & 0xffffu));
+      o[2 * j + 1] = f16_bits_to_f32((uint16_t)(w[j] >> 16));
+    }
+  }
+}
+
+__device__ __forceinline__ void or_flags(uint64_t* flags, const uint64_t* m) {
+  // OR over the workgroup first, then one atomic per word and workgroup
+  __shared__ unsigned long long sflags[MASK_WORDS];
+  if (threadIdx.x < MASK_WORDS) sflags[threadIdx.x] = 0ull;
+  __syncthreads();
+#pragma unroll
+  for (int wd = 0; wd < MASK_WORDS; ++wd) {
+    unsigned long long v = m[wd];
+    for (int o = 32; o > 0; o >>= 1) v |= __shfl_xor(v, o, 64);
+    if ((threadIdx.x & 63) == 0 && v) atomicOr(&sflags[wd], v);
+  }
+  __syncthreads();
+  if (threadIdx.x < MASK_WORDS && sflags[threadIdx.x]) atomicOr((unsigned long long*)&flags[threadIdx.x], sflags[threadIdx.x]);
+}
+
+// 16-bit inputs, groups of g = 8*L consecutive elements (L a power of two <= 64 lanes per group)
+__global__ __launch_bounds__(256) void mse_team_kernel(MseParams p, int64_t ngroups, int ng, int g, int L,
+                                                       int64_t ldw) {
+  const int64_t gtid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t grp = gtid / L;
+  const int sub = (int)(gtid % L);
+  const bool live = grp < ngroups;
+  const QFormat f = make_qformat(p.fmt, p.bits);
+  float xv[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) xv[j] = 0.f;
+  float mn = INFINITY, mx = -INFINITY;
+  if (live) {
+    const int64_t r = grp / ng, gi = grp % ng;
+    const uint4 v = *(const uint4*)((const uint16_t*)p.x + r * ldw + gi * g + (int64_t)sub * 8);
+    unpack8(v, p.dt, xv);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      mn = fminf(mn, xv[j]);
+      mx = fmaxf(mx, xv[j]);
+    }
+  }
+  for (int o = L >> 1; o > 0; o >>= 1) {
+    mn = fminf(mn, __shfl_xor(mn, o, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+  }
+  mn = round_rt(mn * p.expand, p.dt);
+  mx = round_rt(mx * p.expand, p.dt);
+  float best = p.dt == LLMC_BF16 ? 3.3895313892515355e38f : p.dt == LLMC_F16 ? 65504.0f : 3.4028234663852886e38f;
+  uint64_t mask[MASK_WORDS];
+#pragma unroll
+  for (int wd = 0; wd < MASK_WORDS; ++wd) mask[wd] = 0ull;
+  for (int i = 0; i < p.steps; ++i) {
+    const float pi = step_factor(i, p.grid);
+    const float smin = round_rt(mn * pi, p.dt), smax = round_rt(mx * pi, p.dt);
+    float s, zp;
+    int e;
+    qparams_from_minmax(smin, smax, p.dt, f, p.symmetric != 0, p.scale_mode, 1.f, &s, &zp, &e);
+    float err = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) err += elem_error(xv[j], s, zp, !p.symmetric, p.dt, f, p.norm);
+    for (int o = L >> 1; o > 0; o >>= 1) err += __shfl_xor(err, o, 64);
+    err = round_rt(err, p.dt);
+    if (err < best) {
+      best = err;
+#pragma unroll
+      for (int wd = 0; wd < MASK_WORDS; ++wd)
+        if (wd == (i >> 6)) mask[wd] |= 1ull << (i & 63);
+    }
+  }
+  if (!live) {
+#pragma unroll
+    for (int wd = 0; wd < MASK_WORDS; ++wd) mask[wd] = 0ull;
+  }
+  if (live && sub == 0) {
+    store_rt(p.min0, grp, mn, p.dt);
+    store_rt(p.max0, grp, mx, p.dt);
+#pragma unroll
+    for (int wd = 0; wd < MASK_WORDS; ++wd) p.masks[grp * MASK_WORDS + wd] = mask[wd];
+  }
+  or_flags(p.flags, mask);
+}
+
+struct GenericLayout {
+  int mode;  // 0: (n0, n1, G) view with element strides (s0, s1, 1); 1: bh x bw blocks of an [R,K] matrix
+  int64_t n0, G, s0, s1;
+  int R, K, bh, bw, nbc;
+  int64_t ldw;
+};
+
+__device__ __forceinline__ float generic_load(const void* x, int dt, const GenericLayout& l, int64_t n1, int64_t e) {
+  if (l.mode == 0) return load_rt(x, (e / l.G) * l.s0 + n1 * l.s1 + (e % l.G), dt);
+  const int br = (int)(n1 / l.nbc), bc = (int)(n1 % l.nbc);
+  const int rr = br * l.bh + (int)(e / l.bw), cc = bc * l.bw + (int)(e % l.bw);
+  return (rr < l.R && cc < l.K) ? load_rt(x, (int64_t)rr * l.ldw + cc, dt) : 0.f;
+}
+
+__device__ __forceinline__ float block_sum(float v, float* sh) {
+  v = wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return sh[0] + sh[1] + sh[2] + sh[3];
+}
+
+// any layout / dtype: one workgroup per group, values re-read (from L2) at every step
+__global__ __launch_bounds__(256) void mse_generic_kernel(MseParams p, GenericLayout l) {
+  __shared__ float sh[4];
+  __shared__ float shm[8];
+  const int64_t n1 = blockIdx.x;
+  const int64_t total = l.mode == 0 ? l.n0 * l.G : (int64_t)l.bh * l.bw;
+  const QFormat f = make_qformat(p.fmt, p.bits);
+  float mn = INFINITY, mx = -INFINITY;
+  for (int64_t e = threadIdx.x; e < total; e += 256) {
+    const float v = generic_load(p.x, p.dt, l, n1, e);
+    mn = fminf(mn, v);
+    mx = fmaxf(mx, v);
+  }
+  mn = wave_min(mn);
+  mx = wave_max(mx);
+  if ((threadIdx.x & 63) == 0) {
+    shm[threadIdx.x >> 6] = mn;
+    shm[4 + (threadIdx.x >> 6)] = mx;
+  }
+  __syncthreads();
+  mn = fminf(fminf(shm[0], shm[1]), fminf(shm[2], shm[3]));
+  mx = fmaxf(fmaxf(shm[4], shm[5]), fmaxf(shm[6], shm[7]));
+  mn = round_rt(mn * p.expand, p.dt);
+  mx = round_rt(mx * p.expand, p.dt);
+  float best = p.dt == LLMC_BF16 ? 3.3895313892515355e38f : p.dt == LLMC_F16 ? 65504.0f : 3.4028234663852886e38f;
+  uint64_t mask[MASK_WORDS];
+#pragma unroll
+  for (int wd = 0; wd < MASK_WORDS; ++wd) mask[wd] = 0ull;
+  for (int i = 0; i < p.steps; ++i) {
+    const float pi = step_factor(i, p.grid);
+    const float smin = round_rt(mn * pi, p.dt), smax = round_rt(mx * pi, p.dt);
+    float s, zp;
+    int e_;
+    qparams_from_minmax(smin, smax, p.dt, f, p.symmetric != 0, p.scale_mode, 1.f, &s, &zp, &e_);
+    float err = 0.f;
+    for (int64_t e = threadIdx.x; e < total; e += 256)
+      err += elem_error(generic_load(p.x, p.dt, l, n1, e), s, zp, !p.symmetric, p.dt, f, p.norm);
+    err = round_rt(block_sum(err, sh), p.dt);
+    if (err < best) {
+      best = err;
+#pragma unroll
+      for (int wd = 0; wd < MASK_WORDS; ++wd)
+        if (wd == (i >> 6)) mask[wd] |= 1ull << (i & 63);
+    }
+  }
+  if (threadIdx.x == 0) {
+    store_rt(p.min0, n1, mn, p.dt);
+    store_rt(p.max0, n1, mx, p.dt);
+#pragma unroll
+    for (int wd = 0; wd < MASK_WORDS; ++wd) {
+      p.masks[n1 * MASK_WORDS + wd] = mask[wd];
+      if (mask[wd]) atomicOr((unsigned long long*)&p.flags[wd], (unsigned long long)mask[wd]);
+    }
+  }
+}
+
+// replay of the host loop's patience rule on the per-step "any group improved" flags
+__global__ void mse_stop_kernel(const uint64_t* flags, int steps, int patience, int* last_step) {
+  int no_improve = 0, last = steps - 1;
+  for (int i = 0; i < steps; ++i) {
+    if ((flags[i >> 6] >> (i & 63)) & 1ull) {
+      no_improve = 0;
+    } else if (++no_improve >= patience) {
+      last = i;
+      break;
+    }
+  }
+  *last_step = last;
+}
+
+__global__ __launch_bounds__(256) void mse_select_kernel(const uint64_t* __restrict__ masks, int64_t n,
+                                                         const int* __restrict__ last_step,
+                                                         double grid, int dt,
+                                                         const void* __restrict__ min0,
+                                                         const void* __restrict__ max0,
+                                                         void* __restrict__ min_out, void* __restrict__ max_out) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const int last = *last_step;
+  int best = -1;
+  for (int wd = MASK_WORDS - 1; wd >= 0 && best < 0; --wd) {
+    uint64_t m = masks[i * MASK_WORDS + wd];
+    const int lo = wd * 64;
+    if (last < lo) continue;
+    if (last - lo < 63) m &= (2ull << (last - lo)) - 1ull;
+    if (m) best = lo + 63 - __clzll((long long)m);
+  }
+  const float mn = load_rt(min0, i, dt), mx = load_rt(max0, i, dt);
+  // no recorded improvement (e.g. non-finite errors): the reference keeps the un-shrunk range
+  const float pb = best < 0 ? 1.0f : step_factor(best, grid);
+  store_rt(min_out, i, best < 0 ? mn : round_rt(mn * pb, dt), dt);
+  store_rt(max_out, i, best < 0 ? mx : round_rt(mx * pb, dt), dt);
+}
+
+__global__ void mse_zero_flags_kernel(uint64_t* flags) {
+  if (threadIdx.x < MASK_WORDS) flags[threadIdx.x] = 0ull;
+}
+
+inline int64_t align256(int64_t b) { return (b + 255) / 256 * 256; }
+
+// host-side round-to-nearest-even of a scalar to bf16 / f16
+float round_host(float v, int dt) {
+  if (dt == LLMC_BF16) {
+    uint32_t u;
+    memcpy(&u, &v, 4);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    u &= 0xffff0000u;
+    memcpy(&v, &u, 4);
+    return v;
+  }
+  if (dt == LLMC_F16) return (float)(_Float16)v;
+  return v;
+}
+
+struct Workspace {
+  uint64_t* flags;
+  int* last;
+  void* min0;
+  void* max0;
+  uint64_t* masks;
+};
+
+Workspace carve(void* ws, int64_t n) {
+  char* c = (char*)ws;
+  Workspace w;
+  w.flags = (uint64_t*)c; c += 256;
+  w.last = (int*)c; c += 256;
+  w.min0 = c; c += align256(n * 4);
+  w.max0 = c; c += align256(n * 4);
+  w.masks = (uint64_t*)c;
+  return w;
+}
+
+int finish(const MseParams& p, const Workspace& w, int64_t n, int patience, void* min_out, void* max_out,
+           hipStream_t st) {
+  hipLaunchKernelGGL(mse_stop_kernel, dim3(1), dim3(1), 0, st, w.flags, p.steps, patience, w.last);
+  LLMC_LAUNCH_STATUS();
+  hipLaunchKernelGGL(mse_select_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, w.masks, n, w.last,
+                     p.grid, p.dt, w.min0, w.max0, min_out, max_out);
+  LLMC_LAUNCH_STATUS();
+  return 0;
+}
+
+int setup(MseParams& p, Workspace& w, void* workspace, int64_t n, hipStream_t st) {
+  w = carve(workspace, n);
+  hipLaunchKernelGGL(mse_zero_flags_kernel, dim3(1), dim3(64), 0, st, w.flags);
+  LLMC_LAUNCH_STATUS();
+  p.min0 = w.min0;
+  p.max0 = w.max0;
+  p.masks = w.masks;
+  p.flags = w.flags;
+  return 0;
+}
+
+}  // namespace
+
+extern "C" int64_t llmc_mse_workspace_bytes(int64_t n_groups) {
+  return 512 + 2 * align256(n_groups * 4) + align256(n_groups * MASK_WORDS * 8);
+}
+
+static int check_common(int32_t dtype, int32_t fmt, int32_t num_bits, int32_t scale_mode, int32_t steps,
+                        double grid, float norm, float expand, int32_t patience) {
+  LLMC_CHECK_ARG(dtype >= 0 && dtype <= 2, 2);
+  LLMC_CHECK_ARG(fmt >= 0 && fmt <= 2, 100);
+  LLMC_CHECK_ARG(fmt != LLMC_FMT_INT || (num_bits >= 2 && num_bits <= 8), 101);
+  LLMC_CHECK_ARG(scale_mode == LLMC_SCALE_PLAIN || scale_mode == LLMC_SCALE_MXFP4, 102);
+  LLMC_CHECK_ARG(steps >= 0 && steps <= MAX_STEPS, 103);
+  LLMC_CHECK_ARG(grid > 0.0, 104);
+  LLMC_CHECK_ARG(norm > 0.f && expand > 0.f && patience > 0, 105);
+  return 0;
+}
+
+extern "C" int llmc_mse_observe_groups(const void* x, int32_t dtype, int64_t R, int64_t K, int64_t ldw,
+                                       int64_t group, int32_t fmt, int32_t num_bits, int32_t symmetric,
+                                       int32_t scale_mode, int32_t steps, double grid, int32_t patience,
+                                       float norm, float expand, void* min_out, void* max_out, void* workspace,
+                                       int64_t workspace_bytes, void* stream) {
+  LLMC_CHECK_ARG(x && R > 0 && K > 0, 1);
+  int rc = check_common(dtype, fmt, num_bits, scale_mode, steps, grid, norm, expand, patience);
+  if (rc) return rc;
+  LLMC_CHECK_ARG(ldw >= K, 5);
+  LLMC_CHECK_ARG(group > 0 && K % group == 0, 6);
+  LLMC_CHECK_ARG(min_out && max_out, 16);
+  const int64_t n = R * (K / group);
+  LLMC_CHECK_ARG(workspace && (((uintptr_t)workspace) & 255) == 0 && workspace_bytes >= llmc_mse_workspace_bytes(n), 18);
+  hipStream_t st = (hipStream_t)stream;
+  MseParams p;
+  p.x = x; p.dt = dtype; p.fmt = fmt; p.bits = fmt == LLMC_FMT_INT ? num_bits : (fmt == LLMC_FMT_FP8 ? 8 : 4);
+  p.symmetric = symmetric; p.scale_mode = scale_mode; p.steps = steps; p.grid = grid; p.norm = round_host(norm, dtype); p.expand = expand;
+  Workspace w;
+  rc = setup(p, w, workspace, n, st);
+  if (rc) return rc;
+  const int64_t L = group / 8;
+  const bool team = dtype != LLMC_F32 && group % 8 == 0 && L <= 64 && (L & (L - 1)) == 0 && ldw % 8 == 0 &&
+                    (((uintptr_t)x) & 15) == 0;
+  if (team) {
+    const int64_t threads = n * L;
+    hipLaunchKernelGGL(mse_team_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, p, n,
+                       (int)(K / group), (int)group, (int)L, ldw);
+  } else {
+    GenericLayout l = {};
+    l.mode = 0; l.n0 = 1; l.G = group; l.s0 = 0; l.s1 = group; l.ldw = ldw;
+    if (ldw != K) {
+      // rows are not contiguous: one row at a time keeps the strided view valid
+      LLMC_CHECK_ARG(group == K, 5);
+      l.s1 = ldw;
+    }
+    hipLaunchKernelGGL(mse_generic_kernel, dim3((unsigned)n), dim3(256), 0, st, p, l);
+  }
+  LLMC_LAUNCH_STATUS();
+  return finish(p, w, n, patience, min_out, max_out, st);
+}
+
+extern "C" int llmc_mse_observe_strided(const void* x, int32_t dtype, int64_t n0, int64_t n1, int64_t group,
+                                        int64_t stride0, int64_t stride1, int32_t fmt, int32_t num_bits,
+                                        int32_t symmetric, int32_t scale_mode, int32_t steps, double grid,
+                                        int32_t patience, float norm, float expand, void* min_out, void* max_out,
+                                        void* workspace, int64_t workspace_bytes, void* stream) {
+  LLMC_CHECK_ARG(x && n0 > 0 && n1 > 0 && group > 0, 1);
+  int rc = check_common(dtype, fmt, num_bits, scale_mode, steps, grid, norm, expand, patience);
+  if (rc) return rc;
+  LLMC_CHECK_ARG(min_out && max_out, 17);
+  LLMC_CHECK_ARG(workspace && (((uintptr_t)workspace) & 255) == 0 && workspace_bytes >= llmc_mse_workspace_bytes(n1), 19);
+  hipStream_t st = (hipStream_t)stream;
+  MseParams p;
+  p.x = x; p.dt = dtype; p.fmt = fmt; p.bits = fmt == LLMC_FMT_INT ? num_bits : (fmt == LLMC_FMT_FP8 ? 8 : 4);
+  p.symmetric = symmetric; p.scale_mode = scale_mode; p.steps = steps; p.grid = grid; p.norm = round_host(norm, dtype); p.expand = expand;
+  Workspace w;
+  rc = setup(p, w, workspace, n1, st);
+  if (rc) return rc;
+  GenericLayout l = {};
+  l.mode = 0; l.n0 = n0; l.G = group; l.s0 = stride0; l.s1 = stride1;
+  hipLaunchKernelGGL(mse_generic_kernel, dim3((unsigned)n1), dim3(256), 0, st, p, l);
+  LLMC_LAUNCH_STATUS();
+  return finish(p, w, n1, patience, min_out, max_out, st);
+}
+
+extern "C" int llmc_mse_observe_blocks(const void* x, int32_t dtype, int64_t R, int64_t K, int64_t ldw,
+                                       int32_t block_h, int32_t block_w, int32_t fmt, int32_t num_bits,
+                                       int32_t symmetric, int32_t scale_mode, int32_t steps, double grid,
+                                       int32_t patience, float norm, float expand, void* min_out, void* max_out,
+                                       void* workspace, int64_t workspace_bytes, void* stream) {
+  LLMC_CHECK_ARG(x && R > 0 && K > 0, 1);
+  int rc = check_common(dtype, fmt, num_bits, scale_mode, steps, grid, norm, expand, patience);
+  if (rc) return rc;
+  LLMC_CHECK_ARG(block_h > 0 && block_w > 0, 6);
+  const int nbr = (int)((R + block_h - 1) / block_h), nbc = (int)((K + block_w - 1) / block_w);
+  const int64_t n = (int64_t)nbr * nbc;
+  LLMC_CHECK_ARG(min_out && max_out, 17);
+  LLMC_CHECK_ARG(workspace && (((uintptr_t)workspace) & 255) == 0 && workspace_bytes >= llmc_mse_workspace_bytes(n), 19);
+  hipStream_t st = (hipStream_t)stream;
+  MseParams p;
+  p.x = x; p.dt = dtype; p.fmt = fmt; p.bits = fmt == LLMC_FMT_INT ? num_bits : (fmt == LLMC_FMT_FP8 ? 8 : 4);
+  p.symmetric = symmetric; p.scale_mode = scale_mode; p.steps = steps; p.grid = grid; p.norm = round_host(norm, dtype); p.expand = expand;
+  Workspace w;
+  rc = setup(p, w, workspace, n, st);
+  if (rc) return rc;
+  GenericLayout l = {};
+  l.mode = 1; l.R = (int)R; l.K = (int)K; l.bh = block_h; l.bw = block_w; l.nbc = nbc; l.ldw = ldw;
+  hipLaunchKernelGGL(mse_generic_kernel, dim3((unsigned)n), dim3(256), 0, st, p, l);
+  LLMC_LAUNCH_STATUS();
+  return finish(p, w, n, patience, min_out, max_out, st);
+}

@@ -252,3 +252,62 @@ def gptq_quantize(weight, U, scale, zero_point, fmt: int, bits: int, row_div: in
             _stream(weight))
     _lib.check(rc, "llmc_gptq_quantize")
     return out, loss
+
+
+def _mse_common(maxshrink, grid, patience, norm, expand):
+    steps = int(maxshrink * grid)
+    if steps > 256:
+        raise ValueError(f"MSE observer: int(maxshrink*grid)={steps} search steps exceed the supported 256")
+    return steps, float(grid), int(patience), float(norm), float(expand)
+
+
+def mse_observe_groups(w, group: int, fmt: int, bits: int, symmetric: bool, scale_mode: int = SCALE_PLAIN,
+                       maxshrink=0.20, patience=5, grid=100.0, norm=2.4, expand=1.0):
+    """MSE grid search per run of `group` columns of w [R,K] -> (min, max) [R, K/group]."""
+    _require_gpu(w)
+    assert w.ndim == 2 and w.stride(1) == 1
+    R, K = w.shape
+    steps, grid, patience, norm, expand = _mse_common(maxshrink, grid, patience, norm, expand)
+    n = R * (K // group)
+    mn = torch.empty((R, K // group), dtype=w.dtype, device=w.device)
+    mx = torch.empty_like(mn)
+    ws = _workspace(w.device, _lib.lib().llmc_mse_workspace_bytes(n))
+    with torch.cuda.device(w.device):
+        rc = _lib.lib().llmc_mse_observe_groups(
+            w.data_ptr(), _dt(w), R, K, w.stride(0), group, fmt, bits, 1 if symmetric else 0, scale_mode, steps,
+            grid, patience, norm, expand, mn.data_ptr(), mx.data_ptr(), ws.data_ptr(), ws.numel(), _stream(w))
+    _lib.check(rc, "llmc_mse_observe_groups")
+    return mn, mx
+
+
+def mse_observe_strided(x, n0: int, n1: int, group: int, s0: int, s1: int, fmt: int, bits: int, symmetric: bool,
+                        scale_mode: int = SCALE_PLAIN, maxshrink=0.20, patience=5, grid=100.0, norm=2.4, expand=1.0):
+    _require_gpu(x)
+    steps, grid, patience, norm, expand = _mse_common(maxshrink, grid, patience, norm, expand)
+    mn = torch.empty((n1,), dtype=x.dtype, device=x.device)
+    mx = torch.empty_like(mn)
+    ws = _workspace(x.device, _lib.lib().llmc_mse_workspace_bytes(n1))
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().llmc_mse_observe_strided(
+            x.data_ptr(), _dt(x), n0, n1, group, s0, s1, fmt, bits, 1 if symmetric else 0, scale_mode, steps, grid,
+            patience, norm, expand, mn.data_ptr(), mx.data_ptr(), ws.data_ptr(), ws.numel(), _stream(x))
+    _lib.check(rc, "llmc_mse_observe_strided")
+    return mn, mx
+
+
+def mse_observe_blocks(w, bh: int, bw: int, fmt: int, bits: int, symmetric: bool, scale_mode: int = SCALE_PLAIN,
+                       maxshrink=0.20, patience=5, grid=100.0, norm=2.4, expand=1.0):
+    _require_gpu(w)
+    assert w.ndim == 2 and w.stride(1) == 1
+    R, K = w.shape
+    steps, grid, patience, norm, expand = _mse_common(maxshrink, grid, patience, norm, expand)
+    shape = ((R + bh - 1) // bh, (K + bw - 1) // bw)
+    mn = torch.empty(shape, dtype=w.dtype, device=w.device)
+    mx = torch.empty_like(mn)
+    ws = _workspace(w.device, _lib.lib().llmc_mse_workspace_bytes(shape[0] * shape[1]))
+    with torch.cuda.device(w.device):
+        rc = _lib.lib().llmc_mse_observe_blocks(
+            w.data_ptr(), _dt(w), R, K, w.stride(0), bh, bw, fmt, bits, 1 if symmetric else 0, scale_mode, steps,
+            grid, patience, norm, expand, mn.data_ptr(), mx.data_ptr(), ws.data_ptr(), ws.numel(), _stream(w))
+    _lib.check(rc, "llmc_mse_observe_blocks")
+    return mn, mx
