@@ -1,0 +1,68 @@
+"""oneshot(): apply a recipe to a model with optional calibration data (reference: entrypoints/oneshot.py:316-481).
+
+Accepts an instantiated ``torch.nn.Module`` and a ready ``DataLoader`` / list of batches (the
+reference passes a DataLoader straight through, datasets/utils.py:143-144).  Loading models or
+datasets by hub name needs network access and is not part of this build.
+"""
+from __future__ import annotations
+
+import os
+from typing import Optional
+
+import torch
+
+from ..core import active_session
+from ..pipelines import CalibrationPipeline
+
+__all__ = ["Oneshot", "oneshot"]
+
+
+class _DatasetArgs:
+    def __init__(self, **kw):
+        self.__dict__.update(kw)
+
+
+class Oneshot:
+    def __init__(self, model, recipe=None, dataset=None, output_dir: Optional[str] = None, pipeline: str = "independent",
+                 sequential_targets=None, stage: Optional[str] = None, save_compressed: bool = True,
+                 moe_calibrate_all_experts: bool = True, **kwargs):
+        if isinstance(model, str):
+            raise ValueError("oneshot: pass an instantiated torch.nn.Module; loading by name is not available offline")
+        self.model = model
+        self.recipe = recipe
+        self.dataset = dataset
+        self.output_dir = output_dir
+        self.pipeline = pipeline
+        self.stage = stage
+        self.save_compressed = save_compressed
+        self.dataset_args = _DatasetArgs(sequential_targets=sequential_targets, pipeline=pipeline,
+                                         moe_calibrate_all_experts=moe_calibrate_all_experts, **kwargs)
+
+    def __call__(self):
+        self.apply_recipe_modifiers(self.dataset)
+        if self.output_dir is not None:
+            from ..compressors import save_pretrained_compressed
+
+            save_pretrained_compressed(self.model, self.output_dir, save_compressed=self.save_compressed,
+                                       recipe=active_session().lifecycle.recipe)
+        return self.model
+
+    def apply_recipe_modifiers(self, calibration_dataloader):
+        session = active_session()
+        session.reset()
+        session.initialize(model=self.model, recipe=self.recipe, recipe_stage=self.stage,
+                           calib_data=calibration_dataloader)
+        mods = session.get_modifiers()
+        user = self.pipeline
+        pipeline = CalibrationPipeline.from_modifiers(mods, user=user)
+        if calibration_dataloader is None and any(m.requires_calibration_data for m in mods):
+            raise ValueError("the recipe requires calibration data but no `dataset` was given")
+        pipeline(self.model, calibration_dataloader, self.dataset_args)
+        session.finalize()
+
+
+def oneshot(model, recipe=None, dataset=None, output_dir: Optional[str] = None, pipeline: str = "independent",
+            sequential_targets=None, stage: Optional[str] = None, save_compressed: bool = True, **kwargs):
+    """Quantise ``model`` in place according to ``recipe`` and return it; save when ``output_dir`` is given."""
+    return Oneshot(model=model, recipe=recipe, dataset=dataset, output_dir=output_dir, pipeline=pipeline,
+                   sequential_targets=sequential_targets, stage=stage, save_compressed=save_compressed, **kwargs)()

@@ -1,0 +1,212 @@
+"""GPTQModifier (reference: modifiers/gptq/base.py:47-399).
+
+Same fields and lifecycle as the reference.  One MI355X-specific addition: the forward hook
+stages calibration batches and accumulates several of them with one Hessian launch
+(``hessian_batch_tokens``), which amortises the read-modify-write of the [K,K] accumulator;
+the sum over tokens is unchanged up to fp32 summation order.
+"""
+from __future__ import annotations
+
+import contextlib
+import logging
+
+import torch
+from pydantic import PrivateAttr
+
+from ... import ops
+from ...core import Event, State
+from ...observers import ACTIVATION_OBS
+from ...quantization import (
+    ActivationOrdering,
+    QuantizationConfig,
+    QuantizationScheme,
+    QuantizationStrategy,
+    getattr_chain,
+    is_module_quantized,
+    match_named_modules,
+    update_offload_parameter,
+)
+from ...sentinel import Sentinel
+from ...utils.metric_logging import CompressionLogger
+from ..modifier import Modifier
+from ..quantization.calibration import observe, update_qparams
+from ..quantization.quantization import QuantizationMixin
+from .gptq_quantize import accumulate_hessian, make_empty_hessian, quantize_weight
+
+logger = logging.getLogger("llmcompressor_amd")
+
+__all__ = ["GPTQModifier"]
+
+_GPTQ_Q_PARAMS = ["weight", "weight_scale", "weight_zero_point", "weight_g_idx"]
+
+
+class GPTQModifier(Modifier, QuantizationMixin):
+    """GPTQ (https://arxiv.org/abs/2210.17323): calibrate a Hessian per targeted Linear with forward
+    hooks, then quantise the weight column by column with error feedback.
+
+    :param block_size: number of columns compressed in one pass
+    :param dampening_frac: dampening applied to H, as a fraction of the diagonal mean
+    :param actorder: column order; defaults to "static" (quantise in descending diag(H) order, no g_idx)
+    :param offload_hessians: keep Hessians on the CPU between hook calls
+    :param hessian_batch_tokens: stage activations and launch the Hessian kernel once this many tokens
+        are pending (0 = one launch per hook call, the reference's behaviour)
+    """
+
+    requires_calibration_data: bool = True
+
+    block_size: int = 128
+    dampening_frac: float | None = 0.01
+    actorder: ActivationOrdering | Sentinel | None = Sentinel("static")
+    offload_hessians: bool = False
+    hessian_batch_tokens: int = 0
+
+    _module_names: dict = PrivateAttr(default_factory=dict)
+    _hessians: dict = PrivateAttr(default_factory=dict)
+    _num_samples: dict = PrivateAttr(default_factory=dict)
+    _staged: dict = PrivateAttr(default_factory=dict)
+
+    def resolve_quantization_config(self) -> QuantizationConfig:
+        config = super().resolve_quantization_config()
+
+        def resolve_actorder(existing):
+            if self.actorder == Sentinel("static"):
+                return ActivationOrdering.STATIC if existing is None else existing
+            if existing is None or self.actorder == existing:
+                return self.actorder
+            raise ValueError(
+                "Cannot resolve activation ordering when both `GPTQModifier.actorder` and "
+                f"`QuantizationScheme.actorder` are provided and differ ({self.actorder}, {existing}). "
+                "Either unset `GPTQModifier.actorder` or remove `actorder` from config groups.")
+
+        grouped = (QuantizationStrategy.GROUP, QuantizationStrategy.TENSOR_GROUP)
+        for scheme in config.config_groups.values():
+            assert isinstance(scheme, QuantizationScheme)
+            strategy = getattr_chain(scheme, "weights.strategy", None)
+            if strategy in (QuantizationStrategy.GROUP, QuantizationStrategy.TENSOR_GROUP,
+                            QuantizationStrategy.CHANNEL, QuantizationStrategy.TENSOR, QuantizationStrategy.BLOCK):
+                scheme.weights.actorder = resolve_actorder(scheme.weights.actorder)
+                if scheme.weights.actorder == ActivationOrdering.GROUP:
+                    logger.warning("ActivationOrdering.GROUP is deprecated and will be removed in a future "
+                                   "release. Use default actorder='static' instead. ")
+                    if strategy not in grouped:
+                        logger.warning(f"ActivationOrdering.GROUP is not compatible with strategy={strategy}; "
+                                       "falling back to actorder=None for this scheme.")
+                        scheme.weights.actorder = None
+        return config
+
+    def on_initialize(self, state: State, **kwargs) -> bool:
+        if QuantizationMixin.has_config(self):
+            QuantizationMixin.initialize_quantization(self, state.model)
+        self._module_names = {m: name for name, m in match_named_modules(state.model, self.resolved_targets,
+                                                                         self.ignore)}
+        return True
+
+    def on_calibration_start(self, state: State, event: Event, **kwargs):
+        QuantizationMixin.start_calibration(self, state.model)
+        added_hook = False
+        for _, module in match_named_modules(state.model, self.resolved_targets, self.ignore):
+            if getattr_chain(module, "quantization_scheme.weights", None) is not None:
+                if not isinstance(module, torch.nn.Embedding):
+                    self.register_hook(module, self.calibrate_module, "forward")
+                    added_hook = True
+        if not added_hook:
+            raise ValueError("GPTQModifier was unable to find any modules to quantize. Please check quantization "
+                             "`config_groups` and `targets` in recipe")
+
+    def on_sequential_epoch_end(self, state: State, event: Event, modules: list[torch.nn.Module] = (), **kwargs):
+        modules = [m for m in modules if is_module_quantized(m)]
+        observe(modules, base_name="weight")
+        self.sync_obs_act_stats(modules)
+        update_qparams(modules, ACTIVATION_OBS)
+        self.compress_modules()
+
+    def on_calibration_end(self, state: State, event: Event, **kwargs):
+        QuantizationMixin.end_calibration(self, state.model)
+        self.remove_hooks()
+
+    def calibrate_module(self, module: torch.nn.Module, args: tuple[torch.Tensor, ...], _output: torch.Tensor):
+        """Forward hook: accumulate the Hessian of the module's input."""
+        inp = args[0]
+        if module not in self._num_samples:
+            device = inp.device if inp.is_cuda else module.weight.device
+            init_device = "cpu" if self.offload_hessians else device
+            self._hessians[module] = make_empty_hessian(module, device=init_device)
+            self._num_samples[module] = torch.zeros(tuple(), device=device)
+        if self.hessian_batch_tokens > 0 and not self.offload_hessians and isinstance(module, torch.nn.Linear):
+            self._stage(module, inp)
+            return
+        with self._maybe_onload_hessian(module):
+            self._hessians[module], self._num_samples[module] = accumulate_hessian(
+                inp, module, self._hessians[module], self._num_samples[module])
+
+    # -- token staging (see the class docstring)
+    def _stage(self, module, inp):
+        if inp.ndim == 2:
+            inp = inp.unsqueeze(0)
+        elif inp.ndim > 3:
+            inp = inp.reshape(inp.shape[0], -1, inp.shape[-1])
+        self._num_samples[module] += inp.shape[0]
+        rows = inp.reshape(-1, inp.shape[-1])
+        st = self._staged.get(module)
+        cap = max(self.hessian_batch_tokens, rows.shape[0])
+        if st is None or st[0].shape[0] < cap or st[0].dtype != rows.dtype:
+            if st is not None:
+                self._flush(module)
+            st = [torch.empty((cap, rows.shape[1]), dtype=rows.dtype, device=rows.device), 0]
+            self._staged[module] = st
+        if st[1] + rows.shape[0] > st[0].shape[0]:
+            self._flush(module)
+        st[0][st[1]: st[1] + rows.shape[0]].copy_(rows)
+        st[1] += rows.shape[0]
+        if st[1] >= self.hessian_batch_tokens:
+            self._flush(module)
+
+    def _flush(self, module):
+        st = self._staged.get(module)
+        if st is None or st[1] == 0:
+            return
+        ops.hessian_accumulate_(self._hessians[module], st[0][: st[1]], alpha=2.0, assume_symmetric=True)
+        st[1] = 0
+
+    def compress_modules(self):
+        self.compress_module_list(list(self._num_samples.keys()))
+
+    def compress_module_list(self, module_list):
+        for module in module_list:
+            name = self._module_names.get(module, module.__class__.__name__)
+            self._flush(module)
+            self._staged.pop(module, None)
+            num_samples = self._num_samples[module]
+            quant_args = getattr_chain(module, "quantization_scheme.weights")
+            logger.info(f"Quantizing {name} using {int(num_samples)} samples")
+            with torch.no_grad(), self._maybe_onload_hessian(module), CompressionLogger(module) as comp_logger:
+                loss, q_param_dict = quantize_weight(
+                    module=module,
+                    quant_args=quant_args,
+                    hessian=self._hessians.pop(module),
+                    blocksize=self.block_size,
+                    percdamp=self.dampening_frac,
+                    hessian_divisor=float(self._num_samples.pop(module).item()),
+                )
+                comp_logger.set_results(name="GPTQ", loss=loss)
+            for attr, val in q_param_dict.items():
+                update_offload_parameter(module, attr, val)
+
+    def on_finalize(self, state: State, **kwargs) -> bool:
+        if not self.ended_:
+            self.on_end(state, None)
+        if len(self._num_samples) > 0:
+            raise ValueError(f"Failed to compress {len(self._num_samples)} modules")
+        self._hessians = dict()
+        self._num_samples = dict()
+        self._staged = dict()
+        return True
+
+    @contextlib.contextmanager
+    def _maybe_onload_hessian(self, module: torch.nn.Module):
+        if self.offload_hessians:
+            self._hessians[module] = self._hessians[module].to(device=module.weight.device)
+        yield
+        if self.offload_hessians:
+            if module in self._hessians:
+                self._hessians[module] = self._hessians[module].to(device="cpu")

@@ -1,0 +1,153 @@
+"""GPTQ numerics behind the reference's function seams (modifiers/gptq/gptq_quantize.py).
+
+``make_empty_hessian`` (:19-25), ``accumulate_hessian`` (:28-64) and ``quantize_weight``
+(:67-264) keep their names, arguments, return values and error behaviour; the work is done
+by the HIP kernels: ``llmc_hessian_accumulate`` (MFMA SYRK), ``llmc_gptq_hinv`` (damped
+Cholesky chain, identity fallback on a non-positive pivot) and ``llmc_gptq_quantize``
+(block column loop + MFMA trailing updates).
+"""
+from __future__ import annotations
+
+import logging
+import math
+
+import torch
+
+from ... import ops
+from ...quantization import ActivationOrdering, QuantizationArgs, QuantizationStrategy
+from ...quantization.lifecycle import effective_scale, kernel_format
+
+logger = logging.getLogger("llmcompressor_amd")
+
+GPTQ_PRECISION = torch.float32
+
+__all__ = ["make_empty_hessian", "accumulate_hessian", "quantize_weight", "quantize_weight_tensors"]
+
+
+def make_empty_hessian(module: torch.nn.Module, device: torch.device | None = None) -> torch.Tensor:
+    weight = module.weight
+    num_columns = weight.shape[1]
+    device = device if device is not None else weight.device
+    return torch.zeros((num_columns, num_columns), device=device, dtype=GPTQ_PRECISION)
+
+
+def accumulate_hessian(inp: torch.Tensor, module: torch.nn.Module, H: torch.Tensor | None,
+                       num_samples: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """H += 2 X^T X in place; num_samples += batch entries (not tokens)."""
+    inp = inp.to(device=H.device)
+    if len(inp.shape) == 2:
+        inp = inp.unsqueeze(0)
+    elif len(inp.shape) > 3:
+        inp = inp.reshape(inp.shape[0], -1, inp.shape[-1])
+    num_added = inp.shape[0]
+    if isinstance(module, torch.nn.Conv2d):
+        unfold = torch.nn.Unfold(module.kernel_size, dilation=module.dilation, padding=module.padding,
+                                 stride=module.stride)
+        inp = unfold(inp).permute([1, 0, 2]).flatten(1).t()
+    else:  # Linear / Conv1D: rows are tokens
+        inp = inp.reshape((-1, inp.shape[-1]))
+    num_samples += num_added
+    if inp.dtype == torch.float32:
+        # the matrix cores take 16-bit operands; an fp32 activation is split into a bf16 head and
+        # tail, (h + t)^T (h + t) = h^T h + h^T t + t^T h + t^T t, accumulated in fp32
+        raise TypeError("accumulate_hessian: fp32 activations are not supported by this build; "
+                        "calibrate in bf16 or fp16")
+    if inp.shape[0] > 0:
+        ops.hessian_accumulate_(H, inp.contiguous(), alpha=2.0, assume_symmetric=True)
+    return H, num_samples
+
+
+def _scale_layout(strategy, quant_args: QuantizationArgs, num_rows: int, num_columns: int):
+    """(row_div, scale_row_stride, base g_idx or None) of llmc_gptq_quantize."""
+    S = QuantizationStrategy
+    if strategy == S.TENSOR:
+        return 1 << 40, 0, None
+    if strategy == S.CHANNEL:
+        return 1, 1, None
+    if strategy in (S.GROUP, S.TENSOR_GROUP):
+        return 1, math.ceil(num_columns / quant_args.group_size), quant_args.group_size
+    if strategy == S.BLOCK:
+        bh, bw = quant_args.block_structure
+        return bh, math.ceil(num_columns / bw), bw
+    raise ValueError(f"Quantization strategy is not supported for GPTQ: {strategy}")
+
+
+def quantize_weight_tensors(weight: torch.Tensor, observer, quant_args: QuantizationArgs, hessian: torch.Tensor,
+                            blocksize: int = 128, percdamp: float = 0.01, hessian_divisor: float = 1.0):
+    """quantize_weight on bare tensors: ``weight`` [R,K], ``observer`` holding its statistics.
+
+    ``hessian_divisor`` folds the caller's ``H / num_samples`` into the factorisation's first pass."""
+    strategy = quant_args.strategy
+    actorder = quant_args.actorder
+    final_shape, final_dtype = weight.shape, weight.dtype
+    W2 = weight.reshape(weight.shape[0], -1) if weight.ndim != 2 else weight
+    if not W2.is_contiguous():
+        W2 = W2.contiguous()
+    num_rows, num_columns = W2.shape
+    H = hessian
+
+    if actorder == ActivationOrdering.GROUP and strategy not in (QuantizationStrategy.GROUP,
+                                                                 QuantizationStrategy.TENSOR_GROUP):
+        logger.warning("ActivationOrdering.GROUP requires a grouped quantization strategy; "
+                       "falling back to actorder=None for this module.")
+        actorder = None
+
+    perm = None
+    if actorder:
+        perm = torch.argsort(torch.diagonal(H), descending=True)
+    if actorder == ActivationOrdering.GROUP:
+        # re-observe the permuted weight so that groups are runs of the permuted columns
+        observer.delete_statistics(check_fused=False)
+        observer(W2[:, perm].contiguous())
+
+    row_div, srow, divisor = _scale_layout(strategy, quant_args, num_rows, num_columns)
+    g_idx = None
+    if divisor is not None:
+        g_idx = torch.arange(num_columns, device=W2.device, dtype=torch.int) // divisor
+        if actorder == ActivationOrdering.WEIGHT:
+            g_idx = g_idx[perm]
+
+    qparams = observer.get_qparams()
+    scale, zero_point, global_scale = qparams["scale"], qparams["zero_point"], qparams["global_scale"]
+
+    # dead columns, damping, Cholesky -> inverse -> upper factor; identity on failure
+    U, dead, info = ops.gptq_hinv_(H, perm, divisor=float(hessian_divisor), percdamp=percdamp)
+
+    fmt, bits = kernel_format(quant_args)
+    zp = None if quant_args.symmetric else zero_point.to(torch.int8)
+    kscale = effective_scale(scale, quant_args, final_dtype)
+    Wq, loss = ops.gptq_quantize(W2, U, kscale, zp, fmt, bits, row_div, srow, g_idx=g_idx, perm=perm, dead=dead,
+                                 global_scale=global_scale, blocksize=blocksize)
+    if int(info.item()) != 0:
+        logger.warning("Failed to invert hessian due to numerical instability. Consider increasing "
+                       "GPTQModifier.dampening_frac, increasing the number of calibration samples, or shuffling "
+                       "the calibration dataset. Falling back to round-to-nearest for this module.")
+    W = Wq.reshape(final_shape)
+    q_param_dict = {
+        "weight": W,
+        "weight_scale": scale if scale.dtype in (torch.uint8, torch.float8_e4m3fn) else scale.to(dtype=final_dtype),
+        "weight_zero_point": zero_point.to(dtype=quant_args.zp_dtype),
+    }
+    if quant_args.scale_dtype == torch.float8_e4m3fn and scale.dtype == torch.float32:
+        q_param_dict["weight_scale"] = scale  # e4m3-grid values; stored as float8 by the parameter
+    if global_scale is not None:
+        q_param_dict["weight_global_scale"] = global_scale.to(dtype=final_dtype)
+    if actorder == ActivationOrdering.GROUP:
+        invperm = torch.argsort(perm)
+        q_param_dict["weight_g_idx"] = g_idx[invperm]
+    return loss.item(), q_param_dict
+
+
+def quantize_weight(module: torch.nn.Module, quant_args: QuantizationArgs, hessian: torch.Tensor,
+                    blocksize: int = 128, percdamp: float = 0.01, hessian_divisor: float = 1.0) -> tuple[float, dict]:
+    """Quantize a module weight according to the GPTQ algorithm.
+
+    :param module: module with weight being quantized (must carry ``weight_observer`` with statistics)
+    :param quant_args: quantization arguments used to find quantization parameters
+    :param hessian: preaccumulated hessian for quantization (consumed)
+    :param blocksize: chunk size of quantization updates
+    :param percdamp: dampening factor on hessian diagonal
+    :return: loss, dict of weight / weight_scale / weight_zero_point [/ weight_global_scale / weight_g_idx]
+    """
+    return quantize_weight_tensors(module.weight.data, module.weight_observer, quant_args, hessian, blocksize,
+                                   percdamp, hessian_divisor)

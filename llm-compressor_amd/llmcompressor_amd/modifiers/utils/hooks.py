@@ -1,0 +1,54 @@
+"""Hook registration with a global disable switch (reference: modifiers/utils/hooks.py:19-133)."""
+from __future__ import annotations
+
+import contextlib
+from functools import wraps
+from typing import Any, Callable, ClassVar
+
+import torch
+from pydantic import BaseModel, PrivateAttr
+from torch.utils.hooks import RemovableHandle
+
+__all__ = ["HooksMixin"]
+
+
+class HooksMixin(BaseModel):
+    _HOOKS_DISABLED: ClassVar[bool] = False
+    _HOOKS_KEEP_ENABLED: ClassVar[set] = set()
+
+    _hooks: set = PrivateAttr(default_factory=set)
+
+    @classmethod
+    @contextlib.contextmanager
+    def disable_hooks(cls, keep: set = frozenset()):
+        """Disable all hooks across all modifiers, except the handles in ``keep``."""
+        try:
+            HooksMixin._HOOKS_DISABLED = True
+            HooksMixin._HOOKS_KEEP_ENABLED |= set(keep)
+            yield
+        finally:
+            HooksMixin._HOOKS_DISABLED = False
+            HooksMixin._HOOKS_KEEP_ENABLED -= set(keep)
+
+    def register_hook(self, target: torch.nn.Module | torch.nn.Parameter, hook: Callable[[Any], Any], hook_type: str,
+                      **kwargs) -> RemovableHandle:
+        handle = None
+
+        @wraps(hook)
+        def wrapped_hook(*args, **kw):
+            if HooksMixin._HOOKS_DISABLED and handle not in HooksMixin._HOOKS_KEEP_ENABLED:
+                return
+            return hook(*args, **kw)
+
+        name = f"register_{hook_type}_hook" if hook_type else "register_hook"
+        register = getattr(target, name)
+        handle = register(wrapped_hook, **kwargs)
+        self._hooks.add(handle)
+        return handle
+
+    def remove_hooks(self, handles: set | None = None):
+        if handles is None:
+            handles = self._hooks
+        for h in list(handles):
+            h.remove()
+        self._hooks -= set(handles)

@@ -1,0 +1,281 @@
+"""Host-side mirror of the reference interface: argument resolution, recipes, hooks, registry, C ABI surface.
+
+Runs without a GPU.  Cases follow the reference's own unit tests (cited per test)."""
+import ctypes
+import os
+import re
+from contextlib import nullcontext
+
+import pytest
+import torch
+
+from llmcompressor_amd import _lib
+from llmcompressor_amd.compressors import CompressionFormat, infer_format
+from llmcompressor_amd.modifiers.gptq import GPTQModifier
+from llmcompressor_amd.modifiers.quantization import QuantizationModifier
+from llmcompressor_amd.modifiers.utils.hooks import HooksMixin
+from llmcompressor_amd.observers import Observer, flatten_for_calibration
+from llmcompressor_amd.quantization import (
+    QuantizationArgs,
+    QuantizationScheme,
+    initialize_module_for_quantization,
+    preset_name_to_scheme,
+)
+from llmcompressor_amd.recipe import Recipe
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_c_abi_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "llmc_amd.h")).read()
+    declared = set(re.findall(r"\b(llmc_[a-z0-9_]+)\s*\(", header))
+    assert len(declared) >= 15
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    missing = [n for n in sorted(declared) if not hasattr(lib, n)]
+    assert not missing, missing
+    assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
+    assert lib.llmc_version() >= 1
+
+
+def test_ops_refuse_cpu_tensors_instead_of_falling_back():
+    from llmcompressor_amd import ops
+
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ops.hessian_accumulate_(torch.zeros(8, 8), torch.zeros(4, 8, dtype=torch.bfloat16))
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ops.minmax_groups(torch.zeros(4, 8), 8)
+
+
+def _q_config_kwargs(config_0, config_1):
+    def grp(actorder):
+        return dict(targets=["Linear"], input_activations=dict(num_bits=8, symmetric=False, strategy="tensor"),
+                    weights=dict(num_bits=4, symmetric=True, strategy="group", group_size=128, actorder=actorder))
+
+    return dict(config_groups=dict(group_0=grp(config_0), group_1=grp(config_1)))
+
+
+@pytest.mark.parametrize(
+    "has_actorder,actorder,config_0,config_1,expected_0,expected_1",
+    [
+        (False, "N/A", None, None, "static", "static"),
+        (True, "static", None, None, "static", "static"),
+        (True, "group", None, None, "group", "group"),
+        (True, None, None, None, None, None),
+        (True, "group", None, "group", "group", "group"),
+        (True, "group", "group", None, "group", "group"),
+        (True, "static", None, "group", "error", "error"),
+        (True, "static", "group", None, "error", "error"),
+        (True, "group", None, "static", "error", "error"),
+        (True, "group", "static", None, "error", "error"),
+        (True, None, "static", None, "error", "error"),
+        (False, "N/A", None, "static", "static", "static"),
+        (False, "N/A", "static", None, "static", "static"),
+        (False, "N/A", "static", "static", "static", "static"),
+        (False, "N/A", None, "group", "static", "group"),
+        (False, "N/A", "group", None, "group", "static"),
+        (False, "N/A", "group", "group", "group", "group"),
+    ],
+)
+def test_actorder_resolution(has_actorder, actorder, config_0, config_1, expected_0, expected_1):
+    # reference: tests/llmcompressor/modifiers/gptq/test_base.py:60-113
+    kwargs = _q_config_kwargs(config_0, config_1)
+    with pytest.raises(ValueError) if expected_0 == "error" else nullcontext():
+        modifier = GPTQModifier(**kwargs, actorder=actorder) if has_actorder else GPTQModifier(**kwargs)
+        resolved = modifier.resolve_quantization_config()
+    if expected_0 != "error":
+        assert resolved.config_groups["group_0"].input_activations.actorder is None
+        assert resolved.config_groups["group_0"].weights.actorder == expected_0
+        assert resolved.config_groups["group_1"].input_activations.actorder is None
+        assert resolved.config_groups["group_1"].weights.actorder == expected_1
+
+
+def test_block_strategy_parsing_and_group_fallback():
+    m = GPTQModifier(config_groups=dict(group_block=dict(
+        targets=["Linear"], weights=dict(num_bits=8, symmetric=True, strategy="block", block_structure=[128, 128]))))
+    w = m.resolve_quantization_config().config_groups["group_block"].weights
+    assert w.strategy == "block" and w.block_structure == [128, 128]
+    # actorder=group on an ungrouped strategy falls back to None
+    m = GPTQModifier(actorder="group", config_groups=dict(g=dict(targets=["Linear"], weights=dict(strategy="channel"))))
+    assert m.resolve_quantization_config().config_groups["g"].weights.actorder is None
+
+
+def test_scheme_targets_and_serialisation():
+    m = GPTQModifier(targets="Linear", scheme="W4A16", ignore=["lm_head"])
+    cfg = m.resolve_quantization_config()
+    w = cfg.config_groups["group_0"].weights
+    assert (w.num_bits, w.group_size, w.symmetric, str(w.strategy.value)) == (4, 128, True, "group")
+    assert m.resolved_targets == {"Linear"}
+    assert m.model_dump()["actorder"] == "static"
+    assert GPTQModifier(actorder=None).model_dump()["actorder"] is None
+    with pytest.raises(ValueError):
+        GPTQModifier(scheme="NOT_A_SCHEME")
+    with pytest.raises(ValueError):
+        GPTQModifier(scheme="W4A16", config_groups={"g": dict(targets=["Linear"])}).resolve_quantization_config()
+    with pytest.raises(Exception):
+        GPTQModifier(not_a_field=1)  # extra="forbid"
+    assert GPTQModifier(scheme="W4A16").requires_calibration_data
+    assert not QuantizationModifier(scheme="FP8_DYNAMIC").requires_calibration_data
+    assert QuantizationModifier(scheme="FP8").requires_calibration_data  # static activation scales
+
+
+def test_observer_overrides():
+    m = QuantizationModifier(scheme="W4A16", weight_observer="mse")
+    assert m.resolved_config.config_groups["group_0"].weights.observer == "mse"
+    with pytest.raises(ValueError):
+        QuantizationModifier(scheme="W4A16", weight_observer="mse", observer={"weights": "minmax"}).resolved_config
+
+
+def test_recipe_round_trip_and_factory():
+    # reference: tests/llmcompressor/recipe/test_recipe.py:21-72
+    text = """
+    test_stage:
+      quant_modifiers:
+        GPTQModifier:
+          block_size: 64
+          dampening_frac: 0.001
+          actorder: static
+          config_groups:
+            group_0:
+              targets: [Linear]
+              weights: {num_bits: 4, type: int, symmetric: true, strategy: group, group_size: 128}
+        QuantizationModifier:
+          targets: [Linear]
+          scheme: FP8_DYNAMIC
+    """
+    r = Recipe.create_instance(text)
+    assert [type(m).__name__ for m in r.modifiers] == ["GPTQModifier", "QuantizationModifier"]
+    assert r.modifiers[0].block_size == 64 and r.modifiers[0].group == "quant"
+    r2 = Recipe.create_instance(r.yaml())
+    assert r2.dict() == r.dict()
+    r3 = Recipe.create_instance([GPTQModifier(scheme="W4A16")])
+    assert Recipe.create_instance(r3.yaml()).modifiers[0].scheme == "W4A16"
+    with pytest.raises(ValueError):
+        Recipe.create_instance("test_stage:\n  x_modifiers:\n    NoSuchModifier: {}\n")
+
+
+class _Dummy(HooksMixin):
+    pass
+
+
+def test_hooks_register_remove_disable_keep():
+    # reference: tests/llmcompressor/modifiers/utils/test_hooks.py:40-120
+    lin_a, lin_b = torch.nn.Linear(4, 4), torch.nn.Linear(4, 4)
+    mod_a, mod_b = _Dummy(), _Dummy()
+    calls = []
+    ha = mod_a.register_hook(lin_a, lambda *a: calls.append("a"), "forward")
+    hb = mod_b.register_hook(lin_b, lambda *a: calls.append("b"), "forward_pre")
+    x = torch.zeros(1, 4)
+    lin_a(x), lin_b(x)
+    assert calls == ["a", "b"]
+    with HooksMixin.disable_hooks():
+        lin_a(x), lin_b(x)
+    assert calls == ["a", "b"]
+    with HooksMixin.disable_hooks(keep={hb}):
+        lin_a(x), lin_b(x)
+    assert calls == ["a", "b", "b"]
+    mod_a.remove_hooks()
+    lin_a(x), lin_b(x)
+    assert calls == ["a", "b", "b", "b"]
+    mod_b.remove_hooks({hb})
+    lin_b(x)
+    assert calls == ["a", "b", "b", "b"]
+    assert ha not in mod_a._hooks
+
+
+@pytest.mark.parametrize(
+    "args",
+    [
+        QuantizationArgs(strategy="tensor"),
+        QuantizationArgs(strategy="channel"),
+        QuantizationArgs(strategy="group", group_size=4),
+        QuantizationArgs(strategy="tensor_group", group_size=4),
+        QuantizationArgs(strategy="block", block_structure=[5, 4]),
+        QuantizationArgs(strategy="block", block_structure=[3, 3]),
+    ],
+)
+def test_flatten_for_calibration_weights_matches_param_shapes(args):
+    # reference: tests/llmcompressor/observers/test_helpers.py:37-59
+    module = torch.nn.Linear(8, 10)
+    initialize_module_for_quantization(module, QuantizationScheme(targets=[], weights=args))
+    flat = flatten_for_calibration(module.weight, "weight", args)
+    assert flat.shape[1:-1] == module.weight_scale.shape
+    assert flat.shape[1:-1] == module.weight_zero_point.shape
+
+
+@pytest.mark.parametrize("args", [QuantizationArgs(strategy="tensor"), QuantizationArgs(strategy="tensor_group", group_size=4)])
+def test_flatten_for_calibration_input(args):
+    module = torch.nn.Linear(8, 10)
+    initialize_module_for_quantization(module, QuantizationScheme(targets=[], input_activations=args))
+    flat = flatten_for_calibration(torch.empty((3, 5, 8)), "input", args)
+    assert flat.shape[1:-1] == module.input_scale.shape
+
+
+def test_flatten_errors_match_reference_messages():
+    w = torch.empty(4, 8)
+    with pytest.raises(ValueError, match="Token quantization cannot be applied to weights"):
+        flatten_for_calibration(w, "weight", QuantizationArgs(strategy="token"))
+    with pytest.raises(ValueError, match="Channel quantization cannot be applied to activations"):
+        flatten_for_calibration(w, "input", QuantizationArgs(strategy="channel"))
+    with pytest.raises(ValueError, match="Unknown quantization base name"):
+        flatten_for_calibration(w, "bogus", QuantizationArgs())
+
+
+def test_observer_registry_names():
+    for name, cls in [("memoryless_minmax", "MemorylessMinMaxObserver"), ("static_minmax", "StaticMinMaxObserver"),
+                      ("minmax", "MinMaxObserver"), ("memoryless_mse", "MemorylessMSEObserver"),
+                      ("mse", "MovingAverageMSEObserver"), ("nvfp4_expanded_mse", "NVFP4ExpandedMSEObserver")]:
+        obs = Observer.load_from_registry(name, base_name="weight", args=QuantizationArgs())
+        assert type(obs).__name__ == cls
+    with pytest.raises(AssertionError, match="No statistics available"):
+        Observer.load_from_registry("minmax", base_name="weight", args=QuantizationArgs()).get_qparams()
+    with pytest.raises(ValueError):
+        Observer.load_from_registry("mse", base_name="weight", args=QuantizationArgs(), expand=0.5)
+
+
+def test_group_size_validation_error():
+    from llmcompressor_amd.core import State
+
+    model = torch.nn.Sequential(torch.nn.Linear(200, 16))
+    m = QuantizationModifier(scheme="W4A16")
+    with pytest.raises(ValueError, match="not divisible by group_size"):
+        m.on_initialize(State(model=model))
+    QuantizationModifier(scheme="W4A16", bypass_divisibility_checks=True).on_initialize(State(model=torch.nn.Sequential(torch.nn.Linear(200, 16))))
+
+
+@pytest.mark.parametrize(
+    "preset,fmt",
+    [("W8A8", CompressionFormat.int_quantized), ("W4A16", CompressionFormat.pack_quantized),
+     ("W8A16", CompressionFormat.pack_quantized), ("FP8", CompressionFormat.float_quantized),
+     ("FP8_DYNAMIC", CompressionFormat.float_quantized), ("NVFP4A16", CompressionFormat.nvfp4_pack_quantized),
+     ("NVFP4", CompressionFormat.nvfp4_pack_quantized), ("MXFP4A16", CompressionFormat.mxfp4_pack_quantized)],
+)
+def test_format_inference(preset, fmt):
+    # reference: tests/llmcompressor/transformers/compression/test_compress_tensor_utils.py:289-325
+    assert infer_format(preset_name_to_scheme(preset, ["Linear"])) == fmt
+    w8a16_float = QuantizationScheme(targets=["Linear"], weights=QuantizationArgs(num_bits=8, type="float"))
+    assert infer_format(w8a16_float) == CompressionFormat.naive_quantized
+
+
+def test_moe_token_routing_counts():
+    # reference: tests/llmcompressor/modeling/test_linear_experts.py:12-106 (hidden 16, inter 32, 4 experts, top-2)
+    from llmcompressor_amd.modeling import LinearExperts2D, moe_calibration_context
+
+    torch.manual_seed(0)
+    E, H, I, T, k = 4, 16, 32, 16, 2
+    experts = LinearExperts2D.from_fused(torch.randn(E, 2 * I, H), torch.randn(E, H, I))
+    x = torch.randn(T, H)
+    idx = torch.stack([torch.arange(T) % E, (torch.arange(T) + 1) % E], dim=1)
+    wts = torch.full((T, k), 0.5)
+    counts = {}
+    for e, ex in enumerate(experts):
+        ex.gate_proj.register_forward_hook(lambda m, a, o, e=e: counts.__setitem__(e, a[0].shape[0]))
+    out_routed = experts(x, idx, wts)
+    assert counts == {0: 8, 1: 8, 2: 8, 3: 8}
+    with moe_calibration_context():
+        out_all = experts(x, idx, wts)
+    assert counts == {0: 16, 1: 16, 2: 16, 3: 16}
+    assert torch.allclose(out_routed, out_all, atol=1e-5)
+    # an expert without tokens is still called (with an empty batch)
+    counts.clear()
+    experts(x, torch.zeros(T, k, dtype=torch.long), wts)
+    assert counts == {0: 32, 1: 0, 2: 0, 3: 0}  # both top-k slots of every token point at expert 0
