@@ -1,0 +1,375 @@
+"""GPU: the reference-shaped Python interface end to end on the HIP kernels.
+
+Cases follow the reference's own tests (goldens from tests/golden/reference_vectors.json)."""
+import json
+import os
+
+import pytest
+import torch
+
+from oracle import gptq as G
+from oracle import observers as O
+from oracle import qformat as F
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+
+
+def _imports():
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier, accumulate_hessian, make_empty_hessian, quantize_weight
+    from llmcompressor_amd.modifiers.quantization import QuantizationModifier
+    from llmcompressor_amd.modifiers.quantization.calibration import initialize_observer, observe, update_qparams
+    from llmcompressor_amd.observers import Observer
+    from llmcompressor_amd.quantization import (QuantizationArgs, QuantizationScheme, QuantizationStatus, fake_quantize,
+                                                forward_quantize, initialize_module_for_quantization)
+    return locals()
+
+
+def _qargs(d):
+    from llmcompressor_amd.quantization import QuantizationArgs
+
+    return QuantizationArgs(**d)
+
+
+@pytest.mark.parametrize("idx", range(5))
+def test_static_weight_quantization_goldens(golden, idx):
+    # reference: tests/llmcompressor/modifiers/calibration/test_lifecycle.py:16-165
+    L = _imports()
+    case = golden["lifecycle_weight"]["cases"][idx]
+    args = _qargs(case["args"])
+    linear = torch.nn.Linear(6, 4, bias=False).to(DEV)
+    linear.weight.data = torch.arange(24, dtype=torch.bfloat16, device=DEV).reshape(4, 6)
+    scheme = L["QuantizationScheme"](targets=[], weights=args)
+    L["initialize_module_for_quantization"](linear, scheme)
+    assert linear.quantization_scheme is scheme
+    L["initialize_observer"](linear, "weight")
+    linear.weight_observer(linear.weight)
+    mn, mx = linear.weight_observer.min_vals.clone(), linear.weight_observer.max_vals.clone()
+    qp = linear.weight_observer.get_qparams()
+    assert torch.equal(mn.cpu().float(), torch.tensor(case["min"], dtype=torch.float32))
+    assert torch.equal(mx.cpu().float(), torch.tensor(case["max"], dtype=torch.float32))
+    out = L["fake_quantize"](linear.weight.data, qp["scale"], qp["zero_point"], args, global_scale=qp["global_scale"])
+    exp = torch.tensor(case["quant"], dtype=torch.float32).to(torch.bfloat16)
+    assert torch.equal(out.cpu().to(torch.bfloat16), exp)
+    assert torch.nn.functional.mse_loss(out.float().cpu(), linear.weight.data.float().cpu()) <= case["loss"]
+
+
+def test_static_activation_tensor_golden_through_hooks(golden):
+    # reference: test_lifecycle.py:168-273 (int4 tensor activations, identity weight)
+    L = _imports()
+    case = golden["lifecycle_activation"]["cases"][0]
+    args = _qargs(case["args"])
+    x = torch.arange(12, dtype=torch.bfloat16, device=DEV).reshape(1, 2, 6)
+    linear = torch.nn.Linear(6, 6, bias=False).to(DEV)
+    linear.weight.data = torch.eye(6, dtype=torch.bfloat16, device=DEV)
+    L["initialize_module_for_quantization"](linear, L["QuantizationScheme"](targets=[], input_activations=args))
+    L["initialize_observer"](linear, "input")
+    linear.input_observer(x)
+    assert linear.input_observer.min_vals.item() == 0.0 and linear.input_observer.max_vals.item() == 11.0
+    L["update_qparams"](linear, "input")
+    linear.quantization_status = L["QuantizationStatus"].FROZEN
+    out = linear(x)
+    assert torch.equal(out.cpu(), torch.tensor(case["quant"]).to(torch.bfloat16))
+
+
+def test_observer_trajectories(golden):
+    # reference: tests/llmcompressor/modifiers/calibration/test_observers.py:66-123
+    L = _imports()
+    g = golden["observer_trajectories"]
+    observed = torch.tensor(g["observed"], device=DEV)
+    for name, kwargs, exp_min, exp_max in g["cases"]:
+        obs = L["Observer"].load_from_registry(name, base_name="input", args=_qargs(dict(strategy="tensor")), **kwargs)
+        mins, maxs = [], []
+        for row in observed:
+            obs(row)
+            mins.append(obs.min_vals.cpu())
+            maxs.append(obs.max_vals.cpu())
+        assert torch.allclose(torch.stack(mins), torch.tensor(exp_min)), name
+        assert torch.allclose(torch.stack(maxs), torch.tensor(exp_max)), name
+
+
+def test_mse_observer_known_answers_via_registry(golden):
+    # reference: tests/llmcompressor/observers/test_mse.py:9-42
+    L = _imports()
+    g = golden["mse_observer"]
+    tensor = (torch.arange(24).reshape((6, 4)) / 24).to(DEV)
+    for strategy, symmetric, exp_loss in g["cases"]:
+        args = _qargs(dict(num_bits=8, strategy=strategy, symmetric=symmetric,
+                           group_size=(2 if strategy == "group" else None),
+                           block_structure=([3, 2] if strategy == "block" else None), observer="mse"))
+        obs = L["Observer"].load_from_registry("mse", base_name="weight", args=args)
+        qp = obs(tensor).get_qparams()
+        q = L["fake_quantize"](tensor, qp["scale"], qp["zero_point"], args)
+        loss = torch.sum((tensor - q).abs().pow(2)) / tensor.numel()
+        assert loss.item() == pytest.approx(exp_loss, abs=1e-9), (strategy, symmetric)
+
+
+def test_fused_global_scale_and_cooperative_deletion():
+    # reference: tests/llmcompressor/modifiers/utils/test_update_fused_layer_weights.py:72-120,
+    #            tests/llmcompressor/observers/test_fusion_handler.py:184-276
+    L = _imports()
+    from llmcompressor_amd.observers import fuse_weight_observers
+
+    class Attn(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.q_proj = torch.nn.Linear(64, 64, bias=False)
+            self.k_proj = torch.nn.Linear(64, 16, bias=False)
+            self.v_proj = None  # e.g. sliding attention without v_proj: skipped
+
+    torch.manual_seed(0)
+    attn = Attn().to(DEV).to(torch.bfloat16)
+    attn.k_proj.weight.data *= 4
+    args = dict(num_bits=4, type="float", strategy="tensor_group", group_size=16, scale_dtype="float8_e4m3fn")
+    for lin in (attn.q_proj, attn.k_proj):
+        L["initialize_module_for_quantization"](lin, L["QuantizationScheme"](targets=[], weights=_qargs(args)))
+        L["initialize_observer"](lin, "weight")
+    fuse_weight_observers(attn)
+    L["observe"]([attn.q_proj, attn.k_proj], "weight")
+    assert attn.q_proj.weight_observer.has_statistics and attn.k_proj.weight_observer.has_statistics
+    qp_q = attn.q_proj.weight_observer.get_qparams()
+    assert attn.k_proj.weight_observer.has_statistics  # cooperative deletion: partner not done yet
+    qp_k = attn.k_proj.weight_observer.get_qparams()
+    assert not attn.q_proj.weight_observer.has_statistics and not attn.k_proj.weight_observer.has_statistics
+    absmax = max(attn.q_proj.weight.abs().max().item(), attn.k_proj.weight.abs().max().item())
+    assert qp_q["global_scale"].item() == qp_k["global_scale"].item()
+    assert qp_q["global_scale"].item() == pytest.approx(448 * 6 / absmax, rel=1e-2)
+    # identical to the oracle's fused result
+    oa = [F.QArgs(num_bits=4, type="float", strategy="tensor_group", group_size=16, scale_dtype=torch.float8_e4m3fn)
+          for _ in range(2)]
+    oo = [O.Observer("memoryless_minmax", "weight", a) for a in oa]
+    ws = [attn.q_proj.weight.data.cpu(), attn.k_proj.weight.data.cpu()]
+    O.Observer.fuse(zip(oo, ws))
+    exp = [o(w).get_qparams() for o, w in zip(oo, ws)]
+    assert torch.equal(qp_q["scale"].cpu(), exp[0]["scale"]) and torch.equal(qp_k["scale"].cpu(), exp[1]["scale"])
+    assert qp_q["global_scale"].item() == exp[0]["global_scale"].item()
+
+
+@pytest.mark.parametrize("actorder", [None, "weight", "group"])
+def test_quantize_weight_seam_reference_fixtures(actorder):
+    # reference: tests/llmcompressor/modifiers/gptq/test_gptq_quantize.py:21-60
+    L = _imports()
+    torch.manual_seed(3)
+    module = torch.nn.Linear(8, 6, bias=False).to(DEV)
+    args = _qargs(dict(num_bits=4, symmetric=True, strategy="group", group_size=2, actorder=actorder))
+    module.quantization_scheme = L["QuantizationScheme"](targets=["Linear"], weights=args)
+    L["initialize_observer"](module, "weight")
+    L["observe"](module, "weight")
+    hessian = L["make_empty_hessian"](module)
+    hessian += torch.diag(torch.arange(1, 9, dtype=hessian.dtype, device=hessian.device))
+    w0 = module.weight.data.clone().cpu()
+    loss, q = L["quantize_weight"](module=module, quant_args=args, hessian=hessian)
+    assert loss >= 0
+    assert q["weight"].shape == module.weight.shape
+    assert q["weight_scale"].shape == (6, 4) and q["weight_zero_point"].shape == (6, 4)
+    assert ("weight_g_idx" in q) == (actorder == "group")
+    if actorder == "group":
+        assert q["weight_g_idx"].shape == (8,)
+    # same result as the oracle on the same inputs
+    oargs = F.QArgs(num_bits=4, strategy="group", group_size=2, actorder=actorder)
+    oobs = O.Observer("memoryless_minmax", "weight", oargs)
+    oobs(w0)
+    _, exp, _ = G.quantize_weight(w0, oobs, oargs, torch.diag(torch.arange(1, 9, dtype=torch.float32)))
+    assert torch.equal(q["weight"].cpu(), exp["weight"])
+    assert torch.equal(q["weight_scale"].cpu(), exp["weight_scale"])
+    if actorder == "group":
+        assert torch.equal(q["weight_g_idx"].cpu(), exp["weight_g_idx"])
+
+
+def test_quantize_weight_block_and_channel_fixtures():
+    # reference: test_gptq_quantize.py:63-132
+    L = _imports()
+    module = torch.nn.Linear(7, 5, bias=False).to(DEV)
+    args = _qargs(dict(num_bits=8, symmetric=True, strategy="block", block_structure=[2, 4]))
+    module.quantization_scheme = L["QuantizationScheme"](targets=["Linear"], weights=args)
+    L["initialize_observer"](module, "weight")
+    L["observe"](module, "weight")
+    loss, q = L["quantize_weight"](module=module, quant_args=args, hessian=torch.eye(7, device=DEV), blocksize=3)
+    assert loss >= 0 and q["weight_scale"].shape == (3, 2) and q["weight_zero_point"].shape == (3, 2)
+    assert "weight_g_idx" not in q
+    module = torch.nn.Linear(8, 4, bias=False).to(DEV)
+    args = _qargs(dict(num_bits=4, symmetric=True, strategy="channel", actorder="weight"))
+    module.quantization_scheme = L["QuantizationScheme"](targets=["Linear"], weights=args)
+    L["initialize_observer"](module, "weight")
+    L["observe"](module, "weight")
+    H = torch.diag(torch.arange(1, 9, dtype=torch.float32, device=DEV))
+    loss, q = L["quantize_weight"](module=module, quant_args=args, hessian=H, blocksize=4)
+    assert q["weight_scale"].shape[0] == 4 and "weight_g_idx" not in q and loss >= 0
+
+
+class _TinyLayer(torch.nn.Module):
+    def __init__(self, h, inter):
+        super().__init__()
+        self.q_proj = torch.nn.Linear(h, h, bias=False)
+        self.k_proj = torch.nn.Linear(h, h // 2, bias=False)
+        self.gate_proj = torch.nn.Linear(h, inter, bias=False)
+        self.up_proj = torch.nn.Linear(h, inter, bias=False)
+        self.down_proj = torch.nn.Linear(inter, h, bias=False)
+
+    def forward(self, x):
+        a = self.q_proj(x) + torch.nn.functional.pad(self.k_proj(x), (0, x.shape[-1] // 2))
+        x = x + torch.tanh(a)
+        return x + self.down_proj(torch.nn.functional.silu(self.gate_proj(x)) * self.up_proj(x))
+
+
+class _TinyModel(torch.nn.Module):
+    def __init__(self, h=64, inter=128, layers=2, vocab=100):
+        super().__init__()
+        self.embed = torch.nn.Embedding(vocab, h)
+        self.layers = torch.nn.ModuleList([_TinyLayer(h, inter) for _ in range(layers)])
+        self.lm_head = torch.nn.Linear(h, vocab, bias=False)
+
+    def forward(self, input_ids):
+        x = self.embed(input_ids)
+        for layer in self.layers:
+            x = layer(x)
+        return self.lm_head(x)
+
+
+def _tiny(seed=0):
+    torch.manual_seed(seed)
+    return _TinyModel().to(torch.bfloat16)
+
+
+@pytest.mark.parametrize("staging", [0, 256])
+def test_oneshot_gptq_sequential_matches_oracle_layer0(tmp_path, staging):
+    from llmcompressor_amd import oneshot
+    from llmcompressor_amd.compressors import decompress_weight
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+
+    ref = _tiny()
+    model = _tiny().to(DEV)
+    torch.manual_seed(1)
+    data = [torch.randint(0, 100, (1, 48)) for _ in range(12)]
+    recipe = GPTQModifier(targets="Linear", scheme={"W4A16": ["Linear"]}, ignore=["lm_head"], actorder="static",
+                          hessian_batch_tokens=staging,
+                          config_groups=None)
+    recipe = GPTQModifier(targets="Linear", ignore=["lm_head"], hessian_batch_tokens=staging, config_groups={
+        "g": dict(targets=["Linear"], weights=dict(num_bits=4, strategy="group", group_size=32))})
+    out_dir = str(tmp_path / "out")
+    oneshot(model=model, recipe=recipe, dataset=[{"input_ids": d} for d in data], output_dir=out_dir)
+    # layer-0 q_proj: oracle Hessian from the un-quantised embeddings, oracle quantize_weight
+    with torch.no_grad():
+        xs = [ref.embed(d) for d in data]
+    H, n = G.make_empty_hessian(64), torch.zeros(())
+    for x in xs:
+        H, n = G.accumulate_hessian(x, H, n)
+    oargs = F.QArgs(num_bits=4, strategy="group", group_size=32, actorder="weight")
+    w0 = ref.layers[0].q_proj.weight.data
+    oobs = O.Observer("memoryless_minmax", "weight", oargs)
+    oobs(w0)
+    _, exp, _ = G.quantize_weight(w0, oobs, oargs, H / n)
+    got = model.layers[0].q_proj.weight.data.cpu()
+    assert (got == exp["weight"]).float().mean().item() >= 0.999
+    assert torch.equal(model.layers[0].q_proj.weight_scale.data.cpu(), exp["weight_scale"])
+    assert not hasattr(model.layers[0].q_proj, "weight_observer")
+    assert not hasattr(model.lm_head, "quantization_scheme")
+    # later layers were calibrated on the outputs of the quantised earlier layers and are on-grid
+    w1 = model.layers[1].down_proj
+    codes = w1.weight.data.float() / w1.weight_scale.data.float().repeat_interleave(32, dim=1)
+    assert (codes - codes.round()).abs().max() <= 8 * 2.0 ** -8
+    # checkpoint: layout, config, recipe, round trip
+    from safetensors.torch import load_file
+
+    sd = load_file(os.path.join(out_dir, "model.safetensors"))
+    key = "layers.0.q_proj."
+    assert sd[key + "weight_packed"].dtype == torch.int32 and sd[key + "weight_packed"].shape == (64, 8)
+    assert sd[key + "weight_shape"].tolist() == [64, 64] and key + "weight" not in sd
+    assert "lm_head.weight" in sd and key + "weight_g_idx" not in sd
+    cfg = json.load(open(os.path.join(out_dir, "config.json")))["quantization_config"]
+    assert cfg["quant_method"] == "compressed-tensors" and cfg["format"] == "pack-quantized"
+    assert cfg["quantization_status"] == "compressed" and "lm_head" in cfg["ignore"]
+    assert os.path.exists(os.path.join(out_dir, "recipe.yaml"))
+    from llmcompressor_amd.quantization import QuantizationArgs
+
+    deq = decompress_weight({k[len(key):]: v for k, v in sd.items() if k.startswith(key)},
+                            QuantizationArgs(num_bits=4, strategy="group", group_size=32), "pack-quantized")
+    assert torch.equal(deq, got)
+
+
+@pytest.mark.parametrize("scheme,fmt", [("FP8_DYNAMIC", "float-quantized"), ("NVFP4A16", "nvfp4-pack-quantized"),
+                                        ("MXFP4A16", "mxfp4-pack-quantized"), ("W8A16", "pack-quantized")])
+def test_oneshot_datafree_rtn_and_checkpoint_round_trip(tmp_path, scheme, fmt):
+    from llmcompressor_amd import oneshot
+    from llmcompressor_amd.compressors import compress_module, decompress_weight
+    from llmcompressor_amd.modifiers.quantization import QuantizationModifier
+    from llmcompressor_amd.quantization import fake_quantize
+
+    model = _tiny(2).to(DEV)
+    w_before = model.layers[0].gate_proj.weight.data.clone()
+    oneshot(model=model, recipe=QuantizationModifier(targets="Linear", scheme=scheme, ignore=["lm_head"]),
+            output_dir=str(tmp_path / scheme))
+    lin = model.layers[0].gate_proj
+    assert torch.equal(lin.weight.data, w_before)  # RTN keeps the dense weight; packing happens at save
+    args = lin.quantization_scheme.weights
+    gs = getattr(lin, "weight_global_scale", None)
+    fq = fake_quantize(lin.weight.data, lin.weight_scale.data, lin.weight_zero_point.data, args,
+                       global_scale=None if gs is None else gs.data)
+    tensors = compress_module(lin)
+    deq = decompress_weight(tensors, args, fmt)
+    assert torch.equal(deq, fq)
+    # the oracle agrees bit for bit on scales and packed bytes
+    oargs = F.QArgs(num_bits=args.num_bits, type=args.type.value, strategy=args.strategy.value,
+                    group_size=args.group_size, scale_dtype=args.scale_dtype)
+    oobs = [O.Observer("memoryless_minmax", "weight", oargs)]
+    w_cpu = w_before.cpu()
+    if scheme == "NVFP4A16":
+        up = O.Observer("memoryless_minmax", "weight", F.QArgs(**oargs.__dict__))
+        O.Observer.fuse([(oobs[0], w_cpu), (up, model.layers[0].up_proj.weight.data.cpu())])
+    qp = oobs[0](w_cpu).get_qparams()
+    from oracle import pack as P
+
+    exp = P.compress_weight(w_cpu, qp["scale"], qp["zero_point"], oargs, global_scale=qp["global_scale"])
+    if fmt == "float-quantized":
+        assert torch.equal(tensors["weight"].cpu().view(torch.uint8), exp["weight"].view(torch.uint8))
+        assert torch.equal(tensors["weight_scale"].cpu(), exp["weight_scale"])
+    else:
+        assert torch.equal(tensors["weight_packed"].cpu(), exp["weight_packed"])
+        assert torch.equal(tensors["weight_scale"].cpu().view(torch.uint8) if tensors["weight_scale"].dtype != torch.bfloat16 else tensors["weight_scale"].cpu(),
+                           exp["weight_scale"].view(torch.uint8) if exp["weight_scale"].dtype != torch.bfloat16 else exp["weight_scale"])
+    cfg = json.load(open(os.path.join(str(tmp_path / scheme), "config.json")))["quantization_config"]
+    assert cfg["format"] == fmt
+    # quantised forward runs (dynamic per-token activations for FP8_DYNAMIC)
+    with torch.no_grad():
+        y = model(torch.randint(0, 100, (2, 16), device=DEV))
+    assert torch.isfinite(y.float()).all()
+
+
+def test_moe_gptq_zero_token_expert_is_zeroed():
+    """An expert that never receives a token keeps H = 0: every column is dead and its weight is zeroed."""
+    from llmcompressor_amd.core import State, active_session
+    from llmcompressor_amd.modeling import LinearExperts2D
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+
+    torch.manual_seed(0)
+    E, H, I, T = 4, 64, 128, 96
+    experts = LinearExperts2D.from_fused(torch.randn(E, 2 * I, H) * 0.05, torch.randn(E, H, I) * 0.05)
+    experts = experts.to(DEV).to(torch.bfloat16)
+
+    class Wrap(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.layers = torch.nn.ModuleList([experts])
+
+    model = Wrap()
+    mod = GPTQModifier(targets="Linear", config_groups={"g": dict(targets=["Linear"], weights=dict(
+        num_bits=4, strategy="group", group_size=32))})
+    session = active_session()
+    session.reset()
+    session.initialize(model=model, recipe=mod)
+    from llmcompressor_amd.core import LifecycleCallbacks
+
+    LifecycleCallbacks.calibration_start()
+    x = torch.randn(T, H, device=DEV).bfloat16()
+    idx = torch.stack([torch.arange(T) % 3, (torch.arange(T) + 1) % 3], dim=1).to(DEV)  # expert 3 never routed
+    wts = torch.full((T, 2), 0.5, device=DEV, dtype=torch.bfloat16)
+    with torch.no_grad():
+        for _ in range(3):
+            experts(x, idx, wts)
+    LifecycleCallbacks.sequential_epoch_end(modules=list(model.modules()))
+    LifecycleCallbacks.calibration_end()
+    session.finalize()
+    assert torch.count_nonzero(experts[3].gate_proj.weight) == 0
+    assert torch.count_nonzero(experts[3].down_proj.weight) == 0
+    assert torch.count_nonzero(experts[0].gate_proj.weight) > 0
