@@ -77,6 +77,10 @@ __global__ __launch_bounds__(256) void hinv_copyin_kernel(const float* __restric
 }
 
 // Factor the 64x64 diagonal block at (k0,k0) in LDS and replace it by the inverse of its factor.
+// Left-looking (Cholesky-Crout) so nothing is updated ahead of the current column: at step j the
+// 64 four-lane teams each form one dot product over the previous columns -- team t > j for
+// L[t][j], team j for the pivot, team t < j for X[j][t] of X = L^-1 (row j of L is complete by
+// then) -- so factor and inverse advance together with two barriers per column.
 __global__ __launch_bounds__(256) void potf2_inv_kernel(float* __restrict__ A, int Kp, int k0, int K,
                                                         HinvScalars* sc) {
   __shared__ float L[NB][NB + 1];
@@ -87,11 +91,40 @@ __global__ __launch_bounds__(256) void potf2_inv_kernel(float* __restrict__ A, i
     L[i][j] = (j <= i) ? A[(int64_t)(k0 + i) * Kp + k0 + j] : 0.f;
     X[i][j] = 0.f;
   }
+  __syncthreads();
+  const int t = tid >> 2, part = tid & 3;
   for (int j = 0; j < NB; ++j) {
-    __syncthreads();
-    if (tid == 0) {
-      float d = L[j][j];
-      if (!(d > 0.f) || d != d || d > 3.0e38f) {
+    // dot over the previous columns; four independent partial sums keep several LDS loads in flight
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    int k = (t < j ? t : 0) + part;
+    if (t >= j) {
+      const float* rowt = L[t];
+      for (; k + 12 < j; k += 16) {
+        const float a0 = rowt[k], a1 = rowt[k + 4], a2 = rowt[k + 8], a3 = rowt[k + 12];
+        const float b0 = L[j][k], b1 = L[j][k + 4], b2 = L[j][k + 8], b3 = L[j][k + 12];
+        s0 += a0 * b0;
+        s1 += a1 * b1;
+        s2 += a2 * b2;
+        s3 += a3 * b3;
+      }
+      for (; k < j; k += 4) s0 += rowt[k] * L[j][k];
+    } else {
+      for (; k + 12 < j; k += 16) {
+        const float a0 = X[k][t], a1 = X[k + 4][t], a2 = X[k + 8][t], a3 = X[k + 12][t];
+        const float b0 = L[j][k], b1 = L[j][k + 4], b2 = L[j][k + 8], b3 = L[j][k + 12];
+        s0 += a0 * b0;
+        s1 += a1 * b1;
+        s2 += a2 * b2;
+        s3 += a3 * b3;
+      }
+      for (; k < j; k += 4) s0 += X[k][t] * L[j][k];
+    }
+    float s = (s0 + s1) + (s2 + s3);
+    s += __shfl_xor(s, 1, 64);
+    s += __shfl_xor(s, 2, 64);
+    if (t == j && part == 0) {
+      float d = L[j][j] - s;
+      if (!(d > 0.f) || d > 3.0e38f) {
         // first failing pivot, 1-based index in the ORIGINAL (un-reversed) ordering
         if (k0 + j < K) atomicCAS(&sc->info, 0, K - (k0 + j));
         d = 1.f;
@@ -100,25 +133,16 @@ __global__ __launch_bounds__(256) void potf2_inv_kernel(float* __restrict__ A, i
     }
     __syncthreads();
     const float piv = L[j][j];
-    for (int i = j + 1 + tid; i < NB; i += 256) L[i][j] = L[i][j] / piv;
+    if (part == 0) {
+      if (t > j)
+        L[t][j] = (L[t][j] - s) / piv;
+      else if (t < j)
+        X[j][t] = -s / piv;
+      else
+        X[j][j] = 1.f / piv;
+    }
     __syncthreads();
-    const int n = NB - 1 - j;
-    for (int e = tid; e < n * n; e += 256) {
-      const int i = j + 1 + e / n, c = j + 1 + e % n;
-      if (c <= i) L[i][c] -= L[i][j] * L[c][j];
-    }
   }
-  __syncthreads();
-  // column tid of X = L^-1 by forward substitution; a thread only ever reads its own column of X
-  if (tid < NB) {
-    const int j = tid;
-    for (int i = j; i < NB; ++i) {
-      float s = (i == j) ? 1.f : 0.f;
-      for (int k = j; k < i; ++k) s -= L[i][k] * X[k][j];
-      X[i][j] = s / L[i][i];
-    }
-  }
-  __syncthreads();
   for (int e = tid; e < NB * NB; e += 256) {
     const int i = e / NB, j = e % NB;
     A[(int64_t)(k0 + i) * Kp + k0 + j] = (j <= i) ? X[i][j] : 0.f;
@@ -175,25 +199,46 @@ extern "C" int llmc_gptq_hinv(float* H, int64_t ldh, int64_t K, const int32_t* p
                      divisor, sc, A);
   LLMC_LAUNCH_STATUS();
 
-  // right-looking blocked Cholesky; diagonal blocks end up holding inv(L_kk)
-  for (int k0 = 0; k0 < Kp; k0 += NB) {
-    hipLaunchKernelGGL(potf2_inv_kernel, dim3(1), dim3(256), 0, st, A, Kp, k0, (int)K, sc);
-    LLMC_LAUNCH_STATUS();
-    const int M = Kp - k0 - NB;
-    if (M <= 0) break;
-    float* A21 = A + (int64_t)(k0 + NB) * Kp + k0;
-    GemmF32 g = {};
-    // panel: A21 <- A21 * inv(L_kk)^T   (in place: one tile column, each workgroup owns its rows)
-    g.A = A21; g.lda = Kp; g.B = A + (int64_t)k0 * Kp + k0; g.ldb = Kp; g.C = A21; g.ldc = Kp;
-    g.M = M; g.N = NB; g.Kc = NB; g.alpha = 1.f; g.beta = 0.f; g.trans_b = 1; g.batch = 1;
-    int rc = llmc_gemm_f32(g, st);
-    if (rc) return rc;
-    // trailing: A22 <- A22 - A21 A21^T   (lower triangle only)
-    GemmF32 s = {};
-    s.A = A21; s.lda = Kp; s.B = A21; s.ldb = Kp; s.C = A + (int64_t)(k0 + NB) * Kp + k0 + NB; s.ldc = Kp;
-    s.M = M; s.N = M; s.Kc = NB; s.alpha = -1.f; s.beta = 1.f; s.trans_b = 1; s.c_lower = 1; s.batch = 1;
-    rc = llmc_gemm_f32(s, st);
-    if (rc) return rc;
+  // Blocked Cholesky, two levels: inside a 256-wide outer panel the 64-wide steps (diagonal block
+  // factored + inverted in LDS, panel solve as a GEMM) only update the panel's own remaining
+  // columns; the trailing matrix then gets one rank-256 update per outer panel, which cuts its
+  // read-modify-write traffic 4x compared with rank-64 updates.  Diagonal blocks end up holding
+  // inv(L_kk).
+  constexpr int NBO = 256;
+  for (int k0 = 0; k0 < Kp; k0 += NBO) {
+    const int pw = (Kp - k0) < NBO ? (Kp - k0) : NBO;
+    for (int kk = 0; kk < pw; kk += NB) {
+      const int c0 = k0 + kk;
+      hipLaunchKernelGGL(potf2_inv_kernel, dim3(1), dim3(256), 0, st, A, Kp, c0, (int)K, sc);
+      LLMC_LAUNCH_STATUS();
+      const int M = Kp - c0 - NB;
+      if (M <= 0) break;
+      float* A21 = A + (int64_t)(c0 + NB) * Kp + c0;
+      GemmF32 g = {};
+      // panel: A21 <- A21 * inv(L_kk)^T   (in place: one tile column, each workgroup owns its rows)
+      g.A = A21; g.lda = Kp; g.B = A + (int64_t)c0 * Kp + c0; g.ldb = Kp; g.C = A21; g.ldc = Kp;
+      g.M = M; g.N = NB; g.Kc = NB; g.alpha = 1.f; g.beta = 0.f; g.trans_b = 1; g.batch = 1;
+      int rc = llmc_gemm_f32(g, st);
+      if (rc) return rc;
+      const int nrem = k0 + pw - (c0 + NB);
+      if (nrem > 0) {
+        // remaining columns of this outer panel: C[M, nrem] -= A21 * A21[:nrem]^T (lower part)
+        GemmF32 u = {};
+        u.A = A21; u.lda = Kp; u.B = A21; u.ldb = Kp; u.C = A + (int64_t)(c0 + NB) * Kp + c0 + NB; u.ldc = Kp;
+        u.M = M; u.N = nrem; u.Kc = NB; u.alpha = -1.f; u.beta = 1.f; u.trans_b = 1; u.c_lower = 1; u.batch = 1;
+        rc = llmc_gemm_f32(u, st);
+        if (rc) return rc;
+      }
+    }
+    const int M2 = Kp - (k0 + pw);
+    if (M2 > 0) {
+      float* P = A + (int64_t)(k0 + pw) * Kp + k0;
+      GemmF32 t = {};
+      t.A = P; t.lda = Kp; t.B = P; t.ldb = Kp; t.C = A + (int64_t)(k0 + pw) * ((int64_t)Kp + 1); t.ldc = Kp;
+      t.M = M2; t.N = M2; t.Kc = pw; t.alpha = -1.f; t.beta = 1.f; t.trans_b = 1; t.c_lower = 1; t.batch = 1;
+      const int rc = llmc_gemm_f32(t, st);
+      if (rc) return rc;
+    }
   }
 
   // inverse by recursive doubling: [[X11,0],[X21,X22]] with X21 = -X22 * L21 * X11

@@ -22,26 +22,17 @@ __device__ __forceinline__ float4 ld4(const float* p, int valid, bool vec) {
   return v;
 }
 
-template <int BM, int BN>
-__global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32 g, int vec) {
+// FAST: the tile lies fully inside C, the contraction range is a multiple of BK and all rows are
+// 16-byte aligned, so every load is an unconditional float4 and the main loop is one basic block.
+template <int BM, int BN, bool TRANS_B, bool FAST>
+__device__ __forceinline__ void gemm_tile(const GemmF32& g, const float* A, const float* B, float* C, int m0,
+                                          int n0, int k_begin, int k_end, float* As, float* Bs) {
   constexpr int LDA_S = BM + 4, LDB_S = BN + 4;
   constexpr int MI = BM / 64, NI = BN / 64;
   constexpr int A_LD = BM / 64;  // float4 loads per thread for the A slab
   constexpr int B_LD = BN / 64;
-  __shared__ float As[BK * LDA_S];
-  __shared__ float Bs[BK * LDB_S];
-
-  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
-  if (g.c_lower && n0 > m0 + BM - 1) return;
-  const float* A = g.A + (int64_t)blockIdx.z * g.stride_a;
-  const float* B = g.B + (int64_t)blockIdx.z * g.stride_b;
-  float* C = g.C + (int64_t)blockIdx.z * g.stride_c;
-
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  const int k_begin = g.b_lower_tri ? (n0 / BK) * BK : 0;
-  int k_end = g.Kc;
-  if (g.a_lower_tri && m0 + BM < k_end) k_end = m0 + BM;
 
   f32x16_t acc[MI][NI];
 #pragma unroll
@@ -57,17 +48,26 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32 g, int vec) {
     for (int i = 0; i < A_LD; ++i) {
       const int f = tid + i * 256;
       const int m = m0 + f / 4, k = k0 + (f % 4) * 4;
-      ra[i] = (m < g.M) ? ld4(A + (int64_t)m * g.lda + k, k_end - k, vec) : make_float4(0.f, 0.f, 0.f, 0.f);
+      if (FAST)
+        ra[i] = *(const float4*)(A + (int64_t)m * g.lda + k);
+      else
+        ra[i] = (m < g.M) ? ld4(A + (int64_t)m * g.lda + k, k_end - k, false) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
 #pragma unroll
     for (int i = 0; i < B_LD; ++i) {
       const int f = tid + i * 256;
-      if (g.trans_b) {
+      if (TRANS_B) {
         const int n = n0 + f / 4, k = k0 + (f % 4) * 4;
-        rb[i] = (n < g.N) ? ld4(B + (int64_t)n * g.ldb + k, k_end - k, vec) : make_float4(0.f, 0.f, 0.f, 0.f);
+        if (FAST)
+          rb[i] = *(const float4*)(B + (int64_t)n * g.ldb + k);
+        else
+          rb[i] = (n < g.N) ? ld4(B + (int64_t)n * g.ldb + k, k_end - k, false) : make_float4(0.f, 0.f, 0.f, 0.f);
       } else {
         const int k = k0 + f / (BN / 4), n = n0 + (f % (BN / 4)) * 4;
-        rb[i] = (k < k_end) ? ld4(B + (int64_t)k * g.ldb + n, g.N - n, vec) : make_float4(0.f, 0.f, 0.f, 0.f);
+        if (FAST)
+          rb[i] = *(const float4*)(B + (int64_t)k * g.ldb + n);
+        else
+          rb[i] = (k < k_end) ? ld4(B + (int64_t)k * g.ldb + n, g.N - n, false) : make_float4(0.f, 0.f, 0.f, 0.f);
       }
     }
   };
@@ -84,7 +84,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32 g, int vec) {
 #pragma unroll
     for (int i = 0; i < B_LD; ++i) {
       const int f = tid + i * 256;
-      if (g.trans_b) {
+      if (TRANS_B) {
         const int n = f / 4, k = (f % 4) * 4;
         Bs[(k + 0) * LDB_S + n] = rb[i].x;
         Bs[(k + 1) * LDB_S + n] = rb[i].y;
@@ -96,34 +96,35 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32 g, int vec) {
       }
     }
   };
+  auto multiply = [&]() {
+#pragma unroll
+    for (int kk = 0; kk < BK / 2; ++kk) {
+      const int k = 2 * kk + (lane >> 5);
+      float fa[MI], fb[NI];
+#pragma unroll
+      for (int a = 0; a < MI; ++a) fa[a] = As[k * LDA_S + wm * (BM / 2) + a * 32 + (lane & 31)];
+#pragma unroll
+      for (int b = 0; b < NI; ++b) fb[b] = Bs[k * LDB_S + wn * (BN / 2) + b * 32 + (lane & 31)];
+#pragma unroll
+      for (int a = 0; a < MI; ++a)
+#pragma unroll
+        for (int b = 0; b < NI; ++b)
+          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[a], fb[b], acc[a][b], 0, 0, 0);
+    }
+  };
 
   if (k_begin < k_end) {
     load_slab(k_begin);
     store_slab();
     __syncthreads();
-    for (int k0 = k_begin; k0 < k_end; k0 += BK) {
-      const bool more = k0 + BK < k_end;
-      if (more) load_slab(k0 + BK);
-#pragma unroll
-      for (int kk = 0; kk < BK / 2; ++kk) {
-        const int k = 2 * kk + (lane >> 5);
-        float fa[MI], fb[NI];
-#pragma unroll
-        for (int a = 0; a < MI; ++a) fa[a] = As[k * LDA_S + wm * (BM / 2) + a * 32 + (lane & 31)];
-#pragma unroll
-        for (int b = 0; b < NI; ++b) fb[b] = Bs[k * LDB_S + wn * (BN / 2) + b * 32 + (lane & 31)];
-#pragma unroll
-        for (int a = 0; a < MI; ++a)
-#pragma unroll
-          for (int b = 0; b < NI; ++b)
-            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[a], fb[b], acc[a][b], 0, 0, 0);
-      }
+    for (int k0 = k_begin; k0 + BK < k_end; k0 += BK) {
+      load_slab(k0 + BK);
+      multiply();
       __syncthreads();
-      if (more) {
-        store_slab();
-        __syncthreads();
-      }
+      store_slab();
+      __syncthreads();
     }
+    multiply();
   }
 
 #pragma unroll
@@ -131,11 +132,11 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32 g, int vec) {
 #pragma unroll
     for (int b = 0; b < NI; ++b) {
       const int col = n0 + wn * (BN / 2) + b * 32 + (lane & 31);
-      if (col >= g.N) continue;
+      if (!FAST && col >= g.N) continue;
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int row = m0 + wm * (BM / 2) + a * 32 + (v / 4) * 8 + (lane >> 5) * 4 + (v & 3);
-        if (row >= g.M || (g.c_lower && col > row)) continue;
+        if ((!FAST && row >= g.M) || (g.c_lower && col > row)) continue;
         float* cp = C + (int64_t)row * g.ldc + col;
         float r = g.alpha * acc[a][b][v];
         if (g.beta != 0.f) r += g.beta * *cp;
@@ -144,22 +145,47 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32 g, int vec) {
     }
 }
 
+template <int BM, int BN, bool TRANS_B>
+__global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32 g, int vec) {
+  __shared__ float As[BK * (BM + 4)];
+  __shared__ float Bs[BK * (BN + 4)];
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  if (g.c_lower && n0 > m0 + BM - 1) return;
+  const float* A = g.A + (int64_t)blockIdx.z * g.stride_a;
+  const float* B = g.B + (int64_t)blockIdx.z * g.stride_b;
+  float* C = g.C + (int64_t)blockIdx.z * g.stride_c;
+  const int k_begin = g.b_lower_tri ? (n0 / BK) * BK : 0;
+  int k_end = g.Kc;
+  if (g.a_lower_tri && m0 + BM < k_end) k_end = m0 + BM;
+  const bool fast = vec && m0 + BM <= g.M && n0 + BN <= g.N && ((k_end - k_begin) % BK) == 0;
+  if (fast)
+    gemm_tile<BM, BN, TRANS_B, true>(g, A, B, C, m0, n0, k_begin, k_end, As, Bs);
+  else
+    gemm_tile<BM, BN, TRANS_B, false>(g, A, B, C, m0, n0, k_begin, k_end, As, Bs);
+}
+
 }  // namespace
 
 int llmc_gemm_f32(const GemmF32& g, hipStream_t st) {
   if (g.M <= 0 || g.N <= 0 || g.batch <= 0) return 0;
   const int vec = ((g.lda & 3) == 0 && (g.ldb & 3) == 0 && (((uintptr_t)g.A | (uintptr_t)g.B) & 15) == 0 &&
-                   (g.stride_a & 3) == 0 && (g.stride_b & 3) == 0)
+                   (g.stride_a & 3) == 0 && (g.stride_b & 3) == 0 && (g.Kc & 3) == 0)
                       ? 1
                       : 0;
   // 128x128 tiles when they still give the chip enough workgroups, 64x64 otherwise
   const int64_t t128 = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * g.batch;
   if (t128 >= 256 && g.M >= 128 && g.N >= 128) {
     dim3 grid((g.N + 127) / 128, (g.M + 127) / 128, g.batch);
-    hipLaunchKernelGGL((gemm_f32_kernel<128, 128>), grid, dim3(256), 0, st, g, vec);
+    if (g.trans_b)
+      hipLaunchKernelGGL((gemm_f32_kernel<128, 128, true>), grid, dim3(256), 0, st, g, vec);
+    else
+      hipLaunchKernelGGL((gemm_f32_kernel<128, 128, false>), grid, dim3(256), 0, st, g, vec);
   } else {
     dim3 grid((g.N + 63) / 64, (g.M + 63) / 64, g.batch);
-    hipLaunchKernelGGL((gemm_f32_kernel<64, 64>), grid, dim3(256), 0, st, g, vec);
+    if (g.trans_b)
+      hipLaunchKernelGGL((gemm_f32_kernel<64, 64, true>), grid, dim3(256), 0, st, g, vec);
+    else
+      hipLaunchKernelGGL((gemm_f32_kernel<64, 64, false>), grid, dim3(256), 0, st, g, vec);
   }
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : 1000 + (int)e;
