@@ -5,9 +5,10 @@ Workload (BASELINE.json configs[3], one decoder layer per step): GPTQ W4A16 g128
 activation ordering "static", of the seven Linears of a random-init
 Llama-3-8B-shaped decoder layer.  A step is
 
-  Hessian phase : 256 calibration batches x 2048 tokens; per batch one
-                  H += 2 X^T X launch per Linear (q/k/v/o/gate/up on the 4096-wide
-                  input, down on the 14336-wide one) -- 3.21e14 algorithmic FLOP
+  Hessian phase : 256 calibration batches x 2048 tokens through GPTQModifier's forward
+                  hook for each Linear (q/k/v/o/gate/up on the 4096-wide input, down on
+                  the 14336-wide one); the hook stages batches and launches H += 2 X^T X
+                  once per --stage-tokens tokens -- 3.21e14 algorithmic FLOP per step
   quantize phase: per Linear  min-max observer -> scales -> diag argsort ->
                   damped Cholesky chain -> GPTQ column loop -> int4 packing
 
@@ -88,6 +89,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--batches", type=int, default=256, help="calibration batches per step (config: 256)")
     ap.add_argument("--tokens", type=int, default=2048, help="tokens per batch (config: 2048)")
+    ap.add_argument("--stage-tokens", type=int, default=8192,
+                    help="tokens staged per Hessian launch (GPTQModifier.hessian_batch_tokens; 0 = one launch per batch)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -97,57 +100,82 @@ def main():
     import torch
 
     from llmcompressor_amd import ops
+    from llmcompressor_amd.compressors import compress_module
+    from llmcompressor_amd.core import LifecycleCallbacks, active_session
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     B, T = a.batches, a.tokens
     gen = torch.Generator(device=dev).manual_seed(0)
-    weights = {
-        name: (torch.randn(r, k, device=dev, generator=gen) * 0.02).bfloat16() for name, r, k in LINEARS
-    }
+
+    class Layer(torch.nn.Module):  # the seven Linears of one decoder layer (no forward needed here)
+        def __init__(self):
+            super().__init__()
+            for name, r, k in LINEARS:
+                setattr(self, name, torch.nn.Linear(k, r, bias=False, dtype=torch.bfloat16, device=dev))
+
+    layer = Layer()
+    originals = {}
+    for name, r, k in LINEARS:
+        w = (torch.randn(r, k, device=dev, generator=gen) * 0.02).bfloat16()
+        getattr(layer, name).weight.data.copy_(w)
+        originals[name] = w
     # calibration activations, resident in HBM: one stream per distinct Linear input
     x_hidden = torch.empty(B, T, HIDDEN, dtype=torch.bfloat16, device=dev)
     x_inter = torch.empty(B, T, INTER, dtype=torch.bfloat16, device=dev)
     for b in range(B):
         x_hidden[b] = torch.randn(T, HIDDEN, device=dev, generator=gen).bfloat16()
         x_inter[b] = torch.randn(T, INTER, device=dev, generator=gen).bfloat16()
-    hess = {name: torch.zeros(k, k, device=dev) for name, r, k in LINEARS}
-    g_idx_base = {k: (torch.arange(k, dtype=torch.int32, device=dev) // GROUP) for k in (HIDDEN, INTER)}
 
+    # time every launch of the dominant kernel (the 14336-wide Hessian) with events on the launch stream
     dom_events = []
+    dom_tokens = []
+    recording = [False]
+    raw_accumulate = ops.hessian_accumulate_
+
+    def timed_accumulate(H, x, **kw):
+        if recording[0] and H.shape[0] == INTER:
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            out = raw_accumulate(H, x, **kw)
+            e1.record()
+            dom_events.append((e0, e1))
+            dom_tokens.append(x.shape[0])
+            return out
+        return raw_accumulate(H, x, **kw)
+
+    ops.hessian_accumulate_ = timed_accumulate
 
     def step(record: bool):
-        for h in hess.values():
-            h.zero_()
+        for name, r, k in LINEARS:
+            getattr(layer, name).weight.data.copy_(originals[name])
+        recording[0] = record
+        modifier = GPTQModifier(targets="Linear", scheme="W4A16", actorder="static", block_size=128,
+                                dampening_frac=0.01, hessian_batch_tokens=a.stage_tokens)
+        session = active_session()
+        session.reset()
+        session.initialize(model=layer, recipe=modifier)
+        LifecycleCallbacks.calibration_start()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
+        # what the forward hooks do during the calibration pass of this layer
         for b in range(B):
             for name, r, k in LINEARS:
                 x = x_hidden[b] if k == HIDDEN else x_inter[b]
-                if record and k == INTER:
-                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                    e0.record()
-                    ops.hessian_accumulate_(hess[name], x)
-                    e1.record()
-                    dom_events.append((e0, e1))
-                else:
-                    ops.hessian_accumulate_(hess[name], x)
+                modifier.calibrate_module(getattr(layer, name), (x.unsqueeze(0),), None)
+        for m in list(modifier._staged):
+            modifier._flush(m)
         torch.cuda.synchronize()
         t1 = time.perf_counter()
-        out = {}
-        for name, r, k in LINEARS:
-            w = weights[name]
-            mn, mx = ops.minmax_groups(w, GROUP)
-            scale, _, _ = ops.calculate_qparams(mn, mx, ops.FMT_INT, 4, True)
-            perm = torch.argsort(torch.diagonal(hess[name]), descending=True).to(torch.int32)
-            g_idx = g_idx_base[k][perm.long()]
-            U, dead, info = ops.gptq_hinv_(hess[name], perm, divisor=float(B), percdamp=0.01)
-            wq, loss = ops.gptq_quantize(w, U, scale, None, ops.FMT_INT, 4, 1, k // GROUP, g_idx=g_idx, perm=perm,
-                                         dead=dead, blocksize=128)
-            packed = ops.quantize(wq, scale, None, ops.FMT_INT, 4, 1, k // GROUP, GROUP, out_mode=ops.OUT_PACKED)
-            out[name] = (packed, scale, loss)
+        # epoch end: observers -> qparams -> Cholesky chain -> column loop, then pack
+        LifecycleCallbacks.sequential_epoch_end(modules=list(layer.modules()))
+        out = {name: compress_module(getattr(layer, name)) for name, _, _ in LINEARS}
         torch.cuda.synchronize()
         t2 = time.perf_counter()
+        LifecycleCallbacks.calibration_end()
+        session.finalize()
+        recording[0] = False
         return t1 - t0, t2 - t1, out
 
     for _ in range(a.warmup):
@@ -165,7 +193,8 @@ def main():
     flop_step = sum(2.0 * T * k * k for _, _, k in LINEARS) * B
     value = flop_step * a.steps / th / 1e12
     dom_ms = sum(e0.elapsed_time(e1) for e0, e1 in dom_events) / max(1, len(dom_events))
-    dom_flop = 2.0 * T * INTER * INTER
+    dom_T = sum(dom_tokens) / max(1, len(dom_tokens))
+    dom_flop = 2.0 * dom_T * INTER * INTER
     achieved = dom_flop / (dom_ms * 1e-3) / 1e12
     rec = {
         "metric": "GPTQ quantize_weight ms/Linear + Hessian TFLOP/s, Llama-3-8B shapes, W4A16 g128",
@@ -185,12 +214,13 @@ def main():
             f"per step ({B} batches x {T} tokens, 7 Linears: Hessians 6x4096^2 + 14336^2, then quantize_weight + pack)",
             "batches": B,
             "tokens": T,
+            "hessian_tokens_per_launch": int(dom_T),
         },
         "quantize_weight_ms_per_linear": round(tq / a.steps / len(LINEARS) * 1e3, 3),
         "hessian_phase_ms_per_step": round(th / a.steps * 1e3, 2),
         "hessian_algorithmic_flop_per_step": flop_step,
         "roofline": {
-            "kernel": "hessian_syrk_kernel<256> (down_proj Hessian, T=%d, K=%d)" % (T, INTER),
+            "kernel": "hessian_syrk_kernel<256> (down_proj Hessian, %d tokens per launch, K=%d)" % (int(dom_T), INTER),
             "bound": "mfma",
             "achieved": round(achieved, 2),
             "peak": MFMA_BF16_PEAK_TFLOPS,

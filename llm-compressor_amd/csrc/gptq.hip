@@ -50,6 +50,7 @@ struct GptqBlockParams {
   float* loss_rows; // [R]
 };
 
+template <int FMT, int SD, bool HAS_ZP>
 __global__ __launch_bounds__(256) void gptq_block_kernel(GptqBlockParams p) {
   extern __shared__ __attribute__((aligned(16))) float Hs[];  // [GB][GB], zero outside the upper triangle
   const int tid = threadIdx.x;
@@ -60,8 +61,8 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(GptqBlockParams p) {
   const int tl = tid % TEAM;
   const int row = blockIdx.x * ROWS_PER_WG + tid / TEAM;
   const bool live = row < p.R;
-  const QFormat f = make_qformat(p.fmt, p.bits);
-  const bool has_zp = p.zp != nullptr;
+  const QFormat f = make_qformat(FMT, p.bits);  // the format is a compile-time constant here
+  constexpr bool has_zp = HAS_ZP;
   const float gs = p.gscale ? p.gscale[0] : 1.f;
 
   float w[CPL], sv[CPL], zv[CPL], qv[CPL], ev[CPL];
@@ -96,11 +97,11 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(GptqBlockParams p) {
         const float s = __shfl(sv[e], li, TEAM);
         const float zp = has_zp ? __shfl(zv[e], li, TEAM) : 0.f;
         const float qc = quantize_value(wv, s, zp, has_zp, LLMC_F32, f);
-        const float q = dequantize_value(qc, s, zp, has_zp, p.sd);
+        const float q = dequantize_value(qc, s, zp, has_zp, SD);
         const float d = Hs[i * GB + i];
         const float diff = __fsub_rn(wv, q);
         const float err = diff / d;
-        loss += __fmul_rn(diff, diff) / __fmul_rn(d, d);
+        loss += err * err;  // (w-q)^2 / d^2
         const float4 h0 = *(const float4*)&Hs[i * GB + tl * CPL];
         const float4 h1 = *(const float4*)&Hs[i * GB + tl * CPL + 4];
         // product rounded, then subtracted: the reference forms the outer product first
@@ -216,14 +217,29 @@ extern "C" int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R
   p.E = E; p.loss_rows = loss_rows;
 
   const int smem = GB * GB * 4;
-  hipError_t e = hipFuncSetAttribute((const void*)gptq_block_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+  void (*kern)(GptqBlockParams) = nullptr;
+  const bool hz = zero_point != nullptr;
+#define LLMC_PICK(F, S)                                                         \
+  if (p.fmt == F && p.sd == S) kern = hz ? gptq_block_kernel<F, S, true> : gptq_block_kernel<F, S, false>;
+  LLMC_PICK(LLMC_FMT_INT, LLMC_BF16)
+  LLMC_PICK(LLMC_FMT_INT, LLMC_F16)
+  LLMC_PICK(LLMC_FMT_INT, LLMC_F32)
+  LLMC_PICK(LLMC_FMT_FP8, LLMC_BF16)
+  LLMC_PICK(LLMC_FMT_FP8, LLMC_F16)
+  LLMC_PICK(LLMC_FMT_FP8, LLMC_F32)
+  LLMC_PICK(LLMC_FMT_FP4, LLMC_BF16)
+  LLMC_PICK(LLMC_FMT_FP4, LLMC_F16)
+  LLMC_PICK(LLMC_FMT_FP4, LLMC_F32)
+#undef LLMC_PICK
+  if (kern == nullptr) return -17;
+  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
   if (e != hipSuccess) return 1000 + (int)e;
   const unsigned wgs = (unsigned)((R + ROWS_PER_WG - 1) / ROWS_PER_WG);
   for (int64_t i1 = 0; i1 < K; i1 += bs) {
     const int count = (int)((K - i1) < bs ? (K - i1) : bs);
     p.i1 = (int)i1;
     p.count = count;
-    hipLaunchKernelGGL(gptq_block_kernel, dim3(wgs), dim3(256), smem, st, p);
+    hipLaunchKernelGGL(kern, dim3(wgs), dim3(256), smem, st, p);
     LLMC_LAUNCH_STATUS();
     const int64_t i2 = i1 + count;
     if (i2 < K) {
