@@ -89,7 +89,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--batches", type=int, default=256, help="calibration batches per step (config: 256)")
     ap.add_argument("--tokens", type=int, default=2048, help="tokens per batch (config: 2048)")
-    ap.add_argument("--stage-tokens", type=int, default=8192,
+    ap.add_argument("--stage-tokens", type=int, default=16384,
                     help="tokens staged per Hessian launch (GPTQModifier.hessian_batch_tokens; 0 = one launch per batch)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     a = ap.parse_args()

@@ -177,7 +177,12 @@ __global__ __launch_bounds__(256) void hessian_syrk_kernel(float* __restrict__ H
       for (int a = 0; a < MI; ++a) fa[a] = *(const uint4*)(curA + chunk_off(wm * (BT / 2) + a * 32 + (lane & 31), q));
 #pragma unroll
       for (int b = 0; b < MI; ++b) fb[b] = *(const uint4*)(curB + chunk_off(wn * (BT / 2) + b * 32 + (lane & 31), q));
-      if (STORE && ks >= 2) store_cols(nxtA, nxtA + PANEL, (ks - 2) * 4, (ks - 2) * 4 + 4);
+      if (STORE && ks >= 2) {
+        // keep the transposing stores (and the wait for the global loads they consume) in the second
+        // half of the slab: the loads were issued at the end of the previous slab and need the time
+        if (ks == 2) __builtin_amdgcn_sched_barrier(0);
+        store_cols(nxtA, nxtA + PANEL, (ks - 2) * 4, (ks - 2) * 4 + 4);
+      }
 #pragma unroll
       for (int a = 0; a < MI; ++a)
 #pragma unroll
