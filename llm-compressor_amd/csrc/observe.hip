@@ -46,31 +46,31 @@ __device__ __forceinline__ void minmax16(const void* p, float& mn, float& mx) {
   }
 }
 
-// Groups of g = L * N elements, L (power of two <= 64) lanes per group, one 16-byte load per lane.
-template <int DT>
-__global__ __launch_bounds__(256) void minmax_seg_kernel(const void* __restrict__ x, int64_t ldw,
-                                                         int64_t ngroups_total, int ng, int g, int L,
-                                                         void* __restrict__ mn_out,
-                                                         void* __restrict__ mx_out) {
+// Groups of g = L * VPL * N elements: one workgroup walks one row, L (power of two <= 64)
+// neighbouring lanes share a group and each lane loads VPL consecutive 16-byte vectors.
+template <int DT, int VPL>
+__global__ __launch_bounds__(256) void minmax_rows_kernel(const void* __restrict__ x, int64_t ldw, int upr,
+                                                          int ng, int lshift, void* __restrict__ mn_out,
+                                                          void* __restrict__ mx_out) {
   constexpr int N = Vec<DT>::N;
-  const int64_t gtid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const int64_t grp = gtid / L;
-  const int sub = (int)(gtid % L);
-  float mn = INFINITY, mx = -INFINITY;
-  const bool live = grp < ngroups_total;
-  if (live) {
-    const int64_t r = grp / ng, gi = grp % ng;
-    const char* p = (const char*)x + (r * ldw + gi * g + (int64_t)sub * N) * (DT == LLMC_F32 ? 4 : 2);
-    minmax16<DT>(p, mn, mx);
+  const int64_t r = blockIdx.x;
+  const char* row = (const char*)x + r * ldw * (DT == LLMC_F32 ? 4 : 2);
+  const int L = 1 << lshift;
+  for (int u = threadIdx.x; u < upr; u += 256) {
+    float mn = INFINITY, mx = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < VPL; ++k) minmax16<DT>(row + ((int64_t)u * VPL + k) * 16, mn, mx);
+    for (int o = L >> 1; o > 0; o >>= 1) {
+      mn = fminf(mn, __shfl_xor(mn, o, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    }
+    if ((u & (L - 1)) == 0) {
+      const int64_t grp = r * ng + (u >> lshift);
+      store_from_f32<DT>(mn_out, grp, mn);
+      store_from_f32<DT>(mx_out, grp, mx);
+    }
   }
-  for (int o = L >> 1; o > 0; o >>= 1) {
-    mn = fminf(mn, __shfl_xor(mn, o, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, o, 64));
-  }
-  if (live && sub == 0) {
-    store_from_f32<DT>(mn_out, grp, mn);
-    store_from_f32<DT>(mx_out, grp, mx);
-  }
+  (void)N;
 }
 
 // One wave per (group, split): strided 16-byte loads when VEC, element loads otherwise.
@@ -233,11 +233,19 @@ int observe_groups(const void* x, int64_t R, int64_t K, int64_t ldw, int64_t g, 
   const int64_t ng = K / g;
   const int64_t total = R * ng;
   const bool aligned = (((uintptr_t)x) & 15) == 0 && (ldw % N) == 0 && (g % N) == 0;
-  const int64_t L = g / N;
-  if (aligned && L >= 1 && L <= 64 && (L & (L - 1)) == 0) {
-    const int64_t threads = total * L;
-    hipLaunchKernelGGL((minmax_seg_kernel<DT>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st,
-                       x, ldw, total, (int)ng, (int)g, (int)L, mn, mx);
+  const int64_t L = g / N;  // 16-byte vectors per group
+  if (aligned && L >= 1 && L <= 128 && (L & (L - 1)) == 0 && R <= 0x7fffffffLL && K <= (1LL << 30)) {
+    const int vpl = L >= 2 ? 2 : 1;
+    const int lanes = (int)(L / vpl);
+    int lshift = 0;
+    while ((1 << lshift) < lanes) ++lshift;
+    const int upr = (int)(K / (N * vpl));
+    if (vpl == 2)
+      hipLaunchKernelGGL((minmax_rows_kernel<DT, 2>), dim3((unsigned)R), dim3(256), 0, st, x, ldw, upr, (int)ng,
+                         lshift, mn, mx);
+    else
+      hipLaunchKernelGGL((minmax_rows_kernel<DT, 1>), dim3((unsigned)R), dim3(256), 0, st, x, ldw, upr, (int)ng,
+                         lshift, mn, mx);
     LLMC_LAUNCH_STATUS();
     return 0;
   }

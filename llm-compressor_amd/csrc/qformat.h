@@ -84,6 +84,59 @@ __device__ __forceinline__ uint8_t e2m1_index(float mag) {
   return mag < 2.0f ? (uint8_t)(mag * 2.0f) : mag < 4.0f ? (uint8_t)(mag + 2.0f) : mag == 4.0f ? 6 : 7;
 }
 
+// ---- gfx950 conversion instructions.  v_cvt_pk_fp8_f32 rounds to OCP e4m3fn (nearest even) and
+// v_cvt_scalef32_pk_fp4_f32 to e2m1 (ties to the even mantissa); on inputs already clamped to the
+// format's range both give the same bytes as e4m3_encode(e4m3_round(v)) and the e2m1_index /
+// sign-bit-3 nibble above, including the sign bit of a negative value that rounds to zero.
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+// two e4m3 bytes: a in bits 7:0, b in bits 15:8
+__device__ __forceinline__ uint32_t hw_e4m3_pair(float a, float b) {
+  return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false) & 0xffffu;
+}
+__device__ __forceinline__ f32x2_t hw_e4m3_pair_decode(uint32_t w) {
+  return __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false);
+}
+// two e2m1 nibbles in one byte: a in bits 3:0, b in bits 7:4
+__device__ __forceinline__ uint32_t hw_e2m1_pair(float a, float b) {
+  return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(0u, a, b, 1.0f, 0) & 0xffu;
+}
+__device__ __forceinline__ f32x2_t hw_e2m1_pair_decode(uint32_t byte) {
+  return __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(byte, 1.0f, 0);
+}
+
+// ---- division by a value shared by many elements.  The steps are those of the correctly
+// rounded fp32 division sequence (reciprocal with one Newton step, quotient with two residual
+// corrections) with the divisor's part hoisted; they give the IEEE quotient whenever nothing
+// under- or overflows on the way, which `ok` and fastdiv_trusted() bound from the divisor's and
+// the quotient's magnitudes.  Callers redo the division with `/` when the bound fails.
+struct FastDiv {
+  float s, y;
+  bool ok;
+};
+__device__ __forceinline__ FastDiv make_fastdiv(float s) {
+  FastDiv d;
+  d.s = s;
+  const float y0 = __builtin_amdgcn_rcpf(s);
+  const float e = fmaf(-s, y0, 1.0f);
+  d.y = fmaf(e, y0, y0);
+  const float a = fabsf(s);
+  d.ok = a > 0x1p-60f && a < 0x1p60f;
+  return d;
+}
+__device__ __forceinline__ float fastdiv(float x, const FastDiv& d) {
+  float q = x * d.y;
+  float r = fmaf(-d.s, q, x);
+  q = fmaf(r, d.y, q);
+  r = fmaf(-d.s, q, x);
+  return fmaf(r, d.y, q);
+}
+// quotient magnitudes for which fastdiv() is exact given d.ok: below 2^100 nothing overflowed
+// (NaN fails the test too); from 2^-40 up the residuals stayed normal.  An exact zero quotient
+// of a zero dividend is exact as well.
+__device__ __forceinline__ bool fastdiv_big_ok(float q) { return fabsf(q) < 0x1p100f; }
+__device__ __forceinline__ bool fastdiv_small(float q) { return fabsf(q) < 0x1p-40f; }
+
 struct QFormat {
   int fmt;   // LLMC_FMT_*
   float qmin, qmax;

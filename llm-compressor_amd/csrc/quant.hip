@@ -173,6 +173,260 @@ __global__ __launch_bounds__(256) void quantize_kernel(QuantParams p) {
   }
 }
 
+// ---- the common case: 16-bit input with K % 8 == 0, scales in the input's dtype or fp32,
+// power-of-two (or whole-row) column groups, no g_idx, 4/8-bit ints, e4m3 or e2m1.
+// One workgroup walks one row in 16-byte chunks with 32-bit index arithmetic; everything the
+// format decides is a template parameter so the per-element path is branch-free: shared-divisor
+// division, rounding to the quotient's dtype, clamp, and the hardware e4m3/e2m1 conversions.
+template <int XDT>
+__device__ __forceinline__ void unpack8(const uint4& v, float* x) {
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    if (XDT == LLMC_BF16) {
+      x[2 * j] = __uint_as_float(w[j] << 16);
+      x[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+    } else {
+      x[2 * j] = f16_bits_to_f32((uint16_t)(w[j] & 0xffffu));
+      x[2 * j + 1] = f16_bits_to_f32((uint16_t)(w[j] >> 16));
+    }
+  }
+}
+
+// two fp32 values rounded (nearest even) to the 16-bit type DT, packed lo | hi << 16; bf16 goes
+// through the packed conversion instruction
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+template <int DT>
+__device__ __forceinline__ uint32_t pack16(float lo, float hi) {
+  const f32x2_t v = {lo, hi};
+  uint32_t w;
+  if (DT == LLMC_BF16) {
+    const bf16x2_t b = __builtin_convertvector(v, bf16x2_t);
+    __builtin_memcpy(&w, &b, 4);
+  } else {
+    const f16x2_t h = __builtin_convertvector(v, f16x2_t);
+    __builtin_memcpy(&w, &h, 4);
+  }
+  return w;
+}
+template <int DT>
+__device__ __forceinline__ float round16_finite(float f) {
+  if (DT == LLMC_BF16) return (float)(__bf16)f;
+  return (float)(_Float16)f;
+}
+
+// SM: 0 = scales in the input's 16-bit dtype, 1 = fp32 scales, 2 = stored scale / global scale (fp32)
+// A lane handles 16 consecutive columns (two 16-byte loads), which share one scale.
+template <int XDT, int SM, int FMT, bool HAS_ZP, int OUT>
+__global__ __launch_bounds__(256) void quantize_rows_kernel(QuantParams p, int cshift) {
+  constexpr bool S32 = SM != 0;
+  constexpr int PD = S32 ? LLMC_F32 : XDT;  // dtype of the quotient and of the dequantised value
+  constexpr int E = 16;
+  const int64_t r = blockIdx.x;
+  const int upr = (int)(p.K >> 4);
+  const uint16_t* xr = (const uint16_t*)p.x + r * p.ldx;
+  const int64_t srow_off = (p.rdiv == 1 ? r : r / p.rdiv) * p.srow;
+  const QFormat f = make_qformat(FMT, p.bits);
+  float gs = 1.f;
+  if (SM == 2) gs = p.gscale[0];
+
+  for (int u = threadIdx.x; u < upr; u += 256) {
+    const uint4 raw0 = *(const uint4*)(xr + (u << 4));
+    const uint4 raw1 = *(const uint4*)(xr + (u << 4) + 8);
+    const int64_t si = srow_off + ((u << 4) >> cshift);
+    float s;
+    if (SM == 0)
+      s = load_as_f32<XDT>(p.scale, si);
+    else if (SM == 1)
+      s = ((const float*)p.scale)[si];
+    else
+      s = load_rt(p.scale, si, p.scale_dt) / gs;
+    const float zp = HAS_ZP ? (float)p.zp[si] : 0.f;
+    float x[E], v[E];
+    unpack8<XDT>(raw0, x);
+    unpack8<XDT>(raw1, x + 8);
+    const FastDiv d = make_fastdiv(s);
+    bool big = false, small = false;
+#pragma unroll
+    for (int j = 0; j < E; ++j) {
+      v[j] = fastdiv(x[j], d);
+      big = big | !fastdiv_big_ok(v[j]);
+      small = small | fastdiv_small(v[j]);
+    }
+    bool redo = big | !d.ok;
+    if (small) {
+#pragma unroll
+      for (int j = 0; j < E; ++j) redo = redo | (fastdiv_small(v[j]) & (x[j] != 0.f));
+    }
+    if (redo) {
+      // out-of-range divisor or quotient, NaN: the plain division, then the same tail
+#pragma unroll
+      for (int j = 0; j < E; ++j) {
+        v[j] = round_rt(x[j] / s, PD);
+        v[j] = HAS_ZP ? round_rt(v[j] + zp, PD) : v[j] + 0.0f;
+        v[j] = fminf(fmaxf(v[j], f.qmin), f.qmax);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < E; ++j) {
+        if (!S32) v[j] = round16_finite<XDT>(v[j]);
+        if (HAS_ZP)
+          v[j] = S32 ? v[j] + zp : round16_finite<XDT>(v[j] + zp);
+        else if (FMT != LLMC_FMT_INT || OUT == LLMC_OUT_FAKEQUANT)
+          v[j] = v[j] + 0.0f;  // the reference adds a zero zero-point: -0.0 becomes +0.0
+        v[j] = __builtin_amdgcn_fmed3f(v[j], f.qmin, f.qmax);
+      }
+    }
+
+    // element codes: e4m3 bytes / e2m1 nibbles via the conversion instructions
+    uint32_t fp8w[4] = {0u, 0u, 0u, 0u}, fp4w[2] = {0u, 0u};
+    if (FMT == LLMC_FMT_FP8) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) fp8w[j >> 1] |= hw_e4m3_pair(v[2 * j], v[2 * j + 1]) << (16 * (j & 1));
+    } else if (FMT == LLMC_FMT_FP4) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) fp4w[j >> 2] |= hw_e2m1_pair(v[2 * j], v[2 * j + 1]) << (8 * (j & 3));
+    }
+
+    if (OUT == LLMC_OUT_FAKEQUANT) {
+      if (FMT == LLMC_FMT_INT) {
+#pragma unroll
+        for (int j = 0; j < E; ++j) v[j] = rintf(v[j]);
+      } else if (FMT == LLMC_FMT_FP8) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const f32x2_t t = hw_e4m3_pair_decode(fp8w[j >> 1] >> (16 * (j & 1)));
+          v[2 * j] = t.x;
+          v[2 * j + 1] = t.y;
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const f32x2_t t = hw_e2m1_pair_decode(fp4w[j >> 2] >> (8 * (j & 3)));
+          v[2 * j] = t.x;
+          v[2 * j + 1] = t.y;
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < E; ++j) {
+        if (HAS_ZP) v[j] = round_rt(v[j] - zp, PD);
+        v[j] *= s;  // rounding to PD, then to the output's dtype, is one rounding
+      }
+      uint16_t* o = (uint16_t*)p.out + r * p.ldo + (u << 4);
+      *(uint4*)o = make_uint4(pack16<XDT>(v[0], v[1]), pack16<XDT>(v[2], v[3]), pack16<XDT>(v[4], v[5]),
+                              pack16<XDT>(v[6], v[7]));
+      *(uint4*)(o + 8) = make_uint4(pack16<XDT>(v[8], v[9]), pack16<XDT>(v[10], v[11]),
+                                    pack16<XDT>(v[12], v[13]), pack16<XDT>(v[14], v[15]));
+      continue;
+    }
+
+    if (FMT == LLMC_FMT_FP8) {  // bytes either way
+      *(uint4*)((uint8_t*)p.out + r * p.ldo + (u << 4)) = make_uint4(fp8w[0], fp8w[1], fp8w[2], fp8w[3]);
+    } else if (FMT == LLMC_FMT_FP4) {
+      if (OUT == LLMC_OUT_PACKED) {
+        *(uint2*)((uint8_t*)p.out + r * p.ldo + (u << 3)) = make_uint2(fp4w[0], fp4w[1]);
+      } else {  // one nibble per byte
+        uint32_t w[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const uint32_t h = (fp4w[k >> 1] >> (16 * (k & 1))) & 0xffffu;
+          w[k] = (h & 0xfu) | ((h & 0xf0u) << 4) | ((h & 0xf00u) << 8) | ((h & 0xf000u) << 12);
+        }
+        *(uint4*)((uint8_t*)p.out + r * p.ldo + (u << 4)) = make_uint4(w[0], w[1], w[2], w[3]);
+      }
+    } else {
+      // v + 1.5*2^23 rounds v to the nearest-even integer and leaves it, two's complement, in the
+      // low mantissa bits; funnel shifts collect the low 4 or 8 bits of each element
+      uint32_t q[E];
+#pragma unroll
+      for (int j = 0; j < E; ++j) q[j] = __float_as_uint(v[j] + 12582912.0f);
+      if (OUT == LLMC_OUT_CODES || p.bits == 8) {
+        // int8 codes, or int8 fields (offset binary) four to a word: the same byte positions
+        uint32_t w[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int j = 0; j < E; ++j) w[j >> 2] = __builtin_amdgcn_alignbit(q[j], w[j >> 2], 8);
+        if (OUT == LLMC_OUT_CODES) {
+          *(uint4*)((uint8_t*)p.out + r * p.ldo + (u << 4)) = make_uint4(w[0], w[1], w[2], w[3]);
+        } else {
+          const uint32_t m = 0x80808080u;
+          *(uint4*)((uint32_t*)p.out + r * p.ldo + (u << 2)) = make_uint4(w[0] ^ m, w[1] ^ m, w[2] ^ m, w[3] ^ m);
+        }
+      } else {  // sixteen 4-bit fields, offset binary
+        uint32_t w[2] = {0u, 0u};
+#pragma unroll
+        for (int j = 0; j < E; ++j) w[j >> 3] = __builtin_amdgcn_alignbit(q[j], w[j >> 3], 4);
+        *(uint2*)((uint32_t*)p.out + r * p.ldo + (u << 1)) = make_uint2(w[0] ^ 0x88888888u, w[1] ^ 0x88888888u);
+      }
+    }
+  }
+}
+
+template <int XDT, int SM, int FMT, bool HAS_ZP>
+void launch_rows_out(const QuantParams& p, int cshift, hipStream_t st) {
+  const dim3 grid((unsigned)p.R), block(256);
+  if (p.out_mode == LLMC_OUT_FAKEQUANT)
+    hipLaunchKernelGGL((quantize_rows_kernel<XDT, SM, FMT, HAS_ZP, LLMC_OUT_FAKEQUANT>), grid, block, 0, st, p, cshift);
+  else if (p.out_mode == LLMC_OUT_CODES)
+    hipLaunchKernelGGL((quantize_rows_kernel<XDT, SM, FMT, HAS_ZP, LLMC_OUT_CODES>), grid, block, 0, st, p, cshift);
+  else
+    hipLaunchKernelGGL((quantize_rows_kernel<XDT, SM, FMT, HAS_ZP, LLMC_OUT_PACKED>), grid, block, 0, st, p, cshift);
+}
+
+template <int XDT, int SM>
+void launch_rows_fmt(const QuantParams& p, int cshift, hipStream_t st) {
+  if (p.fmt == LLMC_FMT_INT) {
+    if (p.zp)
+      launch_rows_out<XDT, SM, LLMC_FMT_INT, true>(p, cshift, st);
+    else
+      launch_rows_out<XDT, SM, LLMC_FMT_INT, false>(p, cshift, st);
+  } else if (p.fmt == LLMC_FMT_FP8) {
+    launch_rows_out<XDT, SM, LLMC_FMT_FP8, false>(p, cshift, st);
+  } else {
+    launch_rows_out<XDT, SM, LLMC_FMT_FP4, false>(p, cshift, st);
+  }
+}
+
+// launches the row kernel when the call fits its assumptions; false = use the general kernel
+bool try_launch_rows(const QuantParams& p, hipStream_t st) {
+  if (p.x_dt == LLMC_F32 || p.g_idx || p.K % 16 || p.ldx % 8 || ((uintptr_t)p.x & 15)) return false;
+  if (p.R > 0x7fffffffLL || p.K > (1LL << 30)) return false;
+  const int eff = p.gscale ? LLMC_F32 : p.scale_dt;
+  if (eff != LLMC_F32 && eff != p.x_dt) return false;
+  if (p.zp && p.fmt != LLMC_FMT_INT) return false;
+  if (p.fmt == LLMC_FMT_INT && p.bits != 4 && p.bits != 8) return false;
+  int cshift;
+  if (p.cdiv >= p.K) {
+    cshift = 31;
+  } else {
+    if (p.cdiv < 16 || (p.cdiv & (p.cdiv - 1))) return false;
+    cshift = 0;
+    while ((1LL << cshift) < p.cdiv) ++cshift;
+  }
+  if (p.out_mode == LLMC_OUT_FAKEQUANT) {
+    if (p.out_dt != p.x_dt || p.ldo % 8 || ((uintptr_t)p.out & 15)) return false;
+  } else if (p.out_mode == LLMC_OUT_CODES || p.fmt == LLMC_FMT_FP8) {
+    if (p.ldo % 16 || ((uintptr_t)p.out & 15)) return false;  // 16 bytes per lane
+  } else if (p.fmt == LLMC_FMT_FP4) {
+    if (p.ldo % 8 || ((uintptr_t)p.out & 7)) return false;  // 8 bytes per lane
+  } else if (p.bits == 8) {
+    if (p.ldo % 4 || ((uintptr_t)p.out & 15)) return false;  // four int32 words per lane
+  } else {
+    if (p.ldo % 2 || ((uintptr_t)p.out & 7)) return false;  // two int32 words per lane
+  }
+  const int sm = p.gscale ? 2 : (eff == LLMC_F32 ? 1 : 0);
+  if (p.x_dt == LLMC_BF16) {
+    if (sm == 0) launch_rows_fmt<LLMC_BF16, 0>(p, cshift, st);
+    else if (sm == 1) launch_rows_fmt<LLMC_BF16, 1>(p, cshift, st);
+    else launch_rows_fmt<LLMC_BF16, 2>(p, cshift, st);
+  } else {
+    if (sm == 0) launch_rows_fmt<LLMC_F16, 0>(p, cshift, st);
+    else if (sm == 1) launch_rows_fmt<LLMC_F16, 1>(p, cshift, st);
+    else launch_rows_fmt<LLMC_F16, 2>(p, cshift, st);
+  }
+  return true;
+}
+
 // Per-token dynamic quantisation: one workgroup per row.  The row is staged in LDS while
 // its absmax is reduced, so HBM sees one read and one write per element.
 template <int DT>
@@ -259,6 +513,129 @@ __global__ __launch_bounds__(256) void dynamic_token_kernel(const void* __restri
   }
 }
 
+// Per-token dynamic quantisation, rows of up to 8192 elements: one wavefront per row, the row
+// held in registers between the absmax reduction and the quantisation (one HBM read, one write,
+// no LDS, no workgroup barrier).  Lane l of the wave owns 16-byte chunks l, l+64, ...
+template <int DT, int NC, int FMT, int OUT>
+__global__ __launch_bounds__(256) void dynamic_token_wave_kernel(const void* __restrict__ x, int64_t ldx, int64_t N,
+                                                                 int K, int bits, void* __restrict__ out,
+                                                                 int64_t ldo, void* __restrict__ scale_out) {
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= N) return;
+  const uint16_t* xr = (const uint16_t*)x + r * ldx;
+  const int nchunk = K >> 3;
+  uint4 raw[NC];
+  typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
+  u16x2_t m = {0, 0};  // packed max of 15-bit magnitudes (magnitude bits order like the values)
+#pragma unroll
+  for (int i = 0; i < NC; ++i) {
+    const int c = i * 64 + lane;
+    raw[i] = c < nchunk ? *(const uint4*)(xr + (c << 3)) : make_uint4(0, 0, 0, 0);
+  }
+#pragma unroll
+  for (int i = 0; i < NC; ++i) {
+    const uint32_t w[4] = {raw[i].x, raw[i].y, raw[i].z, raw[i].w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t a = w[j] & 0x7fff7fffu;
+      u16x2_t av;
+      __builtin_memcpy(&av, &a, 4);
+      m = __builtin_elementwise_max(m, av);
+    }
+  }
+  uint32_t mm = max((uint32_t)m.x, (uint32_t)m.y);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) mm = max(mm, (uint32_t)__shfl_xor((int)mm, o, 64));
+  const float amax = DT == LLMC_BF16 ? bf16_bits_to_f32((uint16_t)mm) : f16_bits_to_f32((uint16_t)mm);
+  const QFormat f = make_qformat(FMT, bits);
+  float s = round_to<DT>(amax / ((f.qmax - f.qmin) * 0.5f));
+  if (s == 0.f) s = dtype_eps(DT);
+  if (lane == 0) store_from_f32<DT>(scale_out, r, s);
+  const FastDiv d = make_fastdiv(s);
+
+#pragma unroll
+  for (int i = 0; i < NC; ++i) {
+    const int c = i * 64 + lane;
+    if (c >= nchunk) break;
+    float xv[8], v[8];
+    unpack8<DT>(raw[i], xv);
+    bool big = false, small = false;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      v[j] = fastdiv(xv[j], d);
+      big = big | !fastdiv_big_ok(v[j]);
+      small = small | fastdiv_small(v[j]);
+    }
+    bool redo = big | !d.ok;
+    if (small) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) redo = redo | (fastdiv_small(v[j]) & (xv[j] != 0.f));
+    }
+    if (redo) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = fminf(fmaxf(round_to<DT>(xv[j] / s) + 0.0f, f.qmin), f.qmax);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        v[j] = __builtin_amdgcn_fmed3f(round16_finite<DT>(v[j]) + 0.0f, f.qmin, f.qmax);
+    }
+    uint32_t cw[2] = {0u, 0u};  // the eight element bytes
+    if (FMT == LLMC_FMT_FP8) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) cw[j >> 1] |= hw_e4m3_pair(v[2 * j], v[2 * j + 1]) << (16 * (j & 1));
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        cw[j >> 2] = __builtin_amdgcn_alignbit(__float_as_uint(v[j] + 12582912.0f), cw[j >> 2], 8);
+    }
+    if (OUT == LLMC_OUT_CODES) {
+      *(uint2*)((uint8_t*)out + r * ldo + (c << 3)) = make_uint2(cw[0], cw[1]);
+    } else {
+      if (FMT == LLMC_FMT_FP8) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const f32x2_t t = hw_e4m3_pair_decode(cw[j >> 1] >> (16 * (j & 1)));
+          v[2 * j] = t.x;
+          v[2 * j + 1] = t.y;
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = rintf(v[j]);
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] *= s;
+      *(uint4*)((uint16_t*)out + r * ldo + (c << 3)) =
+          make_uint4(pack16<DT>(v[0], v[1]), pack16<DT>(v[2], v[3]), pack16<DT>(v[4], v[5]), pack16<DT>(v[6], v[7]));
+    }
+  }
+}
+
+template <int DT, int NC>
+void launch_token_wave(const void* x, int64_t ldx, int64_t N, int K, int fmt, int bits, int out_mode, void* out,
+                       int64_t ldo, void* scale_out, hipStream_t st) {
+  const dim3 grid((unsigned)((N + 3) / 4)), block(256);
+#define LLMC_TOK(F, O) \
+  hipLaunchKernelGGL((dynamic_token_wave_kernel<DT, NC, F, O>), grid, block, 0, st, x, ldx, N, K, bits, out, ldo, scale_out)
+  if (fmt == LLMC_FMT_FP8) {
+    if (out_mode == LLMC_OUT_CODES) LLMC_TOK(LLMC_FMT_FP8, LLMC_OUT_CODES);
+    else LLMC_TOK(LLMC_FMT_FP8, LLMC_OUT_FAKEQUANT);
+  } else {
+    if (out_mode == LLMC_OUT_CODES) LLMC_TOK(LLMC_FMT_INT, LLMC_OUT_CODES);
+    else LLMC_TOK(LLMC_FMT_INT, LLMC_OUT_FAKEQUANT);
+  }
+#undef LLMC_TOK
+}
+
+template <int DT>
+void launch_token_wave_nc(const void* x, int64_t ldx, int64_t N, int K, int fmt, int bits, int out_mode,
+                          void* out, int64_t ldo, void* scale_out, hipStream_t st) {
+  const int nc = (K / 8 + 63) / 64;
+  if (nc <= 2) launch_token_wave<DT, 2>(x, ldx, N, K, fmt, bits, out_mode, out, ldo, scale_out, st);
+  else if (nc <= 8) launch_token_wave<DT, 8>(x, ldx, N, K, fmt, bits, out_mode, out, ldo, scale_out, st);
+  else launch_token_wave<DT, 16>(x, ldx, N, K, fmt, bits, out_mode, out, ldo, scale_out, st);
+}
+
 __global__ void fill_u32_kernel(uint32_t* p, int64_t n) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i < n) p[i] = 0u;
@@ -297,6 +674,10 @@ extern "C" int llmc_quantize(const void* x, int32_t x_dtype, int64_t R, int64_t 
   p.sd = eff_scale_dt;
   p.out_mode = out_mode; p.out = out; p.out_dt = out_dtype; p.ldo = ldo;
 
+  if (try_launch_rows(p, st)) {
+    LLMC_LAUNCH_STATUS();
+    return 0;
+  }
   bool vec = (K % 8 == 0) && (col_div % 8 == 0) && g_idx == nullptr && (((uintptr_t)x & 15) == 0) &&
              (x_dtype == LLMC_F32 || ldx % 8 == 0);
   if (out_mode == LLMC_OUT_FAKEQUANT)
@@ -337,6 +718,18 @@ extern "C" int llmc_dynamic_per_token_quantize(const void* x, int32_t x_dtype, i
   LLMC_CHECK_ARG(out_mode == LLMC_OUT_FAKEQUANT || out_mode == LLMC_OUT_CODES, 8);
   LLMC_CHECK_ARG(out && scale_out, 9);
   hipStream_t st = (hipStream_t)stream;
+  const bool wave_ok = K % 8 == 0 && K <= 8192 && ldx % 8 == 0 && (((uintptr_t)x) & 15) == 0 &&
+                       (out_mode == LLMC_OUT_CODES ? (ldo % 8 == 0 && (((uintptr_t)out) & 7) == 0)
+                                                   : (ldo % 8 == 0 && (((uintptr_t)out) & 15) == 0));
+  if (wave_ok) {
+    const int nb = fmt == LLMC_FMT_INT ? num_bits : 8;
+    if (x_dtype == LLMC_BF16)
+      launch_token_wave_nc<LLMC_BF16>(x, ldx, N, (int)K, fmt, nb, out_mode, out, ldo, scale_out, st);
+    else
+      launch_token_wave_nc<LLMC_F16>(x, ldx, N, (int)K, fmt, nb, out_mode, out, ldo, scale_out, st);
+    LLMC_LAUNCH_STATUS();
+    return 0;
+  }
   const size_t smem = (size_t)((K + 7) / 8 * 8) * 2;
   auto kern = x_dtype == LLMC_BF16 ? dynamic_token_kernel<LLMC_BF16> : dynamic_token_kernel<LLMC_F16>;
   if (smem > 48 * 1024) {

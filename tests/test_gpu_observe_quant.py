@@ -186,7 +186,63 @@ def test_quantize_with_g_idx_and_fp32_input():
     assert _same(got, exp)
 
 
-@pytest.mark.parametrize("N,K", [(64, 4096), (7, 100), (3, 12288)])
+@pytest.mark.parametrize("case", ["int4_bf16scale", "int8_asym_bf16scale", "fp8_f32scale", "fp4_bf16scale", "fp4_gscale"])
+def test_quantize_every_bf16_value_and_extreme_scales(case):
+    """Every finite-or-infinite bf16 bit pattern as a dividend, against per-row scales from 2^-100 to 2^100:
+    the shared-divisor division of the row kernel must give the bytes the plain division gives
+    (quotients that overflow, underflow, hit ties or vanish included).  NaN inputs are left out:
+    the reference's integer cast of NaN is not defined."""
+    from llmcompressor_amd import ops
+
+    bits = torch.arange(65536, dtype=torch.int32)
+    exp_field = (bits >> 7) & 0xFF
+    keep = ~((exp_field == 0xFF) & ((bits & 0x7F) != 0))
+    vals = bits[keep].to(torch.int16).view(torch.bfloat16)  # 65282 values
+    K = 256
+    vals = vals[: (vals.numel() // K) * K]
+    g = torch.Generator().manual_seed(3)
+    vals = vals[torch.randperm(vals.numel(), generator=g)]
+    w = vals.view(-1, K).repeat(4, 1).contiguous()  # every value meets several scales
+    R = w.shape[0]
+    exps = torch.tensor([-100.0, -70.0, -61.0, -59.0, -40.0, -20.0, -9.0, -5.5, -1.0, 0.0, 0.3, 3.0, 11.0, 40.0, 59.0, 61.0, 100.0])
+    sc = torch.exp2(exps[torch.arange(R) % exps.numel()]) * (1.0 + torch.rand(R, generator=g))
+    kw = dict(global_scale=None)
+    zp = None
+    if case == "int4_bf16scale":
+        args, fmt, nb, scale = F.QArgs(num_bits=4, strategy="channel"), ops.FMT_INT, 4, sc.bfloat16()
+    elif case == "int8_asym_bf16scale":
+        args, fmt, nb, scale = F.QArgs(num_bits=8, strategy="channel", symmetric=False), ops.FMT_INT, 8, sc.bfloat16()
+        zp = torch.randint(-128, 128, (R, 1), generator=g).to(torch.int8)
+    elif case == "fp8_f32scale":
+        args, fmt, nb, scale = F.QArgs(num_bits=8, type="float", strategy="channel"), ops.FMT_FP8, 8, sc.float()
+    elif case == "fp4_bf16scale":
+        args, fmt, nb, scale = F.QArgs(num_bits=4, type="float", strategy="channel"), ops.FMT_FP4, 4, sc.bfloat16()
+    else:
+        args, fmt, nb = F.QArgs(num_bits=4, type="float", strategy="channel"), ops.FMT_FP4, 4
+        scale = sc.clamp(min=2.0**-9, max=448.0).to(E4M3).float()  # an e4m3 scale is never stored as zero
+        kw = dict(global_scale=torch.tensor([37.25]))
+    scale = scale.view(R, 1)
+    ozp = zp.to(scale.dtype) if zp is not None else torch.zeros_like(scale)
+    exp_fq = F.fake_quantize(w, scale, ozp, args, **kw)
+    gkw = {k: (v.cuda() if v is not None else None) for k, v in kw.items()}
+    gzp = zp.cuda() if zp is not None else None
+    fq = ops.quantize(w.cuda(), scale.cuda(), gzp, fmt, nb, 1, 1, 1 << 40, out_mode=ops.OUT_FAKEQUANT, **gkw)
+    fin = torch.isfinite(exp_fq.float())
+    assert torch.equal(torch.isfinite(fq.float().cpu()), fin)
+    assert torch.equal(_bits(fq.cpu())[fin], _bits(exp_fq.to(torch.bfloat16))[fin]), case
+    pk = ops.quantize(w.cuda(), scale.cuda(), gzp, fmt, nb, 1, 1, 1 << 40, out_mode=ops.OUT_PACKED, **gkw)
+    if fmt == ops.FMT_INT:
+        codes = F.quantize(w, scale, ozp, args, dtype=torch.int8)
+        assert _same(pk, P.pack_to_int32(codes, nb)), case
+    elif fmt == ops.FMT_FP8:
+        q8 = F.quantize(w, scale, ozp, args, dtype=E4M3)
+        assert torch.equal(pk.cpu().view(torch.uint8), q8.view(torch.uint8))
+    else:
+        q4 = F.quantize(w, scale, ozp, args, **kw)
+        assert _same(pk, P.pack_fp4_to_uint8(q4)), case
+
+
+@pytest.mark.parametrize("N,K", [(64, 4096), (7, 100), (3, 12288), (5, 512), (9, 8192), (6, 1000)])
 def test_dynamic_per_token_fp8(N, K):
     from llmcompressor_amd import ops
 
