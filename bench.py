@@ -92,6 +92,9 @@ def main():
     ap.add_argument("--stage-tokens", type=int, default=16384,
                     help="tokens staged per Hessian launch (GPTQModifier.hessian_batch_tokens; 0 = one launch per batch)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--probe-dominant", type=int, default=0, metavar="N",
+                    help="counter runs: launch only the dominant kernel N times (14336-wide Hessian, --stage-tokens "
+                    "tokens) and N plain copies of a 1 GiB buffer (the known-size kernel the HBM counters are scaled by)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU figure is produced)", file=sys.stderr)
@@ -106,6 +109,17 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if a.probe_dominant:
+        x = torch.randn(a.stage_tokens or a.tokens, INTER, device=dev).bfloat16()
+        H = torch.zeros(INTER, INTER, device=dev)
+        src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(a.probe_dominant):
+            ops.hessian_accumulate_(H, x)
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(f"probe: {a.probe_dominant} x hessian [{x.shape[0]}x{INTER}] + {a.probe_dominant} x copy of {src.numel() * 4} bytes")
+        return
     B, T = a.batches, a.tokens
     gen = torch.Generator(device=dev).manual_seed(0)
 

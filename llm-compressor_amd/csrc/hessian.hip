@@ -121,94 +121,117 @@ __global__ __launch_bounds__(256) void hessian_syrk_kernel(float* __restrict__ H
       for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
 
   uint4 ra[RT], rb[RT];
-  auto load_slab = [&](int t0) {
+  // RT token rows x 8 features of one panel (features col0 + g_i*8 ..) of the slab starting at t0
+  auto load_panel = [&](uint4* rg, int t0, int col0) {
 #pragma unroll
-    for (int r = 0; r < RT; ++r) {
-      const int t = t0 + g_t * RT + r;
-      ra[r] = load8<ALIGNED>(X, ldx, t, i0 + g_i * 8, T, K);
-      rb[r] = load8<ALIGNED>(X, ldx, t, j0 + g_i * 8, T, K);
+    for (int r = 0; r < RT; ++r) rg[r] = load8<ALIGNED>(X, ldx, t0 + g_t * RT + r, col0 + g_i * 8, T, K);
+  };
+  // registers hold RT token rows x 8 features; LDS wants, per feature, RT consecutive tokens:
+  // column c of the thread's 8 features goes out as one 16-byte (RT == 8) or 8-byte LDS write
+  auto store_col = [&](unsigned char* st, const uint4* rg, int c) {
+    uint32_t o[RT / 2];
+    const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
+#pragma unroll
+    for (int q = 0; q < RT / 2; ++q)
+      o[q] = __builtin_amdgcn_perm(dword_of(rg[2 * q + 1], c >> 1), dword_of(rg[2 * q], c >> 1), sel);
+    const int row = g_i * 8 + c;
+    if constexpr (RT == 8) {
+      *(uint4*)(st + chunk_off(row, g_t)) = make_uint4(o[0], o[1], o[2], o[3]);
+    } else {
+      *(uint2*)(st + chunk_off(row, g_t >> 1) + (g_t & 1) * 8) = make_uint2(o[0], o[1]);
     }
   };
-  // registers hold RT token rows x 8 features; LDS wants, per feature, RT consecutive tokens.
-  // Feature columns [c_lo, c_hi) of this thread's 8 are written.
-  auto store_cols = [&](unsigned char* stA, unsigned char* stB, int c_lo, int c_hi) {
+  auto store_panel = [&](unsigned char* st, const uint4* rg) {
 #pragma unroll
-    for (int c = 0; c < 8; ++c) {
-      if (c < c_lo || c >= c_hi) continue;
-      uint32_t oa[RT / 2], ob[RT / 2];
-      const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
-#pragma unroll
-      for (int q = 0; q < RT / 2; ++q) {
-        oa[q] = __builtin_amdgcn_perm(dword_of(ra[2 * q + 1], c >> 1), dword_of(ra[2 * q], c >> 1), sel);
-        ob[q] = __builtin_amdgcn_perm(dword_of(rb[2 * q + 1], c >> 1), dword_of(rb[2 * q], c >> 1), sel);
-      }
-      const int row = g_i * 8 + c;
-      if constexpr (RT == 8) {
-        const int off = chunk_off(row, g_t);
-        *(uint4*)(stA + off) = make_uint4(oa[0], oa[1], oa[2], oa[3]);
-        *(uint4*)(stB + off) = make_uint4(ob[0], ob[1], ob[2], ob[3]);
-      } else {
-        const int off = chunk_off(row, g_t >> 1) + (g_t & 1) * 8;
-        *(uint2*)(stA + off) = make_uint2(oa[0], oa[1]);
-        *(uint2*)(stB + off) = make_uint2(ob[0], ob[1]);
-      }
-    }
+    for (int c = 0; c < 8; ++c) store_col(st, rg, c);
   };
-  // one slab of MFMAs from stage `cur`; when STORE, the second half also transposes the
-  // register-held next slab into stage `nxt` so the LDS writes hide under the matrix ops
-  // zero the token rows of the register-held slab that lie past T (only the last slab has any)
-  auto mask_tail = [&](int t0) {
+  // zero the token rows of a register-held panel that lie past T (only the last slab has any)
+  auto mask_tail = [&](uint4* rg, int t0) {
     if (!ALIGNED) return;  // the element-wise loader already zero-fills
 #pragma unroll
     for (int r = 0; r < RT; ++r) {
       const bool ok = t0 + g_t * RT + r < T;
-      ra[r].x = ok ? ra[r].x : 0u; ra[r].y = ok ? ra[r].y : 0u; ra[r].z = ok ? ra[r].z : 0u; ra[r].w = ok ? ra[r].w : 0u;
-      rb[r].x = ok ? rb[r].x : 0u; rb[r].y = ok ? rb[r].y : 0u; rb[r].z = ok ? rb[r].z : 0u; rb[r].w = ok ? rb[r].w : 0u;
+      rg[r].x = ok ? rg[r].x : 0u; rg[r].y = ok ? rg[r].y : 0u; rg[r].z = ok ? rg[r].z : 0u; rg[r].w = ok ? rg[r].w : 0u;
     }
   };
-  auto compute = [&](unsigned char* curA, unsigned char* nxtA, auto store_tag) {
+  // One slab of matrix ops from stage `cur`, written out as an explicit software pipeline: the
+  // slab is four groups of 16 tokens, each group NSTEP steps of two MFMAs, and every step also
+  // issues its share of (1) the LDS reads of the next group's operand fragments (double-buffered
+  // in registers), (2) when STORE, the transposing LDS writes of the next slab -- first panel
+  // during group 0, second during group 2 -- and (3) the global loads that refill each register
+  // set during the following group (slab after next, starting at token t2).  A scheduling fence
+  // after every step keeps the compiler from regrouping them; with one wave per SIMD nothing
+  // else would cover a stall.
+  auto compute = [&](unsigned char* curA, unsigned char* nxtA, int t2, auto store_tag, auto mask_tag) {
     constexpr bool STORE = decltype(store_tag)::value;
+    constexpr bool MASK = decltype(mask_tag)::value;
+    constexpr int MPS = 2, NSTEP = MI * MI / MPS;  // matrix ops per step, steps per 16-token group
+    constexpr int FPS = 2 * MI / NSTEP, CPS = 8 / NSTEP, LPS = RT / NSTEP;
     unsigned char* curB = curA + PANEL;
+    uint4 fa[2][MI], fb[2][MI];
+    auto read_frag = [&](int ks, int f) {  // fragment f of group ks: f < MI -> A rows, else B rows
+      const int q = ks * 2 + (lane >> 5);
+      if (f < MI)
+        fa[ks & 1][f] = *(const uint4*)(curA + chunk_off(wm * (BT / 2) + f * 32 + (lane & 31), q));
+      else
+        fb[ks & 1][f - MI] = *(const uint4*)(curB + chunk_off(wn * (BT / 2) + (f - MI) * 32 + (lane & 31), q));
+    };
+#pragma unroll
+    for (int f = 0; f < 2 * MI; ++f) read_frag(0, f);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
-      uint4 fa[MI], fb[MI];
-      const int q = ks * 2 + (lane >> 5);
+      if (STORE && MASK && ks == 0) mask_tail(ra, t2 - BK);
+      if (STORE && MASK && ks == 2) mask_tail(rb, t2 - BK);
 #pragma unroll
-      for (int a = 0; a < MI; ++a) fa[a] = *(const uint4*)(curA + chunk_off(wm * (BT / 2) + a * 32 + (lane & 31), q));
+      for (int st = 0; st < NSTEP; ++st) {
+        if (ks + 1 < BK / 16) {
 #pragma unroll
-      for (int b = 0; b < MI; ++b) fb[b] = *(const uint4*)(curB + chunk_off(wn * (BT / 2) + b * 32 + (lane & 31), q));
-      if (STORE && ks >= 2) {
-        // keep the transposing stores (and the wait for the global loads they consume) in the second
-        // half of the slab: the loads were issued at the end of the previous slab and need the time
-        if (ks == 2) __builtin_amdgcn_sched_barrier(0);
-        store_cols(nxtA, nxtA + PANEL, (ks - 2) * 4, (ks - 2) * 4 + 4);
+          for (int f = st * FPS; f < (st + 1) * FPS; ++f) read_frag(ks + 1, f);
+        }
+        if (STORE) {
+#pragma unroll
+          for (int c = st * CPS; c < (st + 1) * CPS; ++c) {
+            if (ks == 0) store_col(nxtA, ra, c);
+            if (ks == 2) store_col(nxtA + PANEL, rb, c);
+          }
+#pragma unroll
+          for (int r = st * LPS; r < (st + 1) * LPS; ++r) {
+            if (ks == 1) ra[r] = load8<ALIGNED>(X, ldx, t2 + g_t * RT + r, i0 + g_i * 8, T, K);
+            if (ks == 3) rb[r] = load8<ALIGNED>(X, ldx, t2 + g_t * RT + r, j0 + g_i * 8, T, K);
+          }
+        }
+#pragma unroll
+        for (int m = st * MPS; m < (st + 1) * MPS; ++m)
+          acc[m / MI][m % MI] = Mfma<DT>::run(fa[ks & 1][m / MI], fb[ks & 1][m % MI], acc[m / MI][m % MI]);
+        __builtin_amdgcn_sched_barrier(0);
       }
-#pragma unroll
-      for (int a = 0; a < MI; ++a)
-#pragma unroll
-        for (int b = 0; b < MI; ++b) acc[a][b] = Mfma<DT>::run(fa[a], fb[b], acc[a][b]);
     }
   };
 
   const int nslab = (T + BK - 1) / BK;
-  load_slab(0);
-  mask_tail(0);
-  store_cols(smem, smem + PANEL, 0, 8);
-  load_slab(nslab > 1 ? BK : 0);
+  load_panel(ra, 0, i0);
+  load_panel(rb, 0, j0);
+  mask_tail(ra, 0);
+  mask_tail(rb, 0);
+  store_panel(smem, ra);
+  store_panel(smem + PANEL, rb);
+  load_panel(ra, BK, i0);  // (clamped in-bounds when there is no second slab)
+  load_panel(rb, BK, j0);
   __syncthreads();
-  // steady state: slab s multiplied, slab s+1 (full) transposed into the other stage, slab s+2 in flight
+  // steady state: slab s multiplied, slab s+1 transposed into the other stage, slab s+2 in flight
   for (int s = 0; s + 2 < nslab; ++s) {
-    compute(smem + (s & 1) * 2 * PANEL, smem + ((s + 1) & 1) * 2 * PANEL, std::true_type{});
-    load_slab((s + 2) * BK);
+    compute(smem + (s & 1) * 2 * PANEL, smem + ((s + 1) & 1) * 2 * PANEL, (s + 2) * BK, std::true_type{},
+            std::false_type{});
     __syncthreads();
   }
   if (nslab >= 2) {
     const int s = nslab - 2;
-    mask_tail((s + 1) * BK);
-    compute(smem + (s & 1) * 2 * PANEL, smem + ((s + 1) & 1) * 2 * PANEL, std::true_type{});
+    compute(smem + (s & 1) * 2 * PANEL, smem + ((s + 1) & 1) * 2 * PANEL, (s + 2) * BK, std::true_type{},
+            std::true_type{});
     __syncthreads();
   }
-  compute(smem + ((nslab - 1) & 1) * 2 * PANEL, smem, std::false_type{});
+  compute(smem + ((nslab - 1) & 1) * 2 * PANEL, smem, 0, std::false_type{}, std::false_type{});
 
   // 32x32 accumulator layout: lane holds column n = lane&31; register v holds row
   // (v/4)*8 + (lane>>5)*4 + (v&3), i.e. 4 consecutive rows per register quad.  Seen from the
