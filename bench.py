@@ -40,6 +40,9 @@ LINEARS = [  # name, out_features, in_features
 ]
 GROUP = 128
 MFMA_BF16_PEAK_TFLOPS = 2500.0
+# HBM bytes per launch of the dominant kernel from FETCH_SIZE / WRITE_SIZE counter runs scaled by a
+# 1 GiB copy (profiles/hessian_syrk_k14336_t16384_hbm_traffic.md), keyed by tokens per launch
+DOMINANT_TRAFFIC_BYTES = {16384: 7.30e9}
 
 
 def cpu_baseline(tokens: int):
@@ -240,7 +243,8 @@ def main():
             "peak": MFMA_BF16_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved / MFMA_BF16_PEAK_TFLOPS, 4),
-            "traffic": None,
+            "traffic": DOMINANT_TRAFFIC_BYTES.get(int(dom_T)),
+            "algorithmic_hbm_bytes": 2.0 * dom_T * INTER + 8.0 * INTER * INTER,
             "avg_launch_ms": round(dom_ms, 4),
             "launches_timed": len(dom_events),
         },

@@ -169,7 +169,10 @@ __global__ __launch_bounds__(256) void hessian_syrk_kernel(float* __restrict__ H
     constexpr int FPS = 2 * MI / NSTEP, CPS = 8 / NSTEP, LPS = RT / NSTEP;
     unsigned char* curB = curA + PANEL;
     uint4 fa[2][MI], fb[2][MI];
-    auto read_frag = [&](int ks, int f) {  // fragment f of group ks: f < MI -> A rows, else B rows
+    // fragment number n of group ks, in the order the matrix ops first need them:
+    // A rows 0, then all B rows, then the remaining A rows
+    auto read_frag = [&](int ks, int n) {
+      const int f = n == 0 ? 0 : (n <= MI ? MI + n - 1 : n - MI);  // f < MI -> A rows, else B rows
       const int q = ks * 2 + (lane >> 5);
       if (f < MI)
         fa[ks & 1][f] = *(const uint4*)(curA + chunk_off(wm * (BT / 2) + f * 32 + (lane & 31), q));
