@@ -85,6 +85,69 @@ def cpu_baseline(tokens: int):
     }
 
 
+def probe_bandwidth():
+    """Observer / quantize / pack kernels on a 14336 x 4096 bf16 weight (the gate/up projection) and the
+    per-token activation kernel on 8192 x 4096: algorithmic bytes (one read of the input plus one write of
+    the output) over the event-timed launch, against the 8 TB/s HBM peak.  Prints a table."""
+    import torch
+
+    from llmcompressor_amd import ops
+
+    def timed(fn, n=20):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n * 1e-3
+
+    R, K = INTER, HIDDEN
+    n = R * K
+    w = (torch.randn(R, K, device="cuda") * 0.02).bfloat16()
+    rows = []
+
+    def rep(name, t, nbytes):
+        rows.append((name, t * 1e6, nbytes / t / 1e9, nbytes / t / 8e12))
+
+    dst = torch.empty_like(w)
+    rep("copy (reference), 4 B/elem", timed(lambda: dst.copy_(w)), 4 * n)
+    for g in (16, 32, 128, K):
+        rep(f"min-max observer g={g}, 2 B/elem", timed(lambda: ops.minmax_groups(w, g)), 2 * n)
+    mn, mx = ops.minmax_groups(w, 128)
+    sc, _, _ = ops.calculate_qparams(mn, mx, ops.FMT_INT, 4, True)
+    grp = (1, K // 128, 128)
+    rep("int4 g128 -> packed int32, 2.5 B/elem",
+        timed(lambda: ops.quantize(w, sc, None, ops.FMT_INT, 4, *grp, out_mode=ops.OUT_PACKED)), 2.5 * n)
+    rep("int4 g128 fake-quant, 4 B/elem", timed(lambda: ops.quantize(w, sc, None, ops.FMT_INT, 4, *grp)), 4 * n)
+    mn, mx = ops.minmax_groups(w, K)
+    s8, _, _ = ops.calculate_qparams(mn, mx, ops.FMT_FP8, 8, True)
+    rep("fp8 e4m3 per-channel -> bytes, 3 B/elem",
+        timed(lambda: ops.quantize(w, s8, None, ops.FMT_FP8, 8, 1, 1, 1 << 40, out_mode=ops.OUT_PACKED)), 3 * n)
+    mn, mx = ops.minmax_groups(w, 16)
+    gs = ops.global_scale_from_stats([(mn, mx)])
+    s4, _, _ = ops.calculate_qparams(mn, mx, ops.FMT_FP4, 4, True, ops.SCALE_NVFP4, gs)
+    rep("nvfp4 g16 -> packed nibbles, 2.5 B/elem",
+        timed(lambda: ops.quantize(w, s4, None, ops.FMT_FP4, 4, 1, K // 16, 16, out_mode=ops.OUT_PACKED, global_scale=gs)),
+        2.5 * n)
+    mn, mx = ops.minmax_groups(w, 32)
+    sm, _, _ = ops.calculate_qparams(mn, mx, ops.FMT_FP4, 4, True, ops.SCALE_MXFP4, want_codes=True)
+    rep("mxfp4 g32 -> packed nibbles, 2.5 B/elem",
+        timed(lambda: ops.quantize(w, sm, None, ops.FMT_FP4, 4, 1, K // 32, 32, out_mode=ops.OUT_PACKED)), 2.5 * n)
+    x = torch.randn(8192, HIDDEN, device="cuda").bfloat16()
+    rep("fp8 dynamic per-token fake-quant [8192x4096], 4 B/elem", timed(lambda: ops.dynamic_per_token_quantize(x)),
+        4 * x.numel())
+    rep("fp8 dynamic per-token -> bytes [8192x4096], 3 B/elem",
+        timed(lambda: ops.dynamic_per_token_quantize(x, out_mode=ops.OUT_CODES)), 3 * x.numel())
+    print("| kernel (14336 x 4096 bf16 unless noted) | us | GB/s | of 8 TB/s |")
+    print("|---|---|---|---|")
+    for name, us, gbs, frac in rows:
+        print(f"| {name} | {us:.1f} | {gbs:.0f} | {frac * 100:.1f}% |")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -98,6 +161,8 @@ def main():
     ap.add_argument("--probe-dominant", type=int, default=0, metavar="N",
                     help="counter runs: launch only the dominant kernel N times (14336-wide Hessian, --stage-tokens "
                     "tokens) and N plain copies of a 1 GiB buffer (the known-size kernel the HBM counters are scaled by)")
+    ap.add_argument("--probe-bandwidth", action="store_true",
+                    help="print achieved GB/s of the observer / quantize / pack kernels instead of the bench line")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU figure is produced)", file=sys.stderr)
@@ -112,6 +177,9 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if a.probe_bandwidth:
+        probe_bandwidth()
+        return
     if a.probe_dominant:
         x = torch.randn(a.stage_tokens or a.tokens, INTER, device=dev).bfloat16()
         H = torch.zeros(INTER, INTER, device=dev)
