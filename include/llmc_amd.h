@@ -55,11 +55,19 @@ int llmc_version(void);
  * upper results (H must be bitwise symmetric on entry, which holds for a
  * buffer that started as zeros and was only ever updated by this call);
  * without it the lower tiles are read-modify-written too.
+ * `workspace` (16-byte aligned device memory, llmc_hessian_workspace_bytes(T, K)
+ * bytes; may be NULL/0) lets the tiles that do not fill a whole round of
+ * workgroups be cut along the tokens: the chunks' partial tiles go through the
+ * workspace and are summed in a fixed order, so the result does not depend on
+ * timing.  Without it every tile is one workgroup (slower when the tile count
+ * is not a multiple of the CU count).  The workspace holds no state between calls.
  */
 enum { LLMC_HESSIAN_ASSUME_SYMMETRIC = 1 };
+int64_t llmc_hessian_workspace_bytes(int64_t T, int64_t K);
 int llmc_hessian_accumulate(float* H, int64_t ldh, const void* X, int64_t ldx,
                             int64_t T, int64_t K, int32_t x_dtype, float alpha,
-                            int32_t flags, void* stream);
+                            int32_t flags, void* workspace, int64_t workspace_bytes,
+                            void* stream);
 
 /* ---- a10/a11: min-max observers --------------------------------------------
  * Replace _get_min_max() = torch.amin/amax(observed, dim=(0,-1)) on the

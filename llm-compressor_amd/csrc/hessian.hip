@@ -70,39 +70,168 @@ __device__ __forceinline__ int chunk_off(int i, int q) {
   return i * ROW_BYTES + ((q ^ (i & 7) ^ ((i >> 3) & 7)) << 4);
 }
 
+// Work decomposition.  The upper-triangle tiles are numbered compactly in super-tile order (below).
+// A launch is a list of phases; phase p covers tiles [tile0, tile0+ntiles) and cuts the token range
+// into `split` equal chunks, one workgroup per (chunk, tile).  split == 1 is a whole tile with a
+// read-modify-write epilogue.  With split > 1 every chunk stores its partial tile into the
+// workspace (slot ws_tile0 + tile*split + chunk) and a second kernel sums a tile's chunks in fixed
+// order and runs the same epilogue: that is how the tiles left over after the last full round of
+// 256 workgroups still fill the chip, with results that do not depend on timing.
+constexpr int MAX_PHASES = 4;
+struct Phase {
+  int first_wg, tile0, ntiles, split, ws_tile0;
+};
+struct Plan {
+  int nphase;
+  Phase ph[MAX_PHASES];
+};
+
+// Compact tile number c -> (I, J), J >= I.  Tiles are grouped into SH x SW super-tiles (as many
+// tiles as run concurrently on one XCD), super-tiles row-major over those that reach the upper
+// triangle, tiles row-major inside: workgroups sharing an L2 then touch only about SH + SW feature
+// panels of X per slab instead of two each.
+__device__ __forceinline__ void tile_coords(int c, int nb, int SH, int SW, int& I, int& J) {
+  const int nsi = (nb + SH - 1) / SH, nsj = (nb + SW - 1) / SW;
+  for (int si = 0; si < nsi; ++si) {
+    for (int sj = (SH * si) / SW; sj < nsj; ++sj) {
+      const int c_lo = sj * SW, c_hi = min(nb, c_lo + SW);
+      for (int i = si * SH; i < min(nb, si * SH + SH); ++i) {
+        const int lo = max(c_lo, i);
+        const int n = c_hi - lo;
+        if (n <= 0) continue;
+        if (c < n) {
+          I = i;
+          J = lo + c;
+          return;
+        }
+        c -= n;
+      }
+    }
+  }
+  I = J = -1;
+}
+
+// Adds alpha * acc to the BT x BT tile of H at (i0, j0) and to its mirror image.
+// 32x32 accumulator layout: lane holds column n = lane&31; register v holds row
+// (v/4)*8 + (lane>>5)*4 + (v&3), i.e. 4 consecutive rows per register quad.  Seen from the
+// mirrored tile H[j][i] a quad is 4 consecutive floats of one row, so the read-modify-write
+// runs there with 16-byte accesses (4x fewer, 4x larger requests in flight); the tile
+// H[i][j] itself then only needs stores, which are row-contiguous across lanes.
+template <int BT, bool FAST_EPI>
+__device__ __forceinline__ void tile_epilogue(float* __restrict__ H, int64_t ldh, int K, float alpha,
+                                              int assume_sym, int i0, int j0, f32x16_t (&acc)[BT / 64][BT / 64],
+                                              int a_only = -1) {  // >= 0: only MFMA tile row a_only
+  constexpr int MI = BT / 64;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const bool diag = i0 == j0;
+  if (FAST_EPI && i0 + BT <= K && j0 + BT <= K) {
+    // interior tile: no bounds checks, so the 16-byte loads of a whole row of MFMA tiles are
+    // issued back to back before the first use
+#pragma unroll
+    for (int a = 0; a < MI; ++a) {
+      if (a_only >= 0 && a != a_only) continue;
+      float4 old[MI][4];
+#pragma unroll
+      for (int b = 0; b < MI; ++b) {
+        const int col = j0 + wn * (BT / 2) + b * 32 + (lane & 31);
+        const int rbase = i0 + wm * (BT / 2) + a * 32 + (lane >> 5) * 4;
+#pragma unroll
+        for (int vq = 0; vq < 4; ++vq) old[b][vq] = *(const float4*)(H + (int64_t)col * ldh + rbase + vq * 8);
+      }
+#pragma unroll
+      for (int b = 0; b < MI; ++b) {
+        const int col = j0 + wn * (BT / 2) + b * 32 + (lane & 31);
+        const int rbase = i0 + wm * (BT / 2) + a * 32 + (lane >> 5) * 4;
+#pragma unroll
+        for (int vq = 0; vq < 4; ++vq) {
+          const int r0 = rbase + vq * 8;
+          float4 o;
+          o.x = old[b][vq].x + alpha * acc[a][b][vq * 4 + 0];
+          o.y = old[b][vq].y + alpha * acc[a][b][vq * 4 + 1];
+          o.z = old[b][vq].z + alpha * acc[a][b][vq * 4 + 2];
+          o.w = old[b][vq].w + alpha * acc[a][b][vq * 4 + 3];
+          *(float4*)(H + (int64_t)col * ldh + r0) = o;
+          if (!diag) {
+            H[(int64_t)(r0 + 0) * ldh + col] = o.x;
+            H[(int64_t)(r0 + 1) * ldh + col] = o.y;
+            H[(int64_t)(r0 + 2) * ldh + col] = o.z;
+            H[(int64_t)(r0 + 3) * ldh + col] = o.w;
+          }
+        }
+      }
+    }
+    return;
+  }
+#pragma unroll
+  for (int a = 0; a < MI; ++a) {
+    if (a_only >= 0 && a != a_only) continue;
+#pragma unroll
+    for (int b = 0; b < MI; ++b) {
+      const int col = j0 + wn * (BT / 2) + b * 32 + (lane & 31);
+      const int rbase = i0 + wm * (BT / 2) + a * 32 + (lane >> 5) * 4;
+      if (col < K) {
+#pragma unroll
+        for (int vq = 0; vq < 4; ++vq) {
+          const int r0 = rbase + vq * 8;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int row = r0 + e;
+            if (row < K) {
+              float* hp = H + (int64_t)row * ldh + col;
+              const float out = *hp + alpha * acc[a][b][vq * 4 + e];
+              *hp = out;
+              if (!diag) {
+                float* mp = H + (int64_t)col * ldh + row;
+                *mp = assume_sym ? out : *mp + alpha * acc[a][b][vq * 4 + e];
+              }
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
 // BT x BT output tile, 256 threads = 2x2 waves, each wave (BT/2)x(BT/2) = MI x MI MFMA tiles.
 // LDS holds two stages of the two feature-major panels; global loads for slab s+2 are in
 // flight while slab s is multiplied and slab s+1 is transposed into the other stage.
 template <int BT, int DT, bool ALIGNED, bool FAST_EPI>
 __global__ __launch_bounds__(256) void hessian_syrk_kernel(float* __restrict__ H, int64_t ldh,
-                                                            const uint16_t* __restrict__ X, int64_t ldx,
-                                                            int T, int K, float alpha, int assume_sym,
-                                                            int vec_ok, int nb, int nslots) {
+                                                            const uint16_t* __restrict__ Xfull, int64_t ldx,
+                                                            int Tfull, int K, float alpha, int assume_sym,
+                                                            int nb, Plan plan, float* __restrict__ ws) {
   constexpr int RT = BT / 32;  // token rows per thread per panel
   constexpr int GI = BT / 8;   // 8-feature groups per panel
   constexpr int MI = BT / 64;
   constexpr int PANEL = BT * ROW_BYTES;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];  // [2 stages][A,B][BT][128 B]
 
-  // Tile order.  Workgroups are dealt round-robin to the 8 XCDs (each with a private L2), so
-  // block b runs on XCD b%8; p makes every XCD walk a contiguous range of tile slots.  Slots are
-  // grouped into SH x SW super-tiles (as many tiles as run concurrently on one XCD), so the
-  // workgroups sharing an L2 touch only SH + SW feature panels of X per slab instead of one each.
+  // Which (tile, token chunk).  Workgroups are dealt round-robin to the 8 XCDs (each with a private
+  // L2), so block b runs on XCD b%8 (phases start at multiples of 8); `item` makes every XCD walk a
+  // contiguous range of the phase's items, chunk-major, so the workgroups that share an L2 work on
+  // neighbouring tiles over the same tokens.
   constexpr int SH = BT == 256 ? 4 : 8, SW = 8;
-  const int per_xcd = (nslots + 7) / 8;
-  const int p = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-  if (p >= nslots) return;
-  const int nsj = (nb + SW - 1) / SW;
-  int su = p / (SH * SW), SI = 0;
-  // super-row SI holds super-columns (SH*SI)/SW .. nsj-1 (those that reach the upper triangle)
-  while (su >= nsj - (SH * SI) / SW) {
-    su -= nsj - (SH * SI) / SW;
-    ++SI;
-  }
-  const int SJ = (SH * SI) / SW + su;
-  const int I = SI * SH + (p % (SH * SW)) / SW;
-  const int J = SJ * SW + p % SW;
-  if (I >= nb || J >= nb || J < I) return;
+  int pi = 0;
+  while (pi + 1 < plan.nphase && (int)blockIdx.x >= plan.ph[pi + 1].first_wg) ++pi;
+  const Phase ph = plan.ph[pi];
+  const int bl = blockIdx.x - ph.first_wg;
+  const int items = ph.ntiles * ph.split;
+  const int per_xcd = (items + 7) / 8;
+  const int item = (bl % 8) * per_xcd + bl / 8;
+  if (item >= items || bl / 8 >= per_xcd) return;
+  const int chunk = item / ph.ntiles;
+  const int nslab_all = (Tfull + BK - 1) / BK;
+  const int cs = (nslab_all + ph.split - 1) / ph.split;  // slabs per chunk
+  const int s_begin = chunk * cs;
+  if (s_begin >= nslab_all) return;
+  const int t_begin = s_begin * BK;
+  const int T = min(Tfull, (s_begin + cs) * BK) - t_begin;  // tokens of this chunk
+  const uint16_t* X = Xfull + (int64_t)t_begin * ldx;
+  const bool partial = ph.split > 1;
+  int I, J;
+  tile_coords(ph.tile0 + item % ph.ntiles, nb, SH, SW, I, J);
+  if (I < 0) return;
   const int i0 = I * BT, j0 = J * BT;
   const bool diag = (I == J);
 
@@ -236,87 +365,180 @@ __global__ __launch_bounds__(256) void hessian_syrk_kernel(float* __restrict__ H
   }
   compute(smem + ((nslab - 1) & 1) * 2 * PANEL, smem, 0, std::false_type{}, std::false_type{});
 
-  // 32x32 accumulator layout: lane holds column n = lane&31; register v holds row
-  // (v/4)*8 + (lane>>5)*4 + (v&3), i.e. 4 consecutive rows per register quad.  Seen from the
-  // mirrored tile H[j][i] a quad is 4 consecutive floats of one row, so the read-modify-write
-  // runs there with 16-byte accesses (4x fewer, 4x larger requests in flight); the tile
-  // H[i][j] itself then only needs stores, which are row-contiguous across lanes.
-  if (FAST_EPI && i0 + BT <= K && j0 + BT <= K) {
-    // interior tile: no bounds checks, so the 16-byte loads of a whole row of MFMA tiles are
-    // issued back to back before the first use
+  if (partial) {
+    // partial tile: raw accumulators to the workspace in register order (16 bytes per lane, coalesced)
+    float* slot = ws + (int64_t)(ph.ws_tile0 + (item % ph.ntiles) * ph.split + chunk) * (BT * BT);
 #pragma unroll
-    for (int a = 0; a < MI; ++a) {
-      float4 old[MI][4];
+    for (int a = 0; a < MI; ++a)
 #pragma unroll
-      for (int b = 0; b < MI; ++b) {
-        const int col = j0 + wn * (BT / 2) + b * 32 + (lane & 31);
-        const int rbase = i0 + wm * (BT / 2) + a * 32 + (lane >> 5) * 4;
+      for (int b = 0; b < MI; ++b)
 #pragma unroll
-        for (int vq = 0; vq < 4; ++vq) old[b][vq] = *(const float4*)(H + (int64_t)col * ldh + rbase + vq * 8);
-      }
-#pragma unroll
-      for (int b = 0; b < MI; ++b) {
-        const int col = j0 + wn * (BT / 2) + b * 32 + (lane & 31);
-        const int rbase = i0 + wm * (BT / 2) + a * 32 + (lane >> 5) * 4;
-#pragma unroll
-        for (int vq = 0; vq < 4; ++vq) {
-          const int r0 = rbase + vq * 8;
-          float4 o;
-          o.x = old[b][vq].x + alpha * acc[a][b][vq * 4 + 0];
-          o.y = old[b][vq].y + alpha * acc[a][b][vq * 4 + 1];
-          o.z = old[b][vq].z + alpha * acc[a][b][vq * 4 + 2];
-          o.w = old[b][vq].w + alpha * acc[a][b][vq * 4 + 3];
-          *(float4*)(H + (int64_t)col * ldh + r0) = o;
-          if (!diag) {
-            H[(int64_t)(r0 + 0) * ldh + col] = o.x;
-            H[(int64_t)(r0 + 1) * ldh + col] = o.y;
-            H[(int64_t)(r0 + 2) * ldh + col] = o.z;
-            H[(int64_t)(r0 + 3) * ldh + col] = o.w;
-          }
-        }
-      }
-    }
+        for (int vq = 0; vq < 4; ++vq)
+          *(float4*)(slot + (((a * MI + b) * 4 + vq) * 256 + tid) * 4) =
+              make_float4(acc[a][b][vq * 4], acc[a][b][vq * 4 + 1], acc[a][b][vq * 4 + 2], acc[a][b][vq * 4 + 3]);
     return;
   }
+  tile_epilogue<BT, FAST_EPI>(H, ldh, K, alpha, assume_sym, i0, j0, acc);
+}
+
+// Sums the chunks of a split tile in fixed order and applies the tile epilogue; one workgroup per
+// (tile, row of MFMA tiles), the loads of two chunks in flight at a time.
+template <int BT, bool FAST_EPI>
+__global__ __launch_bounds__(256) void hessian_reduce_kernel(float* __restrict__ H, int64_t ldh, int Tfull, int K,
+                                                              float alpha, int assume_sym, int nb, Plan plan,
+                                                              int first_split_phase, const float* __restrict__ ws) {
+  constexpr int MI = BT / 64;
+  constexpr int SH = BT == 256 ? 4 : 8, SW = 8;
+  int pi = first_split_phase, t = blockIdx.x / MI;
+  const int a = blockIdx.x % MI;
+  while (t >= plan.ph[pi].ntiles) t -= plan.ph[pi++].ntiles;
+  const Phase ph = plan.ph[pi];
+  int I, J;
+  tile_coords(ph.tile0 + t, nb, SH, SW, I, J);
+  if (I < 0) return;
+  const int nslab_all = (Tfull + BK - 1) / BK;
+  const int cs = (nslab_all + ph.split - 1) / ph.split;
+  int nchunk = ph.split;
+  while (nchunk > 0 && (nchunk - 1) * cs >= nslab_all) --nchunk;  // trailing chunks without tokens wrote nothing
+  float4 sum[MI][4];
 #pragma unroll
-  for (int a = 0; a < MI; ++a) {
+  for (int b = 0; b < MI; ++b)
 #pragma unroll
-    for (int b = 0; b < MI; ++b) {
-      const int col = j0 + wn * (BT / 2) + b * 32 + (lane & 31);
-      const int rbase = i0 + wm * (BT / 2) + a * 32 + (lane >> 5) * 4;
-      if (col < K) {
+    for (int vq = 0; vq < 4; ++vq) sum[b][vq] = make_float4(0.f, 0.f, 0.f, 0.f);
+  const float* base = ws + (int64_t)(ph.ws_tile0 + t * ph.split) * (BT * BT) + (a * MI * 4 * 256 + threadIdx.x) * 4;
+  auto load = [&](int chunk, float4 (&p)[MI][4]) {
 #pragma unroll
-        for (int vq = 0; vq < 4; ++vq) {
-          const int r0 = rbase + vq * 8;
+    for (int b = 0; b < MI; ++b)
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int row = r0 + e;
-            if (row < K) {
-              float* hp = H + (int64_t)row * ldh + col;
-              const float out = *hp + alpha * acc[a][b][vq * 4 + e];
-              *hp = out;
-              if (!diag) {
-                float* mp = H + (int64_t)col * ldh + row;
-                *mp = assume_sym ? out : *mp + alpha * acc[a][b][vq * 4 + e];
-              }
-            }
-          }
-        }
+      for (int vq = 0; vq < 4; ++vq)
+        p[b][vq] = *(const float4*)(base + (int64_t)chunk * (BT * BT) + ((b * 4 + vq) * 256) * 4);
+  };
+  auto add = [&](const float4 (&p)[MI][4]) {
+#pragma unroll
+    for (int b = 0; b < MI; ++b)
+#pragma unroll
+      for (int vq = 0; vq < 4; ++vq) {
+        sum[b][vq].x += p[b][vq].x;
+        sum[b][vq].y += p[b][vq].y;
+        sum[b][vq].z += p[b][vq].z;
+        sum[b][vq].w += p[b][vq].w;
       }
-    }
+  };
+  int chunk = 0;
+  for (; chunk + 1 < nchunk; chunk += 2) {
+    float4 p0[MI][4], p1[MI][4];
+    load(chunk, p0);
+    load(chunk + 1, p1);
+    add(p0);
+    add(p1);
   }
+  if (chunk < nchunk) {
+    float4 p0[MI][4];
+    load(chunk, p0);
+    add(p0);
+  }
+  f32x16_t acc[MI][MI];
+#pragma unroll
+  for (int aa = 0; aa < MI; ++aa)
+#pragma unroll
+    for (int b = 0; b < MI; ++b)
+#pragma unroll
+      for (int vq = 0; vq < 4; ++vq) {
+        const bool mine = aa == a;
+        acc[aa][b][vq * 4] = mine ? sum[b][vq].x : 0.f;
+        acc[aa][b][vq * 4 + 1] = mine ? sum[b][vq].y : 0.f;
+        acc[aa][b][vq * 4 + 2] = mine ? sum[b][vq].z : 0.f;
+        acc[aa][b][vq * 4 + 3] = mine ? sum[b][vq].w : 0.f;
+      }
+  tile_epilogue<BT, FAST_EPI>(H, ldh, K, alpha, assume_sym, I * BT, J * BT, acc, a);
+}
+
+constexpr int NUM_WG = 256;  // workgroups that run at once: one per CU (LDS and registers allow no more)
+
+struct Choice {
+  int bt = 0;
+  Plan plan;
+  int first_split_phase = 0;  // == plan.nphase when no phase is split
+  int nsplit_tiles = 0;
+  int64_t ws_bytes = 0;
+  double time_us = 0;
+  int grid = 0;
+};
+
+// Phases for BT-wide tiles.  Whole rounds of NUM_WG tiles first.  When `split`, the R tiles left
+// over are cut along the tokens so that they fill a round too: R <= 128 -> one phase of
+// floor(256/R) chunks per tile; R > 128 -> 128 tiles in two chunks, then the rest as before.  A
+// chunk keeps at least 4 slabs.  time_us is a rough model (measured microseconds per slab and per
+// epilogue of one tile, partial tiles through the workspace at 2 TB/s) used only to pick between
+// candidates.
+Choice make_choice(int bt, int64_t T, int64_t K, bool split) {
+  Choice c;
+  c.bt = bt;
+  const int nb = (int)((K + bt - 1) / bt);
+  const int nt = nb * (nb + 1) / 2;
+  const int nslab = (int)((T + BK - 1) / BK);
+  const double slab_us = bt == 256 ? 1.75 : 0.6, epi_us = bt == 256 ? 35.0 : 10.0, chunk_epi_us = 5.0;
+  Plan& plan = c.plan;
+  plan.nphase = 0;
+  int wg = 0, tile0 = 0, ws_tile = 0;
+  auto push = [&](int ntiles, int sp) {
+    Phase& p = plan.ph[plan.nphase++];
+    p.first_wg = wg;
+    p.tile0 = tile0;
+    p.ntiles = ntiles;
+    p.split = sp;
+    p.ws_tile0 = ws_tile;
+    const int items = ntiles * sp;
+    wg += ((items + 7) / 8) * 8;
+    tile0 += ntiles;
+    if (sp > 1) ws_tile += items;
+    const int rounds = (items + NUM_WG - 1) / NUM_WG;
+    c.time_us += rounds * (((nslab + sp - 1) / sp) * slab_us + (sp > 1 ? chunk_epi_us : epi_us));
+  };
+  int slimit = nslab / 4;
+  if (slimit > 16) slimit = 16;
+  int rem = nt;
+  if (!split || slimit < 2) {
+    push(nt, 1);
+    rem = 0;
+  } else {
+    const int whole = (rem / NUM_WG) * NUM_WG;
+    if (whole > 0) push(whole, 1);
+    rem -= whole;
+  }
+  c.first_split_phase = plan.nphase;
+  if (rem > NUM_WG / 2) {
+    push(NUM_WG / 2, 2);
+    rem -= NUM_WG / 2;
+  }
+  if (rem > 0) {
+    int sp = NUM_WG / rem;
+    if (sp > slimit) sp = slimit;
+    push(rem, sp);  // (sp == 1 cannot happen here: rem <= 128 and slimit >= 2)
+  }
+  c.nsplit_tiles = nt - (c.first_split_phase < plan.nphase ? plan.ph[c.first_split_phase].tile0 : nt);
+  c.ws_bytes = (int64_t)ws_tile * bt * bt * 4;
+  c.time_us += c.ws_bytes * 2 / 2e6 + (ws_tile ? 20.0 : 0.0);  // partial tiles written and read back, reduce kernel
+  c.grid = wg;
+  return c;
+}
+
+// the fastest of {128, 256}-wide tiles x {whole tiles, token chunks} that fits the workspace
+Choice choose(int64_t T, int64_t K, int64_t ws_avail) {
+  Choice best;
+  for (int bt : {256, 128})
+    for (int split = 0; split < 2; ++split) {
+      const Choice c = make_choice(bt, T, K, split != 0);
+      if (c.ws_bytes > ws_avail) continue;
+      if (best.bt == 0 || c.time_us < best.time_us) best = c;
+    }
+  return best;
 }
 
 template <int BT, int DT>
-int launch(float* H, int64_t ldh, const void* X, int64_t ldx, int64_t T, int64_t K, float alpha,
-           int flags, hipStream_t st) {
+int launch(const Choice& c, float* H, int64_t ldh, const void* X, int64_t ldx, int64_t T, int64_t K, float alpha,
+           int flags, float* ws, hipStream_t st) {
   const int nb = (int)((K + BT - 1) / BT);
-  constexpr int SH = BT == 256 ? 4 : 8, SW = 8;  // must match the kernel
-  const int nsi = (nb + SH - 1) / SH, nsj = (nb + SW - 1) / SW;
-  int nsuper = 0;
-  for (int si = 0; si < nsi; ++si) nsuper += nsj - (SH * si) / SW;
-  const int nslots = nsuper * SH * SW;
-  const int grid = ((nslots + 7) / 8) * 8;
   const bool aligned = (K % 8 == 0) && (ldx % 8 == 0) && (((uintptr_t)X & 15) == 0);
   const int sym = (flags & LLMC_HESSIAN_ASSUME_SYMMETRIC) ? 1 : 0;
   const int vec_ok = ((ldh & 3) == 0 && ((uintptr_t)H & 15) == 0) ? 1 : 0;
@@ -329,17 +551,31 @@ int launch(float* H, int64_t ldh, const void* X, int64_t ldx, int64_t T, int64_t
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return 1000 + (int)e;
   }
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), smem, st, H, ldh, (const uint16_t*)X, ldx, (int)T,
-                     (int)K, alpha, sym, vec_ok, nb, nslots);
+  hipLaunchKernelGGL(kern, dim3(c.grid), dim3(256), smem, st, H, ldh, (const uint16_t*)X, ldx, (int)T,
+                     (int)K, alpha, sym, nb, c.plan, ws);
   LLMC_LAUNCH_STATUS();
+  if (c.nsplit_tiles > 0) {
+    if (fast)
+      hipLaunchKernelGGL((hessian_reduce_kernel<BT, true>), dim3(c.nsplit_tiles * (BT / 64)), dim3(256), 0, st, H, ldh,
+                         (int)T, (int)K, alpha, sym, nb, c.plan, c.first_split_phase, ws);
+    else
+      hipLaunchKernelGGL((hessian_reduce_kernel<BT, false>), dim3(c.nsplit_tiles * (BT / 64)), dim3(256), 0, st, H, ldh,
+                         (int)T, (int)K, alpha, sym, nb, c.plan, c.first_split_phase, ws);
+    LLMC_LAUNCH_STATUS();
+  }
   return 0;
 }
 
 }  // namespace
 
+extern "C" int64_t llmc_hessian_workspace_bytes(int64_t T, int64_t K) {
+  if (T <= 0 || K <= 0 || K >= (1 << 30)) return 0;
+  return choose(T, K, INT64_MAX).ws_bytes;
+}
+
 extern "C" int llmc_hessian_accumulate(float* H, int64_t ldh, const void* X, int64_t ldx, int64_t T,
                                        int64_t K, int32_t x_dtype, float alpha, int32_t flags,
-                                       void* stream) {
+                                       void* workspace, int64_t workspace_bytes, void* stream) {
   LLMC_CHECK_ARG(H != nullptr, 1);
   LLMC_CHECK_ARG(K > 0 && K < (1 << 30) && ldh >= K, 2);
   LLMC_CHECK_ARG(T >= 0 && T < (1ll << 31), 5);
@@ -347,15 +583,18 @@ extern "C" int llmc_hessian_accumulate(float* H, int64_t ldh, const void* X, int
   LLMC_CHECK_ARG(X != nullptr, 3);
   LLMC_CHECK_ARG(ldx >= K, 4);
   LLMC_CHECK_ARG(x_dtype == LLMC_BF16 || x_dtype == LLMC_F16, 7);
+  LLMC_CHECK_ARG(workspace_bytes >= 0 && (workspace_bytes == 0 || workspace != nullptr), 10);
+  LLMC_CHECK_ARG((((uintptr_t)workspace) & 15) == 0, 10);
   hipStream_t st = (hipStream_t)stream;
-  // 256-wide tiles once there are enough of them to fill 256 CUs; 128-wide below that
-  const int64_t nb256 = (K + 255) / 256;
-  const bool big = nb256 * (nb256 + 1) / 2 >= 512;
+  // 256-wide tiles need half the LDS traffic per matrix op of 128-wide ones; token chunks spread a
+  // tile count that is not a multiple of the CU count over the whole chip
+  const Choice c = choose(T, K, workspace ? workspace_bytes : 0);
+  float* ws = (float*)workspace;
   if (x_dtype == LLMC_BF16)
-    return big ? launch<256, LLMC_BF16>(H, ldh, X, ldx, T, K, alpha, flags, st)
-               : launch<128, LLMC_BF16>(H, ldh, X, ldx, T, K, alpha, flags, st);
-  return big ? launch<256, LLMC_F16>(H, ldh, X, ldx, T, K, alpha, flags, st)
-             : launch<128, LLMC_F16>(H, ldh, X, ldx, T, K, alpha, flags, st);
+    return c.bt == 256 ? launch<256, LLMC_BF16>(c, H, ldh, X, ldx, T, K, alpha, flags, ws, st)
+                       : launch<128, LLMC_BF16>(c, H, ldh, X, ldx, T, K, alpha, flags, ws, st);
+  return c.bt == 256 ? launch<256, LLMC_F16>(c, H, ldh, X, ldx, T, K, alpha, flags, ws, st)
+                     : launch<128, LLMC_F16>(c, H, ldh, X, ldx, T, K, alpha, flags, ws, st);
 }
 
 extern "C" int llmc_version(void) { return 1; }

@@ -50,7 +50,8 @@ _F32 = ctypes.c_float
 # name -> argtypes; every function returns int
 SIGNATURES = {
     "llmc_version": [],
-    "llmc_hessian_accumulate": [_P, _I64, _P, _I64, _I64, _I64, _I32, _F32, _I32, _P],
+    "llmc_hessian_workspace_bytes": [_I64, _I64],
+    "llmc_hessian_accumulate": [_P, _I64, _P, _I64, _I64, _I64, _I32, _F32, _I32, _P, _I64, _P],
     "llmc_minmax_groups": [_P, _I32, _I64, _I64, _I64, _I64, _P, _P, _P, _I64, _P],
     "llmc_minmax_blocks": [_P, _I32, _I64, _I64, _I64, _I32, _I32, _P, _P, _P],
     "llmc_minmax_strided": [_P, _I32, _I64, _I64, _I64, _I64, _I64, _P, _P, _P],
@@ -80,6 +81,7 @@ SIGNATURES.update({
 })
 # functions whose return type is not int
 RESTYPES = {
+    "llmc_hessian_workspace_bytes": ctypes.c_int64,
     "llmc_minmax_workspace_bytes": ctypes.c_int64,
     "llmc_gptq_hinv_workspace_bytes": ctypes.c_int64,
     "llmc_mse_workspace_bytes": ctypes.c_int64,

@@ -72,3 +72,53 @@ def test_hessian_config1_shape_additivity():
     ref = 2 * x.float().t() @ x.float()
     assert _rel(H, ref) < TOL
     assert torch.equal(H, H.t())
+
+
+@pytest.mark.parametrize("T,K", [(1024, 1024), (2048, 4096), (1100, 1288), (4096, 2304)])
+def test_hessian_token_chunks(T, K):
+    """Shapes whose tiles do not fill the chip: tiles are cut along the tokens, the partial tiles go
+    through the workspace and are summed in fixed order.  Same tolerance, still bitwise symmetric and
+    reproducible; without the workspace every tile is one workgroup."""
+    from llmcompressor_amd import ops
+
+    torch.manual_seed(T + K)
+    x = torch.randn(T, K, device="cuda").bfloat16()
+    x[:, 5] *= 30
+    ref = 2 * (x.double().t() @ x.double())
+    H = torch.zeros(K, K, device="cuda")
+    ops.hessian_accumulate_(H, x)
+    assert _rel(H, ref) < TOL
+    assert torch.equal(H, H.t())
+    ops.hessian_accumulate_(H, x)  # a second launch on top of a mirrored result
+    assert _rel(H, 2 * ref) < TOL
+    assert torch.equal(H, H.t())
+    Hd = [torch.zeros(K, K, device="cuda") for _ in range(2)]
+    for h in Hd:
+        ops.hessian_accumulate_(h, x)
+        ops.hessian_accumulate_(h, x)
+    assert torch.equal(Hd[0], Hd[1]) and torch.equal(Hd[0], H)
+    Hn = torch.zeros(K, K, device="cuda")
+    ops.hessian_accumulate_(Hn, x, use_workspace=False)
+    assert _rel(Hn, ref) < TOL and torch.equal(Hn, Hn.t())
+    Hu = torch.randn(K, K, device="cuda")  # not symmetric: both triangles are read-modify-written
+    Hu0 = Hu.clone()
+    ops.hessian_accumulate_(Hu, x, assume_symmetric=False)
+    assert _rel(Hu - Hu0, ref) < 1e-4
+    if T <= 2048 and K <= 1288:  # the CPU oracle at a size it finishes quickly
+        Hc, _ = G.accumulate_hessian(x.cpu(), G.make_empty_hessian(K), torch.zeros(()))
+        assert _rel(H.cpu(), 2 * Hc) < TOL
+
+
+def test_hessian_full_size_token_chunks():
+    """K = 14336 at 4096 tokens: 1536 whole tiles + 60 tiles in chunks; checked on sampled rows."""
+    from llmcompressor_amd import ops
+
+    torch.manual_seed(1)
+    K, T = 14336, 4096
+    x = torch.randn(T, K, device="cuda").bfloat16()
+    H = torch.zeros(K, K, device="cuda")
+    ops.hessian_accumulate_(H, x)
+    rows = torch.tensor([0, 255, 256, 4095, 7000, 13000, 14080, 14335], device="cuda")
+    ref = 2 * (x[:, rows].double().t() @ x.double())
+    assert _rel(H[rows], ref) < TOL
+    assert torch.equal(H, H.t())
