@@ -245,10 +245,11 @@ def main():
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         # what the forward hooks do during the calibration pass of this layer
+        mods = [(getattr(layer, name), k == INTER) for name, _, k in LINEARS]
         for b in range(B):
-            for name, r, k in LINEARS:
-                x = x_hidden[b] if k == HIDDEN else x_inter[b]
-                modifier.calibrate_module(getattr(layer, name), (x.unsqueeze(0),), None)
+            args_h, args_i = (x_hidden[b:b + 1],), (x_inter[b:b + 1],)
+            for mod, wide in mods:
+                modifier.calibrate_module(mod, args_i if wide else args_h, None)
         for m in list(modifier._staged):
             modifier._flush(m)
         torch.cuda.synchronize()

@@ -76,76 +76,80 @@ __global__ __launch_bounds__(256) void hinv_copyin_kernel(const float* __restric
   A[(int64_t)i * Kp + j] = v;
 }
 
-// Factor the 64x64 diagonal block at (k0,k0) in LDS and replace it by the inverse of its factor.
-// Left-looking (Cholesky-Crout) so nothing is updated ahead of the current column: at step j the
-// 64 four-lane teams each form one dot product over the previous columns -- team t > j for
-// L[t][j], team j for the pivot, team t < j for X[j][t] of X = L^-1 (row j of L is complete by
-// then) -- so factor and inverse advance together with two barriers per column.
+// Factor the 64x64 diagonal block at (k0,k0) and replace it by the inverse of its factor.
+// The block and the growing inverse X = L^-1 live in registers: thread (ty, tx) of a 16 x 16 grid
+// owns the 4x4 sub-blocks L[4ty.., 4tx..] and X[4ty.., 4tx..].  Right-looking, one barrier per
+// column j: the owners publish column j of the partly factored block and row j of X through LDS
+// (unscaled; the pivot d is element j of the column), then every thread applies
+//   L[i][c] -= L[i][j] L[c][j] / d,   X[i][c] -= (L[i][j] / sqrt d) (X[j][c] / sqrt d)   for i, c > j
+// to its sub-blocks, so factor and inverse advance together.
 __global__ __launch_bounds__(256) void potf2_inv_kernel(float* __restrict__ A, int Kp, int k0, int K,
                                                         HinvScalars* sc) {
-  __shared__ float L[NB][NB + 1];
-  __shared__ float X[NB][NB + 1];
-  const int tid = threadIdx.x;
-  for (int e = tid; e < NB * NB; e += 256) {
-    const int i = e / NB, j = e % NB;
-    L[i][j] = (j <= i) ? A[(int64_t)(k0 + i) * Kp + k0 + j] : 0.f;
-    X[i][j] = 0.f;
-  }
-  __syncthreads();
-  const int t = tid >> 2, part = tid & 3;
-  for (int j = 0; j < NB; ++j) {
-    // dot over the previous columns; four independent partial sums keep several LDS loads in flight
-    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
-    int k = (t < j ? t : 0) + part;
-    if (t >= j) {
-      const float* rowt = L[t];
-      for (; k + 12 < j; k += 16) {
-        const float a0 = rowt[k], a1 = rowt[k + 4], a2 = rowt[k + 8], a3 = rowt[k + 12];
-        const float b0 = L[j][k], b1 = L[j][k + 4], b2 = L[j][k + 8], b3 = L[j][k + 12];
-        s0 += a0 * b0;
-        s1 += a1 * b1;
-        s2 += a2 * b2;
-        s3 += a3 * b3;
-      }
-      for (; k < j; k += 4) s0 += rowt[k] * L[j][k];
-    } else {
-      for (; k + 12 < j; k += 16) {
-        const float a0 = X[k][t], a1 = X[k + 4][t], a2 = X[k + 8][t], a3 = X[k + 12][t];
-        const float b0 = L[j][k], b1 = L[j][k + 4], b2 = L[j][k + 8], b3 = L[j][k + 12];
-        s0 += a0 * b0;
-        s1 += a1 * b1;
-        s2 += a2 * b2;
-        s3 += a3 * b3;
-      }
-      for (; k < j; k += 4) s0 += X[k][t] * L[j][k];
+  __shared__ __attribute__((aligned(16))) float colbuf[2][NB];
+  __shared__ __attribute__((aligned(16))) float xrow[2][NB];
+  const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+  float Lb[4][4], Xb[4][4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const float4 v = *(const float4*)(A + (int64_t)(k0 + 4 * ty + r) * Kp + k0 + 4 * tx);
+    const float e[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      Lb[r][c] = (4 * tx + c <= 4 * ty + r) ? e[c] : 0.f;
+      Xb[r][c] = (4 * tx + c == 4 * ty + r) ? 1.f : 0.f;
     }
-    float s = (s0 + s1) + (s2 + s3);
-    s += __shfl_xor(s, 1, 64);
-    s += __shfl_xor(s, 2, 64);
-    if (t == j && part == 0) {
-      float d = L[j][j] - s;
+  }
+  for (int jb = 0; jb < NB / 4; ++jb) {
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+      const int j = 4 * jb + jj;
+      const int buf = jj & 1;
+      if (tx == jb) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) colbuf[buf][4 * ty + r] = Lb[r][jj];
+      }
+      if (ty == jb) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) xrow[buf][4 * tx + c] = Xb[jj][c];
+      }
+      __syncthreads();
+      float d = colbuf[buf][j];
       if (!(d > 0.f) || d > 3.0e38f) {
         // first failing pivot, 1-based index in the ORIGINAL (un-reversed) ordering
-        if (k0 + j < K) atomicCAS(&sc->info, 0, K - (k0 + j));
+        if (tid == 0 && k0 + j < K) atomicCAS(&sc->info, 0, K - (k0 + j));
         d = 1.f;
       }
-      L[j][j] = sqrtf(d);
+      const float rinv = 1.f / sqrtf(d);
+      const float4 cr = *(const float4*)&colbuf[buf][4 * ty];
+      const float4 cc = *(const float4*)&colbuf[buf][4 * tx];
+      const float4 xr4 = *(const float4*)&xrow[buf][4 * tx];
+      const float lr[4] = {cr.x * rinv, cr.y * rinv, cr.z * rinv, cr.w * rinv};
+      const float lc[4] = {cc.x * rinv, cc.y * rinv, cc.z * rinv, cc.w * rinv};
+      const float xr[4] = {xr4.x * rinv, xr4.y * rinv, xr4.z * rinv, xr4.w * rinv};
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int i = 4 * ty + r;
+        const float lri = i > j ? lr[r] : 0.f;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          const float lcc = 4 * tx + c > j ? lc[c] : 0.f;
+          Lb[r][c] -= lri * lcc;
+          Xb[r][c] -= lri * xr[c];
+        }
+        if (tx == jb && i >= j) Lb[r][jj] = i == j ? d * rinv : lr[r];  // column j is final
+      }
+      if (ty == jb) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) Xb[jj][c] = xr[c];  // row j of the inverse is final
+      }
     }
-    __syncthreads();
-    const float piv = L[j][j];
-    if (part == 0) {
-      if (t > j)
-        L[t][j] = (L[t][j] - s) / piv;
-      else if (t < j)
-        X[j][t] = -s / piv;
-      else
-        X[j][j] = 1.f / piv;
-    }
-    __syncthreads();
   }
-  for (int e = tid; e < NB * NB; e += 256) {
-    const int i = e / NB, j = e % NB;
-    A[(int64_t)(k0 + i) * Kp + k0 + j] = (j <= i) ? X[i][j] : 0.f;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    float e[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) e[c] = (4 * tx + c <= 4 * ty + r) ? Xb[r][c] : 0.f;
+    *(float4*)(A + (int64_t)(k0 + 4 * ty + r) * Kp + k0 + 4 * tx) = make_float4(e[0], e[1], e[2], e[3]);
   }
 }
 

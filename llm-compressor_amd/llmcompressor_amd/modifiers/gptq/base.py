@@ -139,25 +139,24 @@ class GPTQModifier(Modifier, QuantizationMixin):
             self._hessians[module], self._num_samples[module] = accumulate_hessian(
                 inp, module, self._hessians[module], self._num_samples[module])
 
-    # -- token staging (see the class docstring)
+    # -- token staging (see the class docstring).  The hook runs once per Linear per batch, so it is
+    # kept to one device copy: the sample count is kept on the host until the flush.
     def _stage(self, module, inp):
-        if inp.ndim == 2:
-            inp = inp.unsqueeze(0)
-        elif inp.ndim > 3:
-            inp = inp.reshape(inp.shape[0], -1, inp.shape[-1])
-        self._num_samples[module] += inp.shape[0]
-        rows = inp.reshape(-1, inp.shape[-1])
+        k = inp.shape[-1]
+        n = inp.numel() // k
         st = self._staged.get(module)
-        cap = max(self.hessian_batch_tokens, rows.shape[0])
-        if st is None or st[0].shape[0] < cap or st[0].dtype != rows.dtype:
+        if st is None or st[0].shape[0] < n or st[0].dtype != inp.dtype or st[0].device != inp.device:
             if st is not None:
                 self._flush(module)
-            st = [torch.empty((cap, rows.shape[1]), dtype=rows.dtype, device=rows.device), 0]
+            cap = max(self.hessian_batch_tokens, n)
+            st = [torch.empty((cap, k), dtype=inp.dtype, device=inp.device), 0, 0]
             self._staged[module] = st
-        if st[1] + rows.shape[0] > st[0].shape[0]:
+        elif st[1] + n > st[0].shape[0]:
             self._flush(module)
-        st[0][st[1]: st[1] + rows.shape[0]].copy_(rows)
-        st[1] += rows.shape[0]
+        used = st[1]
+        st[0].narrow(0, used, n).copy_(inp.reshape(n, k))
+        st[1] = used + n
+        st[2] += 1 if inp.ndim == 2 else inp.shape[0]  # accumulate_hessian counts a 2-D input as one sample
         if st[1] >= self.hessian_batch_tokens:
             self._flush(module)
 
@@ -165,8 +164,10 @@ class GPTQModifier(Modifier, QuantizationMixin):
         st = self._staged.get(module)
         if st is None or st[1] == 0:
             return
-        ops.hessian_accumulate_(self._hessians[module], st[0][: st[1]], alpha=2.0, assume_symmetric=True)
+        ops.hessian_accumulate_(self._hessians[module], st[0].narrow(0, 0, st[1]), alpha=2.0, assume_symmetric=True)
+        self._num_samples[module] += st[2]
         st[1] = 0
+        st[2] = 0
 
     def compress_modules(self):
         self.compress_module_list(list(self._num_samples.keys()))
