@@ -14,6 +14,7 @@
 namespace {
 
 constexpr int GB = 128;       // widest column block held on chip
+constexpr int GROUP = 4;      // column blocks whose updates of the far columns are applied together
 constexpr int TEAM = 16;      // lanes per row
 constexpr int CPL = GB / TEAM;  // columns per lane (8)
 constexpr int ROWS_PER_WG = 256 / TEAM;
@@ -46,7 +47,8 @@ struct GptqBlockParams {
   int64_t row_div, srow;
   int fmt, bits;
   int sd;           // dtype the dequantised value is formed in
-  float* E;         // [R, GB] scaled errors of this block
+  float* E;         // scaled errors of this block, row stride ldE
+  int ldE;
   float* loss_rows; // [R]
 };
 
@@ -126,7 +128,7 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(GptqBlockParams p) {
     for (int e = 0; e < CPL; ++e) {
       const int cb = tl * CPL + e;
       if (cb < p.count) p.Wf[(int64_t)row * p.K + p.i1 + cb] = qv[e];
-      p.E[(int64_t)row * GB + cb] = ev[e];
+      p.E[(int64_t)row * p.ldE + cb] = ev[e];
     }
     if (tl == 0) p.loss_rows[row] += loss * 0.5f;
   }
@@ -163,7 +165,7 @@ inline int64_t align256(int64_t b) { return (b + 255) / 256 * 256; }
 }  // namespace
 
 extern "C" int64_t llmc_gptq_quantize_workspace_bytes(int64_t R, int64_t K) {
-  return align256(R * K * 4) + align256(R * GB * 4) + align256(R * 4);
+  return align256(R * K * 4) + align256(R * GROUP * GB * 4) + align256(R * 4);
 }
 
 extern "C" int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R, int64_t K, int64_t ldw,
@@ -195,7 +197,7 @@ extern "C" int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R
 
   float* Wf = (float*)workspace;
   float* E = (float*)((char*)workspace + align256(R * K * 4));
-  float* loss_rows = (float*)((char*)E + align256(R * GB * 4));
+  float* loss_rows = (float*)((char*)E + align256(R * GROUP * GB * 4));
 
   dim3 grid2((unsigned)((K + 255) / 256), (unsigned)R);
 #define LLMC_PREP(DT) \
@@ -235,17 +237,35 @@ extern "C" int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
   if (e != hipSuccess) return 1000 + (int)e;
   const unsigned wgs = (unsigned)((R + ROWS_PER_WG - 1) / ROWS_PER_WG);
-  for (int64_t i1 = 0; i1 < K; i1 += bs) {
-    const int count = (int)((K - i1) < bs ? (K - i1) : bs);
-    p.i1 = (int)i1;
-    p.count = count;
-    hipLaunchKernelGGL(kern, dim3(wgs), dim3(256), smem, st, p);
-    LLMC_LAUNCH_STATUS();
-    const int64_t i2 = i1 + count;
-    if (i2 < K) {
+  // Lazy updates on two levels.  After a block is quantised its scaled errors E_b update only the
+  // columns left in its group of GROUP blocks (what the next block needs); the columns beyond the
+  // group get the whole group's errors in one rank-(GROUP*bs) product.  Same sums as updating
+  // everything after every block, regrouped -- but the big part of W is read and written a
+  // quarter as often, which is what bounds a rank-128 update.
+  const int ldE = GROUP * GB;
+  p.ldE = ldE;
+  for (int64_t g0 = 0; g0 < K; g0 += (int64_t)GROUP * bs) {
+    const int64_t gend = (g0 + (int64_t)GROUP * bs) < K ? g0 + (int64_t)GROUP * bs : K;
+    for (int64_t i1 = g0; i1 < gend; i1 += bs) {
+      const int count = (int)((gend - i1) < bs ? (gend - i1) : bs);
+      p.i1 = (int)i1;
+      p.count = count;
+      p.E = E + (i1 - g0);
+      hipLaunchKernelGGL(kern, dim3(wgs), dim3(256), smem, st, p);
+      LLMC_LAUNCH_STATUS();
+      const int64_t i2 = i1 + count;
+      if (i2 < gend) {
+        GemmF32 g = {};
+        g.A = p.E; g.lda = ldE; g.B = U + i1 * ldu + i2; g.ldb = ldu; g.C = Wf + i2; g.ldc = K;
+        g.M = (int)R; g.N = (int)(gend - i2); g.Kc = count; g.alpha = -1.f; g.beta = 1.f; g.batch = 1;
+        const int rc = llmc_gemm_f32(g, st);
+        if (rc) return rc;
+      }
+    }
+    if (gend < K) {
       GemmF32 g = {};
-      g.A = E; g.lda = GB; g.B = U + i1 * ldu + i2; g.ldb = ldu; g.C = Wf + i2; g.ldc = K;
-      g.M = (int)R; g.N = (int)(K - i2); g.Kc = count; g.alpha = -1.f; g.beta = 1.f; g.batch = 1;
+      g.A = E; g.lda = ldE; g.B = U + g0 * ldu + gend; g.ldb = ldu; g.C = Wf + gend; g.ldc = K;
+      g.M = (int)R; g.N = (int)(K - gend); g.Kc = (int)(gend - g0); g.alpha = -1.f; g.beta = 1.f; g.batch = 1;
       const int rc = llmc_gemm_f32(g, st);
       if (rc) return rc;
     }
