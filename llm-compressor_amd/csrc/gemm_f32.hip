@@ -114,13 +114,21 @@ __device__ __forceinline__ void gemm_tile(const GemmF32& g, const float* A, cons
   };
 
   if (k_begin < k_end) {
+    // two LDS stages: slab k+1 is fetched into registers before slab k is multiplied and
+    // written to the other stage after it, one barrier per slab
+    constexpr int STAGE_A = BK * LDA_S, STAGE_B = BK * LDB_S;
+    float* const As0 = As;
+    float* const Bs0 = Bs;
     load_slab(k_begin);
     store_slab();
     __syncthreads();
+    int cur = 0;
     for (int k0 = k_begin; k0 + BK < k_end; k0 += BK) {
       load_slab(k0 + BK);
       multiply();
-      __syncthreads();
+      cur ^= 1;
+      As = As0 + cur * STAGE_A;
+      Bs = Bs0 + cur * STAGE_B;
       store_slab();
       __syncthreads();
     }
@@ -145,10 +153,13 @@ __device__ __forceinline__ void gemm_tile(const GemmF32& g, const float* A, cons
     }
 }
 
-template <int BM, int BN, bool TRANS_B>
+// ALL_FAST: the host has checked that every tile of the launch takes the unconditional path
+// (M, N multiples of the tile, contraction ranges multiples of BK, 16-byte aligned rows), so the
+// bounds-checked variant is not even instantiated: fewer registers, more waves per SIMD.
+template <int BM, int BN, bool TRANS_B, bool ALL_FAST>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32 g, int vec) {
-  __shared__ float As[BK * (BM + 4)];
-  __shared__ float Bs[BK * (BN + 4)];
+  __shared__ float As[2 * BK * (BM + 4)];
+  __shared__ float Bs[2 * BK * (BN + 4)];
   const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
   if (g.c_lower && n0 > m0 + BM - 1) return;
   const float* A = g.A + (int64_t)blockIdx.z * g.stride_a;
@@ -157,11 +168,15 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32 g, int vec) {
   const int k_begin = g.b_lower_tri ? (n0 / BK) * BK : 0;
   int k_end = g.Kc;
   if (g.a_lower_tri && m0 + BM < k_end) k_end = m0 + BM;
-  const bool fast = vec && m0 + BM <= g.M && n0 + BN <= g.N && ((k_end - k_begin) % BK) == 0;
-  if (fast)
+  if (ALL_FAST) {
     gemm_tile<BM, BN, TRANS_B, true>(g, A, B, C, m0, n0, k_begin, k_end, As, Bs);
-  else
-    gemm_tile<BM, BN, TRANS_B, false>(g, A, B, C, m0, n0, k_begin, k_end, As, Bs);
+  } else {
+    const bool fast = vec && m0 + BM <= g.M && n0 + BN <= g.N && ((k_end - k_begin) % BK) == 0;
+    if (fast)
+      gemm_tile<BM, BN, TRANS_B, true>(g, A, B, C, m0, n0, k_begin, k_end, As, Bs);
+    else
+      gemm_tile<BM, BN, TRANS_B, false>(g, A, B, C, m0, n0, k_begin, k_end, As, Bs);
+  }
 }
 
 }  // namespace
@@ -174,19 +189,21 @@ int llmc_gemm_f32(const GemmF32& g, hipStream_t st) {
                       : 0;
   // 128x128 tiles when they still give the chip enough workgroups, 64x64 otherwise
   const int64_t t128 = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * g.batch;
-  if (t128 >= 256 && g.M >= 128 && g.N >= 128) {
-    dim3 grid((g.N + 127) / 128, (g.M + 127) / 128, g.batch);
-    if (g.trans_b)
-      hipLaunchKernelGGL((gemm_f32_kernel<128, 128, true>), grid, dim3(256), 0, st, g, vec);
-    else
-      hipLaunchKernelGGL((gemm_f32_kernel<128, 128, false>), grid, dim3(256), 0, st, g, vec);
+  const bool big = t128 >= 256 && g.M >= 128 && g.N >= 128;
+  const int bt = big ? 128 : 64;
+  // every tile unconditional?  (a_lower_tri / b_lower_tri cut the contraction at tile edges, which
+  // are multiples of BK for both tile sizes)
+  const bool all_fast = vec && g.M % bt == 0 && g.N % bt == 0 && g.Kc % BK == 0;
+  dim3 grid((g.N + bt - 1) / bt, (g.M + bt - 1) / bt, g.batch);
+#define LLMC_GEMM(BT, TB, AF) hipLaunchKernelGGL((gemm_f32_kernel<BT, BT, TB, AF>), grid, dim3(256), 0, st, g, vec)
+  if (big) {
+    if (g.trans_b) { if (all_fast) LLMC_GEMM(128, true, true); else LLMC_GEMM(128, true, false); }
+    else { if (all_fast) LLMC_GEMM(128, false, true); else LLMC_GEMM(128, false, false); }
   } else {
-    dim3 grid((g.N + 63) / 64, (g.M + 63) / 64, g.batch);
-    if (g.trans_b)
-      hipLaunchKernelGGL((gemm_f32_kernel<64, 64, true>), grid, dim3(256), 0, st, g, vec);
-    else
-      hipLaunchKernelGGL((gemm_f32_kernel<64, 64, false>), grid, dim3(256), 0, st, g, vec);
+    if (g.trans_b) { if (all_fast) LLMC_GEMM(64, true, true); else LLMC_GEMM(64, true, false); }
+    else { if (all_fast) LLMC_GEMM(64, false, true); else LLMC_GEMM(64, false, false); }
   }
+#undef LLMC_GEMM
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : 1000 + (int)e;
 }
