@@ -69,6 +69,16 @@ int llmc_hessian_accumulate(float* H, int64_t ldh, const void* X, int64_t ldx,
                             int32_t flags, void* workspace, int64_t workspace_bytes,
                             void* stream);
 
+/* Grouped form for the per-expert Hessians of an MoE layer (the 128 x 3 accumulate_hessian calls
+ * that LinearExperts2D.forward triggers per batch, modeling/moe/linear_experts.py:235-268): n
+ * independent problems of one width K in one launch.  H, X and T are HOST arrays of n device
+ * pointers / token counts (they are passed to the kernel by value, 128 problems per launch); all
+ * problems share ldh, ldx and the dtype; K % 8 == 0 and every X[i] 16-byte aligned.  A problem
+ * with T[i] == 0 (an expert that received no token) leaves its Hessian untouched. */
+int llmc_hessian_accumulate_grouped(float* const* H, int64_t ldh, const void* const* X, int64_t ldx,
+                                    const int64_t* T, int32_t n, int64_t K, int32_t x_dtype,
+                                    float alpha, int32_t flags, void* stream);
+
 /* ---- a10/a11: min-max observers --------------------------------------------
  * Replace _get_min_max() = torch.amin/amax(observed, dim=(0,-1)) on the
  * flattened weight (src/llmcompressor/observers/min_max.py:70-74 with

@@ -196,11 +196,32 @@ __device__ __forceinline__ void tile_epilogue(float* __restrict__ H, int64_t ldh
 // BT x BT output tile, 256 threads = 2x2 waves, each wave (BT/2)x(BT/2) = MI x MI MFMA tiles.
 // LDS holds two stages of the two feature-major panels; global loads for slab s+2 are in
 // flight while slab s is multiplied and slab s+1 is transposed into the other stage.
-template <int BT, int DT, bool ALIGNED, bool FAST_EPI>
+// Up to GROUP_MAX independent problems of one width K in one launch (blockIdx.y = problem), each
+// with its own Hessian, activation block and token count -- the per-expert Hessians of an MoE
+// layer.  The pointer table travels in the kernel arguments, so the call needs no device-side
+// table and no copy.  Problems without tokens leave their Hessian untouched.
+constexpr int GROUP_MAX = 128;
+struct GroupArgs {
+  static constexpr bool grouped = true;
+  float* H[GROUP_MAX];
+  const uint16_t* X[GROUP_MAX];
+  int T[GROUP_MAX];
+};
+struct NoGroup {
+  static constexpr bool grouped = false;
+};
+
+template <int BT, int DT, bool ALIGNED, bool FAST_EPI, class GRP>
 __global__ __launch_bounds__(256) void hessian_syrk_kernel(float* __restrict__ H, int64_t ldh,
                                                             const uint16_t* __restrict__ Xfull, int64_t ldx,
                                                             int Tfull, int K, float alpha, int assume_sym,
-                                                            int nb, Plan plan, float* __restrict__ ws) {
+                                                            int nb, Plan plan, float* __restrict__ ws, GRP grp) {
+  if constexpr (GRP::grouped) {
+    Tfull = grp.T[blockIdx.y];
+    if (Tfull <= 0) return;
+    H = grp.H[blockIdx.y];
+    Xfull = grp.X[blockIdx.y];
+  }
   constexpr int RT = BT / 32;  // token rows per thread per panel
   constexpr int GI = BT / 8;   // 8-feature groups per panel
   constexpr int MI = BT / 64;
@@ -371,11 +392,14 @@ __global__ __launch_bounds__(256) void hessian_syrk_kernel(float* __restrict__ H
 #pragma unroll
     for (int a = 0; a < MI; ++a)
 #pragma unroll
-      for (int b = 0; b < MI; ++b)
+      for (int b = 0; b < MI; ++b) {
 #pragma unroll
         for (int vq = 0; vq < 4; ++vq)
           *(float4*)(slot + (((a * MI + b) * 4 + vq) * 256 + tid) * 4) =
               make_float4(acc[a][b][vq * 4], acc[a][b][vq * 4 + 1], acc[a][b][vq * 4 + 2], acc[a][b][vq * 4 + 3]);
+        // one MFMA tile at a time: moving all 256 accumulators out of the AGPRs at once spills
+        __builtin_amdgcn_sched_barrier(0);
+      }
     return;
   }
   tile_epilogue<BT, FAST_EPI>(H, ldh, K, alpha, assume_sym, i0, j0, acc);
@@ -545,14 +569,14 @@ int launch(const Choice& c, float* H, int64_t ldh, const void* X, int64_t ldx, i
   constexpr int smem = 4 * BT * ROW_BYTES;
   // 16-byte read-modify-write epilogue needs a symmetric H and 16-byte aligned rows
   const bool fast = sym && vec_ok;
-  auto kern = aligned ? (fast ? hessian_syrk_kernel<BT, DT, true, true> : hessian_syrk_kernel<BT, DT, true, false>)
-                      : (fast ? hessian_syrk_kernel<BT, DT, false, true> : hessian_syrk_kernel<BT, DT, false, false>);
+  auto kern = aligned ? (fast ? hessian_syrk_kernel<BT, DT, true, true, NoGroup> : hessian_syrk_kernel<BT, DT, true, false, NoGroup>)
+                      : (fast ? hessian_syrk_kernel<BT, DT, false, true, NoGroup> : hessian_syrk_kernel<BT, DT, false, false, NoGroup>);
   if (smem > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return 1000 + (int)e;
   }
   hipLaunchKernelGGL(kern, dim3(c.grid), dim3(256), smem, st, H, ldh, (const uint16_t*)X, ldx, (int)T,
-                     (int)K, alpha, sym, nb, c.plan, ws);
+                     (int)K, alpha, sym, nb, c.plan, ws, NoGroup{});
   LLMC_LAUNCH_STATUS();
   if (c.nsplit_tiles > 0) {
     if (fast)
@@ -595,6 +619,66 @@ extern "C" int llmc_hessian_accumulate(float* H, int64_t ldh, const void* X, int
                        : launch<128, LLMC_BF16>(c, H, ldh, X, ldx, T, K, alpha, flags, ws, st);
   return c.bt == 256 ? launch<256, LLMC_F16>(c, H, ldh, X, ldx, T, K, alpha, flags, ws, st)
                      : launch<128, LLMC_F16>(c, H, ldh, X, ldx, T, K, alpha, flags, ws, st);
+}
+
+template <int BT, int DT>
+int launch_grouped(const GroupArgs& grp, int n, int64_t ldh, int64_t ldx, int64_t K, float alpha, int sym, bool fast,
+                   hipStream_t st) {
+  const Choice c = make_choice(BT, /*T=*/64, K, /*split=*/false);  // whole tiles: one phase over all of them
+  const int nb = (int)((K + BT - 1) / BT);
+  constexpr int smem = 4 * BT * ROW_BYTES;
+  auto kern = fast ? hessian_syrk_kernel<BT, DT, true, true, GroupArgs> : hessian_syrk_kernel<BT, DT, true, false, GroupArgs>;
+  if (smem > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return 1000 + (int)e;
+  }
+  hipLaunchKernelGGL(kern, dim3(c.grid, n), dim3(256), smem, st, (float*)nullptr, ldh, (const uint16_t*)nullptr, ldx, 0,
+                     (int)K, alpha, sym, nb, c.plan, (float*)nullptr, grp);
+  LLMC_LAUNCH_STATUS();
+  return 0;
+}
+
+extern "C" int llmc_hessian_accumulate_grouped(float* const* H, int64_t ldh, const void* const* X, int64_t ldx,
+                                               const int64_t* T, int32_t n, int64_t K, int32_t x_dtype,
+                                               float alpha, int32_t flags, void* stream) {
+  LLMC_CHECK_ARG(H != nullptr && n >= 0, 1);
+  LLMC_CHECK_ARG(K > 0 && K < (1 << 30) && K % 8 == 0 && ldh >= K, 2);
+  LLMC_CHECK_ARG(X != nullptr, 3);
+  LLMC_CHECK_ARG(ldx >= K && ldx % 8 == 0, 4);
+  LLMC_CHECK_ARG(T != nullptr, 5);
+  LLMC_CHECK_ARG(x_dtype == LLMC_BF16 || x_dtype == LLMC_F16, 8);
+  hipStream_t st = (hipStream_t)stream;
+  const int sym = (flags & LLMC_HESSIAN_ASSUME_SYMMETRIC) ? 1 : 0;
+  bool fast = sym && (ldh & 3) == 0;
+  for (int i = 0; i < n; ++i) {
+    LLMC_CHECK_ARG(T[i] >= 0 && T[i] < (1ll << 31), 5);
+    if (T[i] == 0) continue;
+    LLMC_CHECK_ARG(H[i] != nullptr, 1);
+    LLMC_CHECK_ARG(X[i] != nullptr && (((uintptr_t)X[i]) & 15) == 0, 3);
+    if (((uintptr_t)H[i]) & 15) fast = false;
+  }
+  const bool big = K >= 512;
+  for (int base = 0; base < n; base += GROUP_MAX) {
+    const int cnt = (n - base) < GROUP_MAX ? (n - base) : GROUP_MAX;
+    GroupArgs grp;
+    bool any = false;
+    for (int i = 0; i < cnt; ++i) {
+      grp.H[i] = H[base + i];
+      grp.X[i] = (const uint16_t*)X[base + i];
+      grp.T[i] = (int)T[base + i];
+      any = any || T[base + i] > 0;
+    }
+    if (!any) continue;
+    int rc;
+    if (x_dtype == LLMC_BF16)
+      rc = big ? launch_grouped<256, LLMC_BF16>(grp, cnt, ldh, ldx, K, alpha, sym, fast, st)
+               : launch_grouped<128, LLMC_BF16>(grp, cnt, ldh, ldx, K, alpha, sym, fast, st);
+    else
+      rc = big ? launch_grouped<256, LLMC_F16>(grp, cnt, ldh, ldx, K, alpha, sym, fast, st)
+               : launch_grouped<128, LLMC_F16>(grp, cnt, ldh, ldx, K, alpha, sym, fast, st);
+    if (rc) return rc;
+  }
+  return 0;
 }
 
 extern "C" int llmc_version(void) { return 1; }

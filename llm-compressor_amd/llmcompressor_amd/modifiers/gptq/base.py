@@ -50,6 +50,10 @@ class GPTQModifier(Modifier, QuantizationMixin):
     :param offload_hessians: keep Hessians on the CPU between hook calls
     :param hessian_batch_tokens: stage activations and launch the Hessian kernel once this many tokens
         are pending (0 = one launch per hook call, the reference's behaviour)
+
+    Expert Linears inside a ``LinearExperts2D`` block are handled together: while the block's forward
+    runs, their hook calls are only recorded, and when it returns all experts' Hessians of one width
+    are updated by a single grouped launch (384 tiny launches per batch become three).
     """
 
     requires_calibration_data: bool = True
@@ -64,6 +68,7 @@ class GPTQModifier(Modifier, QuantizationMixin):
     _hessians: dict = PrivateAttr(default_factory=dict)
     _num_samples: dict = PrivateAttr(default_factory=dict)
     _staged: dict = PrivateAttr(default_factory=dict)
+    _group_pending: list | None = PrivateAttr(default=None)
 
     def resolve_quantization_config(self) -> QuantizationConfig:
         config = super().resolve_quantization_config()
@@ -112,6 +117,12 @@ class GPTQModifier(Modifier, QuantizationMixin):
         if not added_hook:
             raise ValueError("GPTQModifier was unable to find any modules to quantize. Please check quantization "
                              "`config_groups` and `targets` in recipe")
+        from llmcompressor_amd.modeling.moe import LinearExperts2D
+
+        for module in state.model.modules():
+            if isinstance(module, LinearExperts2D):
+                self.register_hook(module, self._begin_expert_group, "forward_pre")
+                self.register_hook(module, self._end_expert_group, "forward")
 
     def on_sequential_epoch_end(self, state: State, event: Event, modules: list[torch.nn.Module] = (), **kwargs):
         modules = [m for m in modules if is_module_quantized(m)]
@@ -132,12 +143,33 @@ class GPTQModifier(Modifier, QuantizationMixin):
             init_device = "cpu" if self.offload_hessians else device
             self._hessians[module] = make_empty_hessian(module, device=init_device)
             self._num_samples[module] = torch.zeros(tuple(), device=device)
+        if (self._group_pending is not None and isinstance(module, torch.nn.Linear) and inp.is_cuda
+                and not self.offload_hessians and inp.dtype in (torch.bfloat16, torch.float16)):
+            self._group_pending.append((module, inp))
+            return
         if self.hessian_batch_tokens > 0 and not self.offload_hessians and isinstance(module, torch.nn.Linear):
             self._stage(module, inp)
             return
         with self._maybe_onload_hessian(module):
             self._hessians[module], self._num_samples[module] = accumulate_hessian(
                 inp, module, self._hessians[module], self._num_samples[module])
+
+    # -- expert groups (see the class docstring)
+    def _begin_expert_group(self, _module, _args):
+        if self._group_pending is None:
+            self._group_pending = []
+
+    def _end_expert_group(self, _module, _args, _output):
+        pending, self._group_pending = self._group_pending, None
+        by_width = {}
+        for module, inp in pending or ():
+            # accumulate_hessian counts a 2-D input as one sample, a batched one by its batch entries
+            self._num_samples[module] += 1 if inp.ndim == 2 else inp.shape[0]
+            x = inp.reshape(-1, inp.shape[-1])
+            by_width.setdefault((x.shape[1], x.dtype), []).append((self._hessians[module], x))
+        for group in by_width.values():
+            ops.hessian_accumulate_grouped_([h for h, _ in group], [x for _, x in group], alpha=2.0,
+                                            assume_symmetric=True)
 
     # -- token staging (see the class docstring).  The hook runs once per Linear per batch, so it is
     # kept to one device copy: the sample count is kept on the host until the flush.

@@ -51,6 +51,50 @@ def hessian_accumulate_(H: torch.Tensor, x: torch.Tensor, alpha: float = 2.0, as
     return H
 
 
+def hessian_accumulate_grouped_(Hs, xs, alpha: float = 2.0, assume_symmetric: bool = True):
+    """One launch for many independent problems of the same width (the per-expert Hessians of an MoE
+    layer): Hs[i] (fp32 [K,K], in place) += alpha * xs[i]^T xs[i] with xs[i] = [T_i, K], T_i >= 0.
+    All Hs share a row stride, all xs a row stride and dtype; every xs[i] is 16-byte aligned."""
+    import ctypes
+
+    assert len(Hs) == len(xs)
+    if not Hs:
+        return Hs
+    H0 = Hs[0]
+    K = H0.shape[0]
+    x_ref = next((x for x in xs if x.shape[0] > 0), None)
+    if x_ref is None:
+        return Hs
+    _require_gpu(H0, x_ref)
+    if x_ref.dtype not in (torch.bfloat16, torch.float16):
+        raise TypeError(f"hessian_accumulate_grouped_: unsupported activation dtype {x_ref.dtype}")
+    n = len(Hs)
+    hp = (ctypes.c_void_p * n)()
+    xp = (ctypes.c_void_p * n)()
+    tc = (ctypes.c_int64 * n)()
+    keep = []
+    for i, (H, x) in enumerate(zip(Hs, xs)):
+        assert H.dtype == torch.float32 and H.shape == (K, K) and H.stride(1) == 1 and H.stride(0) == H0.stride(0)
+        assert x.ndim == 2 and x.shape[1] == K and H.device == H0.device
+        tc[i] = x.shape[0]
+        hp[i] = H.data_ptr()
+        if x.shape[0] > 0:
+            if x.dtype != x_ref.dtype:
+                raise TypeError("hessian_accumulate_grouped_: mixed activation dtypes")
+            if x.stride(1) != 1 or x.stride(0) != x_ref.stride(0) or x.data_ptr() % 16:
+                x = x.contiguous()
+                if x.stride(0) != x_ref.stride(0):
+                    raise ValueError("hessian_accumulate_grouped_: activation blocks need one common row stride")
+                keep.append(x)
+            xp[i] = x.data_ptr()
+    with torch.cuda.device(H0.device):
+        rc = _lib.lib().llmc_hessian_accumulate_grouped(
+            hp, H0.stride(0), xp, x_ref.stride(0), tc, n, K, _DT[x_ref.dtype], float(alpha),
+            1 if assume_symmetric else 0, _stream(H0))
+    _lib.check(rc, "llmc_hessian_accumulate_grouped")
+    return Hs
+
+
 FMT_INT, FMT_FP8, FMT_FP4 = 0, 1, 2
 SCALE_PLAIN, SCALE_NVFP4, SCALE_MXFP4 = 0, 1, 2
 OUT_FAKEQUANT, OUT_CODES, OUT_PACKED = 0, 1, 2

@@ -122,3 +122,50 @@ def test_hessian_full_size_token_chunks():
     ref = 2 * (x[:, rows].double().t() @ x.double())
     assert _rel(H[rows], ref) < TOL
     assert torch.equal(H, H.t())
+
+
+def test_hessian_grouped_moe_shapes():
+    """Config-5 shapes: 128 experts with routed token counts (some zero), widths 2048 and 768, one launch
+    per projection; each expert's Hessian equals the single-problem entry point's, bit for bit where that
+    one also runs whole tiles, and an expert without tokens keeps its Hessian."""
+    from llmcompressor_amd import ops
+
+    g = torch.Generator().manual_seed(0)
+    E = 128
+    w = 1.0 / torch.arange(1, E + 1, dtype=torch.float64) ** 1.1
+    idx = torch.multinomial(w / w.sum(), 4096 * 8, replacement=True, generator=g)
+    n_e = torch.bincount(idx, minlength=E)
+    n_e[5] = 0
+    n_e[77] = 0
+    for K in (2048, 768):
+        x_all = torch.randn(int(n_e.sum()), K, generator=g).bfloat16().cuda()
+        offs = torch.cat([torch.zeros(1, dtype=torch.long), torch.cumsum(n_e, 0)])
+        xs = [x_all[int(offs[e]): int(offs[e + 1])] for e in range(E)]
+        H = torch.zeros(E, K, K, device="cuda")
+        H[5] = 3.0  # must stay as it is
+        ops.hessian_accumulate_grouped_([H[e] for e in range(E)], xs)
+        assert torch.equal(H[5], torch.full_like(H[5], 3.0)) and torch.count_nonzero(H[77]) == 0
+        for e in (0, 1, 17, 64, 127):
+            ref = 2 * (xs[e].double().t() @ xs[e].double())
+            if n_e[e] > 0:
+                assert _rel(H[e], ref) < TOL, (K, e)
+            assert torch.equal(H[e], H[e].t())
+            single = torch.zeros(K, K, device="cuda")
+            if n_e[e] > 0:
+                ops.hessian_accumulate_(single, xs[e], use_workspace=False)
+            assert _rel(H[e], single) < 1e-6 if n_e[e] > 0 else torch.count_nonzero(H[e]) == 0
+        # second launch accumulates on top
+        ops.hessian_accumulate_grouped_([H[e] for e in range(E)], xs)
+        ref = 4 * (xs[0].double().t() @ xs[0].double())
+        assert _rel(H[0], ref) < TOL
+    # the oracle on a small grouped case, f16 inputs, more problems than one launch holds
+    K, E = 96, 150
+    xs = [torch.randn(int(t), K, generator=g).half().cuda() for t in torch.randint(0, 40, (E,), generator=g)]
+    Hs = [torch.zeros(K, K, device="cuda") for _ in range(E)]
+    ops.hessian_accumulate_grouped_(Hs, xs)
+    for e in (0, 3, 129, 149):
+        Hc, _ = G.accumulate_hessian(xs[e].cpu(), G.make_empty_hessian(K), torch.zeros(()))
+        if xs[e].shape[0]:
+            assert _rel(Hs[e].cpu(), Hc) < TOL
+        else:
+            assert torch.count_nonzero(Hs[e]) == 0

@@ -364,9 +364,25 @@ def test_moe_gptq_zero_token_expert_is_zeroed():
     x = torch.randn(T, H, device=DEV).bfloat16()
     idx = torch.stack([torch.arange(T) % 3, (torch.arange(T) + 1) % 3], dim=1).to(DEV)  # expert 3 never routed
     wts = torch.full((T, 2), 0.5, device=DEV, dtype=torch.bfloat16)
-    with torch.no_grad():
-        for _ in range(3):
-            experts(x, idx, wts)
+    calls = []
+    from llmcompressor_amd import ops
+    raw_grouped = ops.hessian_accumulate_grouped_
+    ops.hessian_accumulate_grouped_ = lambda Hs, xs, **kw: (calls.append(len(Hs)), raw_grouped(Hs, xs, **kw))[1]
+    try:
+        with torch.no_grad():
+            for _ in range(3):
+                experts(x, idx, wts)
+    finally:
+        ops.hessian_accumulate_grouped_ = raw_grouped
+    # the experts' hook calls were flushed as grouped launches: per forward one for the gate/up width
+    # (2 x 4 problems) and one for the down width (4 problems)
+    assert sorted(calls) == [4, 4, 4, 8, 8, 8]
+    routed0 = x[(idx == 0).any(dim=1)].double()
+    H0 = mod._hessians[experts[0].gate_proj]
+    ref = 3 * 2 * (routed0.t() @ routed0)
+    assert ((H0.double() - ref).norm() / ref.norm()).item() < 1e-5
+    assert float(mod._num_samples[experts[0].gate_proj]) == 3.0 and float(mod._num_samples[experts[3].up_proj]) == 3.0
+    assert torch.count_nonzero(mod._hessians[experts[3].gate_proj]) == 0
     LifecycleCallbacks.sequential_epoch_end(modules=list(model.modules()))
     LifecycleCallbacks.calibration_end()
     session.finalize()
