@@ -9,6 +9,9 @@
 // the operand shape of v_mfma_f32_32x32x16_{bf16,f16}.  bf16 x bf16 products
 // are exact in fp32 and the accumulation is fp32, so the result differs from
 // an fp32 GEMM on the upcast inputs only by summation order.
+#include <stdlib.h>
+#include <string.h>
+
 #include <type_traits>
 
 #include "common.h"
@@ -493,7 +496,7 @@ struct Choice {
 // over are cut along the tokens so that they fill a round too: R <= 128 -> one phase of
 // floor(256/R) chunks per tile; R > 128 -> 128 tiles in two chunks, then the rest as before.  A
 // chunk keeps at least 4 slabs.  time_us is a rough model (measured microseconds per slab and per
-// epilogue of one tile, partial tiles through the workspace at 2 TB/s) used only to pick between
+// epilogue of one tile, partial tiles through the workspace at 3 TB/s) used only to pick between
 // candidates.
 Choice make_choice(int bt, int64_t T, int64_t K, bool split) {
   Choice c;
@@ -501,7 +504,7 @@ Choice make_choice(int bt, int64_t T, int64_t K, bool split) {
   const int nb = (int)((K + bt - 1) / bt);
   const int nt = nb * (nb + 1) / 2;
   const int nslab = (int)((T + BK - 1) / BK);
-  const double slab_us = bt == 256 ? 1.75 : 0.6, epi_us = bt == 256 ? 35.0 : 10.0, chunk_epi_us = 5.0;
+  const double slab_us = bt == 256 ? 1.75 : 0.7, epi_us = bt == 256 ? 35.0 : 10.0, chunk_epi_us = 5.0;
   Plan& plan = c.plan;
   plan.nphase = 0;
   int wg = 0, tile0 = 0, ws_tile = 0;
@@ -542,7 +545,7 @@ Choice make_choice(int bt, int64_t T, int64_t K, bool split) {
   }
   c.nsplit_tiles = nt - (c.first_split_phase < plan.nphase ? plan.ph[c.first_split_phase].tile0 : nt);
   c.ws_bytes = (int64_t)ws_tile * bt * bt * 4;
-  c.time_us += c.ws_bytes * 2 / 2e6 + (ws_tile ? 20.0 : 0.0);  // partial tiles written and read back, reduce kernel
+  c.time_us += c.ws_bytes * 2 / 3e6 + (ws_tile ? 15.0 : 0.0);  // partial tiles written and read back, reduce kernel
   c.grid = wg;
   return c;
 }
@@ -550,6 +553,12 @@ Choice make_choice(int bt, int64_t T, int64_t K, bool split) {
 // the fastest of {128, 256}-wide tiles x {whole tiles, token chunks} that fits the workspace
 Choice choose(int64_t T, int64_t K, int64_t ws_avail) {
   Choice best;
+#ifdef LLMC_HESSIAN_EXPERIMENT
+  if (const char* f = getenv("LLMC_HESSIAN_FORCE")) {  // "256,1" = tile width, split
+    const int bt = atoi(f), sp = atoi(strchr(f, ',') + 1);
+    return make_choice(bt, T, K, sp != 0);
+  }
+#endif
   for (int bt : {256, 128})
     for (int split = 0; split < 2; ++split) {
       const Choice c = make_choice(bt, T, K, split != 0);
