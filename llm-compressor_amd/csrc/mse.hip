@@ -137,6 +137,186 @@ __global__ __launch_bounds__(256) void mse_team_kernel(MseParams p, int64_t ngro
   or_flags(p.flags, mask);
 }
 
+// ---- 16-bit inputs: the same arithmetic with everything the format decides fixed at compile time,
+// the division by the step's scale done with the shared-divisor sequence (exact, see qformat.h), the
+// e4m3 / e2m1 rounding done by the conversion instructions, and the power evaluated as
+// 2^(norm*log2 a) in extended precision.
+
+// a^norm (a >= 0) rounded to DT.  a = m*2^E; norm*E is exact in fp32 (norm has at most 11
+// significant bits, E at most 8) and splits into an integer I and a fraction r, so
+// a^norm = 2^I * 2^(r + norm*log2 m) with the second exponent small: the hardware log2/exp2 (1 ulp
+// each) leave a few ulps of error in total.  If rounding to DT could fall either way within 16 ulps
+// the library powf decides, so the rounded value matches the reference's pow-then-round.
+template <int DT>
+__device__ __forceinline__ float pow_round16(float a, float norm) {
+  const float m = __builtin_amdgcn_frexp_mantf(a);
+  const int E = __builtin_amdgcn_frexp_expf(a);
+  const float y = norm * (float)E;
+  const float I = rintf(y);
+  const float t = fmaf(norm, __builtin_amdgcn_logf(m), y - I);
+  const float pf = ldexpf(__builtin_amdgcn_exp2f(t), (int)I);
+  const uint32_t w = pack16<DT>(pf * 0.99999809265136719f, pf * 1.0000019073486328f);  // 1 -+ 2^-19
+  if ((w & 0xffffu) != (w >> 16)) return round_rt(powf(a, norm), DT);
+  return DT == LLMC_BF16 ? __uint_as_float(w << 16) : f16_bits_to_f32((uint16_t)(w & 0xffffu));
+}
+
+template <int DT>
+__device__ __forceinline__ void unpack8t(const uint4& v, float* x) {
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    if (DT == LLMC_BF16) {
+      x[2 * j] = __uint_as_float(w[j] << 16);
+      x[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+    } else {
+      x[2 * j] = f16_bits_to_f32((uint16_t)(w[j] & 0xffffu));
+      x[2 * j + 1] = f16_bits_to_f32((uint16_t)(w[j] >> 16));
+    }
+  }
+}
+
+// sum over 8 elements of |fq(x) - x|^norm, every intermediate rounded to DT
+template <int DT, int FMT, bool HAS_ZP>
+__device__ __forceinline__ float chunk_error(const float (&x)[8], float s, float zp, const QFormat& f, float norm) {
+  float v[8];
+  const FastDiv d = make_fastdiv(s);
+  bool big = false, small = false;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    v[j] = fastdiv(x[j], d);
+    big = big | !fastdiv_big_ok(v[j]);
+    small = small | fastdiv_small(v[j]);
+  }
+  bool redo = big | !d.ok;
+  if (small) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) redo = redo | (fastdiv_small(v[j]) & (x[j] != 0.f));
+  }
+  if (redo) {
+    float err = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float q = quantize_value(x[j], s, zp, HAS_ZP, DT, f);
+      const float dq = dequantize_value(q, s, zp, HAS_ZP, DT);
+      const float a = fabsf(round_rt(dq - x[j], DT));
+      err += round_rt(norm == 2.0f ? a * a : powf(a, norm), DT);
+    }
+    return err;
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    v[j] = round16_finite<DT>(v[j]);
+    v[j] = HAS_ZP ? round16_finite<DT>(v[j] + zp) : v[j] + 0.0f;
+    v[j] = __builtin_amdgcn_fmed3f(v[j], f.qmin, f.qmax);
+    if (FMT == LLMC_FMT_INT) v[j] = rintf(v[j]);
+  }
+  if (FMT == LLMC_FMT_FP8) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const f32x2_t t = hw_e4m3_pair_decode(hw_e4m3_pair(v[2 * j], v[2 * j + 1]));
+      v[2 * j] = t.x;
+      v[2 * j + 1] = t.y;
+    }
+  } else if (FMT == LLMC_FMT_FP4) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const f32x2_t t = hw_e2m1_pair_decode(hw_e2m1_pair(v[2 * j], v[2 * j + 1]));
+      v[2 * j] = t.x;
+      v[2 * j + 1] = t.y;
+    }
+  }
+  float err = 0.f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    float dq = v[j];
+    if (HAS_ZP) dq = round16_finite<DT>(dq - zp);
+    dq = round16_finite<DT>(dq * s);
+    const float a = fabsf(round16_finite<DT>(dq - x[j]));
+    err += norm == 2.0f ? round16_finite<DT>(a * a) : pow_round16<DT>(a, norm);
+  }
+  return err;
+}
+
+// 16-bit inputs, groups of g = 8*L consecutive elements (L a power of two <= 64 lanes per group)
+template <int DT, int FMT, bool SYM>
+__global__ __launch_bounds__(256) void mse_team_fast_kernel(MseParams p, int64_t ngroups, int ng, int g, int lshift,
+                                                            int64_t ldw) {
+  const int L = 1 << lshift;
+  const int64_t gtid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t grp = gtid >> lshift;
+  const int sub = (int)(gtid & (L - 1));
+  const bool live = grp < ngroups;
+  const QFormat f = make_qformat(FMT, p.bits);
+  float xv[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) xv[j] = 0.f;
+  float mn = INFINITY, mx = -INFINITY;
+  if (live) {
+    const int64_t r = grp / ng, gi = grp % ng;
+    const uint4 v = *(const uint4*)((const uint16_t*)p.x + r * ldw + gi * g + (int64_t)sub * 8);
+    unpack8t<DT>(v, xv);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      mn = fminf(mn, xv[j]);
+      mx = fmaxf(mx, xv[j]);
+    }
+  }
+  for (int o = L >> 1; o > 0; o >>= 1) {
+    mn = fminf(mn, __shfl_xor(mn, o, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+  }
+  mn = round_to<DT>(mn * p.expand);
+  mx = round_to<DT>(mx * p.expand);
+  float best = DT == LLMC_BF16 ? 3.3895313892515355e38f : 65504.0f;
+  uint64_t mask[MASK_WORDS];
+#pragma unroll
+  for (int wd = 0; wd < MASK_WORDS; ++wd) mask[wd] = 0ull;
+  for (int i = 0; i < p.steps; ++i) {
+    const float pi = step_factor(i, p.grid);
+    const float smin = round_to<DT>(mn * pi), smax = round_to<DT>(mx * pi);
+    float s, zp;
+    int e;
+    qparams_from_minmax(smin, smax, DT, f, SYM, p.scale_mode, 1.f, &s, &zp, &e);
+    float err = chunk_error<DT, FMT, !SYM>(xv, s, zp, f, p.norm);
+    for (int o = L >> 1; o > 0; o >>= 1) err += __shfl_xor(err, o, 64);
+    err = round_to<DT>(err);
+    if (err < best) {
+      best = err;
+#pragma unroll
+      for (int wd = 0; wd < MASK_WORDS; ++wd)
+        if (wd == (i >> 6)) mask[wd] |= 1ull << (i & 63);
+    }
+  }
+  if (!live) {
+#pragma unroll
+    for (int wd = 0; wd < MASK_WORDS; ++wd) mask[wd] = 0ull;
+  }
+  if (live && sub == 0) {
+    store_from_f32<DT>(p.min0, grp, mn);
+    store_from_f32<DT>(p.max0, grp, mx);
+#pragma unroll
+    for (int wd = 0; wd < MASK_WORDS; ++wd) p.masks[grp * MASK_WORDS + wd] = mask[wd];
+  }
+  or_flags(p.flags, mask);
+}
+
+template <int DT>
+void launch_team_fast(const MseParams& p, int64_t n, int ng, int g, int lshift, int64_t ldw, hipStream_t st) {
+  const int64_t threads = n << lshift;
+  const dim3 grid((unsigned)((threads + 255) / 256)), block(256);
+#define LLMC_MSE(F, S) hipLaunchKernelGGL((mse_team_fast_kernel<DT, F, S>), grid, block, 0, st, p, n, ng, g, lshift, ldw)
+  if (p.fmt == LLMC_FMT_INT) {
+    if (p.symmetric) LLMC_MSE(LLMC_FMT_INT, true);
+    else LLMC_MSE(LLMC_FMT_INT, false);
+  } else if (p.fmt == LLMC_FMT_FP8) {
+    if (p.symmetric) LLMC_MSE(LLMC_FMT_FP8, true);
+    else LLMC_MSE(LLMC_FMT_FP8, false);
+  } else {
+    LLMC_MSE(LLMC_FMT_FP4, true);
+  }
+#undef LLMC_MSE
+}
+
 struct GenericLayout {
   int mode;  // 0: (n0, n1, G) view with element strides (s0, s1, 1); 1: bh x bw blocks of an [R,K] matrix
   int64_t n0, G, s0, s1;
@@ -354,7 +534,14 @@ extern "C" int llmc_mse_observe_groups(const void* x, int32_t dtype, int64_t R, 
   const int64_t L = group / 8;
   const bool team = dtype != LLMC_F32 && group % 8 == 0 && L <= 64 && (L & (L - 1)) == 0 && ldw % 8 == 0 &&
                     (((uintptr_t)x) & 15) == 0;
-  if (team) {
+  if (team && (fmt != LLMC_FMT_FP4 || symmetric)) {
+    int lshift = 0;
+    while ((1 << lshift) < L) ++lshift;
+    if (dtype == LLMC_BF16)
+      launch_team_fast<LLMC_BF16>(p, n, (int)(K / group), (int)group, lshift, ldw, st);
+    else
+      launch_team_fast<LLMC_F16>(p, n, (int)(K / group), (int)group, lshift, ldw, st);
+  } else if (team) {
     const int64_t threads = n * L;
     hipLaunchKernelGGL(mse_team_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, p, n,
                        (int)(K / group), (int)group, (int)L, ldw);

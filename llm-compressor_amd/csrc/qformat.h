@@ -105,6 +105,29 @@ __device__ __forceinline__ f32x2_t hw_e2m1_pair_decode(uint32_t byte) {
   return __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(byte, 1.0f, 0);
 }
 
+// two fp32 values rounded (nearest even) to the 16-bit type DT, packed lo | hi << 16; bf16 goes
+// through the packed conversion instruction
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+template <int DT>
+__device__ __forceinline__ uint32_t pack16(float lo, float hi) {
+  const f32x2_t v = {lo, hi};
+  uint32_t w;
+  if (DT == LLMC_BF16) {
+    const bf16x2_t b = __builtin_convertvector(v, bf16x2_t);
+    __builtin_memcpy(&w, &b, 4);
+  } else {
+    const f16x2_t h = __builtin_convertvector(v, f16x2_t);
+    __builtin_memcpy(&w, &h, 4);
+  }
+  return w;
+}
+template <int DT>
+__device__ __forceinline__ float round16_finite(float f) {
+  if (DT == LLMC_BF16) return (float)(__bf16)f;
+  return (float)(_Float16)f;
+}
+
 // ---- division by a value shared by many elements.  The steps are those of the correctly
 // rounded fp32 division sequence (reciprocal with one Newton step, quotient with two residual
 // corrections) with the divisor's part hoisted; they give the IEEE quotient whenever nothing

@@ -193,29 +193,6 @@ __device__ __forceinline__ void unpack8(const uint4& v, float* x) {
   }
 }
 
-// two fp32 values rounded (nearest even) to the 16-bit type DT, packed lo | hi << 16; bf16 goes
-// through the packed conversion instruction
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
-template <int DT>
-__device__ __forceinline__ uint32_t pack16(float lo, float hi) {
-  const f32x2_t v = {lo, hi};
-  uint32_t w;
-  if (DT == LLMC_BF16) {
-    const bf16x2_t b = __builtin_convertvector(v, bf16x2_t);
-    __builtin_memcpy(&w, &b, 4);
-  } else {
-    const f16x2_t h = __builtin_convertvector(v, f16x2_t);
-    __builtin_memcpy(&w, &h, 4);
-  }
-  return w;
-}
-template <int DT>
-__device__ __forceinline__ float round16_finite(float f) {
-  if (DT == LLMC_BF16) return (float)(__bf16)f;
-  return (float)(_Float16)f;
-}
-
 // SM: 0 = scales in the input's 16-bit dtype, 1 = fp32 scales, 2 = stored scale / global scale (fp32)
 // A lane handles 16 consecutive columns (two 16-byte loads), which share one scale.
 template <int XDT, int SM, int FMT, bool HAS_ZP, int OUT>
