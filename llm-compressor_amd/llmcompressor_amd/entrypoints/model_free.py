@@ -1,0 +1,382 @@
+"""Data-free PTQ straight from safetensors shards, without a model definition
+(reference: entrypoints/model_free/__init__.py:45-150, process.py:89-241, lifecycle.py:23-62,
+validate.py:22-78, microscale.py:31-89, save_utils.py:24-121).
+
+Every shard is streamed through the GPU: each quantizable ``*.weight`` tensor becomes a bare
+``nn.Linear`` carrying its scheme, the weight observer and ``calculate_qparams`` run on the device,
+``compress_module`` packs it, and the compressed tensors go back to host memory for the output shard.
+Nothing but observer + pack kernels touches the weights, which makes this the bandwidth-bound caller
+of the hot path.  Microscale (tensor-group) schemes fuse the global scale over q/k/v, gate/up, w1/w3
+and wq_a/wkv_a sets; a partner that lives in another shard is read from there and written with its
+primary, as the reference does.  Only local directories are supported (there is no hub access).
+"""
+from __future__ import annotations
+
+import json
+import os
+import re
+import shutil
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+from typing import Dict, Iterable, Iterator, List, Optional, Tuple
+
+import torch
+from safetensors import safe_open
+from safetensors.torch import save_file
+
+from llmcompressor_amd.compressors import compress_module, infer_format
+from llmcompressor_amd.modifiers.quantization.calibration import (
+    apply_calibration_status,
+    freeze_module_quantization,
+    initialize_observer,
+    observe,
+    update_qparams,
+)
+from llmcompressor_amd.observers import FusionHandler
+from llmcompressor_amd.observers.helpers import flatten_for_calibration
+from llmcompressor_amd.quantization import (
+    QuantizationConfig,
+    QuantizationScheme,
+    QuantizationStatus,
+    QuantizationStrategy,
+    preset_name_to_scheme,
+)
+from llmcompressor_amd.quantization.lifecycle import getattr_chain, initialize_module_for_quantization
+from llmcompressor_amd.utils.metric_logging import logger
+
+__all__ = ["model_free_ptq"]
+
+_INDEX_NAME = "model.safetensors.index.json"
+
+# primary weight -> partner weights sharing one global scale (reference: microscale.py:31-52)
+_FUSED_MAPPINGS: Dict[str, List[str]] = {
+    r"^(?P<prefix>.+?)\.(?P<attn>attn|attention|self_attn|self_attention)\.q_proj\.weight$": [
+        "{prefix}.{attn}.k_proj.weight", "{prefix}.{attn}.v_proj.weight"],
+    r"^(?P<prefix>.+?)\.(?P<attn>attn|attention|self_attn)\.wq_a\.weight$": ["{prefix}.{attn}.wkv_a_with_mqa.weight"],
+    r"^(?P<prefix>.+?)\.(?P<mlp>mlp|feed_forward)\.gate_proj\.weight$": ["{prefix}.{mlp}.up_proj.weight"],
+    r"^(?P<prefix>.+?)\.w1\.weight$": ["{prefix}.w3.weight"],
+}
+
+
+# ---------------------------------------------------------------- config
+def _validate_scheme(scheme: QuantizationScheme):
+    if scheme.weights is None:
+        raise ValueError("Must provide a weights quantization scheme to perform weights-only PTQ")
+    input_dynamic = getattr_chain(scheme, "input_activations.dynamic", True)
+    output_dynamic = getattr_chain(scheme, "output_activations.dynamic", True)
+    if input_dynamic is not True or output_dynamic is not True:
+        raise ValueError("Model Free PTQ cannot calibrate activations. Please use `oneshot` instead.")
+    if scheme.weights.observer in ("minmax", "mse"):
+        new_observer = f"static_{scheme.weights.observer}"
+        logger.warning(f"Scheme uses {scheme.weights.observer} weight observer. Using {new_observer} instead")
+        scheme.weights.observer = new_observer
+    if len(scheme.targets) == 0:
+        scheme.targets.append("Linear")
+
+
+def validate_config(config: Optional[QuantizationConfig], scheme, ignore: Iterable[str]) -> QuantizationConfig:
+    if config is not None and scheme is not None:
+        raise ValueError("Please specify either `config` or `scheme`, not both")
+    if config is None and scheme is None:
+        raise ValueError("Please specify either `config` or `scheme`")
+    if scheme is not None:
+        if isinstance(scheme, str):
+            scheme_name, scheme = scheme, preset_name_to_scheme(scheme, [])
+        else:
+            scheme_name = "config_group_0"
+        config = QuantizationConfig(config_groups={scheme_name: scheme},
+                                    quantization_status=QuantizationStatus.INITIALIZED, ignore=list(ignore))
+    elif ignore:
+        config = config.model_copy(update={"ignore": list(config.ignore or []) + list(ignore)})
+    for s in config.config_groups.values():
+        _validate_scheme(s)
+    return config
+
+
+def is_microscale_scheme(scheme: QuantizationScheme) -> bool:
+    return scheme.weights.strategy == QuantizationStrategy.TENSOR_GROUP
+
+
+# ---------------------------------------------------------------- tensor matching
+def _name_matches(module_name: str, pattern: str) -> bool:
+    if pattern.startswith("re:"):
+        return re.match(pattern[3:], module_name) is not None
+    return module_name == pattern or pattern == "Linear"
+
+
+def _is_ignored(module_name: str, ignore: Iterable[str]) -> bool:
+    if module_name.endswith("norm"):
+        return True  # "modules ending with norm are automatically ignored"
+    for pat in ignore:
+        if pat.startswith("re:"):
+            if re.match(pat[3:], module_name):
+                return True
+        elif module_name == pat or module_name.endswith("." + pat):
+            return True
+    return False
+
+
+def _match_tensors_to_schemes(names: Iterable[str], config: QuantizationConfig
+                              ) -> Iterator[Tuple[str, str, QuantizationScheme]]:
+    """(module name, tensor name, scheme) for every quantizable tensor; the first matching group wins."""
+    matched = set()
+    ignore = list(config.ignore or [])
+    for scheme in config.config_groups.values():
+        for name in names:
+            if name in matched or not name.endswith(".weight"):
+                continue
+            module_name = name[: -len(".weight")]
+            if _is_ignored(module_name, ignore):
+                continue
+            if any(_name_matches(module_name, t) for t in scheme.targets):
+                matched.add(name)
+                yield module_name, name, scheme
+
+
+def validate_weight_for_quantization(shape: Tuple[int, ...], dtype: torch.dtype, scheme: QuantizationScheme,
+                                     tensor_name: str):
+    if len(shape) != 2:
+        raise ValueError(f"Unable to quantize tensor `{tensor_name}`: expected 2D linear weight, "
+                         f"but got shape {tuple(shape)}")
+    try:
+        flatten_for_calibration(torch.empty(shape, dtype=dtype, device="meta"), "weight", scheme.weights)
+    except Exception as exc:  # noqa: BLE001 - rethrown with the tensor's name, as the reference does
+        raise ValueError(f"Unable to quantize tensor `{tensor_name}`: {exc}") from exc
+
+
+# ---------------------------------------------------------------- per-tensor lifecycle
+def initialize_quantized_linear(weight: torch.Tensor, scheme: QuantizationScheme, device) -> torch.nn.Module:
+    out_features, in_features = weight.shape
+    module = torch.nn.Linear(in_features, out_features, bias=False, device=device, dtype=weight.dtype)
+    module.weight.data.copy_(weight)
+    initialize_module_for_quantization(module, scheme, force_zero_point=False)
+    return module
+
+
+def calibrate_weight(module: torch.nn.Module):
+    initialize_observer(module, "weight")
+    apply_calibration_status(module)
+    observe(module, base_name="weight")
+    update_qparams(module, base_name="weight")
+    freeze_module_quantization(module)
+
+
+def split_fused_moe_experts(tensors: Dict[str, torch.Tensor]) -> Dict[str, torch.Tensor]:
+    """3-D ``experts.gate_up_proj`` / ``experts.down_proj`` tensors become per-expert 2-D weights
+    (reference: process.py:244-330)."""
+    out: Dict[str, torch.Tensor] = {}
+    for name, t in tensors.items():
+        if t.ndim == 3 and name.endswith("experts.gate_up_proj"):
+            prefix = name[: -len("gate_up_proj")]
+            inter = t.shape[1] // 2
+            for e in range(t.shape[0]):
+                out[f"{prefix}{e}.gate_proj.weight"] = t[e, :inter].contiguous()
+                out[f"{prefix}{e}.up_proj.weight"] = t[e, inter:].contiguous()
+        elif t.ndim == 3 and name.endswith("experts.down_proj"):
+            prefix = name[: -len("down_proj")]
+            for e in range(t.shape[0]):
+                out[f"{prefix}{e}.down_proj.weight"] = t[e].contiguous()
+        else:
+            out[name] = t
+    return out
+
+
+def _store_compressed(tensors: Dict[str, torch.Tensor], name: str, module_name: str, module: torch.nn.Module):
+    del tensors[name]
+    for key, value in compress_module(module).items():
+        tensors[f"{module_name}.{key}"] = value.to("cpu")
+
+
+def process_file(inverse_weight_map: Dict[str, Optional[List[str]]], save_path: str, config: QuantizationConfig,
+                 device) -> Tuple[int, Dict[str, str]]:
+    """Quantize and compress the tensors of one output shard.  ``inverse_weight_map`` maps a source
+    file to the tensor names to read from it (None = all)."""
+    tensors: Dict[str, torch.Tensor] = {}
+    for path, wanted in inverse_weight_map.items():
+        with safe_open(path, framework="pt", device="cpu") as f:
+            for key in (f.keys() if wanted is None else wanted):
+                tensors[key] = f.get_tensor(key)
+    tensors = split_fused_moe_experts(tensors)
+
+    fused_index: Dict[str, int] = {}
+    nfused = 0
+    for primary_pat, partner_templates in _FUSED_MAPPINGS.items():
+        for name in tensors:
+            m = re.match(primary_pat, name)
+            if m is None:
+                continue
+            members = [name] + [t.format(**m.groupdict()) for t in partner_templates]
+            members = [n for n in members if n in tensors]
+            for n in members:
+                fused_index[n] = nfused
+            nfused += 1
+    fused_modules: Dict[int, Dict[str, Tuple[str, torch.nn.Module]]] = {}
+
+    for module_name, name, scheme in list(_match_tensors_to_schemes(list(tensors), config)):
+        w = tensors[name]
+        validate_weight_for_quantization(tuple(w.shape), w.dtype, scheme, name)
+        module = initialize_quantized_linear(w.to(device), scheme, device)
+        if is_microscale_scheme(scheme) and name in fused_index:
+            initialize_observer(module, "weight")
+            apply_calibration_status(module)
+            fused_modules.setdefault(fused_index[name], {})[name] = (module_name, module)
+            continue
+        calibrate_weight(module)
+        _store_compressed(tensors, name, module_name, module)
+
+    for named in fused_modules.values():
+        mods = [m for _, m in named.values()]
+        FusionHandler.fuse([(m.weight_observer, m) for m in mods])
+        observe(mods, base_name="weight")
+        update_qparams(mods, base_name="weight")
+        for name, (module_name, module) in named.items():
+            freeze_module_quantization(module)
+            _store_compressed(tensors, name, module_name, module)
+
+    tensors = {k: v.contiguous() for k, v in tensors.items()}
+    save_file(tensors, save_path)
+    total_size = sum(t.numel() * t.element_size() for t in tensors.values())
+    return total_size, {key: os.path.basename(save_path) for key in tensors}
+
+
+# ---------------------------------------------------------------- driver
+def _checkpoint_files(model_stub) -> Dict[str, str]:
+    root = Path(model_stub)
+    if not root.is_dir():
+        raise ValueError(f"model_free_ptq needs a local directory with safetensors files, got {model_stub!r} "
+                         "(there is no hub access)")
+    return {str(p.relative_to(root)): str(p) for p in sorted(root.rglob("*")) if p.is_file()}
+
+
+def _build_jobs(model_files: Dict[str, str], save_directory: str, config: QuantizationConfig):
+    shards = {rel: path for rel, path in model_files.items() if rel.endswith(".safetensors")}
+    location: Dict[str, str] = {}
+    for rel, path in shards.items():
+        with safe_open(path, framework="pt", device="cpu") as f:
+            for key in f.keys():
+                location[key] = rel
+    micro = any(is_microscale_scheme(s) for s in config.config_groups.values())
+    moved: Dict[str, str] = {}  # partner tensor -> shard of its primary
+    if micro:
+        for primary_pat, partner_templates in _FUSED_MAPPINGS.items():
+            for name, rel in location.items():
+                m = re.match(primary_pat, name)
+                if m is None:
+                    continue
+                for t in partner_templates:
+                    partner = t.format(**m.groupdict())
+                    if partner in location and location[partner] != rel:
+                        moved[partner] = rel
+    jobs = []
+    for rel, path in shards.items():
+        own = [k for k, r in location.items() if r == rel and k not in moved]
+        iwm: Dict[str, Optional[List[str]]] = {path: own if moved else None}
+        for partner, dst in moved.items():
+            if dst == rel:
+                iwm.setdefault(shards[location[partner]], [])
+                if iwm[shards[location[partner]]] is not None:
+                    iwm[shards[location[partner]]].append(partner)
+        jobs.append((iwm, os.path.join(save_directory, rel)))
+    return jobs, location
+
+
+def update_config(save_directory: str, config: QuantizationConfig):
+    """Write ``quantization_config`` into ``config.json`` (reference: save_utils.py:24-121)."""
+    groups, formats = {}, set()
+    for gname, scheme in config.config_groups.items():
+        fmt = infer_format(scheme)
+        formats.add(fmt)
+        d = scheme.model_dump(mode="json")
+        d["format"] = fmt
+        groups[gname] = d
+    fmt = formats.pop() if len(formats) == 1 else ("mixed-precision" if formats else "dense")
+    qconfig = {
+        "version": config.version,
+        "quant_method": "compressed-tensors",
+        "transform_config": {},
+        "config_groups": groups,
+        "kv_cache_scheme": None if config.kv_cache_scheme is None else config.kv_cache_scheme.model_dump(mode="json"),
+        "ignore": list(config.ignore or []),
+        "quantization_status": QuantizationStatus.COMPRESSED.value,
+        "format": fmt,
+        "global_compression_ratio": None,
+    }
+    path = os.path.join(save_directory, "config.json")
+    if os.path.exists(path):
+        with open(path) as f:
+            data = json.load(f)
+        data["quantization_config"] = qconfig
+        with open(path, "w") as f:
+            json.dump(data, f, indent=2, sort_keys=True)
+    else:
+        logger.warning(f"Could not find config file in {save_directory}. Please set quantization_config to: \n"
+                       f"{json.dumps(qconfig, indent=2, sort_keys=True)}")
+    return qconfig
+
+
+def model_free_ptq(model_stub, save_directory, scheme=None, config: Optional[QuantizationConfig] = None,
+                   ignore: Iterable[str] = tuple(), max_workers: int = 1, device=None, converter=None):
+    """Quantize a checkpoint of safetensors files without a model definition.
+
+    :param model_stub: path to a local directory with the weights files
+    :param save_directory: directory to save quantized weights to
+    :param scheme: weight quantization scheme or preset scheme name (mutually exclusive with config)
+    :param config: quantization config with one or more schemes (mutually exclusive with scheme)
+    :param ignore: modules to ignore; modules ending with "norm" are ignored automatically
+    :param max_workers: worker threads; shards are independent jobs on the one device
+    :param device: device for quantization (default cuda:0)
+    :param converter: not supported
+    """
+    if converter is not None:
+        raise NotImplementedError("checkpoint converters are not part of this build")
+    model_files = _checkpoint_files(model_stub)
+    config = validate_config(config, scheme, ignore)
+    device = torch.device(device if device is not None else "cuda:0")
+    if isinstance(device, (list, tuple)):
+        device = torch.device(device[0])
+    os.makedirs(save_directory, exist_ok=True)
+
+    for rel, path in model_files.items():
+        if not rel.endswith("safetensors") and rel != _INDEX_NAME:
+            dst = Path(save_directory) / rel
+            dst.parent.mkdir(parents=True, exist_ok=True)
+            shutil.copyfile(path, dst)
+
+    jobs, location = _build_jobs(model_files, save_directory, config)
+
+    # validate first (shapes only, nothing is loaded)
+    for rel, path in model_files.items():
+        if rel.endswith(".safetensors"):
+            with safe_open(path, framework="pt", device="cpu") as f:
+                keys = list(f.keys())
+                for _, name, sch in _match_tensors_to_schemes(keys, config):
+                    sl = f.get_slice(name)
+                    shape = tuple(sl.get_shape())
+                    if len(shape) == 2:
+                        dtype = getattr(torch, {"BF16": "bfloat16", "F16": "float16", "F32": "float32"}.get(
+                            sl.get_dtype(), "float32"))
+                        validate_weight_for_quantization(shape, dtype, sch, name)
+                    else:
+                        validate_weight_for_quantization(shape, torch.float32, sch, name)
+
+    total_size, weight_map = 0, {}
+
+    def run(job):
+        iwm, save_path = job
+        Path(save_path).parent.mkdir(parents=True, exist_ok=True)
+        return process_file(iwm, save_path, config, device)
+
+    if max_workers > 1:
+        with ThreadPoolExecutor(max_workers=max_workers) as pool:
+            results = list(pool.map(run, jobs))
+    else:
+        results = [run(j) for j in jobs]
+    for size, wm in results:
+        total_size += size
+        weight_map.update(wm)
+
+    update_config(save_directory, config)
+    if len(jobs) > 1 or _INDEX_NAME in model_files:
+        with open(os.path.join(save_directory, _INDEX_NAME), "w") as f:
+            json.dump({"metadata": {"total_size": total_size}, "weight_map": weight_map}, f, indent=2, sort_keys=True)
+    return total_size, weight_map

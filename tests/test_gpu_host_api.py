@@ -389,3 +389,139 @@ def test_moe_gptq_zero_token_expert_is_zeroed():
     assert torch.count_nonzero(experts[3].gate_proj.weight) == 0
     assert torch.count_nonzero(experts[3].down_proj.weight) == 0
     assert torch.count_nonzero(experts[0].gate_proj.weight) > 0
+
+
+def _write_checkpoint(root, seed=0):
+    """A two-shard toy checkpoint: q/k/v of layer 0 split across the shards, one fused-experts tensor."""
+    import json
+    import os
+
+    from safetensors.torch import save_file
+
+    g = torch.Generator().manual_seed(seed)
+
+    def w(r, c):
+        return (torch.randn(r, c, generator=g) * 0.05).bfloat16()
+
+    s0 = {
+        "model.embed_tokens.weight": w(50, 64),
+        "model.layers.0.self_attn.q_proj.weight": w(64, 64),
+        "model.layers.0.self_attn.o_proj.weight": w(64, 64),
+        "model.layers.0.input_layernorm.weight": torch.ones(64, dtype=torch.bfloat16),
+        "model.layers.0.mlp.gate_proj.weight": w(128, 64),
+        "model.layers.0.mlp.up_proj.weight": w(128, 64),
+    }
+    s1 = {
+        "model.layers.0.self_attn.k_proj.weight": w(32, 64),
+        "model.layers.0.self_attn.v_proj.weight": w(32, 64),
+        "model.layers.0.mlp.down_proj.weight": w(64, 128),
+        "model.layers.1.mlp.experts.gate_up_proj": (torch.randn(2, 64, 32, generator=g) * 0.05).bfloat16(),
+        "model.layers.1.mlp.experts.down_proj": (torch.randn(2, 32, 32, generator=g) * 0.05).bfloat16(),
+        "model.norm.weight": torch.ones(64, dtype=torch.bfloat16),
+        "lm_head.weight": w(50, 64),
+    }
+    os.makedirs(root, exist_ok=True)
+    save_file(s0, os.path.join(root, "model-00001-of-00002.safetensors"))
+    save_file(s1, os.path.join(root, "model-00002-of-00002.safetensors"))
+    wm = {k: "model-00001-of-00002.safetensors" for k in s0}
+    wm.update({k: "model-00002-of-00002.safetensors" for k in s1})
+    with open(os.path.join(root, "model.safetensors.index.json"), "w") as f:
+        json.dump({"metadata": {}, "weight_map": wm}, f)
+    with open(os.path.join(root, "config.json"), "w") as f:
+        json.dump({"model_type": "toy"}, f)
+    with open(os.path.join(root, "tokenizer.json"), "w") as f:
+        f.write("{}")
+    return {**s0, **s1}
+
+
+@pytest.mark.parametrize("scheme", ["FP8_DYNAMIC", "INT4_G32", "NVFP4A16"])
+def test_model_free_ptq_round_trip(tmp_path, scheme):
+    """Shard-streaming PTQ: every Linear weight of the toy checkpoint comes back packed, bit-identical to the
+    oracle's observer + quantise + pack on the same tensor; ignored and norm tensors are copied; fused sets share
+    one global scale even when split across shards."""
+    import json
+
+    from safetensors import safe_open
+
+    from llmcompressor_amd import model_free_ptq
+    from oracle import observers as OO
+    from oracle import pack as OP
+    from oracle import qformat as OF
+
+    src, dst = str(tmp_path / "src"), str(tmp_path / "dst")
+    orig = _write_checkpoint(src)
+    ignore = ["model.embed_tokens", "lm_head"]
+    if scheme == "INT4_G32":
+        from llmcompressor_amd.quantization import QuantizationArgs, QuantizationScheme
+
+        sch = QuantizationScheme(targets=["Linear"], weights=QuantizationArgs(num_bits=4, strategy="group", group_size=32))
+        total, wmap = model_free_ptq(src, dst, scheme=sch, ignore=ignore, device="cuda:0")
+    else:
+        total, wmap = model_free_ptq(src, dst, scheme=scheme, ignore=ignore, device="cuda:0")
+    out = {}
+    for fn in sorted(set(wmap.values())):
+        with safe_open(f"{dst}/{fn}", framework="pt") as f:
+            for k in f.keys():
+                assert k not in out, f"{k} written twice"
+                out[k] = f.get_tensor(k)
+    assert set(wmap) == set(out) and total == sum(t.numel() * t.element_size() for t in out.values())
+    cfg = json.load(open(f"{dst}/config.json"))
+    q = cfg["quantization_config"]
+    assert q["quant_method"] == "compressed-tensors" and q["quantization_status"] == "compressed"
+    assert q["ignore"] == ignore and cfg["model_type"] == "toy"
+    assert (tmp_path / "dst" / "tokenizer.json").exists()
+    for k in ("model.embed_tokens.weight", "lm_head.weight", "model.norm.weight", "model.layers.0.input_layernorm.weight"):
+        assert torch.equal(out[k], orig[k])
+    # fused experts were split into per-expert Linears
+    assert "model.layers.1.mlp.experts.gate_up_proj" not in out
+    assert any(k.startswith("model.layers.1.mlp.experts.1.up_proj.") for k in out)
+
+    def oracle_args():
+        if scheme == "FP8_DYNAMIC":
+            return OF.QArgs(num_bits=8, type="float", strategy="channel"), "float-quantized"
+        if scheme == "INT4_G32":
+            return OF.QArgs(num_bits=4, strategy="group", group_size=32), "pack-quantized"
+        return OF.QArgs(num_bits=4, type="float", strategy="tensor_group", group_size=16,
+                        scale_dtype=torch.float8_e4m3fn), "nvfp4-pack-quantized"
+
+    args, fmt = oracle_args()
+    assert q["format"] == fmt
+    name = "model.layers.0.self_attn.o_proj"
+    w = orig[name + ".weight"]
+    obs = OO.Observer("memoryless_minmax", "weight", args)
+    obs(w)
+    qp = obs.get_qparams()
+    if scheme == "FP8_DYNAMIC":
+        codes = OF.quantize(w, qp["scale"], qp["zero_point"], args, dtype=torch.float8_e4m3fn)
+        assert torch.equal(out[name + ".weight"].view(torch.uint8), codes.view(torch.uint8))
+        assert torch.equal(out[name + ".weight_scale"], qp["scale"])
+    elif scheme == "INT4_G32":
+        codes = OF.quantize(w, qp["scale"], qp["zero_point"], args, dtype=torch.int8)
+        assert torch.equal(out[name + ".weight_packed"], OP.pack_to_int32(codes, 4))
+        assert torch.equal(out[name + ".weight_scale"], qp["scale"])
+        assert out[name + ".weight_shape"].tolist() == [64, 64]
+    elif scheme == "NVFP4A16":
+        # q/k/v share the global scale of the set's largest |w|, although k and v live in the other shard
+        names = [f"model.layers.0.self_attn.{p}_proj" for p in "qkv"]
+        amax = max(orig[n + ".weight"].abs().max() for n in names)
+        gs = OF.generate_gparam(-amax.reshape(1), amax.reshape(1))
+        for n in names:
+            assert torch.equal(out[n + ".weight_global_scale"].reshape(1).float(), gs.reshape(1).float()), n
+            assert wmap[n + ".weight_packed"] == "model-00001-of-00002.safetensors"  # written with the primary
+            wq = orig[n + ".weight"]
+            o2 = OO.Observer("memoryless_minmax", "weight", args)
+            o2(wq)
+            mn, mx = o2.min_vals, o2.max_vals
+            s, z = OF.calculate_qparams(mn, mx, args, global_scale=gs)
+            q4 = OF.quantize(wq, s, z, args, global_scale=gs)
+            assert torch.equal(out[n + ".weight_packed"], OP.pack_fp4_to_uint8(q4)), n
+
+
+def test_model_free_ptq_rejects_indivisible_groups(tmp_path):
+    from llmcompressor_amd import model_free_ptq
+
+    src = str(tmp_path / "src")
+    _write_checkpoint(src)
+    with pytest.raises(ValueError, match="Unable to quantize tensor"):
+        model_free_ptq(src, str(tmp_path / "dst"), scheme="W4A16", ignore=["model.embed_tokens", "lm_head"],
+                       device="cuda:0")

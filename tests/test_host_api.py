@@ -279,3 +279,32 @@ def test_moe_token_routing_counts():
     counts.clear()
     experts(x, torch.zeros(T, k, dtype=torch.long), wts)
     assert counts == {0: 32, 1: 0, 2: 0, 3: 0}  # both top-k slots of every token point at expert 0
+
+
+def test_model_free_config_and_matching():
+    """model_free_ptq host logic: scheme/config validation, ignore rules, first-match-wins targets
+    (reference: entrypoints/model_free/validate.py:22-78, process.py:44-60)."""
+    from llmcompressor_amd.entrypoints.model_free import _match_tensors_to_schemes, validate_config
+    from llmcompressor_amd.quantization import QuantizationArgs, QuantizationConfig, QuantizationScheme
+
+    with pytest.raises(ValueError, match="either `config` or `scheme`"):
+        validate_config(None, None, [])
+    with pytest.raises(ValueError, match="not both"):
+        validate_config(QuantizationConfig(config_groups={}), "FP8_DYNAMIC", [])
+    static_act = QuantizationScheme(targets=["Linear"], weights=QuantizationArgs(num_bits=8),
+                                    input_activations=QuantizationArgs(num_bits=8, dynamic=False))
+    with pytest.raises(ValueError, match="cannot calibrate activations"):
+        validate_config(None, static_act, [])
+    cfg = validate_config(None, "FP8_DYNAMIC", ["lm_head", "re:.*embed.*"])
+    assert list(cfg.config_groups) == ["FP8_DYNAMIC"] and cfg.ignore == ["lm_head", "re:.*embed.*"]
+    names = ["model.embed_tokens.weight", "model.layers.0.self_attn.q_proj.weight", "model.layers.0.self_attn.q_proj.bias",
+             "model.layers.0.post_attention_layernorm.weight", "model.norm.weight", "lm_head.weight",
+             "model.layers.0.mlp.down_proj.weight"]
+    got = [m for m, _, _ in _match_tensors_to_schemes(names, cfg)]
+    assert got == ["model.layers.0.self_attn.q_proj", "model.layers.0.mlp.down_proj"]
+    # two groups: the first that matches a tensor wins
+    a = QuantizationScheme(targets=["re:.*q_proj$"], weights=QuantizationArgs(num_bits=4, strategy="group", group_size=32))
+    b = QuantizationScheme(targets=["Linear"], weights=QuantizationArgs(num_bits=8, strategy="channel"))
+    cfg2 = validate_config(QuantizationConfig(config_groups={"a": a, "b": b}), None, ["lm_head", "model.embed_tokens"])
+    got2 = {m: s.weights.num_bits for m, _, s in _match_tensors_to_schemes(names, cfg2)}
+    assert got2 == {"model.layers.0.self_attn.q_proj": 4, "model.layers.0.mlp.down_proj": 8}
