@@ -97,6 +97,9 @@ def find_decoder_layers(model: torch.nn.Module, sequential_targets=None) -> List
     return list(best)
 
 
+from .cache import IntermediatesCache  # noqa: E402
+
+
 class _StopForward(Exception):
     pass
 
@@ -126,20 +129,24 @@ class SequentialPipeline(CalibrationPipeline):
                         pass
             finally:
                 handle.remove()
-            states = captured
+            # the activations between layers live in a device-resident cache (no CPU offload)
+            offload = getattr(dataset_args, "sequential_offload_device", None) if dataset_args is not None else None
+            cache = IntermediatesCache.empty(len(captured), offload_device=offload)
+            for i, (args, kwargs) in enumerate(captured):
+                cache.update(i, {"args": tuple(args), "kwargs": dict(kwargs)})
+            del captured
             for idx, layer in enumerate(layers):
                 # pass 1: calibrate (hooks fire: Hessians / activation observers)
-                for args, kwargs in states:
-                    layer(*args, **kwargs)
+                for inputs in cache.iter_prefetch():
+                    layer(*inputs["args"], **inputs["kwargs"])
                 LifecycleCallbacks.sequential_epoch_end(modules=list(layer.modules()))
                 # pass 2: propagate through the compressed layer without triggering hooks
-                nxt = []
                 with HooksMixin.disable_hooks():
-                    for args, kwargs in states:
-                        out = layer(*args, **kwargs)
+                    for i in range(len(cache)):
+                        inputs = cache.fetch(i)
+                        out = layer(*inputs["args"], **inputs["kwargs"])
                         hidden = out[0] if isinstance(out, (tuple, list)) else out
-                        nxt.append(((hidden,) + tuple(args[1:]), kwargs))
-                states = nxt
+                        cache.update(i, {"args": (hidden,) + tuple(inputs["args"][1:])})
             # modules outside the layer list (e.g. lm_head) that modifiers may target
             rest = [m for m in model.modules() if not any(m is x for l in layers for x in l.modules())]
             LifecycleCallbacks.sequential_epoch_end(modules=rest)
