@@ -41,8 +41,8 @@ LINEARS = [  # name, out_features, in_features
 GROUP = 128
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch of the dominant kernel from FETCH_SIZE / WRITE_SIZE counter runs scaled by a
-# 1 GiB copy (profiles/hessian_syrk_k14336_t16384_hbm_traffic.md), keyed by tokens per launch
-DOMINANT_TRAFFIC_BYTES = {16384: 7.30e9}
+# 1 GiB copy (profiles/hessian_syrk_k14336_t65536_hbm_traffic.md), keyed by tokens per launch
+DOMINANT_TRAFFIC_BYTES = {16384: 7.30e9, 65536: 29.6e9}
 
 
 def cpu_baseline(tokens: int):
@@ -155,7 +155,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=1)
     ap.add_argument("--batches", type=int, default=256, help="calibration batches per step (config: 256)")
     ap.add_argument("--tokens", type=int, default=2048, help="tokens per batch (config: 2048)")
-    ap.add_argument("--stage-tokens", type=int, default=16384,
+    ap.add_argument("--stage-tokens", type=int, default=65536,
                     help="tokens staged per Hessian launch (GPTQModifier.hessian_batch_tokens; 0 = one launch per batch)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--probe-dominant", type=int, default=0, metavar="N",
