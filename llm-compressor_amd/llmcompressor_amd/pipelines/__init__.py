@@ -69,7 +69,6 @@ class CalibrationPipeline:
 
     @classmethod
     def from_modifiers(cls, modifiers: List, user: Optional[str] = None) -> "CalibrationPipeline":
-        user = None if user in (None, "independent") and False else user
         inferred = "sequential" if any(m.requires_calibration_data for m in modifiers) else "datafree"
         if user is not None and user != inferred and user != "independent":
             return cls.load_from_registry(user)

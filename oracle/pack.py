@@ -66,8 +66,6 @@ def compress_weight(weight, scale, zero_point, args: QArgs, global_scale=None, g
     out = {}
     if args.type == "int":
         q = quantize(weight, scale, zero_point, args, dtype=torch.int8, g_idx=g_idx)
-        if args.num_bits == 8 and False:
-            out["weight"] = q
         out["weight_packed"] = pack_to_int32(q, args.num_bits)
         out["weight_shape"] = torch.tensor([R, K], dtype=torch.int64)
         out["weight_scale"] = scale

@@ -179,3 +179,61 @@ def test_gptq_zero_hessian_zeroes_weight_and_failure_is_rtn():
     wq, _ = ops.gptq_quantize(w.cuda(), U, scale.cuda(), None, ops.FMT_INT, 4, 1, K // g, g_idx=g_idx, dead=dead)
     rtn = F.fake_quantize(w.float(), scale, zp, args).to(torch.bfloat16)
     assert torch.equal(wq.cpu(), rtn)
+
+
+@pytest.mark.parametrize("R,K,T", [(1024, 4096, 8192), (512, 14336, 32768)])
+def test_gptq_full_size_properties(R, K, T):
+    """Llama-3-8B widths (the oracle would take minutes here): size-independent properties.
+    Every output value lies on its group's int4 grid; GPTQ's layer reconstruction error beats
+    round-to-nearest's; rescaling H leaves the codes unchanged; a narrower block width regroups the
+    same fp32 sums (>= 99.9 % identical); U^T U (H/n + damp I) = I on sampled columns."""
+    from llmcompressor_amd import ops
+
+    torch.manual_seed(K)
+    g = 128
+    w = (torch.randn(R, K, device="cuda") * 0.02).bfloat16()
+    x = torch.randn(T, K, device="cuda")
+    x[:, torch.randperm(K, device="cuda")[: K // 100]] *= 20
+    x = x.bfloat16()
+    H = torch.zeros(K, K, device="cuda")
+    ops.hessian_accumulate_(H, x)
+    mn, mx = ops.minmax_groups(w, g)
+    scale, _, _ = ops.calculate_qparams(mn, mx, ops.FMT_INT, 4, True)
+    perm = torch.argsort(torch.diag(H), descending=True)
+    g_idx = (torch.arange(K, dtype=torch.int32, device="cuda") // g)[perm]
+
+    def run(Hin, blocksize=128, divisor=float(T)):
+        U, dead, info = ops.gptq_hinv_(Hin.clone(), perm, divisor=divisor)
+        assert int(info.item()) == 0
+        wq, loss = ops.gptq_quantize(w, U, scale, None, ops.FMT_INT, 4, 1, K // g, g_idx=g_idx, perm=perm, dead=dead,
+                                     blocksize=blocksize)
+        return wq, loss, U
+
+    wq, loss, U = run(H)
+    # grid membership: q = wq / scale is an integer in [-8, 7] and q * scale reproduces wq in bf16
+    s_full = scale.repeat_interleave(g, dim=1)
+    q = (wq.float() / s_full.float()).round()
+    assert q.min() >= -8 and q.max() <= 7
+    assert torch.equal((q.to(torch.bfloat16) * s_full), wq)
+    # reconstruction error vs round-to-nearest with the same scales
+    rtn = ops.quantize(w, scale, None, ops.FMT_INT, 4, 1, K // g, g)
+    xs = x.float()
+    e_gptq = ((w.float() - wq.float()) @ xs.t()).norm().item()
+    e_rtn = ((w.float() - rtn.float()) @ xs.t()).norm().item()
+    assert e_gptq < 0.9 * e_rtn, (e_gptq, e_rtn)
+    assert float(loss) > 0
+    # codes are invariant to a positive rescaling of H (damping is relative)
+    wq_s, _, _ = run(H * 3.0)
+    assert (wq_s == wq).float().mean().item() >= CODE_AGREEMENT
+    # block width only regroups fp32 sums
+    wq_b, _, _ = run(H, blocksize=64)
+    assert (wq_b == wq).float().mean().item() >= CODE_AGREEMENT
+    # U^T U = (P^T H P / n + damp I)^-1 on sampled columns
+    Hp = (H[perm][:, perm] / T).double()
+    damp = 0.01 * torch.diag(Hp).mean()
+    Hp += damp * torch.eye(K, device="cuda", dtype=torch.float64)
+    cols = torch.tensor([0, 1, K // 2, K - 2, K - 1], device="cuda")
+    Ud = U.double()
+    got = Ud.t() @ (Ud @ Hp[:, cols])
+    want = torch.eye(K, device="cuda", dtype=torch.float64)[:, cols]
+    assert (got - want).abs().max().item() < 5e-3
