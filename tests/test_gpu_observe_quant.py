@@ -288,3 +288,49 @@ def test_full_size_properties():
     fq8 = ops.quantize(w, s8, None, ops.FMT_FP8, 8, 1, 1, 1 << 40)
     c8 = ops.quantize(w, s8, None, ops.FMT_FP8, 8, 1, 1, 1 << 40, out_mode=ops.OUT_PACKED)
     assert torch.equal((c8.to(torch.bfloat16) * s8), fq8)
+
+
+def test_full_size_microscale_and_mse_properties():
+    """Config-3 shapes (14336 x 4096): NVFP4 / MXFP4 packed bytes decode to the fake-quantised weight;
+    the MSE observer's ranges lie inside the min-max ranges and do not quantise worse than min-max."""
+    from llmcompressor_amd import ops
+
+    torch.manual_seed(1)
+    R, K = 14336, 4096
+    w = (torch.randn(R, K, device="cuda") * 0.02).bfloat16()
+    e2m1 = torch.tensor([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0], device="cuda")
+    grid = torch.cat([e2m1, -e2m1])
+
+    def decode(pk):
+        lo, hi = (pk & 0xF).long(), (pk >> 4).long()
+        return torch.stack([grid[lo], grid[hi]], dim=-1).reshape(R, K)
+
+    # NVFP4: group 16, e4m3 scales times a global scale
+    mn, mx = ops.minmax_groups(w, 16)
+    gs = ops.global_scale_from_stats([(mn, mx)])
+    s4, _, codes = ops.calculate_qparams(mn, mx, ops.FMT_FP4, 4, True, ops.SCALE_NVFP4, gs, want_codes=True)
+    assert torch.equal(codes.view(torch.float8_e4m3fn).float(), s4.float())  # stored scales are e4m3 values
+    fq = ops.quantize(w, s4, None, ops.FMT_FP4, 4, 1, K // 16, 16, global_scale=gs)
+    pk = ops.quantize(w, s4, None, ops.FMT_FP4, 4, 1, K // 16, 16, out_mode=ops.OUT_PACKED, global_scale=gs)
+    eff = (s4.float() / gs).repeat_interleave(16, dim=1)
+    assert torch.equal((decode(pk) * eff).to(torch.bfloat16), fq)
+    fq2 = ops.quantize(fq, s4, None, ops.FMT_FP4, 4, 1, K // 16, 16, global_scale=gs)
+    assert torch.equal(fq2, fq)  # idempotent
+    # MXFP4: group 32, power-of-two scales
+    mn, mx = ops.minmax_groups(w, 32)
+    sm, _, e8 = ops.calculate_qparams(mn, mx, ops.FMT_FP4, 4, True, ops.SCALE_MXFP4, want_codes=True)
+    assert torch.equal(torch.exp2(e8.float() - 127).to(torch.bfloat16), sm)
+    fqm = ops.quantize(w, sm, None, ops.FMT_FP4, 4, 1, K // 32, 32)
+    pkm = ops.quantize(w, sm, None, ops.FMT_FP4, 4, 1, K // 32, 32, out_mode=ops.OUT_PACKED)
+    assert torch.equal((decode(pkm) * sm.float().repeat_interleave(32, dim=1)).to(torch.bfloat16), fqm)
+    # MSE observer (default grid) vs min-max, int4 group 128
+    mn, mx = ops.minmax_groups(w, 128)
+    mmn, mmx = ops.mse_observe_groups(w, 128, ops.FMT_INT, 4, True, ops.SCALE_PLAIN)
+    assert bool((mmn >= mn).all()) and bool((mmx <= mx).all())
+
+    def qerr(a, b):
+        s, _, _ = ops.calculate_qparams(a, b, ops.FMT_INT, 4, True)
+        f = ops.quantize(w, s, None, ops.FMT_INT, 4, 1, K // 128, 128)
+        return (f.float() - w.float()).abs().pow(2.4).sum().item()
+
+    assert qerr(mmn, mmx) <= 1.0001 * qerr(mn, mx)
