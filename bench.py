@@ -12,9 +12,14 @@ Llama-3-8B-shaped decoder layer.  A step is
   quantize phase: per Linear  min-max observer -> scales -> diag argsort ->
                   damped Cholesky chain -> GPTQ column loop -> int4 packing
 
-All inputs are resident in HBM before the timed region.  `value` is the Hessian
-phase's algorithmic TFLOP/s (2*T*K^2 per launch); `quantize_weight_ms_per_linear`
-is the second half of the metric.  Prints ONE JSON line.
+All inputs are resident in HBM before the timed region: one activation stream per distinct
+Linear input of the layer (q/k/v share theirs, o_proj has its own, gate/up share theirs, down_proj
+has its own).  `value` is the Hessian phase's algorithmic TFLOP/s (2*T*K^2 per Linear per batch)
+with one Hessian accumulated per Linear, as the reference does; `quantize_weight_ms_per_linear` is
+the second half of the metric.  `shared_input_hessians` repeats the step with
+GPTQModifier(share_identical_inputs=True), where q/k/v and gate/up accumulate one Hessian per
+shared input (identical results, 3 of the 6 narrow products removed) -- same algorithmic FLOP
+count over the shorter time.  Prints ONE JSON line.
 """
 from __future__ import annotations
 
@@ -181,6 +186,8 @@ def main():
         probe_bandwidth()
         return
     if a.probe_dominant:
+        from llmcompressor_amd import ops
+
         x = torch.randn(a.stage_tokens or a.tokens, INTER, device=dev).bfloat16()
         H = torch.zeros(INTER, INTER, device=dev)
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
@@ -207,11 +214,13 @@ def main():
         getattr(layer, name).weight.data.copy_(w)
         originals[name] = w
     # calibration activations, resident in HBM: one stream per distinct Linear input
-    x_hidden = torch.empty(B, T, HIDDEN, dtype=torch.bfloat16, device=dev)
-    x_inter = torch.empty(B, T, INTER, dtype=torch.bfloat16, device=dev)
+    streams = {"attn_in": HIDDEN, "attn_out": HIDDEN, "mlp_in": HIDDEN, "mlp_mid": INTER}
+    xs = {k: torch.empty(B, T, w, dtype=torch.bfloat16, device=dev) for k, w in streams.items()}
     for b in range(B):
-        x_hidden[b] = torch.randn(T, HIDDEN, device=dev, generator=gen).bfloat16()
-        x_inter[b] = torch.randn(T, INTER, device=dev, generator=gen).bfloat16()
+        for k, w in streams.items():
+            xs[k][b] = torch.randn(T, w, device=dev, generator=gen).bfloat16()
+    input_of = {"q_proj": "attn_in", "k_proj": "attn_in", "v_proj": "attn_in", "o_proj": "attn_out",
+                "gate_proj": "mlp_in", "up_proj": "mlp_in", "down_proj": "mlp_mid"}
 
     # time every launch of the dominant kernel (the 14336-wide Hessian) with events on the launch stream
     dom_events = []
@@ -232,12 +241,13 @@ def main():
 
     ops.hessian_accumulate_ = timed_accumulate
 
-    def step(record: bool):
+    def step(record: bool, share: bool = False):
         for name, r, k in LINEARS:
             getattr(layer, name).weight.data.copy_(originals[name])
         recording[0] = record
         modifier = GPTQModifier(targets="Linear", scheme="W4A16", actorder="static", block_size=128,
-                                dampening_frac=0.01, hessian_batch_tokens=a.stage_tokens)
+                                dampening_frac=0.01, hessian_batch_tokens=a.stage_tokens,
+                                share_identical_inputs=share)
         session = active_session()
         session.reset()
         session.initialize(model=layer, recipe=modifier)
@@ -245,11 +255,11 @@ def main():
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         # what the forward hooks do during the calibration pass of this layer
-        mods = [(getattr(layer, name), k == INTER) for name, _, k in LINEARS]
+        mods = [(getattr(layer, name), input_of[name]) for name, _, _ in LINEARS]
         for b in range(B):
-            args_h, args_i = (x_hidden[b:b + 1],), (x_inter[b:b + 1],)
-            for mod, wide in mods:
-                modifier.calibrate_module(mod, args_i if wide else args_h, None)
+            args_of = {k: (x[b:b + 1],) for k, x in xs.items()}
+            for mod, stream in mods:
+                modifier.calibrate_module(mod, args_of[stream], None)
         for m in list(modifier._staged):
             modifier._flush(m)
         torch.cuda.synchronize()
@@ -275,6 +285,14 @@ def main():
         tq += q
     torch.cuda.synchronize()
     wall = time.perf_counter() - wall0
+
+    # the same step with one Hessian per shared input (results identical, checked below)
+    sh_h = sh_q = 0.0
+    for _ in range(a.steps):
+        h, q, out_shared = step(False, share=True)
+        sh_h += h
+        sh_q += q
+    same = all(torch.equal(out[n][k], out_shared[n][k]) for n in out for k in out[n])
 
     flop_step = sum(2.0 * T * k * k for _, _, k in LINEARS) * B
     value = flop_step * a.steps / th / 1e12
@@ -305,6 +323,13 @@ def main():
         "quantize_weight_ms_per_linear": round(tq / a.steps / len(LINEARS) * 1e3, 3),
         "hessian_phase_ms_per_step": round(th / a.steps * 1e3, 2),
         "hessian_algorithmic_flop_per_step": flop_step,
+        "shared_input_hessians": {
+            "value": round(flop_step * a.steps / sh_h / 1e12, 2),
+            "unit": "TFLOP/s",
+            "hessian_phase_ms_per_step": round(sh_h / a.steps * 1e3, 2),
+            "quantize_weight_ms_per_linear": round(sh_q / a.steps / len(LINEARS) * 1e3, 3),
+            "packed_weights_identical": bool(same),
+        },
         "roofline": {
             "kernel": "hessian_syrk_kernel<256> (down_proj Hessian, %d tokens per launch, K=%d)" % (int(dom_T), INTER),
             "bound": "mfma",

@@ -51,6 +51,10 @@ class GPTQModifier(Modifier, QuantizationMixin):
     :param hessian_batch_tokens: stage activations and launch the Hessian kernel once this many tokens
         are pending (0 = one launch per hook call, the reference's behaviour)
 
+    :param share_identical_inputs: Linears that are fed the very same tensor on every call (q/k/v, gate/up)
+        have the same Hessian; accumulate it once and hand each of them a copy when it is compressed.
+        Results are identical; off by default, as the reference accumulates one Hessian per module.
+
     Expert Linears inside a ``LinearExperts2D`` block are handled together: while the block's forward
     runs, their hook calls are only recorded, and when it returns all experts' Hessians of one width
     are updated by a single grouped launch (384 tiny launches per batch become three).
@@ -63,12 +67,15 @@ class GPTQModifier(Modifier, QuantizationMixin):
     actorder: ActivationOrdering | Sentinel | None = Sentinel("static")
     offload_hessians: bool = False
     hessian_batch_tokens: int = 0
+    share_identical_inputs: bool = False
 
     _module_names: dict = PrivateAttr(default_factory=dict)
     _hessians: dict = PrivateAttr(default_factory=dict)
     _num_samples: dict = PrivateAttr(default_factory=dict)
     _staged: dict = PrivateAttr(default_factory=dict)
     _group_pending: list | None = PrivateAttr(default=None)
+    _leader: dict = PrivateAttr(default_factory=dict)  # follower module -> module whose Hessian it shares
+    _recent_input: tuple | None = PrivateAttr(default=None)  # (tensor kept alive, its version, leader)
 
     def resolve_quantization_config(self) -> QuantizationConfig:
         config = super().resolve_quantization_config()
@@ -138,6 +145,8 @@ class GPTQModifier(Modifier, QuantizationMixin):
     def calibrate_module(self, module: torch.nn.Module, args: tuple[torch.Tensor, ...], _output: torch.Tensor):
         """Forward hook: accumulate the Hessian of the module's input."""
         inp = args[0]
+        if self.share_identical_inputs and self._follows_recent_input(module, inp):
+            return
         if module not in self._num_samples:
             device = inp.device if inp.is_cuda else module.weight.device
             init_device = "cpu" if self.offload_hessians else device
@@ -153,6 +162,28 @@ class GPTQModifier(Modifier, QuantizationMixin):
         with self._maybe_onload_hessian(module):
             self._hessians[module], self._num_samples[module] = accumulate_hessian(
                 inp, module, self._hessians[module], self._num_samples[module])
+
+    # -- shared Hessians (see ``share_identical_inputs``)
+    def _follows_recent_input(self, module, inp) -> bool:
+        """True when `module` just received the tensor that the previous hook call accumulated for
+        another module of the same width; then only its sample count advances.  The previous input is
+        kept referenced, so no later tensor can take its address while it is being compared."""
+        recent = self._recent_input
+        same = (recent is not None and recent[2] is not module and inp.data_ptr() == recent[0].data_ptr()
+                and inp.shape == recent[0].shape and inp.dtype == recent[0].dtype and inp.stride() == recent[0].stride()
+                and inp._version == recent[1] and isinstance(module, torch.nn.Linear)
+                and module.in_features == recent[2].in_features)
+        leader = self._leader.get(module)
+        if same and (leader is recent[2] or (leader is None and module not in self._num_samples)):
+            self._leader[module] = recent[2]
+            n = 1 if inp.ndim == 2 else inp.shape[0]
+            self._num_samples[module] = self._num_samples.get(module, 0) + n
+            return True
+        if leader is not None:
+            raise RuntimeError("share_identical_inputs: a module that shared its input with another one received a "
+                               "different tensor on a later call; disable share_identical_inputs for this model")
+        self._recent_input = (inp, inp._version, module)
+        return False
 
     # -- expert groups (see the class docstring)
     def _begin_expert_group(self, _module, _args):
@@ -205,6 +236,14 @@ class GPTQModifier(Modifier, QuantizationMixin):
         self.compress_module_list(list(self._num_samples.keys()))
 
     def compress_module_list(self, module_list):
+        for module in module_list:  # followers get their own copy of the shared Hessian
+            leader = self._leader.pop(module, None)
+            if leader is not None:
+                self._flush(leader)
+                self._hessians[module] = self._hessians[leader].clone()
+                self._num_samples[module] = torch.tensor(float(self._num_samples[module]),
+                                                         device=self._hessians[module].device)
+        self._recent_input = None
         for module in module_list:
             name = self._module_names.get(module, module.__class__.__name__)
             self._flush(module)
@@ -233,6 +272,8 @@ class GPTQModifier(Modifier, QuantizationMixin):
         self._hessians = dict()
         self._num_samples = dict()
         self._staged = dict()
+        self._leader = dict()
+        self._recent_input = None
         return True
 
     @contextlib.contextmanager

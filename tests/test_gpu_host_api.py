@@ -525,3 +525,62 @@ def test_model_free_ptq_rejects_indivisible_groups(tmp_path):
     with pytest.raises(ValueError, match="Unable to quantize tensor"):
         model_free_ptq(src, str(tmp_path / "dst"), scheme="W4A16", ignore=["model.embed_tokens", "lm_head"],
                        device="cuda:0")
+
+
+def test_gptq_shared_input_hessians_are_identical():
+    """share_identical_inputs: q/k/v (and gate/up) see one tensor per batch; accumulating their Hessian once
+    gives bit-identical weights and the same sample counts as one Hessian per module."""
+    from llmcompressor_amd.core import LifecycleCallbacks, active_session
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+
+    class Block(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            g = torch.Generator().manual_seed(0)
+            for name, r in (("q_proj", 64), ("k_proj", 32), ("v_proj", 32), ("o_proj", 64)):
+                lin = torch.nn.Linear(64, r, bias=False, dtype=torch.bfloat16)
+                lin.weight.data = (torch.randn(r, 64, generator=g) * 0.05).bfloat16()
+                setattr(self, name, lin)
+
+        def forward(self, x):
+            q, k, v = self.q_proj(x), self.k_proj(x), self.v_proj(x)
+            return self.o_proj(q + torch.cat([k, v], dim=-1))
+
+    class Wrap(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.layers = torch.nn.ModuleList([Block()])
+
+    xs = [torch.randn(2, 24, 64, generator=torch.Generator().manual_seed(i)).bfloat16().to(DEV) for i in range(4)]
+    results = []
+    for share in (False, True):
+        model = Wrap().to(DEV)
+        calls = []
+        from llmcompressor_amd import ops
+        raw = ops.hessian_accumulate_
+        ops.hessian_accumulate_ = lambda H, x, **kw: (calls.append(1), raw(H, x, **kw))[1]
+        try:
+            mod = GPTQModifier(targets="Linear", share_identical_inputs=share, config_groups={"g": dict(
+                targets=["Linear"], weights=dict(num_bits=4, strategy="group", group_size=32))})
+            session = active_session()
+            session.reset()
+            session.initialize(model=model, recipe=mod)
+            LifecycleCallbacks.calibration_start()
+            with torch.no_grad():
+                for x in xs:
+                    model.layers[0](x)
+            if share:
+                blk = model.layers[0]
+                assert mod._leader[blk.k_proj] is blk.q_proj and mod._leader[blk.v_proj] is blk.q_proj
+                assert blk.o_proj not in mod._leader and blk.k_proj not in mod._hessians
+            LifecycleCallbacks.sequential_epoch_end(modules=list(model.modules()))
+            LifecycleCallbacks.calibration_end()
+            session.finalize()
+        finally:
+            ops.hessian_accumulate_ = raw
+        results.append((len(calls), {n: p.detach().clone() for n, p in model.named_parameters()}))
+    (n_raw, w_raw), (n_shared, w_shared) = results
+    assert n_raw == 4 * 4 and n_shared == 4 * 2  # q/k/v collapse to one accumulation per batch
+    assert w_raw.keys() == w_shared.keys()
+    for n in w_raw:
+        assert torch.equal(w_raw[n], w_shared[n]), n
