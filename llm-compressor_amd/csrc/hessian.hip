@@ -307,6 +307,17 @@ __global__ __launch_bounds__(256) void hessian_syrk_kernel(float* __restrict__ H
       rg[r].x = ok ? rg[r].x : 0u; rg[r].y = ok ? rg[r].y : 0u; rg[r].z = ok ? rg[r].z : 0u; rg[r].w = ok ? rg[r].w : 0u;
     }
   };
+  // fragment number n of 16-token group ks of the stage at `stA`, in the order the matrix ops first
+  // need them: A rows 0, then all B rows, then the remaining A rows.  Two register sets (ks & 1).
+  uint4 fa[2][MI], fb[2][MI];
+  auto read_frag = [&](const unsigned char* stA, int ks, int n) {
+    const int f = n == 0 ? 0 : (n <= MI ? MI + n - 1 : n - MI);  // f < MI -> A rows, else B rows
+    const int q = ks * 2 + (lane >> 5);
+    if (f < MI)
+      fa[ks & 1][f] = *(const uint4*)(stA + chunk_off(wm * (BT / 2) + f * 32 + (lane & 31), q));
+    else
+      fb[ks & 1][f - MI] = *(const uint4*)(stA + PANEL + chunk_off(wn * (BT / 2) + (f - MI) * 32 + (lane & 31), q));
+  };
   // One slab of matrix ops from stage `cur`, written out as an explicit software pipeline: the
   // slab is four groups of 16 tokens, each group NSTEP steps of two MFMAs, and every step also
   // issues its share of (1) the LDS reads of the next group's operand fragments (double-buffered
@@ -315,35 +326,27 @@ __global__ __launch_bounds__(256) void hessian_syrk_kernel(float* __restrict__ H
   // set during the following group (slab after next, starting at token t2).  A scheduling fence
   // after every step keeps the compiler from regrouping them; with one wave per SIMD nothing
   // else would cover a stall.
+  // The fragments of the slab's first group are already in registers.  The workgroup barrier
+  // sits after the third group: by then every wave has issued all its reads of stage `cur` and all
+  // its writes of stage `nxt`, so the fourth group can already fetch the next slab's first
+  // fragments from `nxt` and the slab boundary costs neither a barrier wait nor an LDS round trip.
   auto compute = [&](unsigned char* curA, unsigned char* nxtA, int t2, auto store_tag, auto mask_tag) {
     constexpr bool STORE = decltype(store_tag)::value;
     constexpr bool MASK = decltype(mask_tag)::value;
     constexpr int MPS = 2, NSTEP = MI * MI / MPS;  // matrix ops per step, steps per 16-token group
     constexpr int FPS = 2 * MI / NSTEP, CPS = 8 / NSTEP, LPS = RT / NSTEP;
-    unsigned char* curB = curA + PANEL;
-    uint4 fa[2][MI], fb[2][MI];
-    // fragment number n of group ks, in the order the matrix ops first need them:
-    // A rows 0, then all B rows, then the remaining A rows
-    auto read_frag = [&](int ks, int n) {
-      const int f = n == 0 ? 0 : (n <= MI ? MI + n - 1 : n - MI);  // f < MI -> A rows, else B rows
-      const int q = ks * 2 + (lane >> 5);
-      if (f < MI)
-        fa[ks & 1][f] = *(const uint4*)(curA + chunk_off(wm * (BT / 2) + f * 32 + (lane & 31), q));
-      else
-        fb[ks & 1][f - MI] = *(const uint4*)(curB + chunk_off(wn * (BT / 2) + (f - MI) * 32 + (lane & 31), q));
-    };
-#pragma unroll
-    for (int f = 0; f < 2 * MI; ++f) read_frag(0, f);
-    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
       if (STORE && MASK && ks == 0) mask_tail(ra, t2 - BK);
       if (STORE && MASK && ks == 2) mask_tail(rb, t2 - BK);
 #pragma unroll
       for (int st = 0; st < NSTEP; ++st) {
-        if (ks + 1 < BK / 16) {
 #pragma unroll
-          for (int f = st * FPS; f < (st + 1) * FPS; ++f) read_frag(ks + 1, f);
+        for (int f = st * FPS; f < (st + 1) * FPS; ++f) {
+          if (ks + 1 < BK / 16)
+            read_frag(curA, ks + 1, f);
+          else if (STORE)
+            read_frag(nxtA, 0, f);
         }
         if (STORE) {
 #pragma unroll
@@ -362,6 +365,10 @@ __global__ __launch_bounds__(256) void hessian_syrk_kernel(float* __restrict__ H
           acc[m / MI][m % MI] = Mfma<DT>::run(fa[ks & 1][m / MI], fb[ks & 1][m % MI], acc[m / MI][m % MI]);
         __builtin_amdgcn_sched_barrier(0);
       }
+      if (STORE && ks == 2) {
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
   };
 
@@ -375,17 +382,17 @@ __global__ __launch_bounds__(256) void hessian_syrk_kernel(float* __restrict__ H
   load_panel(ra, BK, i0);  // (clamped in-bounds when there is no second slab)
   load_panel(rb, BK, j0);
   __syncthreads();
+#pragma unroll
+  for (int f = 0; f < 2 * MI; ++f) read_frag(smem, 0, f);
+  __builtin_amdgcn_sched_barrier(0);
   // steady state: slab s multiplied, slab s+1 transposed into the other stage, slab s+2 in flight
-  for (int s = 0; s + 2 < nslab; ++s) {
+  for (int s = 0; s + 2 < nslab; ++s)
     compute(smem + (s & 1) * 2 * PANEL, smem + ((s + 1) & 1) * 2 * PANEL, (s + 2) * BK, std::true_type{},
             std::false_type{});
-    __syncthreads();
-  }
   if (nslab >= 2) {
     const int s = nslab - 2;
     compute(smem + (s & 1) * 2 * PANEL, smem + ((s + 1) & 1) * 2 * PANEL, (s + 2) * BK, std::true_type{},
             std::true_type{});
-    __syncthreads();
   }
   compute(smem + ((nslab - 1) & 1) * 2 * PANEL, smem, 0, std::false_type{}, std::false_type{});
 
