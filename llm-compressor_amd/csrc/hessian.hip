@@ -330,9 +330,16 @@ __global__ __launch_bounds__(256) void hessian_syrk_kernel(float* __restrict__ H
   // sits after the third group: by then every wave has issued all its reads of stage `cur` and all
   // its writes of stage `nxt`, so the fourth group can already fetch the next slab's first
   // fragments from `nxt` and the slab boundary costs neither a barrier wait nor an LDS round trip.
-  auto compute = [&](unsigned char* curA, unsigned char* nxtA, int t2, auto store_tag, auto mask_tag) {
+  // Row pointers of the slab the steady state loads next (token t2 + g_t*RT, this thread's 8 features
+  // of either panel): while that slab is a full one no clamping is needed and a load is one 64-bit
+  // add away from them.
+  const uint16_t* pA = X + (int64_t)(2 * BK + g_t * RT) * ldx + min(i0 + g_i * 8, K - 8);
+  const uint16_t* pB = X + (int64_t)(2 * BK + g_t * RT) * ldx + min(j0 + g_i * 8, K - 8);
+  auto compute = [&](unsigned char* curA, unsigned char* nxtA, int t2, auto store_tag, auto mask_tag,
+                     auto direct_tag) {
     constexpr bool STORE = decltype(store_tag)::value;
     constexpr bool MASK = decltype(mask_tag)::value;
+    constexpr bool DIRECT = decltype(direct_tag)::value && ALIGNED;  // unclamped loads through pA / pB
     constexpr int MPS = 2, NSTEP = MI * MI / MPS;  // matrix ops per step, steps per 16-token group
     constexpr int FPS = 2 * MI / NSTEP, CPS = 8 / NSTEP, LPS = RT / NSTEP;
 #pragma unroll
@@ -356,8 +363,13 @@ __global__ __launch_bounds__(256) void hessian_syrk_kernel(float* __restrict__ H
           }
 #pragma unroll
           for (int r = st * LPS; r < (st + 1) * LPS; ++r) {
-            if (ks == 1) ra[r] = load8<ALIGNED>(X, ldx, t2 + g_t * RT + r, i0 + g_i * 8, T, K);
-            if (ks == 3) rb[r] = load8<ALIGNED>(X, ldx, t2 + g_t * RT + r, j0 + g_i * 8, T, K);
+            if (DIRECT) {
+              if (ks == 1) ra[r] = *(const uint4*)(pA + (int64_t)r * ldx);
+              if (ks == 3) rb[r] = *(const uint4*)(pB + (int64_t)r * ldx);
+            } else {
+              if (ks == 1) ra[r] = load8<ALIGNED>(X, ldx, t2 + g_t * RT + r, i0 + g_i * 8, T, K);
+              if (ks == 3) rb[r] = load8<ALIGNED>(X, ldx, t2 + g_t * RT + r, j0 + g_i * 8, T, K);
+            }
           }
         }
 #pragma unroll
@@ -385,16 +397,25 @@ __global__ __launch_bounds__(256) void hessian_syrk_kernel(float* __restrict__ H
 #pragma unroll
   for (int f = 0; f < 2 * MI; ++f) read_frag(smem, 0, f);
   __builtin_amdgcn_sched_barrier(0);
-  // steady state: slab s multiplied, slab s+1 transposed into the other stage, slab s+2 in flight
-  for (int s = 0; s + 2 < nslab; ++s)
+  // steady state: slab s multiplied, slab s+1 transposed into the other stage, slab s+2 in flight;
+  // first the iterations whose slab s+2 is a full one (direct loads), then at most one with clamped loads
+  const int nfull = T / BK;
+  int s = 0;
+  for (; s + 2 < nslab && s + 3 <= nfull; ++s) {
     compute(smem + (s & 1) * 2 * PANEL, smem + ((s + 1) & 1) * 2 * PANEL, (s + 2) * BK, std::true_type{},
-            std::false_type{});
-  if (nslab >= 2) {
-    const int s = nslab - 2;
-    compute(smem + (s & 1) * 2 * PANEL, smem + ((s + 1) & 1) * 2 * PANEL, (s + 2) * BK, std::true_type{},
-            std::true_type{});
+            std::false_type{}, std::true_type{});
+    pA += (int64_t)BK * ldx;
+    pB += (int64_t)BK * ldx;
   }
-  compute(smem + ((nslab - 1) & 1) * 2 * PANEL, smem, 0, std::false_type{}, std::false_type{});
+  for (; s + 2 < nslab; ++s)
+    compute(smem + (s & 1) * 2 * PANEL, smem + ((s + 1) & 1) * 2 * PANEL, (s + 2) * BK, std::true_type{},
+            std::false_type{}, std::false_type{});
+  if (nslab >= 2) {
+    s = nslab - 2;
+    compute(smem + (s & 1) * 2 * PANEL, smem + ((s + 1) & 1) * 2 * PANEL, (s + 2) * BK, std::true_type{},
+            std::true_type{}, std::false_type{});
+  }
+  compute(smem + ((nslab - 1) & 1) * 2 * PANEL, smem, 0, std::false_type{}, std::false_type{}, std::false_type{});
 
   if (partial) {
     // partial tile: raw accumulators to the workspace in register order (16 bytes per lane, coalesced)
