@@ -123,8 +123,25 @@ __device__ __forceinline__ void tile_coords(int c, int nb, int SH, int SW, int& 
 template <int BT, bool FAST_EPI>
 __device__ __forceinline__ void tile_epilogue(float* __restrict__ H, int64_t ldh, int K, float alpha,
                                               int assume_sym, int i0, int j0, f32x16_t (&acc)[BT / 64][BT / 64],
-                                              int a_only = -1) {  // >= 0: only MFMA tile row a_only
+                                              int a_only = -1,              // >= 0: only MFMA tile row a_only
+                                              float* __restrict__ slot = nullptr) {  // partial tile: raw store
   constexpr int MI = BT / 64;
+  if (slot) {
+    // a token chunk's partial tile: raw accumulators in register order (16 bytes per lane, coalesced)
+#pragma unroll
+    for (int a = 0; a < MI; ++a) {
+#pragma unroll
+      for (int b = 0; b < MI; ++b) {
+#pragma unroll
+        for (int vq = 0; vq < 4; ++vq)
+          *(float4*)(slot + (((a * MI + b) * 4 + vq) * 256 + threadIdx.x) * 4) =
+              make_float4(acc[a][b][vq * 4], acc[a][b][vq * 4 + 1], acc[a][b][vq * 4 + 2], acc[a][b][vq * 4 + 3]);
+        // one MFMA tile at a time: moving many accumulators out of the AGPRs at once spills
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    return;
+  }
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const bool diag = i0 == j0;
@@ -417,23 +434,8 @@ __global__ __launch_bounds__(256) void hessian_syrk_kernel(float* __restrict__ H
   }
   compute(smem + ((nslab - 1) & 1) * 2 * PANEL, smem, 0, std::false_type{}, std::false_type{}, std::false_type{});
 
-  if (partial) {
-    // partial tile: raw accumulators to the workspace in register order (16 bytes per lane, coalesced)
-    float* slot = ws + (int64_t)(ph.ws_tile0 + (item % ph.ntiles) * ph.split + chunk) * (BT * BT);
-#pragma unroll
-    for (int a = 0; a < MI; ++a)
-#pragma unroll
-      for (int b = 0; b < MI; ++b) {
-#pragma unroll
-        for (int vq = 0; vq < 4; ++vq)
-          *(float4*)(slot + (((a * MI + b) * 4 + vq) * 256 + tid) * 4) =
-              make_float4(acc[a][b][vq * 4], acc[a][b][vq * 4 + 1], acc[a][b][vq * 4 + 2], acc[a][b][vq * 4 + 3]);
-        // one MFMA tile at a time: moving all 256 accumulators out of the AGPRs at once spills
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    return;
-  }
-  tile_epilogue<BT, FAST_EPI>(H, ldh, K, alpha, assume_sym, i0, j0, acc);
+  float* slot = partial ? ws + (int64_t)(ph.ws_tile0 + (item % ph.ntiles) * ph.split + chunk) * (BT * BT) : nullptr;
+  tile_epilogue<BT, FAST_EPI>(H, ldh, K, alpha, assume_sym, i0, j0, acc, -1, slot);
 }
 
 // Sums the chunks of a split tile in fixed order and applies the tile epilogue; one workgroup per
