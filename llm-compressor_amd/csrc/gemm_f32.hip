@@ -135,6 +135,40 @@ __device__ __forceinline__ void gemm_tile(const GemmF32& g, const float* A, cons
     multiply();
   }
 
+  // Epilogue.  A tile wholly inside C (and, for a lower-triangular C, wholly below the diagonal) needs no
+  // per-element tests.  It uses buffer addressing: one descriptor for the wave's strip of C, the row offset
+  // in a scalar register and a single per-lane byte offset, so no 64-bit address is kept per element; the
+  // 16 values of a 32x32 sub-tile are fetched together, then combined and stored -- one memory round trip
+  // per sub-tile instead of one per element.
+  if (FAST && !(g.c_lower && n0 + BN - 1 > m0)) {
+    const int wm_u = __builtin_amdgcn_readfirstlane(wm), wn_u = __builtin_amdgcn_readfirstlane(wn);
+    float* const c0 = C + (int64_t)(m0 + wm_u * (BM / 2)) * g.ldc + n0 + wn_u * (BN / 2);
+    const int lane_bytes = ((lane >> 5) * 4 * (int)g.ldc + (lane & 31)) * 4;
+    const int row_bytes = (int)g.ldc * 4;
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(c0, 0, 0x7fffffff, 0x00020000);
+#pragma unroll
+    for (int a = 0; a < MI; ++a)
+#pragma unroll
+      for (int b = 0; b < NI; ++b) {
+        float cv[16];
+        if (g.beta != 0.f) {
+#pragma unroll
+          for (int v = 0; v < 16; ++v)
+            cv[v] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                rsrc, lane_bytes, (a * 32 + (v / 4) * 8 + (v & 3)) * row_bytes + b * 128, 0));
+        }
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          float r = g.alpha * acc[a][b][v];
+          if (g.beta != 0.f) r += g.beta * cv[v];
+          __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, r), rsrc, lane_bytes,
+                                                (a * 32 + (v / 4) * 8 + (v & 3)) * row_bytes + b * 128, 0);
+        }
+      }
+    return;
+  }
+
+  // edge and diagonal tiles: element by element
 #pragma unroll
   for (int a = 0; a < MI; ++a)
 #pragma unroll

@@ -9,6 +9,7 @@ from __future__ import annotations
 
 import contextlib
 import logging
+import threading
 
 import torch
 from pydantic import PrivateAttr
@@ -55,6 +56,9 @@ class GPTQModifier(Modifier, QuantizationMixin):
         have the same Hessian; accumulate it once and hand each of them a copy when it is compressed.
         Results are identical; off by default, as the reference accumulates one Hessian per module.
 
+    :param compress_concurrency: how many modules of one ``compress_module_list`` call are quantised at the
+        same time, each on its own HIP stream (1 = one after the other, the reference's behaviour)
+
     Expert Linears inside a ``LinearExperts2D`` block are handled together: while the block's forward
     runs, their hook calls are only recorded, and when it returns all experts' Hessians of one width
     are updated by a single grouped launch (384 tiny launches per batch become three).
@@ -68,6 +72,7 @@ class GPTQModifier(Modifier, QuantizationMixin):
     offload_hessians: bool = False
     hessian_batch_tokens: int = 0
     share_identical_inputs: bool = False
+    compress_concurrency: int = 4
 
     _module_names: dict = PrivateAttr(default_factory=dict)
     _hessians: dict = PrivateAttr(default_factory=dict)
@@ -76,6 +81,7 @@ class GPTQModifier(Modifier, QuantizationMixin):
     _group_pending: list | None = PrivateAttr(default=None)
     _leader: dict = PrivateAttr(default_factory=dict)  # follower module -> module whose Hessian it shares
     _recent_input: tuple | None = PrivateAttr(default=None)  # (tensor kept alive, its version, leader)
+    _streams: list = PrivateAttr(default_factory=list)
 
     def resolve_quantization_config(self) -> QuantizationConfig:
         config = super().resolve_quantization_config()
@@ -244,25 +250,75 @@ class GPTQModifier(Modifier, QuantizationMixin):
                 self._num_samples[module] = torch.tensor(float(self._num_samples[module]),
                                                          device=self._hessians[module].device)
         self._recent_input = None
-        for module in module_list:
-            name = self._module_names.get(module, module.__class__.__name__)
+        for module in module_list:  # pending activations go in on the calibration stream
             self._flush(module)
             self._staged.pop(module, None)
-            num_samples = self._num_samples[module]
-            quant_args = getattr_chain(module, "quantization_scheme.weights")
-            logger.info(f"Quantizing {name} using {int(num_samples)} samples")
-            with torch.no_grad(), self._maybe_onload_hessian(module), CompressionLogger(module) as comp_logger:
-                loss, q_param_dict = quantize_weight(
-                    module=module,
-                    quant_args=quant_args,
-                    hessian=self._hessians.pop(module),
-                    blocksize=self.block_size,
-                    percdamp=self.dampening_frac,
-                    hessian_divisor=float(self._num_samples.pop(module).item()),
-                )
-                comp_logger.set_results(name="GPTQ", loss=loss)
-            for attr, val in q_param_dict.items():
-                update_offload_parameter(module, attr, val)
+        jobs = list(module_list)
+        workers = min(int(self.compress_concurrency), len(jobs))
+        on_gpu = all(m.weight.is_cuda and self._hessians[m].is_cuda for m in jobs)
+        if workers <= 1 or not on_gpu or self.offload_hessians:
+            for module in jobs:
+                self._compress_one(module)
+            return
+        # Modules are independent, and each one's Cholesky chain and column loop are long runs of
+        # small, serially dependent kernels that leave most of the chip idle.  Quantise several at once,
+        # one host thread and one HIP stream each, most expensive first so that the widest module does
+        # not start last.  Per module the kernels and their order are unchanged, so are the results.
+        device = jobs[0].weight.device
+        jobs.sort(key=lambda m: -(float(m.weight.shape[1]) ** 3 + float(m.weight.shape[0]) * m.weight.shape[1] ** 2))
+        main = torch.cuda.current_stream(device)
+        ready = main.record_event()
+        while len(self._streams) < workers:
+            self._streams.append(torch.cuda.Stream(device=device))
+        lock = threading.Lock()
+        errors = []
+
+        def worker(stream):
+            try:
+                with torch.cuda.device(device), torch.cuda.stream(stream):
+                    stream.wait_event(ready)
+                    while True:
+                        with lock:
+                            if not jobs or errors:
+                                return
+                            module = jobs.pop(0)
+                        self._compress_one(module, produced_on=stream, consumed_on=main)
+            except BaseException as err:  # re-raised on the calling thread
+                errors.append(err)
+
+        threads = [threading.Thread(target=worker, args=(s,), daemon=True) for s in self._streams[:workers]]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        for s in self._streams[:workers]:
+            main.wait_stream(s)
+        if errors:
+            raise errors[0]
+
+    def _compress_one(self, module, produced_on=None, consumed_on=None):
+        name = self._module_names.get(module, module.__class__.__name__)
+        hessian = self._hessians.pop(module)
+        num_samples = self._num_samples.pop(module)
+        if produced_on is not None:  # allocated on the calibration stream, last read on this one
+            hessian.record_stream(produced_on)
+        logger.info(f"Quantizing {name} using {int(num_samples)} samples")
+        with torch.no_grad(), CompressionLogger(module) as comp_logger:
+            if self.offload_hessians:
+                hessian = hessian.to(device=module.weight.device)
+            loss, q_param_dict = quantize_weight(
+                module=module,
+                quant_args=getattr_chain(module, "quantization_scheme.weights"),
+                hessian=hessian,
+                blocksize=self.block_size,
+                percdamp=self.dampening_frac,
+                hessian_divisor=float(num_samples),
+            )
+            comp_logger.set_results(name="GPTQ", loss=loss)
+        for attr, val in q_param_dict.items():
+            if consumed_on is not None and val.is_cuda:  # allocated on this stream, read by later forwards
+                val.record_stream(consumed_on)
+            update_offload_parameter(module, attr, val)
 
     def on_finalize(self, state: State, **kwargs) -> bool:
         if not self.ended_:

@@ -584,3 +584,93 @@ def test_gptq_shared_input_hessians_are_identical():
     assert w_raw.keys() == w_shared.keys()
     for n in w_raw:
         assert torch.equal(w_raw[n], w_shared[n]), n
+
+
+def test_gptq_concurrent_module_compression_is_identical():
+    """compress_concurrency: modules quantised on separate streams give bit-identical parameters to the
+    one-after-the-other order, the streams used are distinct, and an error in one module is raised."""
+    from llmcompressor_amd.core import LifecycleCallbacks, active_session
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+    import llmcompressor_amd.modifiers.gptq.base as base
+
+    class Block(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            g = torch.Generator().manual_seed(1)
+            for name, r, k in (("a", 96, 256), ("b", 32, 256), ("c", 256, 256), ("d", 64, 512), ("e", 512, 64),
+                               ("f", 128, 128)):
+                lin = torch.nn.Linear(k, r, bias=False, dtype=torch.bfloat16)
+                lin.weight.data = (torch.randn(r, k, generator=g) * 0.05).bfloat16()
+                setattr(self, name, lin)
+
+        def forward(self, x):
+            h = self.c(x) + torch.cat([self.a(x), self.b(x), self.f(x[..., :128])], dim=-1)
+            return self.e(self.d(torch.cat([h, x], dim=-1)))
+
+    class Wrap(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.layers = torch.nn.ModuleList([Block()])
+
+    xs = [torch.randn(2, 300, 256, generator=torch.Generator().manual_seed(i)).bfloat16().to(DEV) for i in range(3)]
+    results = []
+    for conc in (1, 4):
+        model = Wrap().to(DEV)
+        streams = []
+        raw = base.quantize_weight
+
+        def spy(**kw):
+            streams.append(torch.cuda.current_stream().cuda_stream)
+            return raw(**kw)
+
+        base.quantize_weight = spy
+        try:
+            mod = GPTQModifier(targets="Linear", compress_concurrency=conc, hessian_batch_tokens=512,
+                               config_groups={"g": dict(targets=["Linear"], weights=dict(
+                                   num_bits=4, strategy="group", group_size=32, symmetric=False))})
+            session = active_session()
+            session.reset()
+            session.initialize(model=model, recipe=mod)
+            LifecycleCallbacks.calibration_start()
+            with torch.no_grad():
+                for x in xs:
+                    model.layers[0](x)
+            LifecycleCallbacks.sequential_epoch_end(modules=list(model.modules()))
+            LifecycleCallbacks.calibration_end()
+            session.finalize()
+        finally:
+            base.quantize_weight = raw
+        torch.cuda.synchronize()
+        results.append((streams, {n: p.detach().clone() for n, p in model.named_parameters()}))
+    (s1, w1), (s4, w4) = results
+    assert len(s1) == 6 and len(set(s1)) == 1
+    assert len(s4) == 6 and len(set(s4)) > 1 and s1[0] not in s4
+    assert w1.keys() == w4.keys()
+    for n in w1:
+        assert torch.equal(w1[n], w4[n]), n
+
+    # a failure inside one module's compression surfaces on the caller's thread
+    model = Wrap().to(DEV)
+    raw = base.quantize_weight
+
+    def failing(**kw):
+        if kw["module"] is model.layers[0].d:
+            raise RuntimeError("boom")
+        return raw(**kw)
+
+    base.quantize_weight = failing
+    try:
+        mod = GPTQModifier(targets="Linear", compress_concurrency=3, config_groups={"g": dict(
+            targets=["Linear"], weights=dict(num_bits=4, strategy="group", group_size=32))})
+        session = active_session()
+        session.reset()
+        session.initialize(model=model, recipe=mod)
+        LifecycleCallbacks.calibration_start()
+        with torch.no_grad():
+            model.layers[0](xs[0])
+        with pytest.raises(RuntimeError, match="boom"):
+            LifecycleCallbacks.sequential_epoch_end(modules=list(model.modules()))
+    finally:
+        base.quantize_weight = raw
+        active_session().reset()
+    torch.cuda.synchronize()
