@@ -147,6 +147,15 @@ def probe_bandwidth():
         4 * x.numel())
     rep("fp8 dynamic per-token -> bytes [8192x4096], 3 B/elem",
         timed(lambda: ops.dynamic_per_token_quantize(x, out_mode=ops.OUT_CODES)), 3 * x.numel())
+    # the MSE grid search is arithmetic-bound (every candidate scale re-quantises the group): its figure
+    # of merit is candidate evaluations per second; the GB/s column is its one read of the weight
+    for name, kw, fmt, bits, g in (("mse observer int4 g128, 20 candidates", {}, ops.FMT_INT, 4, 128),
+                                   ("mse observer fp4 g16, 20 candidates", {}, ops.FMT_FP4, 4, 16),
+                                   ("mse observer fp4 g16, 80 candidates (maxshrink 0.8, no early stop)",
+                                    dict(maxshrink=0.8, patience=100), ops.FMT_FP4, 4, 16)):
+        t = timed(lambda: ops.mse_observe_groups(w, g, fmt, bits, True, ops.SCALE_PLAIN, **kw), n=5)
+        cands = 80 if kw else 20
+        rep(f"{name}: {n * cands / t / 1e12:.2f} T element-candidates/s", t, 2 * n)
     print("| kernel (14336 x 4096 bf16 unless noted) | us | GB/s | of 8 TB/s |")
     print("|---|---|---|---|")
     for name, us, gbs, frac in rows:

@@ -60,7 +60,10 @@ int llmc_version(void);
  * workgroups be cut along the tokens: the chunks' partial tiles go through the
  * workspace and are summed in a fixed order, so the result does not depend on
  * timing.  Without it every tile is one workgroup (slower when the tile count
- * is not a multiple of the CU count).  The workspace holds no state between calls.
+ * is not a multiple of the CU count).  Its first 64 KiB hold progress words with
+ * which workgroups that share an L2 pace each other over long token loops (fewer
+ * re-fetches of X; the result does not depend on them).  The workspace holds no
+ * state between calls; calls that overlap in time need workspaces of their own.
  */
 enum { LLMC_HESSIAN_ASSUME_SYMMETRIC = 1 };
 int64_t llmc_hessian_workspace_bytes(int64_t T, int64_t K);

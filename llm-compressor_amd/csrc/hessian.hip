@@ -81,6 +81,11 @@ __device__ __forceinline__ int chunk_off(int i, int q) {
 // order and runs the same epilogue: that is how the tiles left over after the last full round of
 // 256 workgroups still fill the chip, with results that do not depend on timing.
 constexpr int MAX_PHASES = 4;
+constexpr int PACE_SLABS = 4;          // slabs between two pacing ticks
+constexpr int PACE_WINDOW = 2;         // ticks a workgroup may be ahead of the slowest member of its group
+constexpr int PACE_SPIN_LIMIT = 24;    // polls before a workgroup gives up pacing
+constexpr int PACE_MAX_GROUPS = 512;   // 32 slots each, at the head of the workspace
+constexpr int PACE_BYTES = PACE_MAX_GROUPS * 32 * 4;
 struct Phase {
   int first_wg, tile0, ntiles, split, ws_tile0;
 };
@@ -235,7 +240,8 @@ template <int BT, int DT, bool ALIGNED, bool FAST_EPI, class GRP>
 __global__ __launch_bounds__(256) void hessian_syrk_kernel(float* __restrict__ H, int64_t ldh,
                                                             const uint16_t* __restrict__ Xfull, int64_t ldx,
                                                             int Tfull, int K, float alpha, int assume_sym,
-                                                            int nb, Plan plan, float* __restrict__ ws, GRP grp) {
+                                                            int nb, Plan plan, float* __restrict__ ws, GRP grp,
+                                                            unsigned* __restrict__ pace) {
   if constexpr (GRP::grouped) {
     Tfull = grp.T[blockIdx.y];
     if (Tfull <= 0) return;
@@ -277,6 +283,18 @@ __global__ __launch_bounds__(256) void hessian_syrk_kernel(float* __restrict__ H
   const bool diag = (I == J);
 
   const int tid = threadIdx.x;
+  // Pacing.  The 32 workgroups that run together on one XCD share feature panels through that XCD's
+  // L2, but only while they work on nearby slabs; nothing in the kernel keeps them together (the
+  // loads run two slabs ahead, so a workgroup that is ahead is not slowed by its cache misses), and
+  // over a thousand slabs they drift apart until every panel is fetched once per workgroup.  Every
+  // PACE_SLABS slabs a workgroup publishes its tick number in its own slot of the group's 128-byte
+  // line and its first wave reads all 32 slots; a slab later, when the values have arrived, it holds
+  // the workgroup back while it is more than PACE_WINDOW ticks ahead of the slowest member.  Plain
+  // stores and loads to distinct words, no read-modify-write.  The wait is bounded: a workgroup that
+  // times out (its group is not resident together) stops pacing for good.
+  unsigned* const my_group = pace + 32 * ((bl % 8) + 8 * ((bl / 8) / 32));
+  const int my_member = (bl / 8) % 32;
+  bool pacing = pace != nullptr && pi == 0 && ph.split == 1 && ph.ntiles % (8 * 32) == 0 && tid < 64;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
@@ -418,7 +436,33 @@ __global__ __launch_bounds__(256) void hessian_syrk_kernel(float* __restrict__ H
   // first the iterations whose slab s+2 is a full one (direct loads), then at most one with clamped loads
   const int nfull = T / BK;
   int s = 0;
-  for (; s + 2 < nslab && s + 3 <= nfull; ++s) {
+  const int ndirect = max(0, min(nslab - 2, nfull - 2));  // iterations whose slab s+2 is a full one
+  unsigned seen = 0xffffffffu;  // the group's slots as read one period ago (lane m: member m)
+  for (; s + PACE_SLABS <= ndirect; s += PACE_SLABS) {
+    if (pacing) {  // uniform over the first wave, false in the others
+      const unsigned my_tick = (unsigned)(s / PACE_SLABS);
+      int spins = 0;
+      while (true) {
+        // lanes 32..63 hold 0xffffffff; any member more than PACE_WINDOW ticks behind holds us back
+        if (__builtin_amdgcn_ballot_w64(my_tick > seen && my_tick - seen > (unsigned)PACE_WINDOW) == 0) break;
+        if (++spins == PACE_SPIN_LIMIT) {
+          pacing = false;
+          break;
+        }
+        __builtin_amdgcn_s_sleep(8);
+        if (tid < 32) seen = __hip_atomic_load(my_group + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      if (tid == 0) __hip_atomic_store(my_group + my_member, my_tick + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (tid < 32) seen = __hip_atomic_load(my_group + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    for (int i = 0; i < PACE_SLABS; ++i) {
+      compute(smem + ((s + i) & 1) * 2 * PANEL, smem + ((s + i + 1) & 1) * 2 * PANEL, (s + i + 2) * BK,
+              std::true_type{}, std::false_type{}, std::true_type{});
+      pA += (int64_t)BK * ldx;
+      pB += (int64_t)BK * ldx;
+    }
+  }
+  for (; s < ndirect; ++s) {
     compute(smem + (s & 1) * 2 * PANEL, smem + ((s + 1) & 1) * 2 * PANEL, (s + 2) * BK, std::true_type{},
             std::false_type{}, std::true_type{});
     pA += (int64_t)BK * ldx;
@@ -598,9 +642,13 @@ Choice choose(int64_t T, int64_t K, int64_t ws_avail) {
   return best;
 }
 
+__global__ void zero_u32_kernel(unsigned* p, int n) {
+  for (int i = threadIdx.x; i < n; i += blockDim.x) p[i] = 0u;
+}
+
 template <int BT, int DT>
 int launch(const Choice& c, float* H, int64_t ldh, const void* X, int64_t ldx, int64_t T, int64_t K, float alpha,
-           int flags, float* ws, hipStream_t st) {
+           int flags, float* ws, unsigned* pace, hipStream_t st) {
   const int nb = (int)((K + BT - 1) / BT);
   const bool aligned = (K % 8 == 0) && (ldx % 8 == 0) && (((uintptr_t)X & 15) == 0);
   const int sym = (flags & LLMC_HESSIAN_ASSUME_SYMMETRIC) ? 1 : 0;
@@ -614,8 +662,16 @@ int launch(const Choice& c, float* H, int64_t ldh, const void* X, int64_t ldx, i
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return 1000 + (int)e;
   }
+  // pacing slots: 32 per (round of whole tiles, XCD); only worth it for long token loops
+  const Phase& p0 = c.plan.ph[0];
+  const int pace_groups = (p0.split == 1 && p0.ntiles % NUM_WG == 0) ? p0.ntiles / 32 : 0;
+  if (pace_groups == 0 || pace_groups > PACE_MAX_GROUPS || T < 64 * BK) pace = nullptr;
+  if (pace) {
+    hipLaunchKernelGGL(zero_u32_kernel, dim3(1), dim3(256), 0, st, pace, pace_groups * 32);
+    LLMC_LAUNCH_STATUS();
+  }
   hipLaunchKernelGGL(kern, dim3(c.grid), dim3(256), smem, st, H, ldh, (const uint16_t*)X, ldx, (int)T,
-                     (int)K, alpha, sym, nb, c.plan, ws, NoGroup{});
+                     (int)K, alpha, sym, nb, c.plan, ws, NoGroup{}, pace);
   LLMC_LAUNCH_STATUS();
   if (c.nsplit_tiles > 0) {
     if (fast)
@@ -633,7 +689,7 @@ int launch(const Choice& c, float* H, int64_t ldh, const void* X, int64_t ldx, i
 
 extern "C" int64_t llmc_hessian_workspace_bytes(int64_t T, int64_t K) {
   if (T <= 0 || K <= 0 || K >= (1 << 30)) return 0;
-  return choose(T, K, INT64_MAX).ws_bytes;
+  return choose(T, K, INT64_MAX).ws_bytes + PACE_BYTES;
 }
 
 extern "C" int llmc_hessian_accumulate(float* H, int64_t ldh, const void* X, int64_t ldx, int64_t T,
@@ -651,13 +707,17 @@ extern "C" int llmc_hessian_accumulate(float* H, int64_t ldh, const void* X, int
   hipStream_t st = (hipStream_t)stream;
   // 256-wide tiles need half the LDS traffic per matrix op of 128-wide ones; token chunks spread a
   // tile count that is not a multiple of the CU count over the whole chip
-  const Choice c = choose(T, K, workspace ? workspace_bytes : 0);
-  float* ws = (float*)workspace;
+  // workspace layout: [pacing counters, PACE_BYTES][partial tiles of the token chunks]
+  const int64_t avail = workspace ? workspace_bytes : 0;
+  const bool pace_room = avail >= PACE_BYTES;
+  const Choice c = choose(T, K, pace_room ? avail - PACE_BYTES : avail);
+  unsigned* pace = pace_room ? (unsigned*)workspace : nullptr;
+  float* ws = (float*)((char*)workspace + (pace_room ? PACE_BYTES : 0));
   if (x_dtype == LLMC_BF16)
-    return c.bt == 256 ? launch<256, LLMC_BF16>(c, H, ldh, X, ldx, T, K, alpha, flags, ws, st)
-                       : launch<128, LLMC_BF16>(c, H, ldh, X, ldx, T, K, alpha, flags, ws, st);
-  return c.bt == 256 ? launch<256, LLMC_F16>(c, H, ldh, X, ldx, T, K, alpha, flags, ws, st)
-                     : launch<128, LLMC_F16>(c, H, ldh, X, ldx, T, K, alpha, flags, ws, st);
+    return c.bt == 256 ? launch<256, LLMC_BF16>(c, H, ldh, X, ldx, T, K, alpha, flags, ws, pace, st)
+                       : launch<128, LLMC_BF16>(c, H, ldh, X, ldx, T, K, alpha, flags, ws, pace, st);
+  return c.bt == 256 ? launch<256, LLMC_F16>(c, H, ldh, X, ldx, T, K, alpha, flags, ws, pace, st)
+                     : launch<128, LLMC_F16>(c, H, ldh, X, ldx, T, K, alpha, flags, ws, pace, st);
 }
 
 template <int BT, int DT>
@@ -672,7 +732,7 @@ int launch_grouped(const GroupArgs& grp, int n, int64_t ldh, int64_t ldx, int64_
     if (e != hipSuccess) return 1000 + (int)e;
   }
   hipLaunchKernelGGL(kern, dim3(c.grid, n), dim3(256), smem, st, (float*)nullptr, ldh, (const uint16_t*)nullptr, ldx, 0,
-                     (int)K, alpha, sym, nb, c.plan, (float*)nullptr, grp);
+                     (int)K, alpha, sym, nb, c.plan, (float*)nullptr, grp, (unsigned*)nullptr);
   LLMC_LAUNCH_STATUS();
   return 0;
 }
