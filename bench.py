@@ -249,6 +249,20 @@ def main():
         return raw_accumulate(H, x, **kw)
 
     ops.hessian_accumulate_ = timed_accumulate
+    raw_segments = ops.hessian_accumulate_segments_
+
+    def timed_segments(H, xs_, **kw):  # the same kernel, fed the hook's buffers in place (no staging copy)
+        if recording[0] and H.shape[0] == INTER and len(xs_) <= ops.SEGMENTS_MAX:
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            out = raw_segments(H, xs_, **kw)
+            e1.record()
+            dom_events.append((e0, e1))
+            dom_tokens.append(sum(x.shape[0] for x in xs_))
+            return out
+        return raw_segments(H, xs_, **kw)
+
+    ops.hessian_accumulate_segments_ = timed_segments
 
     def step(record: bool, share: bool = False):
         for name, r, k in LINEARS:
@@ -269,7 +283,7 @@ def main():
             args_of = {k: (x[b:b + 1],) for k, x in xs.items()}
             for mod, stream in mods:
                 modifier.calibrate_module(mod, args_of[stream], None)
-        for m in list(modifier._staged):
+        for m in list(modifier._num_samples):
             modifier._flush(m)
         torch.cuda.synchronize()
         t1 = time.perf_counter()

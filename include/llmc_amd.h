@@ -82,6 +82,18 @@ int llmc_hessian_accumulate_grouped(float* const* H, int64_t ldh, const void* co
                                     const int64_t* T, int32_t n, int64_t K, int32_t x_dtype,
                                     float alpha, int32_t flags, void* stream);
 
+/* Segmented form: the token rows of ONE problem lie in n_seg separate buffers (the calibration
+ * batches exactly as GPTQModifier.calibrate_module receives them, modifiers/gptq/base.py:240-262),
+ * so that accumulating several batches with one launch does not need them copied together first.
+ * X is a HOST array of n_seg (<= 64) device pointers, each 16-byte aligned and holding seg_tokens
+ * rows of stride ldx (seg_tokens % 64 == 0); the last buffer holds last_tokens <= seg_tokens rows.
+ * K % 8 == 0 and ldx % 8 == 0.  The result is bit-identical to llmc_hessian_accumulate on the
+ * concatenation.  Workspace as for llmc_hessian_accumulate with T = total rows. */
+int llmc_hessian_accumulate_segments(float* H, int64_t ldh, const void* const* X, int32_t n_seg,
+                                     int64_t seg_tokens, int64_t last_tokens, int64_t ldx, int64_t K,
+                                     int32_t x_dtype, float alpha, int32_t flags, void* workspace,
+                                     int64_t workspace_bytes, void* stream);
+
 /* ---- a10/a11: min-max observers --------------------------------------------
  * Replace _get_min_max() = torch.amin/amax(observed, dim=(0,-1)) on the
  * flattened weight (src/llmcompressor/observers/min_max.py:70-74 with

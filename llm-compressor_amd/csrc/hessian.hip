@@ -228,12 +228,24 @@ __device__ __forceinline__ void tile_epilogue(float* __restrict__ H, int64_t ldh
 constexpr int GROUP_MAX = 128;
 struct GroupArgs {
   static constexpr bool grouped = true;
+  static constexpr bool segmented = false;
   float* H[GROUP_MAX];
   const uint16_t* X[GROUP_MAX];
   int T[GROUP_MAX];
 };
 struct NoGroup {
   static constexpr bool grouped = false;
+  static constexpr bool segmented = false;
+};
+// One problem whose token rows lie in up to SEG_MAX separate buffers of seg_tokens rows each (a
+// multiple of the slab depth, so no slab straddles two buffers; the last one may hold fewer): the
+// calibration batches as the forward hook received them, without first copying them together.
+constexpr int SEG_MAX = 64;
+struct SegArgs {
+  static constexpr bool grouped = false;
+  static constexpr bool segmented = true;
+  const uint16_t* X[SEG_MAX];
+  int seg_tokens;
 };
 
 template <int BT, int DT, bool ALIGNED, bool FAST_EPI, class GRP>
@@ -310,9 +322,30 @@ __global__ __launch_bounds__(256) void hessian_syrk_kernel(float* __restrict__ H
 
   uint4 ra[RT], rb[RT];
   // RT token rows x 8 features of one panel (features col0 + g_i*8 ..) of the slab starting at t0
+  // Segmented input: address of token t0 of this chunk (t0 a slab start, uniform over the workgroup, so
+  // the table of buffers is indexed by a scalar).  A slab that does not exist maps to the last one.
+  auto slab_base = [&](int t0) -> const uint16_t* {
+    if constexpr (GRP::segmented) {
+      const int g = __builtin_amdgcn_readfirstlane(t_begin + min(t0, ((T - 1) / BK) * BK));
+      const int sg = g / grp.seg_tokens;
+      return grp.X[sg] + (int64_t)(g - sg * grp.seg_tokens) * ldx;
+    } else {
+      return X + (int64_t)t0 * ldx;
+    }
+  };
+  // row r of this thread's RT token rows of the slab at t0, features col0 + g_i*8 .. (+8)
+  auto load_row = [&](int t0, int r, int col0) -> uint4 {
+    if constexpr (GRP::segmented) {
+      const int t0c = min(t0, ((T - 1) / BK) * BK);
+      const int tt = min(t0 + g_t * RT + r, T - 1) - t0c;  // rows past T: the last row (masked by the caller)
+      return *(const uint4*)(slab_base(t0) + (int64_t)tt * ldx + min(col0 + g_i * 8, K - 8));
+    } else {
+      return load8<ALIGNED>(X, ldx, t0 + g_t * RT + r, col0 + g_i * 8, T, K);
+    }
+  };
   auto load_panel = [&](uint4* rg, int t0, int col0) {
 #pragma unroll
-    for (int r = 0; r < RT; ++r) rg[r] = load8<ALIGNED>(X, ldx, t0 + g_t * RT + r, col0 + g_i * 8, T, K);
+    for (int r = 0; r < RT; ++r) rg[r] = load_row(t0, r, col0);
   };
   // registers hold RT token rows x 8 features; LDS wants, per feature, RT consecutive tokens:
   // column c of the thread's 8 features goes out as one 16-byte (RT == 8) or 8-byte LDS write
@@ -368,8 +401,21 @@ __global__ __launch_bounds__(256) void hessian_syrk_kernel(float* __restrict__ H
   // Row pointers of the slab the steady state loads next (token t2 + g_t*RT, this thread's 8 features
   // of either panel): while that slab is a full one no clamping is needed and a load is one 64-bit
   // add away from them.
-  const uint16_t* pA = X + (int64_t)(2 * BK + g_t * RT) * ldx + min(i0 + g_i * 8, K - 8);
-  const uint16_t* pB = X + (int64_t)(2 * BK + g_t * RT) * ldx + min(j0 + g_i * 8, K - 8);
+  const uint16_t* pA = slab_base(2 * BK) + (int64_t)(g_t * RT) * ldx + min(i0 + g_i * 8, K - 8);
+  const uint16_t* pB = slab_base(2 * BK) + (int64_t)(g_t * RT) * ldx + min(j0 + g_i * 8, K - 8);
+  // after the iteration that loaded slab s+2: on to slab s+3, which may begin another buffer
+  auto advance = [&](int s_done) {
+    if constexpr (GRP::segmented) {
+      const int g = __builtin_amdgcn_readfirstlane(t_begin + (s_done + 3) * BK);
+      if (g % grp.seg_tokens == 0) {
+        pA = slab_base((s_done + 3) * BK) + (int64_t)(g_t * RT) * ldx + min(i0 + g_i * 8, K - 8);
+        pB = slab_base((s_done + 3) * BK) + (int64_t)(g_t * RT) * ldx + min(j0 + g_i * 8, K - 8);
+        return;
+      }
+    }
+    pA += (int64_t)BK * ldx;
+    pB += (int64_t)BK * ldx;
+  };
   auto compute = [&](unsigned char* curA, unsigned char* nxtA, int t2, auto store_tag, auto mask_tag,
                      auto direct_tag) {
     constexpr bool STORE = decltype(store_tag)::value;
@@ -402,8 +448,8 @@ __global__ __launch_bounds__(256) void hessian_syrk_kernel(float* __restrict__ H
               if (ks == 1) ra[r] = *(const uint4*)(pA + (int64_t)r * ldx);
               if (ks == 3) rb[r] = *(const uint4*)(pB + (int64_t)r * ldx);
             } else {
-              if (ks == 1) ra[r] = load8<ALIGNED>(X, ldx, t2 + g_t * RT + r, i0 + g_i * 8, T, K);
-              if (ks == 3) rb[r] = load8<ALIGNED>(X, ldx, t2 + g_t * RT + r, j0 + g_i * 8, T, K);
+              if (ks == 1) ra[r] = load_row(t2, r, i0);
+              if (ks == 3) rb[r] = load_row(t2, r, j0);
             }
           }
         }
@@ -458,15 +504,13 @@ __global__ __launch_bounds__(256) void hessian_syrk_kernel(float* __restrict__ H
     for (int i = 0; i < PACE_SLABS; ++i) {
       compute(smem + ((s + i) & 1) * 2 * PANEL, smem + ((s + i + 1) & 1) * 2 * PANEL, (s + i + 2) * BK,
               std::true_type{}, std::false_type{}, std::true_type{});
-      pA += (int64_t)BK * ldx;
-      pB += (int64_t)BK * ldx;
+      advance(s + i);
     }
   }
   for (; s < ndirect; ++s) {
     compute(smem + (s & 1) * 2 * PANEL, smem + ((s + 1) & 1) * 2 * PANEL, (s + 2) * BK, std::true_type{},
             std::false_type{}, std::true_type{});
-    pA += (int64_t)BK * ldx;
-    pB += (int64_t)BK * ldx;
+    advance(s);
   }
   for (; s + 2 < nslab; ++s)
     compute(smem + (s & 1) * 2 * PANEL, smem + ((s + 1) & 1) * 2 * PANEL, (s + 2) * BK, std::true_type{},
@@ -648,9 +692,9 @@ __global__ void zero_u32_kernel(unsigned* p, int n) {
 
 template <int BT, int DT>
 int launch(const Choice& c, float* H, int64_t ldh, const void* X, int64_t ldx, int64_t T, int64_t K, float alpha,
-           int flags, float* ws, unsigned* pace, hipStream_t st) {
+           int flags, float* ws, unsigned* pace, hipStream_t st, const SegArgs* segs = nullptr) {
   const int nb = (int)((K + BT - 1) / BT);
-  const bool aligned = (K % 8 == 0) && (ldx % 8 == 0) && (((uintptr_t)X & 15) == 0);
+  const bool aligned = segs || ((K % 8 == 0) && (ldx % 8 == 0) && (((uintptr_t)X & 15) == 0));
   const int sym = (flags & LLMC_HESSIAN_ASSUME_SYMMETRIC) ? 1 : 0;
   const int vec_ok = ((ldh & 3) == 0 && ((uintptr_t)H & 15) == 0) ? 1 : 0;
   constexpr int smem = 4 * BT * ROW_BYTES;
@@ -670,8 +714,18 @@ int launch(const Choice& c, float* H, int64_t ldh, const void* X, int64_t ldx, i
     hipLaunchKernelGGL(zero_u32_kernel, dim3(1), dim3(256), 0, st, pace, pace_groups * 32);
     LLMC_LAUNCH_STATUS();
   }
-  hipLaunchKernelGGL(kern, dim3(c.grid), dim3(256), smem, st, H, ldh, (const uint16_t*)X, ldx, (int)T,
-                     (int)K, alpha, sym, nb, c.plan, ws, NoGroup{}, pace);
+  if (segs) {
+    auto skern = fast ? hessian_syrk_kernel<BT, DT, true, true, SegArgs> : hessian_syrk_kernel<BT, DT, true, false, SegArgs>;
+    if (smem > 48 * 1024) {
+      hipError_t e = hipFuncSetAttribute((const void*)skern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+      if (e != hipSuccess) return 1000 + (int)e;
+    }
+    hipLaunchKernelGGL(skern, dim3(c.grid), dim3(256), smem, st, H, ldh, (const uint16_t*)nullptr, ldx, (int)T,
+                       (int)K, alpha, sym, nb, c.plan, ws, *segs, pace);
+  } else {
+    hipLaunchKernelGGL(kern, dim3(c.grid), dim3(256), smem, st, H, ldh, (const uint16_t*)X, ldx, (int)T,
+                       (int)K, alpha, sym, nb, c.plan, ws, NoGroup{}, pace);
+  }
   LLMC_LAUNCH_STATUS();
   if (c.nsplit_tiles > 0) {
     if (fast)
@@ -718,6 +772,43 @@ extern "C" int llmc_hessian_accumulate(float* H, int64_t ldh, const void* X, int
                        : launch<128, LLMC_BF16>(c, H, ldh, X, ldx, T, K, alpha, flags, ws, pace, st);
   return c.bt == 256 ? launch<256, LLMC_F16>(c, H, ldh, X, ldx, T, K, alpha, flags, ws, pace, st)
                      : launch<128, LLMC_F16>(c, H, ldh, X, ldx, T, K, alpha, flags, ws, pace, st);
+}
+
+extern "C" int llmc_hessian_accumulate_segments(float* H, int64_t ldh, const void* const* X, int32_t n_seg,
+                                                int64_t seg_tokens, int64_t last_tokens, int64_t ldx, int64_t K,
+                                                int32_t x_dtype, float alpha, int32_t flags, void* workspace,
+                                                int64_t workspace_bytes, void* stream) {
+  LLMC_CHECK_ARG(H != nullptr, 1);
+  LLMC_CHECK_ARG(K > 0 && K < (1 << 30) && K % 8 == 0 && ldh >= K, 8);
+  LLMC_CHECK_ARG(X != nullptr, 3);
+  LLMC_CHECK_ARG(n_seg >= 0 && n_seg <= SEG_MAX, 4);
+  if (n_seg == 0) return 0;
+  LLMC_CHECK_ARG(seg_tokens > 0 && seg_tokens % BK == 0 && seg_tokens < (1ll << 30), 5);
+  LLMC_CHECK_ARG(last_tokens > 0 && last_tokens <= seg_tokens, 6);
+  LLMC_CHECK_ARG(ldx >= K && ldx % 8 == 0, 7);
+  LLMC_CHECK_ARG(x_dtype == LLMC_BF16 || x_dtype == LLMC_F16, 9);
+  LLMC_CHECK_ARG(workspace_bytes >= 0 && (workspace_bytes == 0 || workspace != nullptr), 12);
+  LLMC_CHECK_ARG((((uintptr_t)workspace) & 15) == 0, 12);
+  const int64_t T = (int64_t)(n_seg - 1) * seg_tokens + last_tokens;
+  LLMC_CHECK_ARG(T < (1ll << 31), 5);
+  SegArgs segs;
+  for (int i = 0; i < SEG_MAX; ++i) {
+    const void* p = X[i < n_seg ? i : n_seg - 1];
+    LLMC_CHECK_ARG(p != nullptr && (((uintptr_t)p) & 15) == 0, 3);
+    segs.X[i] = (const uint16_t*)p;
+  }
+  segs.seg_tokens = (int)seg_tokens;
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t avail = workspace ? workspace_bytes : 0;
+  const bool pace_room = avail >= PACE_BYTES;
+  const Choice c = choose(T, K, pace_room ? avail - PACE_BYTES : avail);
+  unsigned* pace = pace_room ? (unsigned*)workspace : nullptr;
+  float* ws = (float*)((char*)workspace + (pace_room ? PACE_BYTES : 0));
+  if (x_dtype == LLMC_BF16)
+    return c.bt == 256 ? launch<256, LLMC_BF16>(c, H, ldh, nullptr, ldx, T, K, alpha, flags, ws, pace, st, &segs)
+                       : launch<128, LLMC_BF16>(c, H, ldh, nullptr, ldx, T, K, alpha, flags, ws, pace, st, &segs);
+  return c.bt == 256 ? launch<256, LLMC_F16>(c, H, ldh, nullptr, ldx, T, K, alpha, flags, ws, pace, st, &segs)
+                     : launch<128, LLMC_F16>(c, H, ldh, nullptr, ldx, T, K, alpha, flags, ws, pace, st, &segs);
 }
 
 template <int BT, int DT>

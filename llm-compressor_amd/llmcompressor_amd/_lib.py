@@ -52,6 +52,7 @@ SIGNATURES = {
     "llmc_version": [],
     "llmc_hessian_workspace_bytes": [_I64, _I64],
     "llmc_hessian_accumulate_grouped": [_P, _I64, _P, _I64, _P, _I32, _I64, _I32, _F32, _I32, _P],
+    "llmc_hessian_accumulate_segments": [_P, _I64, _P, _I32, _I64, _I64, _I64, _I64, _I32, _F32, _I32, _P, _I64, _P],
     "llmc_hessian_accumulate": [_P, _I64, _P, _I64, _I64, _I64, _I32, _F32, _I32, _P, _I64, _P],
     "llmc_minmax_groups": [_P, _I32, _I64, _I64, _I64, _I64, _P, _P, _P, _I64, _P],
     "llmc_minmax_blocks": [_P, _I32, _I64, _I64, _I64, _I32, _I32, _P, _P, _P],

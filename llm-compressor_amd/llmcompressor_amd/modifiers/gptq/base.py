@@ -56,6 +56,10 @@ class GPTQModifier(Modifier, QuantizationMixin):
         have the same Hessian; accumulate it once and hand each of them a copy when it is compressed.
         Results are identical; off by default, as the reference accumulates one Hessian per module.
 
+    :param stage_by_reference: while staging, keep references to the hook's input tensors instead of copying
+        them into a staging buffer, and hand the kernel the list of buffers.  Taken only for contiguous
+        bf16/f16 inputs whose token count is a multiple of 64; anything else is copied.  An input that is
+        modified in place before its batch is accumulated raises at the flush (tensor version check)
     :param compress_concurrency: how many modules of one ``compress_module_list`` call are quantised at the
         same time, each on its own HIP stream (1 = one after the other, the reference's behaviour)
 
@@ -73,11 +77,13 @@ class GPTQModifier(Modifier, QuantizationMixin):
     hessian_batch_tokens: int = 0
     share_identical_inputs: bool = False
     compress_concurrency: int = 4
+    stage_by_reference: bool = True
 
     _module_names: dict = PrivateAttr(default_factory=dict)
     _hessians: dict = PrivateAttr(default_factory=dict)
     _num_samples: dict = PrivateAttr(default_factory=dict)
     _staged: dict = PrivateAttr(default_factory=dict)
+    _held: dict = PrivateAttr(default_factory=dict)
     _group_pending: list | None = PrivateAttr(default=None)
     _leader: dict = PrivateAttr(default_factory=dict)  # follower module -> module whose Hessian it shares
     _recent_input: tuple | None = PrivateAttr(default=None)  # (tensor kept alive, its version, leader)
@@ -209,10 +215,30 @@ class GPTQModifier(Modifier, QuantizationMixin):
                                             assume_symmetric=True)
 
     # -- token staging (see the class docstring).  The hook runs once per Linear per batch, so it is
-    # kept to one device copy: the sample count is kept on the host until the flush.
+    # kept cheap: the sample count is kept on the host until the flush.
     def _stage(self, module, inp):
         k = inp.shape[-1]
         n = inp.numel() // k
+        samples = 1 if inp.ndim == 2 else inp.shape[0]  # accumulate_hessian counts a 2-D input as one sample
+        if self.stage_by_reference and inp.is_contiguous():
+            x = inp.view(n, k)
+            held = self._held.get(module)
+            fits = ops.segment_ok(x) and (held is None or not held[0] or (
+                held[0][0].shape == x.shape and held[0][0].dtype == x.dtype))
+            if fits:
+                st = self._staged.get(module)
+                if st is not None and st[1] > 0:
+                    self._flush(module)
+                if held is None:
+                    held = self._held[module] = [[], [], 0]  # views, (tensor, version at hook time), samples
+                held[0].append(x)
+                held[1].append((inp, inp._version))
+                held[2] += samples
+                if len(held[0]) * n >= self.hessian_batch_tokens or len(held[0]) >= ops.SEGMENTS_MAX:
+                    self._flush(module)
+                return
+            if held is not None and held[0]:
+                self._flush(module)
         st = self._staged.get(module)
         if st is None or st[0].shape[0] < n or st[0].dtype != inp.dtype or st[0].device != inp.device:
             if st is not None:
@@ -225,11 +251,21 @@ class GPTQModifier(Modifier, QuantizationMixin):
         used = st[1]
         st[0].narrow(0, used, n).copy_(inp.reshape(n, k))
         st[1] = used + n
-        st[2] += 1 if inp.ndim == 2 else inp.shape[0]  # accumulate_hessian counts a 2-D input as one sample
+        st[2] += samples
         if st[1] >= self.hessian_batch_tokens:
             self._flush(module)
 
     def _flush(self, module):
+        held = self._held.get(module)
+        if held is not None and held[0]:
+            for t, version in held[1]:
+                if t._version != version:
+                    raise RuntimeError(
+                        "GPTQModifier: an activation that was held for Hessian accumulation was modified in place "
+                        "after the forward hook saw it; set stage_by_reference=False for this model")
+            ops.hessian_accumulate_segments_(self._hessians[module], held[0], alpha=2.0, assume_symmetric=True)
+            self._num_samples[module] += held[2]
+            self._held[module] = [[], [], 0]
         st = self._staged.get(module)
         if st is None or st[1] == 0:
             return
@@ -253,6 +289,7 @@ class GPTQModifier(Modifier, QuantizationMixin):
         for module in module_list:  # pending activations go in on the calibration stream
             self._flush(module)
             self._staged.pop(module, None)
+            self._held.pop(module, None)
         jobs = list(module_list)
         workers = min(int(self.compress_concurrency), len(jobs))
         on_gpu = all(m.weight.is_cuda and self._hessians[m].is_cuda for m in jobs)
@@ -328,6 +365,7 @@ class GPTQModifier(Modifier, QuantizationMixin):
         self._hessians = dict()
         self._num_samples = dict()
         self._staged = dict()
+        self._held = dict()
         self._leader = dict()
         self._recent_input = None
         return True

@@ -51,6 +51,55 @@ def hessian_accumulate_(H: torch.Tensor, x: torch.Tensor, alpha: float = 2.0, as
     return H
 
 
+SEGMENTS_MAX = 64  # buffers per llmc_hessian_accumulate_segments launch
+
+
+def segment_ok(x: torch.Tensor) -> bool:
+    """Can `x` ([T, K] view) be one buffer of hessian_accumulate_segments_ (not the last one)?"""
+    return (x.is_cuda and x.ndim == 2 and x.dtype in (torch.bfloat16, torch.float16) and x.stride(1) == 1
+            and x.shape[0] > 0 and x.shape[0] % 64 == 0 and x.shape[1] % 8 == 0 and x.stride(0) % 8 == 0
+            and x.data_ptr() % 16 == 0)
+
+
+def hessian_accumulate_segments_(H: torch.Tensor, xs, alpha: float = 2.0, assume_symmetric: bool = True):
+    """H (fp32 [K,K], in place) += alpha * X^T X where X is the row-wise concatenation of xs, without
+    building it: xs[i] = [T_i, K] with one common row stride and dtype, T_i equal and a multiple of 64
+    for all but the last (which may hold fewer rows).  Bit-identical to hessian_accumulate_ on torch.cat(xs)."""
+    import ctypes
+
+    if not xs:
+        return H
+    x0 = xs[0]
+    _require_gpu(H, x0)
+    K = H.shape[0]
+    assert H.dtype == torch.float32 and H.shape == (K, K) and H.stride(1) == 1
+    seg = x0.shape[0] if len(xs) > 1 else -(-x0.shape[0] // 64) * 64
+    for i, x in enumerate(xs):
+        last = i == len(xs) - 1
+        if not (x.ndim == 2 and x.shape[1] == K and x.dtype == x0.dtype and x.stride(1) == 1
+                and x.stride(0) == x0.stride(0) and x.device == H.device and x.data_ptr() % 16 == 0
+                and (x.shape[0] == seg or (last and 0 < x.shape[0] <= seg))):
+            raise ValueError("hessian_accumulate_segments_: buffers need one width, dtype, row stride and row count "
+                             "(the last may be shorter) and 16-byte alignment")
+    if x0.dtype not in (torch.bfloat16, torch.float16):
+        raise TypeError(f"hessian_accumulate_segments_: unsupported activation dtype {x0.dtype}")
+    if seg % 64 or K % 8 or x0.stride(0) % 8:
+        raise ValueError("hessian_accumulate_segments_: rows per buffer must be a multiple of 64, K and the row "
+                         "stride multiples of 8")
+    with torch.cuda.device(H.device):
+        for b in range(0, len(xs), SEGMENTS_MAX):
+            part = xs[b:b + SEGMENTS_MAX]
+            T = seg * (len(part) - 1) + part[-1].shape[0]
+            xp = (ctypes.c_void_p * len(part))(*[x.data_ptr() for x in part])
+            nws = int(_lib.lib().llmc_hessian_workspace_bytes(T, K))
+            ws = _workspace(H.device, nws) if nws else None
+            rc = _lib.lib().llmc_hessian_accumulate_segments(
+                H.data_ptr(), H.stride(0), xp, len(part), seg, part[-1].shape[0], x0.stride(0), K, _DT[x0.dtype],
+                float(alpha), 1 if assume_symmetric else 0, _ptr(ws), nws, _stream(H))
+            _lib.check(rc, "llmc_hessian_accumulate_segments")
+    return H
+
+
 def hessian_accumulate_grouped_(Hs, xs, alpha: float = 2.0, assume_symmetric: bool = True):
     """One launch for many independent problems of the same width (the per-expert Hessians of an MoE
     layer): Hs[i] (fp32 [K,K], in place) += alpha * xs[i]^T xs[i] with xs[i] = [T_i, K], T_i >= 0.

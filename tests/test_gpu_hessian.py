@@ -169,3 +169,64 @@ def test_hessian_grouped_moe_shapes():
             assert _rel(Hs[e].cpu(), Hc) < TOL
         else:
             assert torch.count_nonzero(Hs[e]) == 0
+
+
+@pytest.mark.parametrize("K,seg,nseg,last,dtype", [
+    (1024, 64, 5, 64, torch.bfloat16),      # every slab in a buffer of its own
+    (1288, 128, 7, 100, torch.bfloat16),    # ragged last buffer, K not a multiple of the tile
+    (4096, 256, 9, 256, torch.float16),     # tiles cut along the tokens: chunk starts inside a buffer list
+    (2304, 192, 64, 1, torch.bfloat16),     # the maximum number of buffers, a single row in the last
+    (512, 2048, 1, 777, torch.bfloat16),    # one buffer only
+])
+def test_hessian_segments_match_concatenation(K, seg, nseg, last, dtype):
+    """llmc_hessian_accumulate_segments on separately allocated buffers is bit-identical to
+    llmc_hessian_accumulate on their concatenation (same plan, same summation order)."""
+    from llmcompressor_amd import ops
+
+    torch.manual_seed(K + seg)
+    xs = []
+    for i in range(nseg):
+        rows = last if i == nseg - 1 else seg
+        # separate allocations in shuffled address order, padded rows (row stride > K)
+        buf = torch.randn(rows, K + 8, device="cuda").to(dtype)
+        xs.append(buf[:, :K])
+        _ = torch.empty(1000 * (i % 3 + 1), device="cuda")
+    cat = torch.cat([x.contiguous() for x in xs], 0)
+    ref = 2 * (cat.double().t() @ cat.double())
+    H0 = torch.randn(K, K, device="cuda")
+    H0 = H0 + H0.t()
+    Ha, Hb = H0.clone(), H0.clone()
+    ops.hessian_accumulate_(Ha, cat)
+    ops.hessian_accumulate_segments_(Hb, xs)
+    assert torch.equal(Ha, Hb)
+    assert _rel(Hb - H0, ref) < 2e-5
+    assert torch.equal(Hb, Hb.t())
+    # more buffers than one launch takes: split by the wrapper
+    if nseg == 64:
+        Hc = H0.clone()
+        ops.hessian_accumulate_segments_(Hc, xs[:-1] + [xs[0]] * 3 + [xs[-1]])
+        cat2 = torch.cat([cat[:-last], xs[0], xs[0], xs[0], cat[-last:]], 0)
+        assert _rel(Hc - H0, 2 * (cat2.double().t() @ cat2.double())) < 2e-5
+    with pytest.raises(ValueError):
+        ops.hessian_accumulate_segments_(Hb, [xs[0][:63], xs[0][:63]])  # rows per buffer not a multiple of 64
+
+
+def test_hessian_segments_full_size():
+    """K = 14336, 32 buffers of 2048 tokens (one staged launch of the bench): bit-identical to the
+    concatenated launch."""
+    from llmcompressor_amd import ops
+
+    torch.manual_seed(3)
+    K, seg, nseg = 14336, 2048, 32
+    big = torch.randn(nseg + 1, seg, K, device="cuda").bfloat16()
+    xs = [big[i] for i in range(nseg)]
+    xs = [xs[(7 * i) % nseg] for i in range(nseg)]  # buffers out of address order
+    cat = torch.cat(xs, 0)
+    Ha = torch.zeros(K, K, device="cuda")
+    Hb = torch.zeros(K, K, device="cuda")
+    ops.hessian_accumulate_(Ha, cat)
+    ops.hessian_accumulate_segments_(Hb, xs)
+    assert torch.equal(Ha, Hb)
+    rows = torch.tensor([0, 255, 256, 7000, 14335], device="cuda")
+    ref = 2 * (cat[:, rows].double().t() @ cat.double())
+    assert _rel(Hb[rows], ref) < TOL

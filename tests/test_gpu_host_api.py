@@ -674,3 +674,75 @@ def test_gptq_concurrent_module_compression_is_identical():
         base.quantize_weight = raw
         active_session().reset()
     torch.cuda.synchronize()
+
+
+def test_gptq_stage_by_reference_matches_copy_staging_and_detects_inplace_writes():
+    """stage_by_reference hands the kernel the hook's buffers instead of a staged copy: same launches, same
+    token order, bit-identical parameters; an activation modified in place before its flush raises."""
+    from llmcompressor_amd import ops
+    from llmcompressor_amd.core import LifecycleCallbacks, active_session
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+
+    class Wrap(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            g = torch.Generator().manual_seed(5)
+            lin = torch.nn.Linear(256, 96, bias=False, dtype=torch.bfloat16)
+            lin.weight.data = (torch.randn(96, 256, generator=g) * 0.05).bfloat16()
+            self.layers = torch.nn.ModuleList([lin])
+
+    # 128-token batches are taken by reference; the 100-token one is not a multiple of 64 and is copied
+    sizes = [128, 128, 128, 100, 128, 128]
+    xs = [torch.randn(1, n, 256, generator=torch.Generator().manual_seed(i)).bfloat16().to(DEV)
+          for i, n in enumerate(sizes)]
+    results = []
+    for by_ref in (False, True):
+        model = Wrap().to(DEV)
+        calls = {"copy": 0, "segments": 0}
+        raw_a, raw_s = ops.hessian_accumulate_, ops.hessian_accumulate_segments_
+        ops.hessian_accumulate_ = lambda H, x, **kw: (calls.__setitem__("copy", calls["copy"] + 1), raw_a(H, x, **kw))[1]
+        ops.hessian_accumulate_segments_ = lambda H, x, **kw: (
+            calls.__setitem__("segments", calls["segments"] + 1), raw_s(H, x, **kw))[1]
+        try:
+            mod = GPTQModifier(targets="Linear", hessian_batch_tokens=256, stage_by_reference=by_ref,
+                               config_groups={"g": dict(targets=["Linear"], weights=dict(
+                                   num_bits=4, strategy="group", group_size=32))})
+            session = active_session()
+            session.reset()
+            session.initialize(model=model, recipe=mod)
+            LifecycleCallbacks.calibration_start()
+            with torch.no_grad():
+                for x in xs:
+                    model.layers[0](x)
+            lin = model.layers[0]
+            LifecycleCallbacks.sequential_epoch_end(modules=list(model.modules()))
+            LifecycleCallbacks.calibration_end()
+            session.finalize()
+        finally:
+            ops.hessian_accumulate_, ops.hessian_accumulate_segments_ = raw_a, raw_s
+        results.append((dict(calls), {n: p.detach().clone() for n, p in model.named_parameters()}))
+    (c_copy, w_copy), (c_ref, w_ref) = results
+    assert c_copy["segments"] == 0 and c_copy["copy"] >= 3
+    assert c_ref["segments"] >= 2 and c_ref["copy"] >= 1
+    for n in w_copy:
+        # the two modes group the batches into launches differently (fp32 summation order of H), so a
+        # rare weight may land on the neighbouring code; scales and zero points do not depend on H
+        if n.endswith("weight"):
+            assert (w_copy[n] != w_ref[n]).float().mean().item() < 1e-3, n
+        else:
+            assert torch.equal(w_copy[n], w_ref[n]), n
+
+    model = Wrap().to(DEV)
+    mod = GPTQModifier(targets="Linear", hessian_batch_tokens=1024, config_groups={"g": dict(
+        targets=["Linear"], weights=dict(num_bits=4, strategy="group", group_size=32))})
+    session = active_session()
+    session.reset()
+    session.initialize(model=model, recipe=mod)
+    LifecycleCallbacks.calibration_start()
+    x = xs[0].clone()
+    with torch.no_grad():
+        model.layers[0](x)
+        x.mul_(2.0)  # the held activation changes before its batch is accumulated
+    with pytest.raises(RuntimeError, match="modified in place"):
+        LifecycleCallbacks.sequential_epoch_end(modules=list(model.modules()))
+    active_session().reset()
