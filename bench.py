@@ -47,7 +47,7 @@ GROUP = 128
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch of the dominant kernel from FETCH_SIZE / WRITE_SIZE counter runs scaled by a
 # 1 GiB copy (profiles/hessian_syrk_k14336_t65536_hbm_traffic.md), keyed by tokens per launch
-DOMINANT_TRAFFIC_BYTES = {16384: 7.30e9, 65536: 29.6e9}
+DOMINANT_TRAFFIC_BYTES = {65536: 30.3e9}
 
 
 def cpu_baseline(tokens: int):
@@ -197,15 +197,17 @@ def main():
     if a.probe_dominant:
         from llmcompressor_amd import ops
 
-        x = torch.randn(a.stage_tokens or a.tokens, INTER, device=dev).bfloat16()
+        # the launch the bench's hook path makes: the batches of one staging period, each in its own buffer
+        nseg = max(1, (a.stage_tokens or a.tokens) // a.tokens)
+        x = torch.randn(nseg, a.tokens, INTER, device=dev).bfloat16()
         H = torch.zeros(INTER, INTER, device=dev)
         src = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
         dst = torch.empty_like(src)
         for _ in range(a.probe_dominant):
-            ops.hessian_accumulate_(H, x)
+            ops.hessian_accumulate_segments_(H, [x[i] for i in range(nseg)])
             dst.copy_(src)
         torch.cuda.synchronize()
-        print(f"probe: {a.probe_dominant} x hessian [{x.shape[0]}x{INTER}] + {a.probe_dominant} x copy of {src.numel() * 4} bytes")
+        print(f"probe: {a.probe_dominant} x hessian [{nseg}x{a.tokens}x{INTER}] + {a.probe_dominant} x copy of {src.numel() * 4} bytes")
         return
     B, T = a.batches, a.tokens
     gen = torch.Generator(device=dev).manual_seed(0)
