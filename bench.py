@@ -162,6 +162,53 @@ def probe_bandwidth():
         print(f"| {name} | {us:.1f} | {gbs:.0f} | {frac * 100:.1f}% |")
 
 
+def probe_sparsegpt():
+    """SparseGPT on the layer's three Linear shapes (Hessian from 8192 tokens): event-timed factorisation and
+    pruning loop per Linear, unstructured 50 % and 2:4, and the CPU oracle on the 4096 x 4096 one.  Prints a table."""
+    import torch
+
+    from llmcompressor_amd import ops
+    from oracle import sparsegpt as S
+
+    def timed(fn, n=3):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n
+
+    print("| Linear (rows x columns) | factorisation ms | unstructured 50% ms | 2:4 ms | zeros (unstructured) |")
+    print("|---|---|---|---|---|")
+    keep = None
+    for R, K in ((HIDDEN, HIDDEN), (INTER, HIDDEN), (HIDDEN, INTER)):
+        torch.manual_seed(0)
+        x = torch.randn(8192, K, device="cuda").bfloat16()
+        W = (torch.randn(R, K, device="cuda") * 0.02).bfloat16()
+        H0 = torch.zeros(K, K, device="cuda")
+        ops.hessian_accumulate_(H0, x)
+        t_f = timed(lambda: ops.gptq_hinv_(H0.clone(), None, divisor=4.0))
+        U, dead, _ = ops.gptq_hinv_(H0.clone(), None, divisor=4.0)
+        t_u = timed(lambda: ops.sparsegpt_sparsify(W, U, 0.5, dead=dead))
+        t_s = timed(lambda: ops.sparsegpt_sparsify(W, U, 0.5, prune_n=2, prune_m=4, dead=dead))
+        Q, _ = ops.sparsegpt_sparsify(W, U, 0.5, dead=dead)
+        print(f"| {R} x {K} | {t_f:.2f} | {t_u:.2f} | {t_s:.2f} | {(Q == 0).float().mean().item():.4f} |")
+        if keep is None:
+            keep = (x.cpu(), W.cpu())
+    x, W = keep
+    torch.set_num_threads(min(os.cpu_count() or 1, 16))
+    H, n = S.make_empty_hessian(HIDDEN), 0
+    for chunk in x.reshape(4, 2048, HIDDEN):
+        H, n = S.accumulate_hessian(chunk, H, n)
+    t0 = time.perf_counter()
+    S.sparsify_weight(W, H, 0.5)
+    print(f"\nCPU oracle, 4096 x 4096 unstructured 50% (factorisation + loop, {torch.get_num_threads()} threads): "
+          f"{(time.perf_counter() - t0) * 1e3:.0f} ms")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -177,6 +224,8 @@ def main():
                     "tokens) and N plain copies of a 1 GiB buffer (the known-size kernel the HBM counters are scaled by)")
     ap.add_argument("--probe-bandwidth", action="store_true",
                     help="print achieved GB/s of the observer / quantize / pack kernels instead of the bench line")
+    ap.add_argument("--probe-sparsegpt", action="store_true",
+                    help="print SparseGPT timings per Linear shape instead of the bench line")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU figure is produced)", file=sys.stderr)
@@ -193,6 +242,9 @@ def main():
     torch.cuda.set_device(dev)
     if a.probe_bandwidth:
         probe_bandwidth()
+        return
+    if a.probe_sparsegpt:
+        probe_sparsegpt()
         return
     if a.probe_dominant:
         from llmcompressor_amd import ops

@@ -235,6 +235,27 @@ int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R, int64_t K
                        void* out_weight, int64_t ldo, float* loss_out, void* workspace,
                        int64_t workspace_bytes, void* stream);
 
+/* ---- SparseGPT (a "next" row: the same Hessian / Cholesky / column-loop skeleton) ----------
+ * Replaces the loop of sparsify_weight (src/llmcompressor/modifiers/pruning/sparsegpt/
+ * sgpt_sparsify.py:125-213); the factor U comes from llmc_gptq_hinv (:97-118 are the same
+ * dead-column / damping / Cholesky chain; pass divisor = number of samples to turn the summed
+ * Hessian into the reference's running average of :48-53).
+ *   prune_n == 0: unstructured.  Per block of `blocksize` columns the elements whose saliency
+ *     w^2 / U[c][c]^2 is <= the int(R * count * sparsity)-th smallest of the block are zeroed
+ *     (:141-156; an exact radix selection replaces the sort).  32 <= blocksize <= 128.
+ *   prune_n : prune_m (m in {2, 4, 8}, blocksize % m == 0): when the column loop reaches a group
+ *     of m columns, the n least salient of its current values are zeroed (:165-176).
+ *   preserve_sparsity_mask: weights that are zero on entry stay zero, are not compensated by the
+ *     trailing updates (:193-198) and count towards the target (:143-151).  The caller checks
+ *     that the existing sparsity does not exceed the target (:127-133 raises).
+ * out_weight receives the pruned weight in w_dtype, *loss_out the sum of (w - q)^2 / d^2 / 2. */
+int64_t llmc_sparsegpt_workspace_bytes(int64_t R, int64_t K);
+int llmc_sparsegpt_sparsify(const void* weight, int32_t w_dtype, int64_t R, int64_t K, int64_t ldw,
+                            const float* U, int64_t ldu, const uint8_t* dead, double sparsity,
+                            int32_t prune_n, int32_t prune_m, int32_t blocksize,
+                            int32_t preserve_sparsity_mask, void* out_weight, int64_t ldo,
+                            float* loss_out, void* workspace, int64_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

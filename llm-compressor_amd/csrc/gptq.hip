@@ -162,7 +162,379 @@ __global__ __launch_bounds__(256) void zero_f32_kernel(float* p, int64_t n) {
 
 inline int64_t align256(int64_t b) { return (b + 255) / 256 * 256; }
 
+// ---------------------------------------------------------------------------------------------
+// SparseGPT: the same blocked column loop with a pruning mask in place of the quantiser.
+//
+// Unstructured pruning takes, per block of columns, the elements whose saliency w^2 / d^2
+// (d = diagonal of the inverse-Hessian factor) is not above the k-th smallest of the whole
+// [R x count] block, k = int(numel * sparsity).  That order statistic is found exactly by a
+// three-pass radix selection on the float bit patterns (11 + 11 + 10 bits; saliencies are
+// non-negative, so their bit patterns order like the values): every pass builds a histogram
+// of the next digit over the elements that match the digits found so far.  The histograms of
+// a block live in their own slice of the workspace, so nothing is cleared between blocks.
+// N:M pruning (M in {2, 4, 8}: a group lies inside one lane's 8 columns) picks, when the loop
+// reaches a group, the N least salient of its current values.
+constexpr int SG_BINS = 2048;
+constexpr int SG_HIST_WORDS = 3 * SG_BINS + 64;  // three histograms + the masked-element count
+constexpr int SG_MIN_BLOCK = 32;                 // narrowest unstructured block (sizes the histogram slices)
+
+struct SgptParams {
+  float* Wf;
+  int R, K;
+  const float* U;
+  int64_t ldu;
+  int i1, count;
+  const uint8_t* mask;   // [R,K] bytes, 1 = was zero before pruning (preserve mode), or NULL
+  unsigned* hist;        // this block's SG_HIST_WORDS words
+  unsigned k;            // rank of the threshold element (0-based) in the ascending order
+  int prune_n, prune_m;  // 0:0 = unstructured
+  float* E;
+  int ldE;
+  float* loss_rows;
+};
+
+__device__ __forceinline__ float sgpt_saliency(float w, float d, bool masked) {
+  const float num = masked ? 0.f : __fmul_rn(w, w);
+  return __fdiv_rn(num, __fmul_rn(d, d));
+}
+
+// First bin whose running total exceeds k; k becomes the rank inside that bin.  All 256 threads of the
+// workgroup take part; `scratch` holds 258 words.
+__device__ __forceinline__ unsigned sgpt_find_bin(const unsigned* __restrict__ hist, int nbins, unsigned& k,
+                                                  unsigned* scratch) {
+  const int tid = threadIdx.x;
+  const int per = nbins / 256;
+  unsigned local = 0;
+  for (int b = 0; b < per; ++b) local += hist[tid * per + b];
+  scratch[tid] = local;
+  __syncthreads();
+  if (tid == 0) {
+    unsigned run = 0;
+    int t = 0;
+    for (; t < 255; ++t) {
+      if (run + scratch[t] > k) break;
+      run += scratch[t];
+    }
+    unsigned bin = (unsigned)(t * per);
+    for (int b = 0; b < per - 1; ++b) {
+      const unsigned h = hist[t * per + b];
+      if (run + h > k) break;
+      run += h;
+      ++bin;
+    }
+    scratch[256] = bin;
+    scratch[257] = k - run;
+  }
+  __syncthreads();
+  const unsigned bin = scratch[256];
+  k = scratch[257];
+  __syncthreads();
+  return bin;
+}
+
+template <int PASS>
+__global__ __launch_bounds__(256) void sgpt_hist_kernel(SgptParams p) {
+  __shared__ unsigned lh[SG_BINS];
+  __shared__ unsigned scratch[258];
+  __shared__ unsigned nmasked;
+  const int tid = threadIdx.x;
+  for (int b = tid; b < SG_BINS; b += 256) lh[b] = 0;
+  if (tid == 0) nmasked = 0;
+  unsigned k = p.k, prefix = 0;
+  if (PASS >= 1) prefix = sgpt_find_bin(p.hist, SG_BINS, k, scratch);
+  if (PASS >= 2) prefix = (prefix << 11) | sgpt_find_bin(p.hist + SG_BINS, SG_BINS, k, scratch);
+  __syncthreads();
+  const int64_t n = (int64_t)p.R * p.count;
+  for (int64_t e = (int64_t)blockIdx.x * 256 + tid; e < n; e += (int64_t)gridDim.x * 256) {
+    const int r = (int)(e / p.count), c = (int)(e % p.count);
+    const int col = p.i1 + c;
+    const bool masked = p.mask && p.mask[(int64_t)r * p.K + col];
+    const float t = sgpt_saliency(p.Wf[(int64_t)r * p.K + col], p.U[(int64_t)col * p.ldu + col], masked);
+    const unsigned bits = __float_as_uint(t);
+    if (PASS == 0) {
+      atomicAdd(&lh[bits >> 21], 1u);
+      if (masked) atomicAdd(&nmasked, 1u);
+    } else if (PASS == 1) {
+      if ((bits >> 21) == prefix) atomicAdd(&lh[(bits >> 10) & 2047u], 1u);
+    } else {
+      if ((bits >> 10) == prefix) atomicAdd(&lh[bits & 1023u], 1u);
+    }
+  }
+  __syncthreads();
+  unsigned* gh = p.hist + PASS * SG_BINS;
+  for (int b = tid; b < SG_BINS; b += 256)
+    if (lh[b]) atomicAdd(&gh[b], lh[b]);
+  if (PASS == 0 && tid == 0 && nmasked) atomicAdd(&p.hist[3 * SG_BINS], nmasked);
+}
+
+template <bool NM>
+__global__ __launch_bounds__(256) void sgpt_block_kernel(SgptParams p) {
+  extern __shared__ __attribute__((aligned(16))) float Hs[];  // [GB][GB], zero outside the upper triangle
+  __shared__ unsigned scratch[258];
+  const int tid = threadIdx.x;
+  for (int e = tid; e < GB * GB; e += 256) {
+    const int i = e / GB, c = e % GB;
+    Hs[e] = (c >= i && c < p.count) ? p.U[(int64_t)(p.i1 + i) * p.ldu + p.i1 + c] : 0.f;
+  }
+  // unstructured: the block's threshold from its three histograms
+  float thresh = 0.f;
+  bool use_thresh = false;
+  if (!NM) {
+    unsigned k = p.k;
+    unsigned bits = sgpt_find_bin(p.hist, SG_BINS, k, scratch);
+    bits = (bits << 11) | sgpt_find_bin(p.hist + SG_BINS, SG_BINS, k, scratch);
+    bits = (bits << 10) | sgpt_find_bin(p.hist + 2 * SG_BINS, 1024, k, scratch);
+    thresh = __uint_as_float(bits);
+    // with a mask to preserve, the mask is only extended when the target asks for more zeros than it holds
+    use_thresh = p.mask == nullptr || p.k > p.hist[3 * SG_BINS];
+  }
+  __syncthreads();
+  const int tl = tid % TEAM;
+  const int row = blockIdx.x * ROWS_PER_WG + tid / TEAM;
+  const bool live = row < p.R;
+
+  float w[CPL], qv[CPL], ev[CPL];
+  unsigned pruned = 0, masked = 0;  // bit e: column tl*CPL + e of the block
+#pragma unroll
+  for (int e = 0; e < CPL; ++e) {
+    const int cb = tl * CPL + e;
+    w[e] = 0.f;
+    qv[e] = 0.f;
+    ev[e] = 0.f;
+    if (live && cb < p.count) {
+      const int c = p.i1 + cb;
+      w[e] = p.Wf[(int64_t)row * p.K + c];
+      if (p.mask && p.mask[(int64_t)row * p.K + c]) masked |= 1u << e;
+    }
+  }
+  __syncthreads();  // Hs complete
+  if (!NM) {
+    if (use_thresh) {
+#pragma unroll
+      for (int e = 0; e < CPL; ++e) {
+        const int cb = tl * CPL + e;
+        if (cb < p.count && sgpt_saliency(w[e], Hs[cb * GB + cb], (masked >> e) & 1u) <= thresh) pruned |= 1u << e;
+      }
+    } else {
+      pruned = masked;
+    }
+  } else {
+    pruned = masked;
+  }
+
+  float loss = 0.f;
+  for (int li = 0; li < TEAM; ++li) {
+    if (li * CPL >= p.count) break;
+#pragma unroll
+    for (int e = 0; e < CPL; ++e) {
+      const int i = li * CPL + e;
+      if (i < p.count) {  // uniform across the workgroup
+        if (NM && (e % p.prune_m) == 0 && tl == li) {
+          // the N least salient of the group's current values (ties: the lower column first)
+          float t[CPL];
+#pragma unroll
+          for (int j = 0; j < CPL; ++j) {
+            const int cb = tl * CPL + j;
+            t[j] = sgpt_saliency(w[j], Hs[(cb < GB ? cb : 0) * GB + (cb < GB ? cb : 0)], (masked >> j) & 1u);
+          }
+#pragma unroll
+          for (int j = 0; j < CPL; ++j) {
+            if (j >= e && j < e + p.prune_m && tl * CPL + j < p.count) {
+              int rank = 0;
+#pragma unroll
+              for (int l = 0; l < CPL; ++l)
+                if (l >= e && l < e + p.prune_m && tl * CPL + l < p.count && (t[l] < t[j] || (t[l] == t[j] && l < j)))
+                  ++rank;
+              if (rank < p.prune_n) pruned |= 1u << j;
+            }
+          }
+        }
+        const float wv = __shfl(w[e], li, TEAM);
+        const unsigned flags = __shfl((int)pruned, li, TEAM);
+        const float q = ((flags >> e) & 1u) ? 0.f : wv;
+        const float d = Hs[i * GB + i];
+        const float diff = __fsub_rn(wv, q);
+        const float err = diff / d;
+        loss += err * err;  // (w-q)^2 / d^2
+        const float4 h0 = *(const float4*)&Hs[i * GB + tl * CPL];
+        const float4 h1 = *(const float4*)&Hs[i * GB + tl * CPL + 4];
+        w[0] = __fsub_rn(w[0], __fmul_rn(err, h0.x));
+        w[1] = __fsub_rn(w[1], __fmul_rn(err, h0.y));
+        w[2] = __fsub_rn(w[2], __fmul_rn(err, h0.z));
+        w[3] = __fsub_rn(w[3], __fmul_rn(err, h0.w));
+        w[4] = __fsub_rn(w[4], __fmul_rn(err, h1.x));
+        w[5] = __fsub_rn(w[5], __fmul_rn(err, h1.y));
+        w[6] = __fsub_rn(w[6], __fmul_rn(err, h1.z));
+        w[7] = __fsub_rn(w[7], __fmul_rn(err, h1.w));
+        if (tl == li) {
+          qv[e] = q;
+          ev[e] = err;
+        }
+      }
+    }
+  }
+
+  if (live) {
+#pragma unroll
+    for (int e = 0; e < CPL; ++e) {
+      const int cb = tl * CPL + e;
+      if (cb < p.count) p.Wf[(int64_t)row * p.K + p.i1 + cb] = qv[e];
+      p.E[(int64_t)row * p.ldE + cb] = ev[e];
+    }
+    if (tl == 0) p.loss_rows[row] += loss * 0.5f;
+  }
+}
+
+// mask[r,c] = (Wf[r,c] == 0): the sparsity pattern to preserve
+__global__ __launch_bounds__(256) void sgpt_mask_kernel(const float* __restrict__ Wf, int64_t n, uint8_t* mask) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) mask[i] = Wf[i] == 0.f ? 1 : 0;
+}
+
+// the trailing updates leave preserved zeros alone: put them back after an unmasked product
+__global__ __launch_bounds__(256) void sgpt_rezero_kernel(float* __restrict__ Wf, const uint8_t* __restrict__ mask,
+                                                          int K, int c0, int c1) {
+  const int c = c0 + blockIdx.x * 256 + threadIdx.x;
+  const int r = blockIdx.y;
+  if (c < c1 && mask[(int64_t)r * K + c]) Wf[(int64_t)r * K + c] = 0.f;
+}
+
+__global__ __launch_bounds__(256) void zero_u32_words_kernel(unsigned* p, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = 0u;
+}
+
 }  // namespace
+
+extern "C" int64_t llmc_sparsegpt_workspace_bytes(int64_t R, int64_t K) {
+  const int64_t slices = (K + SG_MIN_BLOCK - 1) / SG_MIN_BLOCK;
+  return align256(R * K * 4) + align256(R * GROUP * GB * 4) + align256(R * 4) +
+         align256(slices * SG_HIST_WORDS * 4) + align256(R * K);
+}
+
+extern "C" int llmc_sparsegpt_sparsify(const void* weight, int32_t w_dtype, int64_t R, int64_t K, int64_t ldw,
+                                       const float* U, int64_t ldu, const uint8_t* dead, double sparsity,
+                                       int32_t prune_n, int32_t prune_m, int32_t blocksize,
+                                       int32_t preserve_sparsity_mask, void* out_weight, int64_t ldo,
+                                       float* loss_out, void* workspace, int64_t workspace_bytes, void* stream) {
+  LLMC_CHECK_ARG(weight != nullptr, 1);
+  LLMC_CHECK_ARG(w_dtype >= 0 && w_dtype <= 2, 2);
+  LLMC_CHECK_ARG(R > 0 && R < (1ll << 24), 3);
+  LLMC_CHECK_ARG(K > 0 && K < (1ll << 31), 4);
+  LLMC_CHECK_ARG(ldw >= K, 5);
+  LLMC_CHECK_ARG(U != nullptr && ldu >= K, 6);
+  const bool nm = prune_n != 0;
+  LLMC_CHECK_ARG(nm || (sparsity >= 0.0 && sparsity < 1.0), 9);
+  LLMC_CHECK_ARG(!nm || ((prune_m == 2 || prune_m == 4 || prune_m == 8) && prune_n > 0 && prune_n <= prune_m), 11);
+  // the block width decides which elements compete for the unstructured threshold, so it is not
+  // clamped the way the quantiser's is
+  LLMC_CHECK_ARG(blocksize > 0 && blocksize <= GB && (nm ? blocksize % prune_m == 0 : blocksize >= SG_MIN_BLOCK), 12);
+  LLMC_CHECK_ARG(out_weight != nullptr && ldo >= K, 14);
+  LLMC_CHECK_ARG(workspace != nullptr && (((uintptr_t)workspace) & 255) == 0, 17);
+  LLMC_CHECK_ARG(workspace_bytes >= llmc_sparsegpt_workspace_bytes(R, K), 18);
+  hipStream_t st = (hipStream_t)stream;
+  const int bs = blocksize;
+  const int64_t nblocks = (K + bs - 1) / bs;
+
+  char* wp = (char*)workspace;
+  float* Wf = (float*)wp; wp += align256(R * K * 4);
+  float* E = (float*)wp; wp += align256(R * GROUP * GB * 4);
+  float* loss_rows = (float*)wp; wp += align256(R * 4);
+  unsigned* hist = (unsigned*)wp; wp += align256(((K + SG_MIN_BLOCK - 1) / SG_MIN_BLOCK) * SG_HIST_WORDS * 4);
+  uint8_t* mask = preserve_sparsity_mask ? (uint8_t*)wp : nullptr;
+
+  dim3 grid2((unsigned)((K + 255) / 256), (unsigned)R);
+#define LLMC_PREP(DT) \
+  hipLaunchKernelGGL((gptq_prepare_w_kernel<DT>), grid2, dim3(256), 0, st, weight, ldw, (int)R, (int)K, \
+                     (const int32_t*)nullptr, dead, Wf)
+  if (w_dtype == LLMC_BF16) LLMC_PREP(LLMC_BF16);
+  else if (w_dtype == LLMC_F16) LLMC_PREP(LLMC_F16);
+  else LLMC_PREP(LLMC_F32);
+#undef LLMC_PREP
+  LLMC_LAUNCH_STATUS();
+  hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((R + 255) / 256)), dim3(256), 0, st, loss_rows, R);
+  LLMC_LAUNCH_STATUS();
+  if (!nm) {
+    const int64_t words = nblocks * SG_HIST_WORDS;
+    hipLaunchKernelGGL(zero_u32_words_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, st, hist, words);
+    LLMC_LAUNCH_STATUS();
+  }
+  if (mask) {
+    hipLaunchKernelGGL(sgpt_mask_kernel, dim3((unsigned)((R * K + 255) / 256)), dim3(256), 0, st, Wf, R * K, mask);
+    LLMC_LAUNCH_STATUS();
+  }
+
+  SgptParams p;
+  p.Wf = Wf; p.R = (int)R; p.K = (int)K; p.U = U; p.ldu = ldu; p.mask = mask;
+  p.prune_n = prune_n; p.prune_m = nm ? prune_m : 1; p.loss_rows = loss_rows;
+  const int smem = GB * GB * 4;
+  void (*kern)(SgptParams) = nm ? sgpt_block_kernel<true> : sgpt_block_kernel<false>;
+  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+  if (e != hipSuccess) return 1000 + (int)e;
+  const unsigned wgs = (unsigned)((R + ROWS_PER_WG - 1) / ROWS_PER_WG);
+  const int ldE = GROUP * GB;
+  p.ldE = ldE;
+  auto rezero = [&](int64_t c0, int64_t c1) {  // preserved zeros in columns [c0, c1) back to zero
+    if (!mask || c0 >= c1) return;
+    hipLaunchKernelGGL(sgpt_rezero_kernel, dim3((unsigned)((c1 - c0 + 255) / 256), (unsigned)R), dim3(256), 0, st, Wf,
+                       mask, (int)K, (int)c0, (int)c1);
+  };
+  // the same two-level lazy updates as the quantiser's loop
+  int64_t blk = 0;
+  for (int64_t g0 = 0; g0 < K; g0 += (int64_t)GROUP * bs) {
+    const int64_t gend = (g0 + (int64_t)GROUP * bs) < K ? g0 + (int64_t)GROUP * bs : K;
+    for (int64_t i1 = g0; i1 < gend; i1 += bs, ++blk) {
+      const int count = (int)((gend - i1) < bs ? (gend - i1) : bs);
+      p.i1 = (int)i1;
+      p.count = count;
+      p.E = E + (i1 - g0);
+      p.hist = hist + blk * SG_HIST_WORDS;
+      p.k = (unsigned)((double)(R * count) * sparsity);
+      if (!nm) {
+        const unsigned hw = (unsigned)((R * count + 256 * 16 - 1) / (256 * 16));
+        hipLaunchKernelGGL(sgpt_hist_kernel<0>, dim3(hw), dim3(256), 0, st, p);
+        hipLaunchKernelGGL(sgpt_hist_kernel<1>, dim3(hw), dim3(256), 0, st, p);
+        hipLaunchKernelGGL(sgpt_hist_kernel<2>, dim3(hw), dim3(256), 0, st, p);
+        LLMC_LAUNCH_STATUS();
+      }
+      hipLaunchKernelGGL(kern, dim3(wgs), dim3(256), smem, st, p);
+      LLMC_LAUNCH_STATUS();
+      const int64_t i2 = i1 + count;
+      if (i2 < gend) {
+        GemmF32 g = {};
+        g.A = p.E; g.lda = ldE; g.B = U + i1 * ldu + i2; g.ldb = ldu; g.C = Wf + i2; g.ldc = K;
+        g.M = (int)R; g.N = (int)(gend - i2); g.Kc = count; g.alpha = -1.f; g.beta = 1.f; g.batch = 1;
+        const int rc = llmc_gemm_f32(g, st);
+        if (rc) return rc;
+        rezero(i2, gend);
+        LLMC_LAUNCH_STATUS();
+      }
+    }
+    if (gend < K) {
+      GemmF32 g = {};
+      g.A = E; g.lda = ldE; g.B = U + g0 * ldu + gend; g.ldb = ldu; g.C = Wf + gend; g.ldc = K;
+      g.M = (int)R; g.N = (int)(K - gend); g.Kc = (int)(gend - g0); g.alpha = -1.f; g.beta = 1.f; g.batch = 1;
+      const int rc = llmc_gemm_f32(g, st);
+      if (rc) return rc;
+      rezero(gend, K);
+      LLMC_LAUNCH_STATUS();
+    }
+  }
+
+#define LLMC_FIN(DT) \
+  hipLaunchKernelGGL((gptq_finalize_kernel<DT>), grid2, dim3(256), 0, st, Wf, (int)R, (int)K, \
+                     (const int32_t*)nullptr, out_weight, ldo)
+  if (w_dtype == LLMC_BF16) LLMC_FIN(LLMC_BF16);
+  else if (w_dtype == LLMC_F16) LLMC_FIN(LLMC_F16);
+  else LLMC_FIN(LLMC_F32);
+#undef LLMC_FIN
+  LLMC_LAUNCH_STATUS();
+  if (loss_out) {
+    hipLaunchKernelGGL(sum_rows_kernel, dim3(1), dim3(256), 0, st, loss_rows, (int)R, loss_out);
+    LLMC_LAUNCH_STATUS();
+  }
+  return 0;
+}
 
 extern "C" int64_t llmc_gptq_quantize_workspace_bytes(int64_t R, int64_t K) {
   return align256(R * K * 4) + align256(R * GROUP * GB * 4) + align256(R * 4);

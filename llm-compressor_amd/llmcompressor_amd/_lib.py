@@ -52,6 +52,9 @@ SIGNATURES = {
     "llmc_version": [],
     "llmc_hessian_workspace_bytes": [_I64, _I64],
     "llmc_hessian_accumulate_grouped": [_P, _I64, _P, _I64, _P, _I32, _I64, _I32, _F32, _I32, _P],
+    "llmc_sparsegpt_workspace_bytes": [_I64, _I64],
+    "llmc_sparsegpt_sparsify": [_P, _I32, _I64, _I64, _I64, _P, _I64, _P, ctypes.c_double, _I32, _I32, _I32, _I32, _P,
+                                _I64, _P, _P, _I64, _P],
     "llmc_hessian_accumulate_segments": [_P, _I64, _P, _I32, _I64, _I64, _I64, _I64, _I32, _F32, _I32, _P, _I64, _P],
     "llmc_hessian_accumulate": [_P, _I64, _P, _I64, _I64, _I64, _I32, _F32, _I32, _P, _I64, _P],
     "llmc_minmax_groups": [_P, _I32, _I64, _I64, _I64, _I64, _P, _P, _P, _I64, _P],
@@ -88,6 +91,7 @@ RESTYPES = {
     "llmc_gptq_hinv_workspace_bytes": ctypes.c_int64,
     "llmc_mse_workspace_bytes": ctypes.c_int64,
     "llmc_gptq_quantize_workspace_bytes": ctypes.c_int64,
+    "llmc_sparsegpt_workspace_bytes": ctypes.c_int64,
 }
 SIGNATURES["llmc_minmax_workspace_bytes"] = []
 

@@ -16,9 +16,11 @@ class ModifierFactory:
     @staticmethod
     def refresh():
         from .gptq.base import GPTQModifier
+        from .pruning.sparsegpt.base import SparseGPTModifier
         from .quantization.quantization.base import QuantizationModifier
 
-        ModifierFactory._main_registry = {c.__name__: c for c in (GPTQModifier, QuantizationModifier)}
+        ModifierFactory._main_registry = {c.__name__: c for c in (GPTQModifier, QuantizationModifier,
+                                                                  SparseGPTModifier)}
         ModifierFactory._loaded = True
 
     @staticmethod

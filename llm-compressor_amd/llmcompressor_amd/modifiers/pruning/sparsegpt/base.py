@@ -1,0 +1,156 @@
+"""SparseGPTModifier (reference: modifiers/pruning/sparsegpt/base.py:21-173).
+
+Same fields and lifecycle as the reference.  As for GPTQ, the forward hook stages calibration batches and
+accumulates several of them with one Hessian launch (``hessian_batch_tokens``, ``stage_by_reference``), and the
+modules of one ``compress_modules`` call are pruned concurrently on separate streams
+(``compress_concurrency``); neither changes the result beyond fp32 summation order.
+"""
+from __future__ import annotations
+
+import logging
+import threading
+
+import torch
+from pydantic import PrivateAttr
+
+from ....core import State
+from ....quantization import update_offload_parameter
+from ....utils.metric_logging import CompressionLogger
+from ...utils.hessian_staging import HessianStagingMixin
+from .sgpt_base import SparsityModifierBase
+from .sgpt_sparsify import accumulate_hessian, make_empty_hessian, sparsify_weight
+
+logger = logging.getLogger("llmcompressor_amd")
+
+__all__ = ["SparseGPTModifier"]
+
+
+class SparseGPTModifier(SparsityModifierBase, HessianStagingMixin):
+    """One-shot SparseGPT (https://arxiv.org/abs/2301.00774).
+
+    :param sparsity: sparsity to compress the model to (or one value per target layer)
+    :param sparsity_profile: 'owl' for Outlier Weighed Layerwise Sparsity
+    :param mask_structure: "N:M" (M in {2, 4, 8} in this build), "0:0" = unstructured
+    :param block_size: columns compressed in one pass (unstructured: also the set the threshold is taken over)
+    :param dampening_frac: dampening applied to H, as a fraction of the diagonal mean
+    :param preserve_sparsity_mask: keep (and extend) the sparsity pattern the model already has
+    :param offload_hessians: keep Hessians on the CPU between hook calls
+    :param hessian_batch_tokens / stage_by_reference / compress_concurrency: scheduling only, see GPTQModifier
+    """
+
+    block_size: int = 128
+    dampening_frac: float | None = 0.01
+    preserve_sparsity_mask: bool = False
+    offload_hessians: bool = False
+    hessian_batch_tokens: int = 0
+    stage_by_reference: bool = True
+    compress_concurrency: int = 4
+
+    _num_samples: dict = PrivateAttr(default_factory=dict)
+    _hessians: dict = PrivateAttr(default_factory=dict)
+    _staged: dict = PrivateAttr(default_factory=dict)
+    _held: dict = PrivateAttr(default_factory=dict)
+    _streams: list = PrivateAttr(default_factory=list)
+
+    def calibrate_module(self, module: torch.nn.Module, args: tuple[torch.Tensor, ...], _output: torch.Tensor):
+        """Forward hook: accumulate the Hessian of the module's input."""
+        inp = args[0]
+        if module not in self._num_samples:
+            device = inp.device if inp.is_cuda else module.weight.device
+            self._hessians[module] = make_empty_hessian(module, device="cpu" if self.offload_hessians else device)
+            self._num_samples[module] = 0
+        if self.hessian_batch_tokens > 0 and not self.offload_hessians and isinstance(module, torch.nn.Linear):
+            self._stage(module, inp)
+            return
+        if self.offload_hessians:
+            self._hessians[module] = self._hessians[module].to(device=inp.device)
+        self._hessians[module], self._num_samples[module] = accumulate_hessian(
+            inp, module, self._hessians[module], self._num_samples[module])
+        if self.offload_hessians:
+            self._hessians[module] = self._hessians[module].to(device="cpu")
+
+    def compress_modules(self):
+        """Sparsify the modules that have been calibrated."""
+        jobs = list(self._num_samples.keys())
+        for module in jobs:
+            self._flush(module)
+            self._staged.pop(module, None)
+            self._held.pop(module, None)
+        workers = min(int(self.compress_concurrency), len(jobs))
+        if workers <= 1 or self.offload_hessians or not all(m.weight.is_cuda for m in jobs):
+            for module in jobs:
+                self._compress_one(module)
+            return
+        # independent modules, each a long chain of small dependent kernels: several at once, one host thread
+        # and one HIP stream each, most expensive first (same scheme as GPTQModifier.compress_module_list)
+        device = jobs[0].weight.device
+        jobs.sort(key=lambda m: -(float(m.weight.shape[1]) ** 3 + float(m.weight.shape[0]) * m.weight.shape[1] ** 2))
+        main = torch.cuda.current_stream(device)
+        ready = main.record_event()
+        while len(self._streams) < workers:
+            self._streams.append(torch.cuda.Stream(device=device))
+        lock = threading.Lock()
+        errors = []
+
+        def worker(stream):
+            try:
+                with torch.cuda.device(device), torch.cuda.stream(stream):
+                    stream.wait_event(ready)
+                    while True:
+                        with lock:
+                            if not jobs or errors:
+                                return
+                            module = jobs.pop(0)
+                        self._compress_one(module, produced_on=stream, consumed_on=main)
+            except BaseException as err:  # re-raised on the calling thread
+                errors.append(err)
+
+        threads = [threading.Thread(target=worker, args=(s,), daemon=True) for s in self._streams[:workers]]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        for s in self._streams[:workers]:
+            main.wait_stream(s)
+        if errors:
+            raise errors[0]
+
+    def _compress_one(self, module, produced_on=None, consumed_on=None):
+        name = self._module_names[module]
+        sparsity = self._module_sparsities[module]
+        num_samples = self._num_samples[module]
+        logger.info(f"Sparsifying {name} using {num_samples} samples")
+        if self.offload_hessians:
+            self._hessians[module] = self._hessians[module].to(device=module.weight.device)
+        if produced_on is not None:  # allocated on the calibration stream, last read on this one
+            self._hessians[module].record_stream(produced_on)
+        with torch.no_grad(), CompressionLogger(module) as comp_logger:
+            loss, sparsified_weight = sparsify_weight(
+                module=module,
+                hessians_dict=self._hessians,
+                sparsity=sparsity,
+                prune_n=self._prune_n,
+                prune_m=self._prune_m,
+                block_size=self.block_size,
+                dampening_frac=self.dampening_frac,
+                preserve_sparsity_mask=self.preserve_sparsity_mask,
+                num_samples=float(num_samples),
+            )
+            comp_logger.set_results(name="SGPT", loss=loss)
+        if consumed_on is not None and sparsified_weight.is_cuda:
+            sparsified_weight.record_stream(consumed_on)
+        update_offload_parameter(module, "weight", sparsified_weight)
+        del self._num_samples[module]  # the Hessian was consumed by sparsify_weight
+
+    def on_finalize(self, state: State, **kwargs) -> bool:
+        if not self.ended_:
+            self.on_end(state, None)
+        if len(self._num_samples) > 0:
+            raise ValueError(f"Failed to compress {len(self._num_samples)} modules")
+        self._hessians = dict()
+        self._num_samples = dict()
+        self._staged = dict()
+        self._held = dict()
+        self._module_names = dict()
+        self._module_sparsities = dict()
+        return True

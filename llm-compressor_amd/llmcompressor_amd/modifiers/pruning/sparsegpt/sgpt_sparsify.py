@@ -1,0 +1,90 @@
+"""SparseGPT numerics behind the reference's function seams
+(modifiers/pruning/sparsegpt/sgpt_sparsify.py).
+
+``make_empty_hessian`` (:10-16), ``accumulate_hessian`` (:19-56) and ``sparsify_weight`` (:59-213) keep their
+names, arguments and return values.  One difference in representation: the reference keeps the Hessian as a
+running average ``H*n/(n+b) + (2/(n+b)) X^T X``; here H is the plain sum ``2 X^T X`` (one MFMA launch, no
+rescaling pass over the [K,K] matrix per batch) and the division by the sample count is folded into the first
+pass of the factorisation -- the same matrix up to fp32 rounding.  ``sparsify_weight`` therefore takes the
+sample count (``num_samples``, default 1 = the Hessian is already an average).
+"""
+from __future__ import annotations
+
+import logging
+
+import torch
+
+from .... import ops
+
+logger = logging.getLogger("llmcompressor_amd")
+
+SGPT_PRECISION = torch.float32
+
+__all__ = ["make_empty_hessian", "accumulate_hessian", "sparsify_weight", "sparsify_weight_tensors"]
+
+
+def make_empty_hessian(module: torch.nn.Module, device: torch.device | None = None) -> torch.Tensor:
+    weight = module.weight
+    device = device if device is not None else weight.device
+    return torch.zeros((weight.shape[1], weight.shape[1]), device=device, dtype=SGPT_PRECISION)
+
+
+def accumulate_hessian(inp: torch.Tensor, module: torch.nn.Module, H: torch.Tensor,
+                       num_samples: int) -> tuple[torch.Tensor, int]:
+    """H += 2 X^T X in place (a sum, see the module docstring); num_samples += batch entries."""
+    inp = inp.to(device=H.device)
+    if len(inp.shape) == 2:
+        inp = inp.unsqueeze(0)
+    num_added = inp.shape[0]
+    if isinstance(module, torch.nn.Conv2d):
+        unfold = torch.nn.Unfold(module.kernel_size, dilation=module.dilation, padding=module.padding,
+                                 stride=module.stride)
+        inp = unfold(inp).permute([1, 0, 2]).flatten(1).t()
+    else:
+        inp = inp.reshape((-1, inp.shape[-1]))
+    num_samples += num_added
+    if inp.dtype not in (torch.bfloat16, torch.float16):
+        raise TypeError("accumulate_hessian: activations must be bf16 or fp16 in this build")
+    if inp.shape[0] > 0:
+        ops.hessian_accumulate_(H, inp.contiguous(), alpha=2.0, assume_symmetric=True)
+    return H, num_samples
+
+
+def sparsify_weight_tensors(weight: torch.Tensor, hessian: torch.Tensor, sparsity: float, prune_n: int, prune_m: int,
+                            block_size: int, dampening_frac: float, preserve_sparsity_mask: bool,
+                            num_samples: float = 1.0):
+    """sparsify_weight on bare tensors: weight [R, K] (Linear layout), hessian [K, K] = sum of 2 X^T X over
+    ``num_samples`` samples.  Returns (loss tensor [1], pruned weight in weight.dtype, info tensor)."""
+    W = weight if weight.is_contiguous() else weight.contiguous()
+    if preserve_sparsity_mask:
+        current = (W == 0).sum() / W.numel()
+        if float(current) > sparsity:
+            raise ValueError("The target sparsity is lower than the sparsity of the base model. Please retry "
+                             "after turning preserve_sparsity_mask=False")
+    U, dead, info = ops.gptq_hinv_(hessian, None, divisor=float(num_samples), percdamp=dampening_frac)
+    Q, loss = ops.sparsegpt_sparsify(W, U, sparsity, prune_n=prune_n, prune_m=prune_m, dead=dead,
+                                     blocksize=block_size, preserve_sparsity_mask=preserve_sparsity_mask)
+    return loss, Q, info
+
+
+def sparsify_weight(module: torch.nn.Module, hessians_dict: dict, sparsity: float, prune_n: int, prune_m: int,
+                    block_size: int, dampening_frac: float, preserve_sparsity_mask: bool,
+                    num_samples: float = 1.0) -> tuple[float, torch.Tensor]:
+    """Prune ``module.weight`` to the target sparsity; consumes ``hessians_dict[module]``."""
+    final_shape, final_dtype = module.weight.shape, module.weight.dtype
+    W = module.weight.data
+    H = hessians_dict.pop(module)
+    conv1d = module.__class__.__name__ == "Conv1D"
+    if isinstance(module, torch.nn.Conv2d):
+        W = W.flatten(1)
+    elif conv1d:
+        W = W.t()
+    loss, Q, info = sparsify_weight_tensors(W, H, sparsity, prune_n, prune_m, block_size, dampening_frac,
+                                            preserve_sparsity_mask, num_samples)
+    if int(info.item()) != 0:
+        logger.warning("Failed to invert hessian due to numerical instability. Consider increasing "
+                       "SparseGPTModifier.dampening_frac, increasing the number of calibration samples, or "
+                       "shuffling the calibration dataset")
+    if conv1d:
+        Q = Q.t()
+    return loss.item(), Q.reshape(final_shape).to(final_dtype)

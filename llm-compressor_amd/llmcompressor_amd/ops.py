@@ -355,6 +355,33 @@ def gptq_quantize(weight, U, scale, zero_point, fmt: int, bits: int, row_div: in
     return out, loss
 
 
+def sparsegpt_sparsify(weight, U, sparsity: float, prune_n: int = 0, prune_m: int = 0, dead=None,
+                       blocksize: int = 128, preserve_sparsity_mask: bool = False):
+    """The SparseGPT column loop on the factor U of gptq_hinv_.  Returns (pruned weight in weight.dtype,
+    loss fp32 [1])."""
+    _require_gpu(weight, U)
+    assert weight.ndim == 2 and weight.stride(1) == 1 and U.stride(1) == 1
+    R, K = weight.shape
+    if prune_n:
+        if prune_m not in (2, 4, 8) or not 0 < prune_n <= prune_m or blocksize % prune_m or blocksize > 128:
+            raise ValueError(f"sparsegpt_sparsify: unsupported mask structure {prune_n}:{prune_m} for block size "
+                             f"{blocksize} (M must be 2, 4 or 8 and divide the block size, which is at most 128)")
+    elif not (0.0 <= sparsity < 1.0) or not 32 <= blocksize <= 128:
+        raise ValueError(f"sparsegpt_sparsify: sparsity {sparsity} must lie in [0, 1) and the block size "
+                         f"{blocksize} in [32, 128]")
+    out = torch.empty((R, K), dtype=weight.dtype, device=weight.device)
+    loss = torch.empty(1, dtype=torch.float32, device=weight.device)
+    nbytes = _lib.lib().llmc_sparsegpt_workspace_bytes(R, K)
+    ws = _workspace(weight.device, nbytes)
+    with torch.cuda.device(weight.device):
+        rc = _lib.lib().llmc_sparsegpt_sparsify(
+            weight.data_ptr(), _dt(weight), R, K, weight.stride(0), U.data_ptr(), U.stride(0), _ptr(dead),
+            float(sparsity), int(prune_n), int(prune_m), int(blocksize), 1 if preserve_sparsity_mask else 0,
+            out.data_ptr(), K, loss.data_ptr(), ws.data_ptr(), ws.numel(), _stream(weight))
+    _lib.check(rc, "llmc_sparsegpt_sparsify")
+    return out, loss
+
+
 def _mse_common(maxshrink, grid, patience, norm, expand):
     steps = int(maxshrink * grid)
     if steps > 256:

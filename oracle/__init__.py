@@ -29,4 +29,10 @@ closed form or invariant says so here):
   specs): MXFP4 E8M0 scale generation, ``pack_to_int32`` / ``pack_fp4_to_uint8``
   byte layouts, fp8 storage, per-token dynamic FP8 scales, zero-scale epsilon
   substitution.
+* parity unpinned by reference vectors, pinned by mathematics only:
+  ``sparsegpt.accumulate_hessian`` / ``sparsegpt.sparsify_weight`` (the
+  reference's SparseGPT tests need hub models; see ``tests/test_oracle_sparsegpt.py``:
+  closed-form running-average Hessian, diagonal-Hessian == saliency pruning,
+  exact zero counts, un-blocked fp64 textbook elimination, the OBS step against
+  a constrained least-squares solve).
 """

@@ -746,3 +746,59 @@ def test_gptq_stage_by_reference_matches_copy_staging_and_detects_inplace_writes
     with pytest.raises(RuntimeError, match="modified in place"):
         LifecycleCallbacks.sequential_epoch_end(modules=list(model.modules()))
     active_session().reset()
+
+
+@pytest.mark.parametrize("structure,staging", [("0:0", 0), ("2:4", 256), ("0:0", 256)])
+def test_sparsegpt_modifier_matches_oracle(structure, staging):
+    """SparseGPTModifier through the lifecycle events: hooks accumulate the Hessian, the epoch end prunes.
+    The first Linear (whose inputs are the calibration batches themselves) is checked against the oracle."""
+    from oracle import sparsegpt as S
+
+    from llmcompressor_amd.core import LifecycleCallbacks, active_session
+    from llmcompressor_amd.modifiers.factory import ModifierFactory
+
+    class Wrap(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            g = torch.Generator().manual_seed(21)
+            a = torch.nn.Linear(128, 192, bias=False, dtype=torch.bfloat16)
+            b = torch.nn.Linear(192, 64, bias=False, dtype=torch.bfloat16)
+            a.weight.data = (torch.randn(192, 128, generator=g) * 0.05).bfloat16()
+            b.weight.data = (torch.randn(64, 192, generator=g) * 0.05).bfloat16()
+            self.layers = torch.nn.ModuleList([torch.nn.Sequential(a, b)])
+            self.lm_head = torch.nn.Linear(64, 32, bias=False, dtype=torch.bfloat16)
+
+    xs = [torch.randn(2, 64, 128, generator=torch.Generator().manual_seed(i)).bfloat16() for i in range(4)]
+    model = Wrap().to(DEV)
+    W0 = model.layers[0][0].weight.detach().cpu().clone()
+    head0 = model.lm_head.weight.detach().clone()
+    mod = ModifierFactory.create("SparseGPTModifier", sparsity=0.5, mask_structure=structure, block_size=64,
+                                 targets=["Linear"], ignore=["re:.*lm_head"], hessian_batch_tokens=staging)
+    session = active_session()
+    session.reset()
+    session.initialize(model=model, recipe=mod)
+    LifecycleCallbacks.calibration_start()
+    with torch.no_grad():
+        for x in xs:
+            model.lm_head(model.layers[0](x.to(DEV)))
+    LifecycleCallbacks.sequential_epoch_end(modules=list(model.modules()))
+    LifecycleCallbacks.calibration_end()
+    session.finalize()
+    torch.cuda.synchronize()
+
+    H, n = S.make_empty_hessian(128), 0
+    for x in xs:
+        H, n = S.accumulate_hessian(x, H, n)
+    assert n == 8
+    pn, pm = (int(v) for v in structure.split(":"))
+    _, Qo = S.sparsify_weight(W0, H, 0.5, pn, pm, 64, 0.01, False)
+    Qg = model.layers[0][0].weight.detach().cpu()
+    assert ((Qg == 0) == (Qo == 0)).float().mean().item() >= 0.999
+    both = (Qg != 0) & (Qo != 0)
+    assert ((Qg.double() - Qo.double())[both].norm() / Qo.double()[both].norm()).item() < 6e-3
+    Q1 = model.layers[0][1].weight.detach()
+    if pn:
+        assert torch.all((Q1 == 0).reshape(64, 192 // 4, 4).sum(-1) == 2)
+    else:
+        assert abs((Q1 == 0).float().mean().item() - 0.5) < 0.01
+    assert torch.equal(model.lm_head.weight.detach(), head0)  # ignored

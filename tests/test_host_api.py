@@ -347,3 +347,45 @@ def test_intermediates_cache_interface():
     off = IntermediatesCache.empty(1, offload_device="cpu")
     off.update(0, {"h": torch.ones(4)})
     assert off.batch_intermediates[0]["h"].value.device.type == "cpu" and off.fetch(0)["h"].device.type == "cpu"
+
+
+def test_sparsegpt_modifier_fields_and_validation():
+    """SparseGPTModifier keeps the reference's fields, validators and registry name
+    (modifiers/pruning/sparsegpt/{base,sgpt_base}.py)."""
+    import warnings
+
+    from llmcompressor_amd.modifiers.factory import ModifierFactory
+    from llmcompressor_amd.modifiers.pruning import SparseGPTModifier
+
+    m = SparseGPTModifier(sparsity=0.5, mask_structure="2:4")
+    assert (m._prune_n, m._prune_m) == (2, 4) and m.block_size == 128 and m.dampening_frac == 0.01
+    assert m.targets == ["Linear"] and m.requires_calibration_data and not m.preserve_sparsity_mask
+    assert (SparseGPTModifier(sparsity=0.3)._prune_n, SparseGPTModifier(sparsity=0.3)._prune_m) == (0, 0)
+    with pytest.raises(ValueError):
+        SparseGPTModifier(sparsity=0.5, sparsity_profile="owl")  # owl needs owl_m and owl_lmbda too
+    with pytest.raises(ValueError):
+        SparseGPTModifier(sparsity=0.5, sparsity_profile="other")
+    ok = SparseGPTModifier(sparsity=0.5, sparsity_profile="OWL", owl_m=5, owl_lmbda=0.05)
+    assert ok.sparsity_profile == "owl"
+    with warnings.catch_warnings(record=True) as w:
+        warnings.simplefilter("always")
+        assert SparseGPTModifier(sparsity=0.5, sequential_update=False).sequential_update is True
+        assert any(issubclass(x.category, DeprecationWarning) for x in w)
+    made = ModifierFactory.create("SparseGPTModifier", sparsity=0.7, mask_structure="4:8", dampening_frac=0.001)
+    assert isinstance(made, SparseGPTModifier) and made._prune_m == 8
+
+    from llmcompressor_amd.recipe import Recipe
+
+    recipe = Recipe.create_instance("""
+    test_stage:
+      obcq_modifiers:
+        SparseGPTModifier:
+          sparsity: 0.5
+          mask_structure: "2:4"
+          dampening_frac: 0.001
+          block_size: 128
+          targets: ['Linear']
+          ignore: ['re:.*lm_head']
+    """)
+    (mod,) = recipe.modifiers
+    assert isinstance(mod, SparseGPTModifier) and mod.ignore == ["re:.*lm_head"] and mod._prune_n == 2
