@@ -144,6 +144,23 @@ int llmc_mse_observe_blocks(const void* x, int32_t dtype, int64_t R, int64_t K, 
                             int32_t patience, float norm, float expand, void* min_out, void* max_out,
                             void* workspace, int64_t workspace_bytes, void* stream);
 
+/* Importance-weighted search (a "next" row: observers/imatrix.py).
+ *   llmc_sumsq_accumulate: sum[c] += sum_t x[t][c]^2 in fp32 -- the forward-pre hook's
+ *     token_sum = x.float().pow(2).sum(leading dims) (imatrix.py:93-111) without the fp32 copy of x.
+ *   llmc_imatrix_observe_groups: _grid_search (imatrix.py:255-328) on weight [R,K] in groups of `group`
+ *     columns (group = K: per channel): candidates i = 0..steps-1 with p = 1 - i/grid, the error
+ *     |fq(x) - x|^norm formed and summed in fp32 and multiplied by importance[column] (fp32 [K],
+ *     already normalised to mean 1; NULL = uniform), global early stop after `patience` candidates
+ *     without any improvement (0 = never).  Workspace as llmc_mse_workspace_bytes(#groups). */
+int64_t llmc_sumsq_workspace_bytes(int64_t K);
+int llmc_sumsq_accumulate(const void* x, int32_t dtype, int64_t T, int64_t K, int64_t ldx, float* sum,
+                          void* workspace, int64_t workspace_bytes, void* stream);
+int llmc_imatrix_observe_groups(const void* x, int32_t dtype, int64_t R, int64_t K, int64_t ldw,
+                                int64_t group, int32_t fmt, int32_t num_bits, int32_t symmetric,
+                                int32_t scale_mode, int32_t steps, double grid, int32_t patience,
+                                float norm, float expand, const float* importance, void* min_out,
+                                void* max_out, void* workspace, int64_t workspace_bytes, void* stream);
+
 /* ---- a12/a16: qparams ------------------------------------------------------
  * llmc_absmax_accumulate + llmc_generate_gparam replace Observer.get_global_scale()
  * (src/llmcompressor/observers/base.py:78-96; CT generate_gparam): absmax_inout

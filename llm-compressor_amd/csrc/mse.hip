@@ -30,6 +30,10 @@ struct MseParams {
   void* max0;        // [N]
   uint64_t* masks;   // [N][MASK_WORDS]
   uint64_t* flags;   // [MASK_WORDS] zero-initialised
+  // importance-weighted variant (observers/imatrix.py:255-328): the error |fq(x) - x|^norm is formed and
+  // summed in fp32 (values are quantised in dt as before) and weighted per input channel
+  int err32;
+  const float* imp;  // [K] weights, or NULL for uniform
 };
 
 __device__ __forceinline__ float step_factor(int i, double grid) { return (float)(1.0 - (double)i / grid); }
@@ -43,6 +47,18 @@ __device__ __forceinline__ float elem_error(float x, float s, float zp, bool has
   // `norm` arrives already rounded to dt: the eager pow converts its scalar exponent to the tensor dtype
   const float pw = norm == 2.0f ? a * a : powf(a, norm);
   return round_rt(pw, dt);
+}
+
+// fp32 error of the importance-weighted search: fq(x) in dt, then (fq - x), abs, pow in fp32; the
+// eager pow multiplies for exponents 2 and 3
+__device__ __forceinline__ float elem_error32(float x, float s, float zp, bool has_zp, int dt, const QFormat& f,
+                                              float norm) {
+  const float q = quantize_value(x, s, zp, has_zp, dt, f);
+  const float dq = dequantize_value(q, s, zp, has_zp, dt);
+  const float a = fabsf(__fsub_rn(dq, x));
+  if (norm == 2.0f) return __fmul_rn(a, a);
+  if (norm == 3.0f) return __fmul_rn(__fmul_rn(a, a), a);
+  return powf(a, norm);
 }
 
 __device__ __forceinline__ void unpack8(uint4 v, int dt, float* o) {
@@ -103,6 +119,15 @@ __global__ __launch_bounds__(256) void mse_team_kernel(MseParams p, int64_t ngro
   mn = round_rt(mn * p.expand, p.dt);
   mx = round_rt(mx * p.expand, p.dt);
   float best = p.dt == LLMC_BF16 ? 3.3895313892515355e38f : p.dt == LLMC_F16 ? 65504.0f : 3.4028234663852886e38f;
+  if (p.err32) best = 3.4028234663852886e38f;
+  float wt[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) wt[j] = 1.f;
+  if (p.err32 && p.imp && live) {
+    const int64_t gi = grp % ng;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) wt[j] = p.imp[gi * g + (int64_t)sub * 8 + j];
+  }
   uint64_t mask[MASK_WORDS];
 #pragma unroll
   for (int wd = 0; wd < MASK_WORDS; ++wd) mask[wd] = 0ull;
@@ -113,10 +138,18 @@ __global__ __launch_bounds__(256) void mse_team_kernel(MseParams p, int64_t ngro
     int e;
     qparams_from_minmax(smin, smax, p.dt, f, p.symmetric != 0, p.scale_mode, 1.f, &s, &zp, &e);
     float err = 0.f;
+    if (p.err32) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) err += elem_error(xv[j], s, zp, !p.symmetric, p.dt, f, p.norm);
+      for (int j = 0; j < 8; ++j) {
+        const float ej = elem_error32(xv[j], s, zp, !p.symmetric, p.dt, f, p.norm);
+        err += p.imp ? __fmul_rn(ej, wt[j]) : ej;
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) err += elem_error(xv[j], s, zp, !p.symmetric, p.dt, f, p.norm);
+    }
     for (int o = L >> 1; o > 0; o >>= 1) err += __shfl_xor(err, o, 64);
-    err = round_rt(err, p.dt);
+    if (!p.err32) err = round_rt(err, p.dt);
     if (err < best) {
       best = err;
 #pragma unroll
@@ -322,6 +355,7 @@ struct GenericLayout {
   int64_t n0, G, s0, s1;
   int R, K, bh, bw, nbc;
   int64_t ldw;
+  int64_t ng;  // mode 0, weighted search: groups per row (column of element e of group n1 = (n1 % ng)*G + e % G)
 };
 
 __device__ __forceinline__ float generic_load(const void* x, int dt, const GenericLayout& l, int64_t n1, int64_t e) {
@@ -364,6 +398,7 @@ __global__ __launch_bounds__(256) void mse_generic_kernel(MseParams p, GenericLa
   mn = round_rt(mn * p.expand, p.dt);
   mx = round_rt(mx * p.expand, p.dt);
   float best = p.dt == LLMC_BF16 ? 3.3895313892515355e38f : p.dt == LLMC_F16 ? 65504.0f : 3.4028234663852886e38f;
+  if (p.err32) best = 3.4028234663852886e38f;
   uint64_t mask[MASK_WORDS];
 #pragma unroll
   for (int wd = 0; wd < MASK_WORDS; ++wd) mask[wd] = 0ull;
@@ -374,9 +409,17 @@ __global__ __launch_bounds__(256) void mse_generic_kernel(MseParams p, GenericLa
     int e_;
     qparams_from_minmax(smin, smax, p.dt, f, p.symmetric != 0, p.scale_mode, 1.f, &s, &zp, &e_);
     float err = 0.f;
-    for (int64_t e = threadIdx.x; e < total; e += 256)
-      err += elem_error(generic_load(p.x, p.dt, l, n1, e), s, zp, !p.symmetric, p.dt, f, p.norm);
-    err = round_rt(block_sum(err, sh), p.dt);
+    if (p.err32) {
+      for (int64_t e = threadIdx.x; e < total; e += 256) {
+        const float ej = elem_error32(generic_load(p.x, p.dt, l, n1, e), s, zp, !p.symmetric, p.dt, f, p.norm);
+        err += p.imp ? __fmul_rn(ej, p.imp[(n1 % l.ng) * l.G + e % l.G]) : ej;
+      }
+      err = block_sum(err, sh);
+    } else {
+      for (int64_t e = threadIdx.x; e < total; e += 256)
+        err += elem_error(generic_load(p.x, p.dt, l, n1, e), s, zp, !p.symmetric, p.dt, f, p.norm);
+      err = round_rt(block_sum(err, sh), p.dt);
+    }
     if (err < best) {
       best = err;
 #pragma unroll
@@ -525,7 +568,7 @@ extern "C" int llmc_mse_observe_groups(const void* x, int32_t dtype, int64_t R, 
   const int64_t n = R * (K / group);
   LLMC_CHECK_ARG(workspace && (((uintptr_t)workspace) & 255) == 0 && workspace_bytes >= llmc_mse_workspace_bytes(n), 18);
   hipStream_t st = (hipStream_t)stream;
-  MseParams p;
+  MseParams p = {};
   p.x = x; p.dt = dtype; p.fmt = fmt; p.bits = fmt == LLMC_FMT_INT ? num_bits : (fmt == LLMC_FMT_FP8 ? 8 : 4);
   p.symmetric = symmetric; p.scale_mode = scale_mode; p.steps = steps; p.grid = grid; p.norm = round_host(norm, dtype); p.expand = expand;
   Workspace w;
@@ -570,7 +613,7 @@ extern "C" int llmc_mse_observe_strided(const void* x, int32_t dtype, int64_t n0
   LLMC_CHECK_ARG(min_out && max_out, 17);
   LLMC_CHECK_ARG(workspace && (((uintptr_t)workspace) & 255) == 0 && workspace_bytes >= llmc_mse_workspace_bytes(n1), 19);
   hipStream_t st = (hipStream_t)stream;
-  MseParams p;
+  MseParams p = {};
   p.x = x; p.dt = dtype; p.fmt = fmt; p.bits = fmt == LLMC_FMT_INT ? num_bits : (fmt == LLMC_FMT_FP8 ? 8 : 4);
   p.symmetric = symmetric; p.scale_mode = scale_mode; p.steps = steps; p.grid = grid; p.norm = round_host(norm, dtype); p.expand = expand;
   Workspace w;
@@ -597,7 +640,7 @@ extern "C" int llmc_mse_observe_blocks(const void* x, int32_t dtype, int64_t R, 
   LLMC_CHECK_ARG(min_out && max_out, 17);
   LLMC_CHECK_ARG(workspace && (((uintptr_t)workspace) & 255) == 0 && workspace_bytes >= llmc_mse_workspace_bytes(n), 19);
   hipStream_t st = (hipStream_t)stream;
-  MseParams p;
+  MseParams p = {};
   p.x = x; p.dt = dtype; p.fmt = fmt; p.bits = fmt == LLMC_FMT_INT ? num_bits : (fmt == LLMC_FMT_FP8 ? 8 : 4);
   p.symmetric = symmetric; p.scale_mode = scale_mode; p.steps = steps; p.grid = grid; p.norm = round_host(norm, dtype); p.expand = expand;
   Workspace w;
@@ -608,4 +651,102 @@ extern "C" int llmc_mse_observe_blocks(const void* x, int32_t dtype, int64_t R, 
   hipLaunchKernelGGL(mse_generic_kernel, dim3((unsigned)n), dim3(256), 0, st, p, l);
   LLMC_LAUNCH_STATUS();
   return finish(p, w, n, patience, min_out, max_out, st);
+}
+
+// ---- importance-weighted search (observers/imatrix.py) -------------------------------------------
+
+namespace {
+
+// partial[s][c] = sum over the s-th slice of the token rows of x[t][c]^2 (fp32, fixed order)
+__global__ __launch_bounds__(256) void sumsq_partial_kernel(const void* __restrict__ x, int dt, int64_t T, int64_t K,
+                                                            int64_t ldx, int slices, float* __restrict__ partial) {
+  const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (c >= K) return;
+  const int s = blockIdx.y;
+  const int64_t per = (T + slices - 1) / slices;
+  const int64_t t0 = s * per, t1 = (t0 + per) < T ? t0 + per : T;
+  float acc = 0.f;
+  for (int64_t t = t0; t < t1; ++t) {
+    const float v = load_rt(x, t * ldx + c, dt);
+    acc += v * v;
+  }
+  partial[(int64_t)s * K + c] = acc;
+}
+
+__global__ __launch_bounds__(256) void sumsq_finish_kernel(const float* __restrict__ partial, int64_t K, int slices,
+                                                           float* __restrict__ sum) {
+  const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (c >= K) return;
+  float acc = 0.f;
+  for (int s = 0; s < slices; ++s) acc += partial[(int64_t)s * K + c];
+  sum[c] += acc;
+}
+
+constexpr int SUMSQ_SLICES = 32;
+
+}  // namespace
+
+extern "C" int64_t llmc_sumsq_workspace_bytes(int64_t K) { return align256(K * SUMSQ_SLICES * 4); }
+
+extern "C" int llmc_sumsq_accumulate(const void* x, int32_t dtype, int64_t T, int64_t K, int64_t ldx, float* sum,
+                                     void* workspace, int64_t workspace_bytes, void* stream) {
+  LLMC_CHECK_ARG(dtype >= 0 && dtype <= 2, 2);
+  LLMC_CHECK_ARG(T >= 0 && K > 0 && ldx >= K, 3);
+  if (T == 0) return 0;
+  LLMC_CHECK_ARG(x != nullptr && sum != nullptr, 1);
+  LLMC_CHECK_ARG(workspace && (((uintptr_t)workspace) & 255) == 0 && workspace_bytes >= llmc_sumsq_workspace_bytes(K), 7);
+  hipStream_t st = (hipStream_t)stream;
+  const int slices = T < SUMSQ_SLICES ? (int)T : SUMSQ_SLICES;
+  hipLaunchKernelGGL(sumsq_partial_kernel, dim3((unsigned)((K + 255) / 256), (unsigned)slices), dim3(256), 0, st, x,
+                     dtype, T, K, ldx, slices, (float*)workspace);
+  LLMC_LAUNCH_STATUS();
+  hipLaunchKernelGGL(sumsq_finish_kernel, dim3((unsigned)((K + 255) / 256)), dim3(256), 0, st,
+                     (const float*)workspace, K, slices, sum);
+  LLMC_LAUNCH_STATUS();
+  return 0;
+}
+
+extern "C" int llmc_imatrix_observe_groups(const void* x, int32_t dtype, int64_t R, int64_t K, int64_t ldw,
+                                           int64_t group, int32_t fmt, int32_t num_bits, int32_t symmetric,
+                                           int32_t scale_mode, int32_t steps, double grid, int32_t patience,
+                                           float norm, float expand, const float* importance, void* min_out,
+                                           void* max_out, void* workspace, int64_t workspace_bytes,
+                                           void* stream) {
+  LLMC_CHECK_ARG(x && R > 0 && K > 0, 1);
+  // patience 0 = never stop early (imatrix.py:321-325)
+  const int pat = patience > 0 ? patience : 0x7fffffff;
+  int rc = check_common(dtype, fmt, num_bits, scale_mode, steps, grid, norm, expand, pat);
+  if (rc) return rc;
+  LLMC_CHECK_ARG(patience >= 0, 13);
+  LLMC_CHECK_ARG(ldw >= K, 5);
+  LLMC_CHECK_ARG(group > 0 && K % group == 0, 6);
+  LLMC_CHECK_ARG(min_out && max_out, 17);
+  const int64_t n = R * (K / group);
+  LLMC_CHECK_ARG(workspace && (((uintptr_t)workspace) & 255) == 0 && workspace_bytes >= llmc_mse_workspace_bytes(n), 19);
+  hipStream_t st = (hipStream_t)stream;
+  MseParams p = {};
+  p.x = x; p.dt = dtype; p.fmt = fmt; p.bits = fmt == LLMC_FMT_INT ? num_bits : (fmt == LLMC_FMT_FP8 ? 8 : 4);
+  p.symmetric = symmetric; p.scale_mode = scale_mode; p.steps = steps; p.grid = grid; p.norm = norm; p.expand = expand;
+  p.err32 = 1; p.imp = importance;
+  Workspace w;
+  rc = setup(p, w, workspace, n, st);
+  if (rc) return rc;
+  const int64_t L = group / 8;
+  const bool team = dtype != LLMC_F32 && group % 8 == 0 && L <= 64 && (L & (L - 1)) == 0 && ldw % 8 == 0 &&
+                    (((uintptr_t)x) & 15) == 0;
+  if (team) {
+    const int64_t threads = n * L;
+    hipLaunchKernelGGL(mse_team_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, p, n,
+                       (int)(K / group), (int)group, (int)L, ldw);
+  } else {
+    GenericLayout l = {};
+    l.mode = 0; l.n0 = 1; l.G = group; l.s0 = 0; l.s1 = group; l.ldw = ldw; l.ng = K / group;
+    if (ldw != K) {
+      LLMC_CHECK_ARG(group == K, 5);
+      l.s1 = ldw;
+    }
+    hipLaunchKernelGGL(mse_generic_kernel, dim3((unsigned)n), dim3(256), 0, st, p, l);
+  }
+  LLMC_LAUNCH_STATUS();
+  return finish(p, w, n, pat, min_out, max_out, st);
 }

@@ -79,6 +79,10 @@ SIGNATURES.update({
     "llmc_mse_workspace_bytes": [_I64],
     "llmc_mse_observe_groups": [_P, _I32, _I64, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _F64, _I32, _F32,
                                 _F32, _P, _P, _P, _I64, _P],
+    "llmc_sumsq_workspace_bytes": [_I64],
+    "llmc_sumsq_accumulate": [_P, _I32, _I64, _I64, _I64, _P, _P, _I64, _P],
+    "llmc_imatrix_observe_groups": [_P, _I32, _I64, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _F64, _I32, _F32,
+                                    _F32, _P, _P, _P, _P, _I64, _P],
     "llmc_mse_observe_strided": [_P, _I32, _I64, _I64, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _F64, _I32,
                                  _F32, _F32, _P, _P, _P, _I64, _P],
     "llmc_mse_observe_blocks": [_P, _I32, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _F64, _I32,
@@ -92,6 +96,7 @@ RESTYPES = {
     "llmc_mse_workspace_bytes": ctypes.c_int64,
     "llmc_gptq_quantize_workspace_bytes": ctypes.c_int64,
     "llmc_sparsegpt_workspace_bytes": ctypes.c_int64,
+    "llmc_sumsq_workspace_bytes": ctypes.c_int64,
 }
 SIGNATURES["llmc_minmax_workspace_bytes"] = []
 

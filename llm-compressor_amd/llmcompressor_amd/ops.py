@@ -408,6 +408,45 @@ def mse_observe_groups(w, group: int, fmt: int, bits: int, symmetric: bool, scal
     return mn, mx
 
 
+def sumsq_accumulate_(total: torch.Tensor, x: torch.Tensor):
+    """total[K] (fp32, in place) += sum over the rows of x [T, K] of x^2."""
+    _require_gpu(total, x)
+    assert total.dtype == torch.float32 and total.ndim == 1 and x.ndim == 2 and x.shape[1] == total.shape[0]
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    ws = _workspace(x.device, _lib.lib().llmc_sumsq_workspace_bytes(x.shape[1]))
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().llmc_sumsq_accumulate(x.data_ptr(), _dt(x), x.shape[0], x.shape[1], x.stride(0),
+                                              total.data_ptr(), ws.data_ptr(), ws.numel(), _stream(x))
+    _lib.check(rc, "llmc_sumsq_accumulate")
+    return total
+
+
+def imatrix_observe_groups(w, group: int, fmt: int, bits: int, symmetric: bool, scale_mode: int = SCALE_PLAIN,
+                           importance=None, maxshrink=0.95, patience=5, grid=20, norm=3.0, expand=1.0):
+    """Importance-weighted grid search per run of `group` columns of w [R,K] -> (min, max) [R, K/group]."""
+    _require_gpu(w)
+    assert w.ndim == 2 and w.stride(1) == 1
+    R, K = w.shape
+    steps = max(1, int(maxshrink * grid)) + 1
+    if steps > 256:
+        raise ValueError(f"imatrix_observe_groups: {steps} candidates exceed the 256 this build records")
+    if importance is not None:
+        importance = importance.to(device=w.device, dtype=torch.float32).contiguous()
+        assert importance.numel() == K
+    n = R * (K // group)
+    mn = torch.empty((R, K // group), dtype=w.dtype, device=w.device)
+    mx = torch.empty_like(mn)
+    ws = _workspace(w.device, _lib.lib().llmc_mse_workspace_bytes(n))
+    with torch.cuda.device(w.device):
+        rc = _lib.lib().llmc_imatrix_observe_groups(
+            w.data_ptr(), _dt(w), R, K, w.stride(0), group, fmt, bits, 1 if symmetric else 0, scale_mode, steps,
+            float(grid), int(patience), float(norm), float(expand), _ptr(importance), mn.data_ptr(), mx.data_ptr(),
+            ws.data_ptr(), ws.numel(), _stream(w))
+    _lib.check(rc, "llmc_imatrix_observe_groups")
+    return mn, mx
+
+
 def mse_observe_strided(x, n0: int, n1: int, group: int, s0: int, s1: int, fmt: int, bits: int, symmetric: bool,
                         scale_mode: int = SCALE_PLAIN, maxshrink=0.20, patience=5, grid=100.0, norm=2.4, expand=1.0):
     _require_gpu(x)

@@ -34,5 +34,8 @@ closed form or invariant says so here):
   reference's SparseGPT tests need hub models; see ``tests/test_oracle_sparsegpt.py``:
   closed-form running-average Hessian, diagonal-Hessian == saliency pruning,
   exact zero counts, un-blocked fp64 textbook elimination, the OBS step against
-  a constrained least-squares solve).
+  a constrained least-squares solve); ``observers.imatrix_grid_search`` /
+  ``observers.prepare_importance`` (``tests/test_oracle_imatrix.py``: the
+  reference's uniform-importance == plain-search property, brute-force fp64
+  argmin, patience rule).
 """

@@ -112,6 +112,53 @@ def grid_search_mse(observed, args: QArgs, maxshrink=0.20, patience=5, grid=100.
     return best_min, best_max
 
 
+def prepare_importance(imatrix_sum, imatrix_count, observed, args: QArgs):
+    """imatrix.py:126-139: E[x^2] per input channel, normalised to mean 1, laid out like ``observed``."""
+    imp = imatrix_sum / float(imatrix_count)
+    imp = imp.to(torch.float32)
+    imp = imp / (imp.mean() + torch.finfo(torch.float32).tiny)
+    rows = observed.shape[1]
+    return flatten_for_calibration(imp.unsqueeze(0).expand(rows, -1), "weight", args)
+
+
+def imatrix_grid_search(observed, args: QArgs, maxshrink=0.95, patience=5, grid=20, norm=3.0, expand=1.0,
+                        importance_weights=None):
+    """Importance-weighted shrink-factor search, imatrix.py:255-328: candidates i = 0..max(1, int(maxshrink*grid))
+    inclusive, error |fq(x) - x|^norm formed, weighted and summed in fp32, global early stop only when
+    patience > 0.  parity unpinned by reference vectors; pinned by the reference's own property (uniform
+    importance == the plain search on fp32 inputs) and a brute-force fp64 argmin in tests/test_oracle_imatrix.py."""
+    token_args = args.copy(strategy="token")
+    if args.strategy == "tensor_group" and args.scale_dtype is not None:
+        args = args.copy(scale_dtype=None)
+        token_args = token_args.copy(scale_dtype=None)
+    min_val = torch.amin(observed, dim=(0, -1)) * expand
+    max_val = torch.amax(observed, dim=(0, -1)) * expand
+    best_error = torch.full(min_val.shape, torch.finfo(torch.float32).max, dtype=torch.float32)
+    best_min, best_max = min_val.clone(), max_val.clone()
+    no_improve = 0
+    observed_f = observed.float()
+    for i in range(max(1, int(maxshrink * grid)) + 1):
+        p = 1 - i / grid
+        smin, smax = p * min_val, p * max_val
+        scales, zps = calculate_qparams(smin, smax, args, global_scale=None)
+        q = fake_quantize(observed, scales.unsqueeze(-1), zps.unsqueeze(-1), token_args).float()
+        e = (q - observed_f).abs().pow(norm)
+        if importance_weights is not None:
+            e = e * importance_weights
+        err = e.sum(dim=(0, -1))
+        improved = err < best_error
+        if torch.any(improved):
+            best_error[improved] = err[improved]
+            best_min[improved] = smin[improved]
+            best_max[improved] = smax[improved]
+            no_improve = 0
+        else:
+            no_improve += 1
+            if patience > 0 and no_improve >= patience:
+                break
+    return best_min, best_max
+
+
 class Observer:
     """Minimal observer with the reference's statistics / qparams / fusion contract."""
 
