@@ -9,8 +9,6 @@
 // the operand shape of v_mfma_f32_32x32x16_{bf16,f16}.  bf16 x bf16 products
 // are exact in fp32 and the accumulation is fp32, so the result differs from
 // an fp32 GEMM on the upcast inputs only by summation order.
-#include <stdlib.h>
-#include <string.h>
 
 #include <type_traits>
 
@@ -671,12 +669,6 @@ Choice make_choice(int bt, int64_t T, int64_t K, bool split) {
 // the fastest of {128, 256}-wide tiles x {whole tiles, token chunks} that fits the workspace
 Choice choose(int64_t T, int64_t K, int64_t ws_avail) {
   Choice best;
-#ifdef LLMC_HESSIAN_EXPERIMENT
-  if (const char* f = getenv("LLMC_HESSIAN_FORCE")) {  // "256,1" = tile width, split
-    const int bt = atoi(f), sp = atoi(strchr(f, ',') + 1);
-    return make_choice(bt, T, K, sp != 0);
-  }
-#endif
   for (int bt : {256, 128})
     for (int split = 0; split < 2; ++split) {
       const Choice c = make_choice(bt, T, K, split != 0);
