@@ -160,6 +160,19 @@ int llmc_imatrix_observe_groups(const void* x, int32_t dtype, int64_t R, int64_t
                                 int32_t scale_mode, int32_t steps, double grid, int32_t patience,
                                 float norm, float expand, const float* importance, void* min_out,
                                 void* max_out, void* workspace, int64_t workspace_bytes, void* stream);
+/* The same search without weights on the other layouts (the reference routes block-wise weights and
+ * non-weight observers to the uniform fall-back, imatrix.py:141-245); arguments as the llmc_mse_observe_*
+ * twins, patience 0 = never stop. */
+int llmc_imatrix_observe_strided(const void* x, int32_t dtype, int64_t n0, int64_t n1, int64_t group,
+                                 int64_t stride0, int64_t stride1, int32_t fmt, int32_t num_bits,
+                                 int32_t symmetric, int32_t scale_mode, int32_t steps, double grid,
+                                 int32_t patience, float norm, float expand, void* min_out, void* max_out,
+                                 void* workspace, int64_t workspace_bytes, void* stream);
+int llmc_imatrix_observe_blocks(const void* x, int32_t dtype, int64_t R, int64_t K, int64_t ldw,
+                                int32_t block_h, int32_t block_w, int32_t fmt, int32_t num_bits,
+                                int32_t symmetric, int32_t scale_mode, int32_t steps, double grid,
+                                int32_t patience, float norm, float expand, void* min_out, void* max_out,
+                                void* workspace, int64_t workspace_bytes, void* stream);
 
 /* ---- a12/a16: qparams ------------------------------------------------------
  * llmc_absmax_accumulate + llmc_generate_gparam replace Observer.get_global_scale()

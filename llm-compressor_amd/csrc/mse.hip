@@ -602,7 +602,7 @@ extern "C" int llmc_mse_observe_groups(const void* x, int32_t dtype, int64_t R, 
   return finish(p, w, n, patience, min_out, max_out, st);
 }
 
-extern "C" int llmc_mse_observe_strided(const void* x, int32_t dtype, int64_t n0, int64_t n1, int64_t group,
+static int observe_strided_impl(int err32, const void* x, int32_t dtype, int64_t n0, int64_t n1, int64_t group,
                                         int64_t stride0, int64_t stride1, int32_t fmt, int32_t num_bits,
                                         int32_t symmetric, int32_t scale_mode, int32_t steps, double grid,
                                         int32_t patience, float norm, float expand, void* min_out, void* max_out,
@@ -615,7 +615,8 @@ extern "C" int llmc_mse_observe_strided(const void* x, int32_t dtype, int64_t n0
   hipStream_t st = (hipStream_t)stream;
   MseParams p = {};
   p.x = x; p.dt = dtype; p.fmt = fmt; p.bits = fmt == LLMC_FMT_INT ? num_bits : (fmt == LLMC_FMT_FP8 ? 8 : 4);
-  p.symmetric = symmetric; p.scale_mode = scale_mode; p.steps = steps; p.grid = grid; p.norm = round_host(norm, dtype); p.expand = expand;
+  p.symmetric = symmetric; p.scale_mode = scale_mode; p.steps = steps; p.grid = grid;
+  p.norm = err32 ? norm : round_host(norm, dtype); p.expand = expand; p.err32 = err32;
   Workspace w;
   rc = setup(p, w, workspace, n1, st);
   if (rc) return rc;
@@ -626,7 +627,16 @@ extern "C" int llmc_mse_observe_strided(const void* x, int32_t dtype, int64_t n0
   return finish(p, w, n1, patience, min_out, max_out, st);
 }
 
-extern "C" int llmc_mse_observe_blocks(const void* x, int32_t dtype, int64_t R, int64_t K, int64_t ldw,
+extern "C" int llmc_mse_observe_strided(const void* x, int32_t dtype, int64_t n0, int64_t n1, int64_t group,
+                                        int64_t stride0, int64_t stride1, int32_t fmt, int32_t num_bits,
+                                        int32_t symmetric, int32_t scale_mode, int32_t steps, double grid,
+                                        int32_t patience, float norm, float expand, void* min_out, void* max_out,
+                                        void* workspace, int64_t workspace_bytes, void* stream) {
+  return observe_strided_impl(0, x, dtype, n0, n1, group, stride0, stride1, fmt, num_bits, symmetric, scale_mode, steps,
+                              grid, patience, norm, expand, min_out, max_out, workspace, workspace_bytes, stream);
+}
+
+static int observe_blocks_impl(int err32, const void* x, int32_t dtype, int64_t R, int64_t K, int64_t ldw,
                                        int32_t block_h, int32_t block_w, int32_t fmt, int32_t num_bits,
                                        int32_t symmetric, int32_t scale_mode, int32_t steps, double grid,
                                        int32_t patience, float norm, float expand, void* min_out, void* max_out,
@@ -642,7 +652,8 @@ extern "C" int llmc_mse_observe_blocks(const void* x, int32_t dtype, int64_t R, 
   hipStream_t st = (hipStream_t)stream;
   MseParams p = {};
   p.x = x; p.dt = dtype; p.fmt = fmt; p.bits = fmt == LLMC_FMT_INT ? num_bits : (fmt == LLMC_FMT_FP8 ? 8 : 4);
-  p.symmetric = symmetric; p.scale_mode = scale_mode; p.steps = steps; p.grid = grid; p.norm = round_host(norm, dtype); p.expand = expand;
+  p.symmetric = symmetric; p.scale_mode = scale_mode; p.steps = steps; p.grid = grid;
+  p.norm = err32 ? norm : round_host(norm, dtype); p.expand = expand; p.err32 = err32;
   Workspace w;
   rc = setup(p, w, workspace, n, st);
   if (rc) return rc;
@@ -651,6 +662,15 @@ extern "C" int llmc_mse_observe_blocks(const void* x, int32_t dtype, int64_t R, 
   hipLaunchKernelGGL(mse_generic_kernel, dim3((unsigned)n), dim3(256), 0, st, p, l);
   LLMC_LAUNCH_STATUS();
   return finish(p, w, n, patience, min_out, max_out, st);
+}
+
+extern "C" int llmc_mse_observe_blocks(const void* x, int32_t dtype, int64_t R, int64_t K, int64_t ldw,
+                                       int32_t block_h, int32_t block_w, int32_t fmt, int32_t num_bits,
+                                       int32_t symmetric, int32_t scale_mode, int32_t steps, double grid,
+                                       int32_t patience, float norm, float expand, void* min_out, void* max_out,
+                                       void* workspace, int64_t workspace_bytes, void* stream) {
+  return observe_blocks_impl(0, x, dtype, R, K, ldw, block_h, block_w, fmt, num_bits, symmetric, scale_mode, steps, grid,
+                             patience, norm, expand, min_out, max_out, workspace, workspace_bytes, stream);
 }
 
 // ---- importance-weighted search (observers/imatrix.py) -------------------------------------------
@@ -749,4 +769,29 @@ extern "C" int llmc_imatrix_observe_groups(const void* x, int32_t dtype, int64_t
   }
   LLMC_LAUNCH_STATUS();
   return finish(p, w, n, pat, min_out, max_out, st);
+}
+
+// the uniform fall-back of the importance-weighted observer on the other layouts (imatrix.py:141-245 route
+// block-wise weights and non-weight observers to the same search without weights): fp32 error, patience 0 = never stop
+extern "C" int llmc_imatrix_observe_strided(const void* x, int32_t dtype, int64_t n0, int64_t n1, int64_t group,
+                                            int64_t stride0, int64_t stride1, int32_t fmt, int32_t num_bits,
+                                            int32_t symmetric, int32_t scale_mode, int32_t steps, double grid,
+                                            int32_t patience, float norm, float expand, void* min_out,
+                                            void* max_out, void* workspace, int64_t workspace_bytes,
+                                            void* stream) {
+  LLMC_CHECK_ARG(patience >= 0, 14);
+  return observe_strided_impl(1, x, dtype, n0, n1, group, stride0, stride1, fmt, num_bits, symmetric, scale_mode, steps,
+                              grid, patience > 0 ? patience : 0x7fffffff, norm, expand, min_out, max_out, workspace,
+                              workspace_bytes, stream);
+}
+
+extern "C" int llmc_imatrix_observe_blocks(const void* x, int32_t dtype, int64_t R, int64_t K, int64_t ldw,
+                                           int32_t block_h, int32_t block_w, int32_t fmt, int32_t num_bits,
+                                           int32_t symmetric, int32_t scale_mode, int32_t steps, double grid,
+                                           int32_t patience, float norm, float expand, void* min_out,
+                                           void* max_out, void* workspace, int64_t workspace_bytes, void* stream) {
+  LLMC_CHECK_ARG(patience >= 0, 14);
+  return observe_blocks_impl(1, x, dtype, R, K, ldw, block_h, block_w, fmt, num_bits, symmetric, scale_mode, steps, grid,
+                             patience > 0 ? patience : 0x7fffffff, norm, expand, min_out, max_out, workspace,
+                             workspace_bytes, stream);
 }

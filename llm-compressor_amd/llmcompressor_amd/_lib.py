@@ -83,6 +83,10 @@ SIGNATURES.update({
     "llmc_sumsq_accumulate": [_P, _I32, _I64, _I64, _I64, _P, _P, _I64, _P],
     "llmc_imatrix_observe_groups": [_P, _I32, _I64, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _F64, _I32, _F32,
                                     _F32, _P, _P, _P, _P, _I64, _P],
+    "llmc_imatrix_observe_strided": [_P, _I32, _I64, _I64, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _F64, _I32,
+                                     _F32, _F32, _P, _P, _P, _I64, _P],
+    "llmc_imatrix_observe_blocks": [_P, _I32, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _F64, _I32,
+                                    _F32, _F32, _P, _P, _P, _I64, _P],
     "llmc_mse_observe_strided": [_P, _I32, _I64, _I64, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _F64, _I32,
                                  _F32, _F32, _P, _P, _P, _I64, _P],
     "llmc_mse_observe_blocks": [_P, _I32, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _F64, _I32,

@@ -103,10 +103,12 @@ class IMatrixMSEObserver(Observer):
         mode = ops.SCALE_MXFP4 if self.args.is_mx else ops.SCALE_PLAIN
         kw = dict(maxshrink=self.maxshrink, patience=self.patience, grid=self.grid, norm=self.norm,
                   expand=self.expand)
-        if kind != "groups":
-            raise NotImplementedError("imatrix_mse: this build searches weight observers laid out as rows of "
-                                      "column groups (CHANNEL, GROUP, TENSOR_GROUP, TENSOR on a 2-D weight)")
-        mn, mx = ops.imatrix_observe_groups(t, p, fmt, bits, self.args.symmetric, mode, importance=imp, **kw)
+        if kind == "groups":
+            mn, mx = ops.imatrix_observe_groups(t, p, fmt, bits, self.args.symmetric, mode, importance=imp, **kw)
+        elif kind == "blocks":  # no importance here: _validated_importance sent block-wise weights to the fall-back
+            mn, mx = ops.imatrix_observe_blocks(t, p[0], p[1], fmt, bits, self.args.symmetric, mode, **kw)
+        else:
+            mn, mx = ops.imatrix_observe_strided(t, *p, fmt, bits, self.args.symmetric, mode, **kw)
         return mn.reshape(shape), mx.reshape(shape)
 
     def _fallback(self, exc_type, msg: str):

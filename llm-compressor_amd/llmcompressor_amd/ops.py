@@ -478,3 +478,45 @@ def mse_observe_blocks(w, bh: int, bw: int, fmt: int, bits: int, symmetric: bool
             grid, patience, norm, expand, mn.data_ptr(), mx.data_ptr(), ws.data_ptr(), ws.numel(), _stream(w))
     _lib.check(rc, "llmc_mse_observe_blocks")
     return mn, mx
+
+
+def _imatrix_steps(maxshrink, grid):
+    steps = max(1, int(maxshrink * grid)) + 1
+    if steps > 256:
+        raise ValueError(f"imatrix search: {steps} candidates exceed the 256 this build records")
+    return steps
+
+
+def imatrix_observe_strided(x, n0: int, n1: int, group: int, s0: int, s1: int, fmt: int, bits: int, symmetric: bool,
+                            scale_mode: int = SCALE_PLAIN, maxshrink=0.95, patience=5, grid=20, norm=3.0, expand=1.0):
+    """The uniform fp32-error search on an (n0, n1, group) strided view -> (min, max) [n1]."""
+    _require_gpu(x)
+    mn = torch.empty((n1,), dtype=x.dtype, device=x.device)
+    mx = torch.empty_like(mn)
+    ws = _workspace(x.device, _lib.lib().llmc_mse_workspace_bytes(n1))
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().llmc_imatrix_observe_strided(
+            x.data_ptr(), _dt(x), n0, n1, group, s0, s1, fmt, bits, 1 if symmetric else 0, scale_mode,
+            _imatrix_steps(maxshrink, grid), float(grid), int(patience), float(norm), float(expand), mn.data_ptr(),
+            mx.data_ptr(), ws.data_ptr(), ws.numel(), _stream(x))
+    _lib.check(rc, "llmc_imatrix_observe_strided")
+    return mn, mx
+
+
+def imatrix_observe_blocks(w, bh: int, bw: int, fmt: int, bits: int, symmetric: bool, scale_mode: int = SCALE_PLAIN,
+                           maxshrink=0.95, patience=5, grid=20, norm=3.0, expand=1.0):
+    """The uniform fp32-error search on bh x bw blocks of w [R,K] -> (min, max) [ceil(R/bh), ceil(K/bw)]."""
+    _require_gpu(w)
+    assert w.ndim == 2 and w.stride(1) == 1
+    R, K = w.shape
+    shape = ((R + bh - 1) // bh, (K + bw - 1) // bw)
+    mn = torch.empty(shape, dtype=w.dtype, device=w.device)
+    mx = torch.empty_like(mn)
+    ws = _workspace(w.device, _lib.lib().llmc_mse_workspace_bytes(shape[0] * shape[1]))
+    with torch.cuda.device(w.device):
+        rc = _lib.lib().llmc_imatrix_observe_blocks(
+            w.data_ptr(), _dt(w), R, K, w.stride(0), bh, bw, fmt, bits, 1 if symmetric else 0, scale_mode,
+            _imatrix_steps(maxshrink, grid), float(grid), int(patience), float(norm), float(expand), mn.data_ptr(),
+            mx.data_ptr(), ws.data_ptr(), ws.numel(), _stream(w))
+    _lib.check(rc, "llmc_imatrix_observe_blocks")
+    return mn, mx

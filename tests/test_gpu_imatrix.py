@@ -127,3 +127,36 @@ def test_imatrix_fallbacks_and_strict():
         with pytest.raises(ValueError):
             Observer.load_from_registry("imatrix_mse", base_name="weight",
                                         args=QuantizationArgs(observer_kwargs=bad, **base))
+
+
+def test_imatrix_block_and_activation_fall_back_to_uniform_search():
+    """Block-wise weights and non-weight observers take the uniform fp32-error search (imatrix.py:141-245;
+    reference test_block_strategy / test_non_weight_base_name_non_strict_falls_back)."""
+    from llmcompressor_amd.observers import Observer
+    from llmcompressor_amd.quantization import QuantizationArgs
+
+    g = torch.Generator().manual_seed(3)
+    w = (torch.randn(96, 160, generator=g) * 0.05).bfloat16()
+    lin = torch.nn.Linear(160, 96, bias=False, dtype=torch.bfloat16, device=DEV)
+    lin.weight.data.copy_(w)
+    qa = QuantizationArgs(num_bits=4, symmetric=True, strategy="block", block_structure=[32, 64],
+                          observer="imatrix_mse")
+    obs = Observer.load_from_registry("imatrix_mse", base_name="weight", args=qa)
+    obs.attach(lin)
+    obs._imatrix_sum = torch.rand(160, device=DEV) + 0.1
+    obs._imatrix_count = torch.tensor(1, dtype=torch.int64, device=DEV)
+    obs(lin.weight)
+    oa = QArgs(num_bits=4, symmetric=True, strategy="block", block_structure=[32, 64])
+    observed = O.flatten_for_calibration(w, "weight", oa)
+    mn_o, mx_o = O.imatrix_grid_search(observed, oa)
+    same = (obs.min_vals.cpu() == mn_o.reshape(obs.min_vals.shape)) & (obs.max_vals.cpu() == mx_o.reshape(obs.max_vals.shape))
+    assert same.float().mean().item() >= 0.9  # 15 blocks: at most one near-tie may swap
+
+    x = (torch.randn(4, 33, 64, generator=g)).bfloat16()
+    qa = QuantizationArgs(num_bits=8, symmetric=True, strategy="tensor", observer="imatrix_mse")
+    aobs = Observer.load_from_registry("imatrix_mse", base_name="input", args=qa)
+    aobs(x.to(DEV))
+    oa = QArgs(num_bits=8, symmetric=True, strategy="tensor")
+    mn_o, mx_o = O.imatrix_grid_search(O.flatten_for_calibration(x, "input", oa), oa)
+    assert torch.equal(aobs.min_vals.cpu().reshape(-1), mn_o.reshape(-1))
+    assert torch.equal(aobs.max_vals.cpu().reshape(-1), mx_o.reshape(-1))
