@@ -9,7 +9,6 @@ from __future__ import annotations
 
 import contextlib
 import logging
-import threading
 
 import torch
 from pydantic import PrivateAttr
@@ -32,6 +31,7 @@ from ...utils.metric_logging import CompressionLogger
 from ..modifier import Modifier
 from ..quantization.calibration import observe, update_qparams
 from ..quantization.quantization import QuantizationMixin
+from ..utils.concurrent import run_on_streams
 from ..utils.hessian_staging import HessianStagingMixin
 from .gptq_quantize import accumulate_hessian, make_empty_hessian, quantize_weight
 
@@ -88,7 +88,7 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
     _group_pending: list | None = PrivateAttr(default=None)
     _leader: dict = PrivateAttr(default_factory=dict)  # follower module -> module whose Hessian it shares
     _recent_input: tuple | None = PrivateAttr(default=None)  # (tensor kept alive, its version, leader)
-    _streams: list = PrivateAttr(default_factory=list)
+    _streams: dict = PrivateAttr(default_factory=dict)
 
     def resolve_quantization_config(self) -> QuantizationConfig:
         config = super().resolve_quantization_config()
@@ -233,46 +233,16 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
             self._held.pop(module, None)
         jobs = list(module_list)
         workers = min(int(self.compress_concurrency), len(jobs))
-        on_gpu = all(m.weight.is_cuda and self._hessians[m].is_cuda for m in jobs)
+        on_gpu = (all(m.weight.is_cuda and self._hessians[m].is_cuda for m in jobs)
+                  and len({m.weight.device for m in jobs}) == 1)  # one device per call
         if workers <= 1 or not on_gpu or self.offload_hessians:
             for module in jobs:
                 self._compress_one(module)
             return
-        # Modules are independent, and each one's Cholesky chain and column loop are long runs of
-        # small, serially dependent kernels that leave most of the chip idle.  Quantise several at once,
-        # one host thread and one HIP stream each, most expensive first so that the widest module does
-        # not start last.  Per module the kernels and their order are unchanged, so are the results.
-        device = jobs[0].weight.device
+        # several modules at once, one host thread and one HIP stream each, most expensive first so that the
+        # widest module does not start last (see modifiers/utils/concurrent.py); results are unchanged
         jobs.sort(key=lambda m: -(float(m.weight.shape[1]) ** 3 + float(m.weight.shape[0]) * m.weight.shape[1] ** 2))
-        main = torch.cuda.current_stream(device)
-        ready = main.record_event()
-        while len(self._streams) < workers:
-            self._streams.append(torch.cuda.Stream(device=device))
-        lock = threading.Lock()
-        errors = []
-
-        def worker(stream):
-            try:
-                with torch.cuda.device(device), torch.cuda.stream(stream):
-                    stream.wait_event(ready)
-                    while True:
-                        with lock:
-                            if not jobs or errors:
-                                return
-                            module = jobs.pop(0)
-                        self._compress_one(module, produced_on=stream, consumed_on=main)
-            except BaseException as err:  # re-raised on the calling thread
-                errors.append(err)
-
-        threads = [threading.Thread(target=worker, args=(s,), daemon=True) for s in self._streams[:workers]]
-        for t in threads:
-            t.start()
-        for t in threads:
-            t.join()
-        for s in self._streams[:workers]:
-            main.wait_stream(s)
-        if errors:
-            raise errors[0]
+        run_on_streams(jobs, self._compress_one, workers, jobs[0].weight.device, self._streams)
 
     def _compress_one(self, module, produced_on=None, consumed_on=None):
         name = self._module_names.get(module, module.__class__.__name__)

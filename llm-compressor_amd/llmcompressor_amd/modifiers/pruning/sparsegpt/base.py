@@ -8,7 +8,6 @@ modules of one ``compress_modules`` call are pruned concurrently on separate str
 from __future__ import annotations
 
 import logging
-import threading
 
 import torch
 from pydantic import PrivateAttr
@@ -16,6 +15,7 @@ from pydantic import PrivateAttr
 from ....core import State
 from ....quantization import update_offload_parameter
 from ....utils.metric_logging import CompressionLogger
+from ...utils.concurrent import run_on_streams
 from ...utils.hessian_staging import HessianStagingMixin
 from .sgpt_base import SparsityModifierBase
 from .sgpt_sparsify import accumulate_hessian, make_empty_hessian, sparsify_weight
@@ -50,7 +50,7 @@ class SparseGPTModifier(SparsityModifierBase, HessianStagingMixin):
     _hessians: dict = PrivateAttr(default_factory=dict)
     _staged: dict = PrivateAttr(default_factory=dict)
     _held: dict = PrivateAttr(default_factory=dict)
-    _streams: list = PrivateAttr(default_factory=list)
+    _streams: dict = PrivateAttr(default_factory=dict)
 
     def calibrate_module(self, module: torch.nn.Module, args: tuple[torch.Tensor, ...], _output: torch.Tensor):
         """Forward hook: accumulate the Hessian of the module's input."""
@@ -77,43 +77,14 @@ class SparseGPTModifier(SparsityModifierBase, HessianStagingMixin):
             self._staged.pop(module, None)
             self._held.pop(module, None)
         workers = min(int(self.compress_concurrency), len(jobs))
-        if workers <= 1 or self.offload_hessians or not all(m.weight.is_cuda for m in jobs):
+        one_gpu = all(m.weight.is_cuda for m in jobs) and len({m.weight.device for m in jobs}) == 1
+        if workers <= 1 or self.offload_hessians or not one_gpu:
             for module in jobs:
                 self._compress_one(module)
             return
-        # independent modules, each a long chain of small dependent kernels: several at once, one host thread
-        # and one HIP stream each, most expensive first (same scheme as GPTQModifier.compress_module_list)
-        device = jobs[0].weight.device
+        # independent modules, each a long chain of small dependent kernels: several at once, most expensive first
         jobs.sort(key=lambda m: -(float(m.weight.shape[1]) ** 3 + float(m.weight.shape[0]) * m.weight.shape[1] ** 2))
-        main = torch.cuda.current_stream(device)
-        ready = main.record_event()
-        while len(self._streams) < workers:
-            self._streams.append(torch.cuda.Stream(device=device))
-        lock = threading.Lock()
-        errors = []
-
-        def worker(stream):
-            try:
-                with torch.cuda.device(device), torch.cuda.stream(stream):
-                    stream.wait_event(ready)
-                    while True:
-                        with lock:
-                            if not jobs or errors:
-                                return
-                            module = jobs.pop(0)
-                        self._compress_one(module, produced_on=stream, consumed_on=main)
-            except BaseException as err:  # re-raised on the calling thread
-                errors.append(err)
-
-        threads = [threading.Thread(target=worker, args=(s,), daemon=True) for s in self._streams[:workers]]
-        for t in threads:
-            t.start()
-        for t in threads:
-            t.join()
-        for s in self._streams[:workers]:
-            main.wait_stream(s)
-        if errors:
-            raise errors[0]
+        run_on_streams(jobs, self._compress_one, workers, jobs[0].weight.device, self._streams)
 
     def _compress_one(self, module, produced_on=None, consumed_on=None):
         name = self._module_names[module]
