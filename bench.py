@@ -156,6 +156,13 @@ def probe_bandwidth():
         t = timed(lambda: ops.mse_observe_groups(w, g, fmt, bits, True, ops.SCALE_PLAIN, **kw), n=5)
         cands = 80 if kw else 20
         rep(f"{name}: {n * cands / t / 1e12:.2f} T element-candidates/s", t, 2 * n)
+    tot = torch.zeros(HIDDEN, dtype=torch.float32, device="cuda")
+    rep("imatrix hook: sum of squares per channel [8192x4096], 2 B/elem", timed(lambda: ops.sumsq_accumulate_(tot, x)),
+        2 * x.numel())
+    imp = torch.rand(K, device="cuda") + 0.1
+    t = timed(lambda: ops.imatrix_observe_groups(w, 128, ops.FMT_INT, 4, True, importance=imp), n=5)
+    rep(f"imatrix observer int4 g128, 20 candidates, fp32 weighted error: {n * 20 / t / 1e12:.2f} T element-candidates/s",
+        t, 2 * n)
     print("| kernel (14336 x 4096 bf16 unless noted) | us | GB/s | of 8 TB/s |")
     print("|---|---|---|---|")
     for name, us, gbs, frac in rows:

@@ -702,7 +702,42 @@ __global__ __launch_bounds__(256) void sumsq_finish_kernel(const float* __restri
   sum[c] += acc;
 }
 
-constexpr int SUMSQ_SLICES = 32;
+constexpr int SUMSQ_SLICES = 64;
+
+// 16-bit input with 16-byte aligned rows: a workgroup covers 256 columns of one token slice as 32 column
+// groups (16-byte loads) x 8 token lanes, folds the token lanes through LDS and writes one partial row
+__global__ __launch_bounds__(256) void sumsq_partial16_kernel(const uint16_t* __restrict__ x, int dt, int64_t T,
+                                                              int64_t K, int64_t ldx, int slices,
+                                                              float* __restrict__ partial) {
+  __shared__ float red[8][256 + 8];
+  const int cg = threadIdx.x & 31, tl = threadIdx.x >> 5;
+  const int64_t c0 = (int64_t)blockIdx.x * 256 + cg * 8;
+  const int s = blockIdx.y;
+  const int64_t per = (T + slices - 1) / slices;
+  const int64_t t0 = s * per, t1 = (t0 + per) < T ? t0 + per : T;
+  float acc[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+  if (c0 < K) {
+    for (int64_t t = t0 + tl; t < t1; t += 8) {
+      const uint4 v = *(const uint4*)(x + t * ldx + c0);
+      float f[8];
+      unpack8(v, dt, f);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[j] += f[j] * f[j];
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) red[tl][cg * 8 + j] = acc[j];
+  __syncthreads();
+  const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (c < K) {
+    float sum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) sum += red[r][threadIdx.x];
+    partial[(int64_t)s * K + c] = sum;
+  }
+}
 
 }  // namespace
 
@@ -717,8 +752,13 @@ extern "C" int llmc_sumsq_accumulate(const void* x, int32_t dtype, int64_t T, in
   LLMC_CHECK_ARG(workspace && (((uintptr_t)workspace) & 255) == 0 && workspace_bytes >= llmc_sumsq_workspace_bytes(K), 7);
   hipStream_t st = (hipStream_t)stream;
   const int slices = T < SUMSQ_SLICES ? (int)T : SUMSQ_SLICES;
-  hipLaunchKernelGGL(sumsq_partial_kernel, dim3((unsigned)((K + 255) / 256), (unsigned)slices), dim3(256), 0, st, x,
-                     dtype, T, K, ldx, slices, (float*)workspace);
+  const bool wide = dtype != LLMC_F32 && K % 8 == 0 && ldx % 8 == 0 && (((uintptr_t)x) & 15) == 0;
+  if (wide)
+    hipLaunchKernelGGL(sumsq_partial16_kernel, dim3((unsigned)((K + 255) / 256), (unsigned)slices), dim3(256), 0, st,
+                       (const uint16_t*)x, dtype, T, K, ldx, slices, (float*)workspace);
+  else
+    hipLaunchKernelGGL(sumsq_partial_kernel, dim3((unsigned)((K + 255) / 256), (unsigned)slices), dim3(256), 0, st, x,
+                       dtype, T, K, ldx, slices, (float*)workspace);
   LLMC_LAUNCH_STATUS();
   hipLaunchKernelGGL(sumsq_finish_kernel, dim3((unsigned)((K + 255) / 256)), dim3(256), 0, st,
                      (const float*)workspace, K, slices, sum);
