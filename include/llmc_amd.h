@@ -243,6 +243,18 @@ int llmc_gptq_hinv(float* H, int64_t ldh, int64_t K, const int32_t* perm, float 
                    float percdamp, uint8_t* dead_out, void* workspace, int64_t workspace_bytes,
                    int32_t* info_out, void* stream);
 
+/* Grouped form for many small problems of one width (the experts of an MoE layer): the chain of
+ * llmc_gptq_hinv run once for all n problems in lock-step, every kernel carrying one more batch
+ * dimension.  H (and perm, or NULL) are HOST arrays of n device pointers, divisors a HOST array of n
+ * floats; dead_out is device [n, K] bytes (or NULL), U_out device [n, K, ldu] floats (the factors; the
+ * Hessians themselves are left untouched), info_out device [n].  Results are bit-identical to n single
+ * calls. */
+int64_t llmc_gptq_hinv_grouped_workspace_bytes(int64_t n, int64_t K);
+int llmc_gptq_hinv_grouped(const float* const* H, int64_t ldh, int32_t n, int64_t K,
+                           const int32_t* const* perm, const float* divisors, float percdamp,
+                           uint8_t* dead_out, float* U_out, int64_t ldu, void* workspace,
+                           int64_t workspace_bytes, int32_t* info_out, void* stream);
+
 /* ---- a8/a9: GPTQ block column loop ---------------------------------------------
  * Replaces the loop of quantize_weight (gptq_quantize.py:88-92,144-146,167-250):
  * W = float(weight)[:, perm], dead columns zeroed; per block of `blocksize`

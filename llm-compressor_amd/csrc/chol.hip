@@ -13,6 +13,8 @@
 // (4) writes the index-reversed result over H.  A non-positive pivot sets
 // *info and the output becomes the identity (the reference's round-to-nearest
 // fallback) without a host round trip.
+#include <vector>
+
 #include "common.h"
 #include "gemm_f32.h"
 
@@ -25,12 +27,29 @@ struct HinvScalars {
   int info;
 };
 
+// One problem of a grouped call (llmc_gptq_hinv_grouped): the kernels below take an optional array of
+// these and pick theirs by the workgroup index; the work matrices and scalars of problem b then sit at
+// a fixed stride behind those of problem 0.
+struct HinvItem {
+  const float* H;
+  const int32_t* perm;
+  uint8_t* dead;
+  float* U;
+  float div;
+  int pad;
+};
+
 // damp = percdamp * mean(diag(H')) where H' = H/div with zero diagonal entries replaced by 1;
 // dead[c] = 1 where the (permuted) diagonal was zero
 __global__ __launch_bounds__(256) void hinv_stats_kernel(const float* __restrict__ H, int64_t ldh, int K,
                                                          const int32_t* __restrict__ perm, float div,
                                                          float percdamp, uint8_t* __restrict__ dead,
-                                                         HinvScalars* sc) {
+                                                         HinvScalars* sc, const HinvItem* __restrict__ items) {
+  if (items) {
+    const HinvItem it = items[blockIdx.x];
+    H = it.H; perm = it.perm; dead = it.dead; div = it.div;
+    sc += blockIdx.x;
+  }
   __shared__ double red[4];
   double sum = 0.0;
   for (int c = threadIdx.x; c < K; c += 256) {
@@ -55,7 +74,13 @@ __global__ __launch_bounds__(256) void hinv_stats_kernel(const float* __restrict
 __global__ __launch_bounds__(256) void hinv_copyin_kernel(const float* __restrict__ H, int64_t ldh, int K,
                                                           int Kp, const int32_t* __restrict__ perm,
                                                           float div, const HinvScalars* __restrict__ sc,
-                                                          float* __restrict__ A) {
+                                                          float* __restrict__ A, const HinvItem* __restrict__ items) {
+  if (items) {
+    const HinvItem it = items[blockIdx.z];
+    H = it.H; perm = it.perm; div = it.div;
+    sc += blockIdx.z;
+    A += (int64_t)blockIdx.z * Kp * Kp;
+  }
   const int j = blockIdx.x * 256 + threadIdx.x;
   const int i = blockIdx.y;
   if (j >= Kp) return;
@@ -86,6 +111,8 @@ __global__ __launch_bounds__(256) void hinv_copyin_kernel(const float* __restric
 // so factor and inverse advance together.
 __global__ __launch_bounds__(256) void potf2_inv_kernel(float* __restrict__ A, int Kp, int k0, int K,
                                                         HinvScalars* sc) {
+  A += (int64_t)blockIdx.x * Kp * Kp;  // grouped call: one workgroup per problem (a single problem has one workgroup)
+  sc += blockIdx.x;
   __shared__ __attribute__((aligned(16))) float colbuf[2][NB][4];  // panel: row i, columns j0..j0+3
   __shared__ __attribute__((aligned(16))) float xrow[2][4][NB];    // rows j0..j0+3 of X
   const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
@@ -220,7 +247,14 @@ __global__ __launch_bounds__(256) void potf2_inv_kernel(float* __restrict__ A, i
 __global__ __launch_bounds__(256) void hinv_copyout_kernel(const float* __restrict__ X, int Kp, int K,
                                                            const HinvScalars* __restrict__ sc,
                                                            float* __restrict__ U, int64_t ldu,
-                                                           int32_t* __restrict__ info_out) {
+                                                           int32_t* __restrict__ info_out,
+                                                           const HinvItem* __restrict__ items) {
+  if (items) {
+    U = items[blockIdx.z].U;
+    sc += blockIdx.z;
+    X += (int64_t)blockIdx.z * Kp * Kp;
+    if (info_out) info_out += blockIdx.z;
+  }
   const int j = blockIdx.x * 256 + threadIdx.x;
   const int i = blockIdx.y;
   if (i == 0 && j == 0 && info_out) *info_out = sc->info;
@@ -260,10 +294,10 @@ extern "C" int llmc_gptq_hinv(float* H, int64_t ldh, int64_t K, const int32_t* p
   float* T = A + (int64_t)Kp * Kp;
 
   hipLaunchKernelGGL(hinv_stats_kernel, dim3(1), dim3(256), 0, st, H, ldh, (int)K, perm, divisor, percdamp,
-                     dead_out, sc);
+                     dead_out, sc, (const HinvItem*)nullptr);
   LLMC_LAUNCH_STATUS();
   hipLaunchKernelGGL(hinv_copyin_kernel, dim3((Kp + 255) / 256, Kp), dim3(256), 0, st, H, ldh, (int)K, Kp, perm,
-                     divisor, sc, A);
+                     divisor, sc, A, (const HinvItem*)nullptr);
   LLMC_LAUNCH_STATUS();
 
   // Blocked Cholesky, two levels: inside a 256-wide outer panel the 64-wide steps (diagonal block
@@ -340,7 +374,138 @@ extern "C" int llmc_gptq_hinv(float* H, int64_t ldh, int64_t K, const int32_t* p
   }
 
   hipLaunchKernelGGL(hinv_copyout_kernel, dim3((unsigned)((K + 255) / 256), (unsigned)K), dim3(256), 0, st, A, Kp,
-                     (int)K, sc, H, ldh, info_out);
+                     (int)K, sc, H, ldh, info_out, (const HinvItem*)nullptr);
+  LLMC_LAUNCH_STATUS();
+  return 0;
+}
+
+// ---- grouped form: n independent problems of one width in lock-step ---------------------------------
+// The chain of a small Hessian (an MoE expert's: K = 768 or 2048) is a run of tiny kernels that uses a few
+// CUs for microseconds each; run for 128 experts one after the other, the chip idles.  Here every kernel of
+// the chain is launched once for all problems (one more grid dimension / GEMM batch level), so the chain is
+// as long as a single problem's while each launch carries n times the work.
+
+extern "C" int64_t llmc_gptq_hinv_grouped_workspace_bytes(int64_t n, int64_t K) {
+  const int64_t Kp = round_up(K, NB);
+  return round_up(n * (int64_t)sizeof(HinvItem), 256) + round_up(n * (int64_t)sizeof(HinvScalars), 256) +
+         n * (Kp * Kp + Kp * Kp / 4) * 4 + 256;
+}
+
+extern "C" int llmc_gptq_hinv_grouped(const float* const* H, int64_t ldh, int32_t n, int64_t K,
+                                      const int32_t* const* perm, const float* divisors, float percdamp,
+                                      uint8_t* dead_out, float* U_out, int64_t ldu, void* workspace,
+                                      int64_t workspace_bytes, int32_t* info_out, void* stream) {
+  LLMC_CHECK_ARG(H != nullptr && ldh >= K, 1);
+  LLMC_CHECK_ARG(n >= 0 && n <= 4096, 3);
+  if (n == 0) return 0;
+  LLMC_CHECK_ARG(K > 0 && K <= 65536, 4);
+  LLMC_CHECK_ARG(divisors != nullptr, 6);
+  LLMC_CHECK_ARG(U_out != nullptr && ldu >= K, 9);
+  LLMC_CHECK_ARG(workspace != nullptr && (((uintptr_t)workspace) & 255) == 0, 11);
+  LLMC_CHECK_ARG(workspace_bytes >= llmc_gptq_hinv_grouped_workspace_bytes(n, K), 12);
+  hipStream_t st = (hipStream_t)stream;
+  const int Kp = (int)round_up(K, NB);
+  const int64_t mat = (int64_t)Kp * Kp;
+  LLMC_CHECK_ARG((int64_t)n * (Kp / 128 + 1) < 65535, 3);  // deepest GEMM batch in one grid dimension
+
+  char* wp = (char*)workspace;
+  HinvItem* items = (HinvItem*)wp; wp += round_up(n * (int64_t)sizeof(HinvItem), 256);
+  HinvScalars* sc = (HinvScalars*)wp; wp += round_up(n * (int64_t)sizeof(HinvScalars), 256);
+  float* A = (float*)wp;
+  float* T = A + (int64_t)n * mat;
+  std::vector<HinvItem> host(n);
+  for (int b = 0; b < n; ++b) {
+    LLMC_CHECK_ARG(H[b] != nullptr && divisors[b] != 0.f, 1);
+    host[b].H = H[b];
+    host[b].perm = perm ? perm[b] : nullptr;
+    host[b].dead = dead_out ? dead_out + (int64_t)b * K : nullptr;
+    host[b].U = U_out + (int64_t)b * K * ldu;
+    host[b].div = divisors[b];
+    host[b].pad = 0;
+  }
+  // pageable source: the copy has read `host` when the call returns
+  hipError_t me = hipMemcpyAsync(items, host.data(), n * sizeof(HinvItem), hipMemcpyHostToDevice, st);
+  if (me != hipSuccess) return 1000 + (int)me;
+
+  hipLaunchKernelGGL(hinv_stats_kernel, dim3(n), dim3(256), 0, st, (const float*)nullptr, ldh, (int)K,
+                     (const int32_t*)nullptr, 1.f, percdamp, (uint8_t*)nullptr, sc, (const HinvItem*)items);
+  LLMC_LAUNCH_STATUS();
+  hipLaunchKernelGGL(hinv_copyin_kernel, dim3((Kp + 255) / 256, Kp, n), dim3(256), 0, st, (const float*)nullptr, ldh,
+                     (int)K, Kp, (const int32_t*)nullptr, 1.f, sc, A, (const HinvItem*)items);
+  LLMC_LAUNCH_STATUS();
+
+  const int NBO = Kp >= 8192 ? 512 : 256;
+  for (int k0 = 0; k0 < Kp; k0 += NBO) {
+    const int pw = (Kp - k0) < NBO ? (Kp - k0) : NBO;
+    for (int kk = 0; kk < pw; kk += NB) {
+      const int c0 = k0 + kk;
+      hipLaunchKernelGGL(potf2_inv_kernel, dim3(n), dim3(256), 0, st, A, Kp, c0, (int)K, sc);
+      LLMC_LAUNCH_STATUS();
+      const int M = Kp - c0 - NB;
+      if (M <= 0) break;
+      float* A21 = A + (int64_t)(c0 + NB) * Kp + c0;
+      GemmF32 g = {};
+      g.A = A21; g.lda = Kp; g.B = A + (int64_t)c0 * Kp + c0; g.ldb = Kp; g.C = A21; g.ldc = Kp;
+      g.M = M; g.N = NB; g.Kc = NB; g.alpha = 1.f; g.beta = 0.f; g.trans_b = 1;
+      g.batch = n; g.stride_a = mat; g.stride_b = mat; g.stride_c = mat;
+      int rc = llmc_gemm_f32(g, st);
+      if (rc) return rc;
+      const int nrem = k0 + pw - (c0 + NB);
+      if (nrem > 0) {
+        GemmF32 u = {};
+        u.A = A21; u.lda = Kp; u.B = A21; u.ldb = Kp; u.C = A + (int64_t)(c0 + NB) * Kp + c0 + NB; u.ldc = Kp;
+        u.M = M; u.N = nrem; u.Kc = NB; u.alpha = -1.f; u.beta = 1.f; u.trans_b = 1; u.c_lower = 1;
+        u.batch = n; u.stride_a = mat; u.stride_b = mat; u.stride_c = mat;
+        rc = llmc_gemm_f32(u, st);
+        if (rc) return rc;
+      }
+    }
+    const int M2 = Kp - (k0 + pw);
+    if (M2 > 0) {
+      float* P = A + (int64_t)(k0 + pw) * Kp + k0;
+      GemmF32 t = {};
+      t.A = P; t.lda = Kp; t.B = P; t.ldb = Kp; t.C = A + (int64_t)(k0 + pw) * ((int64_t)Kp + 1); t.ldc = Kp;
+      t.M = M2; t.N = M2; t.Kc = pw; t.alpha = -1.f; t.beta = 1.f; t.trans_b = 1; t.c_lower = 1;
+      t.batch = n; t.stride_a = mat; t.stride_b = mat; t.stride_c = mat;
+      const int rc = llmc_gemm_f32(t, st);
+      if (rc) return rc;
+    }
+  }
+
+  for (int64_t s = NB; s < Kp; s *= 2) {
+    const int64_t full = Kp / (2 * s);
+    const int64_t rem = Kp % (2 * s);
+    const int64_t step = 2 * s * ((int64_t)Kp + 1);
+    for (int part = 0; part < 2; ++part) {
+      int64_t base, s2, batch;
+      if (part == 0) {
+        base = 0; s2 = s; batch = full;
+      } else {
+        base = full * 2 * s; s2 = rem - s; batch = 1;
+      }
+      if (batch <= 0 || s2 <= 0) continue;
+      float* X11 = A + base * ((int64_t)Kp + 1);
+      float* X22 = X11 + s * ((int64_t)Kp + 1);
+      float* L21 = X11 + s * (int64_t)Kp;
+      GemmF32 g = {};
+      g.A = L21; g.lda = Kp; g.B = X11; g.ldb = Kp; g.C = T; g.ldc = s;
+      g.M = (int)s2; g.N = (int)s; g.Kc = (int)s; g.alpha = 1.f; g.beta = 0.f; g.b_lower_tri = 1;
+      g.batch = (int)batch; g.stride_a = step; g.stride_b = step; g.stride_c = s * s;
+      g.batch2 = n; g.stride2_a = mat; g.stride2_b = mat; g.stride2_c = mat / 4;
+      int rc = llmc_gemm_f32(g, st);
+      if (rc) return rc;
+      GemmF32 h = {};
+      h.A = X22; h.lda = Kp; h.B = T; h.ldb = s; h.C = L21; h.ldc = Kp;
+      h.M = (int)s2; h.N = (int)s; h.Kc = (int)s2; h.alpha = -1.f; h.beta = 0.f; h.a_lower_tri = 1;
+      h.batch = (int)batch; h.stride_a = step; h.stride_b = s * s; h.stride_c = step;
+      h.batch2 = n; h.stride2_a = mat; h.stride2_b = mat / 4; h.stride2_c = mat;
+      rc = llmc_gemm_f32(h, st);
+      if (rc) return rc;
+    }
+  }
+
+  hipLaunchKernelGGL(hinv_copyout_kernel, dim3((unsigned)((K + 255) / 256), (unsigned)K, (unsigned)n), dim3(256), 0, st,
+                     A, Kp, (int)K, sc, (float*)nullptr, ldu, info_out, (const HinvItem*)items);
   LLMC_LAUNCH_STATUS();
   return 0;
 }

@@ -23,6 +23,10 @@ struct GemmF32 {
   // batching over blockIdx.z
   int batch;
   int64_t stride_a, stride_b, stride_c;
+  // second batch level (independent problems, each with `batch` blocks): blockIdx.z = b + batch * b2;
+  // 0 or 1 = none
+  int batch2;
+  int64_t stride2_a, stride2_b, stride2_c;
 };
 
 // enqueue on `st`; returns 0 or 1000 + hipError_t

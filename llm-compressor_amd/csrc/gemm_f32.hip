@@ -196,9 +196,10 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32 g, int vec) {
   __shared__ float Bs[2 * BK * (BN + 4)];
   const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
   if (g.c_lower && n0 > m0 + BM - 1) return;
-  const float* A = g.A + (int64_t)blockIdx.z * g.stride_a;
-  const float* B = g.B + (int64_t)blockIdx.z * g.stride_b;
-  float* C = g.C + (int64_t)blockIdx.z * g.stride_c;
+  const int b1 = (int)blockIdx.z % g.batch, b2 = (int)blockIdx.z / g.batch;
+  const float* A = g.A + (int64_t)b1 * g.stride_a + (int64_t)b2 * g.stride2_a;
+  const float* B = g.B + (int64_t)b1 * g.stride_b + (int64_t)b2 * g.stride2_b;
+  float* C = g.C + (int64_t)b1 * g.stride_c + (int64_t)b2 * g.stride2_c;
   const int k_begin = g.b_lower_tri ? (n0 / BK) * BK : 0;
   int k_end = g.Kc;
   if (g.a_lower_tri && m0 + BM < k_end) k_end = m0 + BM;
@@ -217,18 +218,20 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32 g, int vec) {
 
 int llmc_gemm_f32(const GemmF32& g, hipStream_t st) {
   if (g.M <= 0 || g.N <= 0 || g.batch <= 0) return 0;
+  const int nb2 = g.batch2 > 1 ? g.batch2 : 1;
   const int vec = ((g.lda & 3) == 0 && (g.ldb & 3) == 0 && (((uintptr_t)g.A | (uintptr_t)g.B) & 15) == 0 &&
-                   (g.stride_a & 3) == 0 && (g.stride_b & 3) == 0 && (g.Kc & 3) == 0)
+                   (g.stride_a & 3) == 0 && (g.stride_b & 3) == 0 && (g.Kc & 3) == 0 &&
+                   (nb2 == 1 || ((g.stride2_a & 3) == 0 && (g.stride2_b & 3) == 0)))
                       ? 1
                       : 0;
   // 128x128 tiles when they still give the chip enough workgroups, 64x64 otherwise
-  const int64_t t128 = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * g.batch;
+  const int64_t t128 = (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * g.batch * nb2;
   const bool big = t128 >= 256 && g.M >= 128 && g.N >= 128;
   const int bt = big ? 128 : 64;
   // every tile unconditional?  (a_lower_tri / b_lower_tri cut the contraction at tile edges, which
   // are multiples of BK for both tile sizes)
   const bool all_fast = vec && g.M % bt == 0 && g.N % bt == 0 && g.Kc % BK == 0;
-  dim3 grid((g.N + bt - 1) / bt, (g.M + bt - 1) / bt, g.batch);
+  dim3 grid((g.N + bt - 1) / bt, (g.M + bt - 1) / bt, g.batch * nb2);
 #define LLMC_GEMM(BT, TB, AF) hipLaunchKernelGGL((gemm_f32_kernel<BT, BT, TB, AF>), grid, dim3(256), 0, st, g, vec)
   if (big) {
     if (g.trans_b) { if (all_fast) LLMC_GEMM(128, true, true); else LLMC_GEMM(128, true, false); }

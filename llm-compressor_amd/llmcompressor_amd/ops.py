@@ -327,6 +327,38 @@ def gptq_hinv_(H: torch.Tensor, perm=None, divisor: float = 1.0, percdamp: float
     return H, dead, info
 
 
+def gptq_hinv_grouped(Hs, perms=None, divisors=None, percdamp: float = 0.01):
+    """gptq_hinv_ for n Hessians of one width in lock-step.  Hs: list of fp32 [K,K] (left untouched); perms:
+    int32 [n,K] tensor or None; divisors: list of floats.  Returns (U [n,K,K] fp32, dead [n,K] uint8, info [n])."""
+    import ctypes
+
+    n = len(Hs)
+    H0 = Hs[0]
+    _require_gpu(H0)
+    K = H0.shape[0]
+    for H in Hs:
+        assert H.dtype == torch.float32 and H.shape == (K, K) and H.stride(1) == 1 and H.stride(0) == H0.stride(0)
+        assert H.device == H0.device
+    U = torch.empty((n, K, K), dtype=torch.float32, device=H0.device)
+    dead = torch.empty((n, K), dtype=torch.uint8, device=H0.device)
+    info = torch.zeros(n, dtype=torch.int32, device=H0.device)
+    hp = (ctypes.c_void_p * n)(*[H.data_ptr() for H in Hs])
+    pp = None
+    if perms is not None:
+        perms = perms.to(torch.int32).contiguous()
+        assert perms.shape == (n, K)
+        pp = (ctypes.c_void_p * n)(*[perms.data_ptr() + 4 * K * b for b in range(n)])
+    dv = (ctypes.c_float * n)(*[float(d) for d in (divisors if divisors is not None else [1.0] * n)])
+    nbytes = _lib.lib().llmc_gptq_hinv_grouped_workspace_bytes(n, K)
+    ws = _workspace(H0.device, nbytes)
+    with torch.cuda.device(H0.device):
+        rc = _lib.lib().llmc_gptq_hinv_grouped(hp, H0.stride(0), n, K, pp, dv, float(percdamp), dead.data_ptr(),
+                                              U.data_ptr(), K, ws.data_ptr(), ws.numel(), info.data_ptr(),
+                                              _stream(H0))
+    _lib.check(rc, "llmc_gptq_hinv_grouped")
+    return U, dead, info
+
+
 def gptq_quantize(weight, U, scale, zero_point, fmt: int, bits: int, row_div: int, scale_row_stride: int,
                   g_idx=None, perm=None, dead=None, global_scale=None, blocksize: int = 128):
     """The GPTQ column loop.  Returns (quantised-dequantised weight in weight.dtype, loss fp32 [1])."""

@@ -237,3 +237,33 @@ def test_gptq_full_size_properties(R, K, T):
     got = Ud.t() @ (Ud @ Hp[:, cols])
     want = torch.eye(K, device="cuda", dtype=torch.float64)[:, cols]
     assert (got - want).abs().max().item() < 5e-3
+
+
+@pytest.mark.parametrize("K,n,actorder", [(768, 5, False), (2048, 3, True), (200, 4, True)])
+def test_hinv_grouped_is_bit_identical_to_single_calls(K, n, actorder):
+    """llmc_gptq_hinv_grouped: the lock-step chain over n problems gives exactly the factors, dead-column
+    flags and failure flags of n single calls (one problem is made indefinite, one has dead columns)."""
+    from llmcompressor_amd import ops
+
+    torch.manual_seed(K + n)
+    Hs = []
+    for b in range(n):
+        x = torch.randn(3 * K if b != 1 else K // 2, K, device="cuda").bfloat16()
+        H = torch.zeros(K, K, device="cuda")
+        ops.hessian_accumulate_(H, x)
+        if b == 2:
+            H[5, :] = 0
+            H[:, 5] = 0
+        if b == n - 1:
+            H = -H  # not positive definite: identity fallback, info != 0
+        Hs.append(H)
+    perms = torch.stack([torch.argsort(torch.diagonal(H), descending=True) for H in Hs]).to(torch.int32) if actorder else None
+    divs = [float(b + 1) for b in range(n)]
+    U, dead, info = ops.gptq_hinv_grouped(Hs, perms, divs, 0.01)
+    for b in range(n):
+        Hc = Hs[b].clone()
+        Ub, db, ib = ops.gptq_hinv_(Hc, perms[b] if actorder else None, divisor=divs[b], percdamp=0.01)
+        assert torch.equal(U[b], Ub), b
+        assert torch.equal(dead[b], db)
+        assert int(info[b]) == int(ib)
+    assert int(info[n - 1]) != 0 and int(info[0]) == 0
