@@ -277,6 +277,21 @@ int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R, int64_t K
                        void* out_weight, int64_t ldo, float* loss_out, void* workspace,
                        int64_t workspace_bytes, void* stream);
 
+/* Grouped form of llmc_gptq_quantize for n problems of one shape and scheme (the expert Linears of an MoE
+ * layer) in lock-step.  weight, scale, zero_point, global_scale, g_idx and out_weight are HOST arrays of n
+ * device pointers (zero_point / global_scale / g_idx may be NULL as in the single call); U is device
+ * [n][K][ldu] with problem stride u_stride (as written by llmc_gptq_hinv_grouped), perm device [n, K] int32
+ * or NULL, dead device [n, K] bytes or NULL, loss_out device [n].  Results are bit-identical to n single calls. */
+int64_t llmc_gptq_quantize_grouped_workspace_bytes(int64_t n, int64_t R, int64_t K);
+int llmc_gptq_quantize_grouped(const void* const* weight, int32_t w_dtype, int32_t n, int64_t R, int64_t K,
+                               int64_t ldw, const float* U, int64_t ldu, int64_t u_stride,
+                               const int32_t* perm, const uint8_t* dead, const void* const* scale,
+                               int32_t scale_dtype, const int8_t* const* zero_point,
+                               const float* const* global_scale, const int32_t* const* g_idx,
+                               int64_t row_div, int64_t scale_row_stride, int32_t fmt, int32_t num_bits,
+                               int32_t blocksize, void* const* out_weight, int64_t ldo, float* loss_out,
+                               void* workspace, int64_t workspace_bytes, void* stream);
+
 /* ---- SparseGPT (a "next" row: the same Hessian / Cholesky / column-loop skeleton) ----------
  * Replaces the loop of sparsify_weight (src/llmcompressor/modifiers/pruning/sparsegpt/
  * sgpt_sparsify.py:125-213); the factor U comes from llmc_gptq_hinv (:97-118 are the same

@@ -8,6 +8,8 @@
 // quantises it, forms err = (w - q)/U[i][i] and subtracts err * U[i][c] from its
 // own 8 columns (U is zero below the diagonal, so no masking is needed).
 // After the block, W[:, i2:] -= Err * U[i1:i2, i2:] runs as an fp32 MFMA GEMM.
+#include <vector>
+
 #include "gemm_f32.h"
 #include "qformat.h"
 
@@ -19,11 +21,29 @@ constexpr int TEAM = 16;      // lanes per row
 constexpr int CPL = GB / TEAM;  // columns per lane (8)
 constexpr int ROWS_PER_WG = 256 / TEAM;
 
+// One problem of a grouped call (llmc_gptq_quantize_grouped); the kernels pick theirs by a grid index and
+// find its work buffers at a fixed stride behind those of problem 0.
+struct GptqItem {
+  const void* weight;
+  const void* scale;
+  const int8_t* zp;
+  const float* gscale;
+  const int32_t* g_idx;
+  void* out;
+};
+
 template <int WDT>
 __global__ __launch_bounds__(256) void gptq_prepare_w_kernel(const void* __restrict__ w, int64_t ldw, int R,
                                                              int K, const int32_t* __restrict__ perm,
                                                              const uint8_t* __restrict__ dead,
-                                                             float* __restrict__ Wf) {
+                                                             float* __restrict__ Wf,
+                                                             const GptqItem* __restrict__ items = nullptr) {
+  if (items) {  // grouped: problem blockIdx.z, perm / dead rows of [n,K] arrays
+    w = items[blockIdx.z].weight;
+    if (perm) perm += (int64_t)blockIdx.z * K;
+    if (dead) dead += (int64_t)blockIdx.z * K;
+    Wf += (int64_t)blockIdx.z * R * K;
+  }
   const int c = blockIdx.x * 256 + threadIdx.x;
   const int r = blockIdx.y;
   if (c >= K) return;
@@ -50,11 +70,23 @@ struct GptqBlockParams {
   float* E;         // scaled errors of this block, row stride ldE
   int ldE;
   float* loss_rows; // [R]
+  // grouped call: problem blockIdx.y takes scale / zp / gscale / g_idx from items and its Wf, U, E and
+  // loss rows at these strides (in elements)
+  const GptqItem* items;
+  int64_t u_stride;
 };
 
 template <int FMT, int SD, bool HAS_ZP>
 __global__ __launch_bounds__(256) void gptq_block_kernel(GptqBlockParams p) {
   extern __shared__ __attribute__((aligned(16))) float Hs[];  // [GB][GB], zero outside the upper triangle
+  if (p.items) {
+    const GptqItem it = p.items[blockIdx.y];
+    p.scale = it.scale; p.zp = it.zp; p.gscale = it.gscale; p.g_idx = it.g_idx;
+    p.Wf += (int64_t)blockIdx.y * p.R * p.K;
+    p.U += (int64_t)blockIdx.y * p.u_stride;
+    p.E += (int64_t)blockIdx.y * p.R * p.ldE;
+    p.loss_rows += (int64_t)blockIdx.y * p.R;
+  }
   const int tid = threadIdx.x;
   for (int e = tid; e < GB * GB; e += 256) {
     const int i = e / GB, c = e % GB;
@@ -137,7 +169,13 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(GptqBlockParams p) {
 template <int WDT>
 __global__ __launch_bounds__(256) void gptq_finalize_kernel(const float* __restrict__ Wf, int R, int K,
                                                             const int32_t* __restrict__ perm,
-                                                            void* __restrict__ out, int64_t ldo) {
+                                                            void* __restrict__ out, int64_t ldo,
+                                                            const GptqItem* __restrict__ items = nullptr) {
+  if (items) {
+    out = items[blockIdx.z].out;
+    if (perm) perm += (int64_t)blockIdx.z * K;
+    Wf += (int64_t)blockIdx.z * R * K;
+  }
   const int c = blockIdx.x * 256 + threadIdx.x;
   const int r = blockIdx.y;
   if (c >= K) return;
@@ -147,6 +185,8 @@ __global__ __launch_bounds__(256) void gptq_finalize_kernel(const float* __restr
 
 __global__ __launch_bounds__(256) void sum_rows_kernel(const float* __restrict__ v, int n, float* out) {
   __shared__ float red[4];
+  v += (int64_t)blockIdx.x * n;  // grouped call: one workgroup per problem
+  out += blockIdx.x;
   float s = 0.f;
   for (int i = threadIdx.x; i < n; i += 256) s += v[i];
   s = wave_sum(s);
@@ -589,6 +629,7 @@ extern "C" int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R
   p.fmt = fmt; p.bits = fmt == LLMC_FMT_INT ? num_bits : (fmt == LLMC_FMT_FP8 ? 8 : 4);
   p.sd = global_scale ? LLMC_F32 : scale_dtype;
   p.E = E; p.loss_rows = loss_rows;
+  p.items = nullptr; p.u_stride = 0;
 
   const int smem = GB * GB * 4;
   void (*kern)(GptqBlockParams) = nullptr;
@@ -652,6 +693,147 @@ extern "C" int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R
   LLMC_LAUNCH_STATUS();
   if (loss_out) {
     hipLaunchKernelGGL(sum_rows_kernel, dim3(1), dim3(256), 0, st, loss_rows, (int)R, loss_out);
+    LLMC_LAUNCH_STATUS();
+  }
+  return 0;
+}
+
+// ---- grouped form: n problems of one shape in lock-step (the expert Linears of an MoE layer) ---------
+// Every kernel of llmc_gptq_quantize is launched once for all problems (one more grid dimension, GEMM batch):
+// the serial chain of column blocks is as long as one problem's while each launch carries n times the rows.
+
+extern "C" int64_t llmc_gptq_quantize_grouped_workspace_bytes(int64_t n, int64_t R, int64_t K) {
+  return align256(n * (int64_t)sizeof(GptqItem)) + align256(n * R * K * 4) + align256(n * R * GROUP * GB * 4) +
+         align256(n * R * 4);
+}
+
+extern "C" int llmc_gptq_quantize_grouped(const void* const* weight, int32_t w_dtype, int32_t n, int64_t R, int64_t K,
+                                          int64_t ldw, const float* U, int64_t ldu, int64_t u_stride,
+                                          const int32_t* perm, const uint8_t* dead, const void* const* scale,
+                                          int32_t scale_dtype, const int8_t* const* zero_point,
+                                          const float* const* global_scale, const int32_t* const* g_idx,
+                                          int64_t row_div, int64_t scale_row_stride, int32_t fmt, int32_t num_bits,
+                                          int32_t blocksize, void* const* out_weight, int64_t ldo, float* loss_out,
+                                          void* workspace, int64_t workspace_bytes, void* stream) {
+  LLMC_CHECK_ARG(weight != nullptr, 1);
+  LLMC_CHECK_ARG(w_dtype >= 0 && w_dtype <= 2, 2);
+  LLMC_CHECK_ARG(n >= 0 && n <= 4096, 3);
+  if (n == 0) return 0;
+  LLMC_CHECK_ARG(R > 0 && R < (1ll << 31), 4);
+  LLMC_CHECK_ARG(K > 0 && K < (1ll << 31) && ldw >= K, 5);
+  LLMC_CHECK_ARG(U != nullptr && ldu >= K && u_stride >= K * ldu, 7);
+  LLMC_CHECK_ARG(scale != nullptr, 12);
+  LLMC_CHECK_ARG(scale_dtype >= 0 && scale_dtype <= 2, 13);
+  LLMC_CHECK_ARG(row_div > 0 && scale_row_stride >= 0, 17);
+  LLMC_CHECK_ARG(fmt >= 0 && fmt <= 2, 19);
+  LLMC_CHECK_ARG(fmt != LLMC_FMT_INT || (num_bits >= 2 && num_bits <= 8), 20);
+  LLMC_CHECK_ARG(blocksize > 0, 21);
+  LLMC_CHECK_ARG(out_weight != nullptr && ldo >= K, 22);
+  LLMC_CHECK_ARG(workspace != nullptr && (((uintptr_t)workspace) & 255) == 0, 25);
+  LLMC_CHECK_ARG(workspace_bytes >= llmc_gptq_quantize_grouped_workspace_bytes(n, R, K), 26);
+  LLMC_CHECK_ARG(n < 65535 && (K + 255) / 256 < 65535, 3);
+  hipStream_t st = (hipStream_t)stream;
+  const int bs = blocksize > GB ? GB : blocksize;
+
+  char* wp = (char*)workspace;
+  GptqItem* items = (GptqItem*)wp; wp += align256(n * (int64_t)sizeof(GptqItem));
+  float* Wf = (float*)wp; wp += align256(n * R * K * 4);
+  float* E = (float*)wp; wp += align256(n * R * GROUP * GB * 4);
+  float* loss_rows = (float*)wp;
+  std::vector<GptqItem> host(n);
+  for (int b = 0; b < n; ++b) {
+    LLMC_CHECK_ARG(weight[b] != nullptr && scale[b] != nullptr && out_weight[b] != nullptr, 1);
+    host[b].weight = weight[b];
+    host[b].scale = scale[b];
+    host[b].zp = zero_point ? zero_point[b] : nullptr;
+    host[b].gscale = global_scale ? global_scale[b] : nullptr;
+    host[b].g_idx = g_idx ? g_idx[b] : nullptr;
+    host[b].out = out_weight[b];
+  }
+  hipError_t me = hipMemcpyAsync(items, host.data(), n * sizeof(GptqItem), hipMemcpyHostToDevice, st);
+  if (me != hipSuccess) return 1000 + (int)me;
+
+  dim3 grid3((unsigned)((K + 255) / 256), (unsigned)R, (unsigned)n);
+#define LLMC_PREP(DT)                                                                                         \
+  hipLaunchKernelGGL((gptq_prepare_w_kernel<DT>), grid3, dim3(256), 0, st, (const void*)nullptr, ldw, (int)R, \
+                     (int)K, perm, dead, Wf, (const GptqItem*)items)
+  if (w_dtype == LLMC_BF16) LLMC_PREP(LLMC_BF16);
+  else if (w_dtype == LLMC_F16) LLMC_PREP(LLMC_F16);
+  else LLMC_PREP(LLMC_F32);
+#undef LLMC_PREP
+  LLMC_LAUNCH_STATUS();
+  hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n * R + 255) / 256)), dim3(256), 0, st, loss_rows, n * R);
+  LLMC_LAUNCH_STATUS();
+
+  GptqBlockParams p;
+  p.Wf = Wf; p.R = (int)R; p.K = (int)K; p.U = U; p.ldu = ldu;
+  p.scale = nullptr; p.scale_dt = scale_dtype; p.zp = nullptr; p.gscale = nullptr; p.g_idx = nullptr;
+  p.row_div = row_div; p.srow = scale_row_stride;
+  p.fmt = fmt; p.bits = fmt == LLMC_FMT_INT ? num_bits : (fmt == LLMC_FMT_FP8 ? 8 : 4);
+  p.sd = global_scale ? LLMC_F32 : scale_dtype;
+  p.E = E; p.loss_rows = loss_rows;
+  p.items = items; p.u_stride = u_stride;
+
+  const int smem = GB * GB * 4;
+  void (*kern)(GptqBlockParams) = nullptr;
+  const bool hz = zero_point != nullptr;
+#define LLMC_PICK(F, S)                                                         \
+  if (p.fmt == F && p.sd == S) kern = hz ? gptq_block_kernel<F, S, true> : gptq_block_kernel<F, S, false>;
+  LLMC_PICK(LLMC_FMT_INT, LLMC_BF16)
+  LLMC_PICK(LLMC_FMT_INT, LLMC_F16)
+  LLMC_PICK(LLMC_FMT_INT, LLMC_F32)
+  LLMC_PICK(LLMC_FMT_FP8, LLMC_BF16)
+  LLMC_PICK(LLMC_FMT_FP8, LLMC_F16)
+  LLMC_PICK(LLMC_FMT_FP8, LLMC_F32)
+  LLMC_PICK(LLMC_FMT_FP4, LLMC_BF16)
+  LLMC_PICK(LLMC_FMT_FP4, LLMC_F16)
+  LLMC_PICK(LLMC_FMT_FP4, LLMC_F32)
+#undef LLMC_PICK
+  if (kern == nullptr) return -19;
+  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+  if (e != hipSuccess) return 1000 + (int)e;
+  const unsigned wgs = (unsigned)((R + ROWS_PER_WG - 1) / ROWS_PER_WG);
+  const int ldE = GROUP * GB;
+  p.ldE = ldE;
+  for (int64_t g0 = 0; g0 < K; g0 += (int64_t)GROUP * bs) {
+    const int64_t gend = (g0 + (int64_t)GROUP * bs) < K ? g0 + (int64_t)GROUP * bs : K;
+    for (int64_t i1 = g0; i1 < gend; i1 += bs) {
+      const int count = (int)((gend - i1) < bs ? (gend - i1) : bs);
+      p.i1 = (int)i1;
+      p.count = count;
+      p.E = E + (i1 - g0);
+      hipLaunchKernelGGL(kern, dim3(wgs, (unsigned)n), dim3(256), smem, st, p);
+      LLMC_LAUNCH_STATUS();
+      const int64_t i2 = i1 + count;
+      if (i2 < gend) {
+        GemmF32 g = {};
+        g.A = p.E; g.lda = ldE; g.B = U + i1 * ldu + i2; g.ldb = ldu; g.C = Wf + i2; g.ldc = K;
+        g.M = (int)R; g.N = (int)(gend - i2); g.Kc = count; g.alpha = -1.f; g.beta = 1.f;
+        g.batch = n; g.stride_a = R * (int64_t)ldE; g.stride_b = u_stride; g.stride_c = R * K;
+        const int rc = llmc_gemm_f32(g, st);
+        if (rc) return rc;
+      }
+    }
+    if (gend < K) {
+      GemmF32 g = {};
+      g.A = E; g.lda = ldE; g.B = U + g0 * ldu + gend; g.ldb = ldu; g.C = Wf + gend; g.ldc = K;
+      g.M = (int)R; g.N = (int)(K - gend); g.Kc = (int)(gend - g0); g.alpha = -1.f; g.beta = 1.f;
+      g.batch = n; g.stride_a = R * (int64_t)ldE; g.stride_b = u_stride; g.stride_c = R * K;
+      const int rc = llmc_gemm_f32(g, st);
+      if (rc) return rc;
+    }
+  }
+
+#define LLMC_FIN(DT)                                                                                          \
+  hipLaunchKernelGGL((gptq_finalize_kernel<DT>), grid3, dim3(256), 0, st, Wf, (int)R, (int)K, perm, (void*)nullptr, \
+                     ldo, (const GptqItem*)items)
+  if (w_dtype == LLMC_BF16) LLMC_FIN(LLMC_BF16);
+  else if (w_dtype == LLMC_F16) LLMC_FIN(LLMC_F16);
+  else LLMC_FIN(LLMC_F32);
+#undef LLMC_FIN
+  LLMC_LAUNCH_STATUS();
+  if (loss_out) {
+    hipLaunchKernelGGL(sum_rows_kernel, dim3((unsigned)n), dim3(256), 0, st, loss_rows, (int)R, loss_out);
     LLMC_LAUNCH_STATUS();
   }
   return 0;

@@ -54,6 +54,9 @@ SIGNATURES = {
     "llmc_hessian_accumulate_grouped": [_P, _I64, _P, _I64, _P, _I32, _I64, _I32, _F32, _I32, _P],
     "llmc_gptq_hinv_grouped_workspace_bytes": [_I64, _I64],
     "llmc_gptq_hinv_grouped": [_P, _I64, _I32, _I64, _P, _P, _F32, _P, _P, _I64, _P, _I64, _P, _P],
+    "llmc_gptq_quantize_grouped_workspace_bytes": [_I64, _I64, _I64],
+    "llmc_gptq_quantize_grouped": [_P, _I32, _I32, _I64, _I64, _I64, _P, _I64, _I64, _P, _P, _P, _I32, _P, _P, _P, _I64,
+                                   _I64, _I32, _I32, _I32, _P, _I64, _P, _P, _I64, _P],
     "llmc_sparsegpt_workspace_bytes": [_I64, _I64],
     "llmc_sparsegpt_sparsify": [_P, _I32, _I64, _I64, _I64, _P, _I64, _P, ctypes.c_double, _I32, _I32, _I32, _I32, _P,
                                 _I64, _P, _P, _I64, _P],
@@ -102,6 +105,7 @@ RESTYPES = {
     "llmc_mse_workspace_bytes": ctypes.c_int64,
     "llmc_gptq_quantize_workspace_bytes": ctypes.c_int64,
     "llmc_sparsegpt_workspace_bytes": ctypes.c_int64,
+    "llmc_gptq_quantize_grouped_workspace_bytes": ctypes.c_int64,
     "llmc_gptq_hinv_grouped_workspace_bytes": ctypes.c_int64,
     "llmc_sumsq_workspace_bytes": ctypes.c_int64,
 }

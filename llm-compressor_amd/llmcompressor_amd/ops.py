@@ -387,6 +387,53 @@ def gptq_quantize(weight, U, scale, zero_point, fmt: int, bits: int, row_div: in
     return out, loss
 
 
+def gptq_quantize_grouped(weights, U, scales, zero_points, fmt: int, bits: int, row_div: int, scale_row_stride: int,
+                          g_idxs=None, perms=None, dead=None, global_scales=None, blocksize: int = 128):
+    """gptq_quantize for n weights of one shape in lock-step.  weights / scales / zero_points / g_idxs /
+    global_scales: lists of n tensors (the last three may be None); U [n,K,K] fp32; perms [n,K] int32 or None;
+    dead [n,K] uint8 or None.  Returns (list of quantised-dequantised weights, loss fp32 [n])."""
+    import ctypes
+
+    n = len(weights)
+    w0 = weights[0]
+    _require_gpu(w0, U)
+    R, K = w0.shape
+    keep = []
+
+    def ptrs(ts, dtype=None):
+        if ts is None:
+            return None
+        arr = (ctypes.c_void_p * n)()
+        for i, t in enumerate(ts):
+            t = t.contiguous() if dtype is None else t.to(dtype).contiguous()
+            keep.append(t)
+            arr[i] = t.data_ptr()
+        return arr
+
+    for w in weights:
+        assert w.shape == (R, K) and w.dtype == w0.dtype and w.stride(1) == 1 and w.stride(0) == w0.stride(0)
+    assert U.shape == (n, K, K) and U.dtype == torch.float32 and U.is_contiguous()
+    for s_ in scales:
+        assert s_.dtype == scales[0].dtype and s_.numel() == scales[0].numel()
+    if perms is not None:
+        perms = perms.to(torch.int32).contiguous()
+    outs = [torch.empty((R, K), dtype=w0.dtype, device=w0.device) for _ in range(n)]
+    loss = torch.empty(n, dtype=torch.float32, device=w0.device)
+    nbytes = _lib.lib().llmc_gptq_quantize_grouped_workspace_bytes(n, R, K)
+    ws = _workspace(w0.device, nbytes)
+    wp = (ctypes.c_void_p * n)(*[w.data_ptr() for w in weights])
+    op = (ctypes.c_void_p * n)(*[o.data_ptr() for o in outs])
+    sp, zp = ptrs(scales), ptrs(zero_points)
+    gp, ip = ptrs(global_scales), ptrs(g_idxs, torch.int32)
+    with torch.cuda.device(w0.device):
+        rc = _lib.lib().llmc_gptq_quantize_grouped(
+            wp, _dt(w0), n, R, K, w0.stride(0), U.data_ptr(), K, K * K, _ptr(perms), _ptr(dead), sp, _dt(keep[0]),
+            zp, gp, ip, row_div, scale_row_stride, fmt, bits, blocksize, op, K, loss.data_ptr(), ws.data_ptr(),
+            ws.numel(), _stream(w0))
+    _lib.check(rc, "llmc_gptq_quantize_grouped")
+    return outs, loss
+
+
 def sparsegpt_sparsify(weight, U, sparsity: float, prune_n: int = 0, prune_m: int = 0, dead=None,
                        blocksize: int = 128, preserve_sparsity_mask: bool = False):
     """The SparseGPT column loop on the factor U of gptq_hinv_.  Returns (pruned weight in weight.dtype,

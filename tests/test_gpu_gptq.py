@@ -267,3 +267,52 @@ def test_hinv_grouped_is_bit_identical_to_single_calls(K, n, actorder):
         assert torch.equal(dead[b], db)
         assert int(info[b]) == int(ib)
     assert int(info[n - 1]) != 0 and int(info[0]) == 0
+
+
+@pytest.mark.parametrize("R,K,n,fmt_case", [(96, 768, 5, "int4_sym"), (64, 512, 4, "int4_asym_actorder"),
+                                            (48, 256, 3, "nvfp4")])
+def test_gptq_quantize_grouped_is_bit_identical_to_single_calls(R, K, n, fmt_case):
+    """llmc_gptq_quantize_grouped on the factors of llmc_gptq_hinv_grouped: identical weights and losses to n
+    single calls (int4 symmetric g128, int4 asymmetric g64 with activation ordering, NVFP4 with global scales)."""
+    from llmcompressor_amd import ops
+
+    torch.manual_seed(R + K)
+    Ws = [(torch.randn(R, K, device="cuda") * 0.05).bfloat16() for _ in range(n)]
+    Hs = []
+    for b in range(n):
+        x = torch.randn(2 * K, K, device="cuda").bfloat16()
+        H = torch.zeros(K, K, device="cuda")
+        ops.hessian_accumulate_(H, x)
+        Hs.append(H)
+    actorder = "actorder" in fmt_case
+    perms = torch.stack([torch.argsort(torch.diagonal(H), descending=True) for H in Hs]).to(torch.int32) if actorder else None
+    scales, zps, gss, gidx = [], [], [], []
+    for b, W in enumerate(Ws):
+        if fmt_case == "nvfp4":
+            mn, mx = ops.minmax_groups(W, 16)
+            gs = ops.global_scale_from_stats([(mn, mx)])
+            s, _, _ = ops.calculate_qparams(mn, mx, ops.FMT_FP4, 4, True, ops.SCALE_NVFP4, gs)
+            scales.append(s.float() if s.dtype not in (torch.float32, torch.bfloat16, torch.float16) else s)
+            gss.append(gs)
+            group = 16
+        else:
+            group = 64 if actorder else 128
+            mn, mx = ops.minmax_groups(W, group)
+            s, z, _ = ops.calculate_qparams(mn, mx, ops.FMT_INT, 4, not actorder)
+            scales.append(s)
+            zps.append(z.to(torch.int8))
+        g = torch.arange(K, dtype=torch.int32, device="cuda") // group
+        gidx.append(g[perms[b].long()] if actorder else g)
+    fmt = ops.FMT_FP4 if fmt_case == "nvfp4" else ops.FMT_INT
+    zp_arg = zps if actorder else None
+    gs_arg = gss if fmt_case == "nvfp4" else None
+    U, dead, info = ops.gptq_hinv_grouped(Hs, perms, [2.0] * n, 0.01)
+    assert int(info.abs().sum()) == 0
+    outs, loss = ops.gptq_quantize_grouped(Ws, U, scales, zp_arg, fmt, 4, 1, K // group, g_idxs=gidx, perms=perms,
+                                           dead=dead, global_scales=gs_arg)
+    for b in range(n):
+        ob, lb = ops.gptq_quantize(Ws[b], U[b], scales[b], zp_arg[b] if zp_arg else None, fmt, 4, 1, K // group,
+                                   g_idx=gidx[b], perm=perms[b] if actorder else None, dead=dead[b],
+                                   global_scale=gs_arg[b] if gs_arg else None)
+        assert torch.equal(outs[b], ob), b
+        assert torch.equal(loss[b:b + 1], lb)
