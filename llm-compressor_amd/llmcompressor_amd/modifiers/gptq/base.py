@@ -33,7 +33,7 @@ from ..quantization.calibration import observe, update_qparams
 from ..quantization.quantization import QuantizationMixin
 from ..utils.concurrent import run_on_streams
 from ..utils.hessian_staging import HessianStagingMixin
-from .gptq_quantize import accumulate_hessian, make_empty_hessian, quantize_weight
+from .gptq_quantize import accumulate_hessian, group_key, make_empty_hessian, quantize_weight, quantize_weight_group
 
 logger = logging.getLogger("llmcompressor_amd")
 
@@ -61,6 +61,9 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
         them into a staging buffer, and hand the kernel the list of buffers.  Taken only for contiguous
         bf16/f16 inputs whose token count is a multiple of 64; anything else is copied.  An input that is
         modified in place before its batch is accumulated raises at the flush (tensor version check)
+    :param group_min_modules: when at least this many Linears of one ``compress_module_list`` call share shape,
+        dtype and scheme (the experts of an MoE layer), they are quantised together in lock-step grouped kernels
+        (0 = never); ``group_max_bytes`` bounds the work buffers of one such call
     :param compress_concurrency: how many modules of one ``compress_module_list`` call are quantised at the
         same time, each on its own HIP stream (1 = one after the other, the reference's behaviour)
 
@@ -78,6 +81,8 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
     hessian_batch_tokens: int = 0
     share_identical_inputs: bool = False
     compress_concurrency: int = 4
+    group_min_modules: int = 8
+    group_max_bytes: int = 8 << 30
     stage_by_reference: bool = True
 
     _module_names: dict = PrivateAttr(default_factory=dict)
@@ -231,7 +236,9 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
             self._flush(module)
             self._staged.pop(module, None)
             self._held.pop(module, None)
-        jobs = list(module_list)
+        jobs = self._compress_groups(list(module_list))
+        if not jobs:
+            return
         workers = min(int(self.compress_concurrency), len(jobs))
         on_gpu = (all(m.weight.is_cuda and self._hessians[m].is_cuda for m in jobs)
                   and len({m.weight.device for m in jobs}) == 1)  # one device per call
@@ -243,6 +250,42 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
         # widest module does not start last (see modifiers/utils/concurrent.py); results are unchanged
         jobs.sort(key=lambda m: -(float(m.weight.shape[1]) ** 3 + float(m.weight.shape[0]) * m.weight.shape[1] ** 2))
         run_on_streams(jobs, self._compress_one, workers, jobs[0].weight.device, self._streams)
+
+    def _compress_groups(self, jobs):
+        """Quantise sets of at least ``group_min_modules`` Linears of one shape and scheme (the experts of an MoE
+        layer) in lock-step and return the modules that are left for the per-module path."""
+        if self.group_min_modules <= 0 or self.offload_hessians:
+            return jobs
+        sets = {}
+        for m in jobs:
+            key = group_key(m, getattr_chain(m, "quantization_scheme.weights"), self._hessians[m])
+            if key is not None:
+                sets.setdefault(key, []).append(m)
+        rest = [m for m in jobs]
+        for members in sets.values():
+            if len(members) < self.group_min_modules:
+                continue
+            K = members[0].weight.shape[1]
+            # bound the lock-step work buffers (factors + work matrices: about 10 K^2 bytes per problem)
+            per_call = max(1, min(len(members), int(self.group_max_bytes // (10 * K * K))))
+            for i in range(0, len(members), per_call):
+                part = members[i:i + per_call]
+                hs = [self._hessians.pop(m) for m in part]
+                counts = [float(self._num_samples.pop(m)) for m in part]
+                names = [self._module_names.get(m, m.__class__.__name__) for m in part]
+                logger.info(f"Quantizing {len(part)} modules in lock-step ({names[0]} .. {names[-1]})")
+                with torch.no_grad():
+                    results = quantize_weight_group(part, hs, counts, self.block_size, self.dampening_frac)
+                failed = torch.stack([r[2] for r in results]).tolist()
+                for m, name, (loss, q_param_dict, _), bad in zip(part, names, results, failed):
+                    if bad:
+                        logger.warning(f"Failed to invert hessian of {name} due to numerical instability. Falling "
+                                       "back to round-to-nearest for this module.")
+                    for attr, val in q_param_dict.items():
+                        update_offload_parameter(m, attr, val)
+            done = set(members)
+            rest = [m for m in rest if m not in done]
+        return rest
 
     def _compress_one(self, module, produced_on=None, consumed_on=None):
         name = self._module_names.get(module, module.__class__.__name__)

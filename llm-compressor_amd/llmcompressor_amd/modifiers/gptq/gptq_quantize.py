@@ -21,7 +21,8 @@ logger = logging.getLogger("llmcompressor_amd")
 
 GPTQ_PRECISION = torch.float32
 
-__all__ = ["make_empty_hessian", "accumulate_hessian", "quantize_weight", "quantize_weight_tensors"]
+__all__ = ["make_empty_hessian", "accumulate_hessian", "quantize_weight", "quantize_weight_tensors",
+           "quantize_weight_group", "group_key"]
 
 
 def make_empty_hessian(module: torch.nn.Module, device: torch.device | None = None) -> torch.Tensor:
@@ -151,3 +152,63 @@ def quantize_weight(module: torch.nn.Module, quant_args: QuantizationArgs, hessi
     """
     return quantize_weight_tensors(module.weight.data, module.weight_observer, quant_args, hessian, blocksize,
                                    percdamp, hessian_divisor)
+
+
+def group_key(module: torch.nn.Module, quant_args: QuantizationArgs, hessian: torch.Tensor):
+    """Modules with equal keys can go through ``quantize_weight_group`` together; None = not eligible."""
+    w = module.weight
+    if not isinstance(module, torch.nn.Linear) or w.ndim != 2 or not w.is_cuda or not hessian.is_cuda:
+        return None
+    actorder = quant_args.actorder
+    if actorder == ActivationOrdering.GROUP:  # re-observes the permuted weight per module
+        return None
+    return (tuple(w.shape), w.dtype, w.device, w.stride(0), hessian.stride(0),
+            quant_args.model_dump_json() if hasattr(quant_args, "model_dump_json") else repr(quant_args))
+
+
+def quantize_weight_group(modules, hessians, hessian_divisors, blocksize: int = 128, percdamp: float = 0.01):
+    """``quantize_weight`` for several Linears of one shape and scheme at once (the experts of an MoE layer):
+    one lock-step Cholesky chain and one lock-step column loop for all of them instead of a chain of tiny
+    kernels per module.  Same results as calling ``quantize_weight`` on each.  Returns a list of
+    (loss tensor, q_param_dict, info tensor)."""
+    n = len(modules)
+    quant_args = getattr(modules[0].quantization_scheme, "weights")
+    strategy, actorder = quant_args.strategy, quant_args.actorder
+    Ws = [m.weight.data if m.weight.data.is_contiguous() else m.weight.data.contiguous() for m in modules]
+    num_rows, num_columns = Ws[0].shape
+    final_dtype = Ws[0].dtype
+    if actorder == ActivationOrdering.GROUP and strategy not in (QuantizationStrategy.GROUP,
+                                                                 QuantizationStrategy.TENSOR_GROUP):
+        actorder = None
+    perms = None
+    if actorder:
+        perms = torch.stack([torch.argsort(torch.diagonal(H), descending=True) for H in hessians])
+    row_div, srow, divisor = _scale_layout(strategy, quant_args, num_rows, num_columns)
+    g_idxs = None
+    if divisor is not None:
+        base = torch.arange(num_columns, device=Ws[0].device, dtype=torch.int) // divisor
+        g_idxs = [base[perms[b]] if actorder == ActivationOrdering.WEIGHT else base for b in range(n)]
+    qps = [m.weight_observer.get_qparams() for m in modules]
+    fmt, bits = kernel_format(quant_args)
+    zps = None if quant_args.symmetric else [qp["zero_point"].to(torch.int8) for qp in qps]
+    kscales = [effective_scale(qp["scale"], quant_args, final_dtype) for qp in qps]
+    has_gs = qps[0]["global_scale"] is not None
+    gss = [qp["global_scale"] for qp in qps] if has_gs else None
+
+    U, dead, info = ops.gptq_hinv_grouped(hessians, perms, hessian_divisors, percdamp)
+    outs, loss = ops.gptq_quantize_grouped(Ws, U, kscales, zps, fmt, bits, row_div, srow, g_idxs=g_idxs, perms=perms,
+                                           dead=dead, global_scales=gss, blocksize=blocksize)
+    results = []
+    for b, (m, qp) in enumerate(zip(modules, qps)):
+        scale, zero_point, global_scale = qp["scale"], qp["zero_point"], qp["global_scale"]
+        q = {
+            "weight": outs[b].reshape(m.weight.shape),
+            "weight_scale": scale if scale.dtype in (torch.uint8, torch.float8_e4m3fn) else scale.to(dtype=final_dtype),
+            "weight_zero_point": zero_point.to(dtype=quant_args.zp_dtype),
+        }
+        if quant_args.scale_dtype == torch.float8_e4m3fn and scale.dtype == torch.float32:
+            q["weight_scale"] = scale
+        if global_scale is not None:
+            q["weight_global_scale"] = global_scale.to(dtype=final_dtype)
+        results.append((loss[b], q, info[b]))
+    return results

@@ -802,3 +802,59 @@ def test_sparsegpt_modifier_matches_oracle(structure, staging):
     else:
         assert abs((Q1 == 0).float().mean().item() - 0.5) < 0.01
     assert torch.equal(model.lm_head.weight.detach(), head0)  # ignored
+
+
+@pytest.mark.parametrize("scheme", [dict(num_bits=4, strategy="group", group_size=32),
+                                    dict(num_bits=4, strategy="channel", symmetric=False, actorder="weight"),
+                                    dict(num_bits=4, type="float", strategy="tensor_group", group_size=16,
+                                         scale_dtype=torch.float8_e4m3fn)])
+def test_moe_gptq_lock_step_groups_match_per_module_path(scheme):
+    """The experts of a LinearExperts2D block quantised in lock-step (grouped Cholesky chain and column loop)
+    end up with exactly the parameters of the per-module path, a never-routed expert included."""
+    from llmcompressor_amd import ops
+    from llmcompressor_amd.core import LifecycleCallbacks, active_session
+    from llmcompressor_amd.modeling import LinearExperts2D
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+
+    E, H, I, T = 10, 64, 128, 160
+    g = torch.Generator().manual_seed(4)
+    gate_up, down = torch.randn(E, 2 * I, H, generator=g) * 0.05, torch.randn(E, H, I, generator=g) * 0.05
+    x = torch.randn(T, H, generator=g).bfloat16().to(DEV)
+    idx = torch.stack([torch.arange(T) % (E - 1), (torch.arange(T) * 7 + 1) % (E - 1)], dim=1).to(DEV)  # expert E-1 idle
+    wts = torch.full((T, 2), 0.5, device=DEV, dtype=torch.bfloat16)
+    results = []
+    for group_min in (0, 4):
+        experts = LinearExperts2D.from_fused(gate_up, down).to(DEV).to(torch.bfloat16)
+
+        class Wrap(torch.nn.Module):
+            def __init__(self):
+                super().__init__()
+                self.layers = torch.nn.ModuleList([experts])
+
+        model = Wrap()
+        calls = []
+        raw = ops.gptq_quantize_grouped
+        ops.gptq_quantize_grouped = lambda *a, **kw: (calls.append(len(a[0])), raw(*a, **kw))[1]
+        try:
+            mod = GPTQModifier(targets="Linear", group_min_modules=group_min,
+                               config_groups={"g": dict(targets=["Linear"], weights=dict(scheme))})
+            session = active_session()
+            session.reset()
+            session.initialize(model=model, recipe=mod)
+            LifecycleCallbacks.calibration_start()
+            with torch.no_grad():
+                for _ in range(2):
+                    experts(x, idx, wts)
+            LifecycleCallbacks.sequential_epoch_end(modules=list(model.modules()))
+            LifecycleCallbacks.calibration_end()
+            session.finalize()
+        finally:
+            ops.gptq_quantize_grouped = raw
+        torch.cuda.synchronize()
+        results.append((calls, {n: p.detach().clone() for n, p in model.named_parameters()}))
+    (c0, p0), (c1, p1) = results
+    assert c0 == [] and sorted(c1) == [E, 2 * E]  # gate+up share a shape (20 problems), down is the other set
+    assert p0.keys() == p1.keys()
+    for n in p0:
+        assert torch.equal(p0[n], p1[n]), n
+    assert torch.count_nonzero(p1[f"layers.0.{E - 1}.down_proj.weight"]) == 0
