@@ -216,6 +216,66 @@ def probe_sparsegpt():
           f"{(time.perf_counter() - t0) * 1e3:.0f} ms")
 
 
+def probe_moe():
+    """One MoE expert layer (128 experts, hidden 2048, intermediate 768, top-8 routing of 4096 tokens: 384 expert
+    Linears) through GPTQModifier W4A16: time of the calibration forward (grouped Hessian launches from the hooks)
+    and of the quantisation of the 384 Linears, with lock-step groups and with the per-module path.  Prints a table."""
+    import torch
+
+    from llmcompressor_amd.core import LifecycleCallbacks, active_session
+    from llmcompressor_amd.modeling.moe import LinearExperts2D
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+
+    E, H, I, T, TOPK = 128, 2048, 768, 4096, 8
+    torch.manual_seed(0)
+
+    class Layer(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.experts = LinearExperts2D(E, H, I, torch.bfloat16, "cuda")
+
+        def forward(self, x, idx, w):
+            return self.experts(x, idx, w)
+
+    class Wrap(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.layers = torch.nn.ModuleList([Layer()])
+
+    model = Wrap()
+    x = torch.randn(T, H, device="cuda").bfloat16()
+    # a skewed router, as trained ones are: expert e is about e^-1.1 as likely as expert 1
+    logits = torch.randn(T, E, device="cuda") + torch.log(1.0 / torch.arange(1, E + 1, device="cuda").float() ** 1.1)
+    w, idx = torch.topk(torch.softmax(logits, -1), TOPK, -1)
+    print("| quantisation of the 384 expert Linears | forward + Hessians ms | quantise ms | ms per Linear |")
+    print("|---|---|---|---|")
+    for label, gmin in (("lock-step groups (default)", 8), ("one module at a time, 4 streams", 0)):
+        best = None
+        for _ in range(3):
+            for p in model.parameters():
+                if p.dtype == torch.bfloat16:
+                    p.data.normal_(0, 0.02)
+            mod = GPTQModifier(targets="Linear", scheme="W4A16", group_min_modules=gmin)
+            s = active_session()
+            s.reset()
+            s.initialize(model=model, recipe=mod)
+            LifecycleCallbacks.calibration_start()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            with torch.no_grad():
+                model.layers[0](x, idx, w.to(x.dtype))
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            LifecycleCallbacks.sequential_epoch_end(modules=list(model.modules()))
+            torch.cuda.synchronize()
+            t2 = time.perf_counter()
+            LifecycleCallbacks.calibration_end()
+            s.finalize()
+            if best is None or t2 - t1 < best[1]:
+                best = (t1 - t0, t2 - t1)
+        print(f"| {label} | {best[0] * 1e3:.1f} | {best[1] * 1e3:.1f} | {best[1] * 1e3 / (3 * E):.2f} |")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -233,6 +293,8 @@ def main():
                     help="print achieved GB/s of the observer / quantize / pack kernels instead of the bench line")
     ap.add_argument("--probe-sparsegpt", action="store_true",
                     help="print SparseGPT timings per Linear shape instead of the bench line")
+    ap.add_argument("--probe-moe", action="store_true",
+                    help="print the timings of one 128-expert MoE layer through GPTQModifier instead of the bench line")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU figure is produced)", file=sys.stderr)
@@ -252,6 +314,9 @@ def main():
         return
     if a.probe_sparsegpt:
         probe_sparsegpt()
+        return
+    if a.probe_moe:
+        probe_moe()
         return
     if a.probe_dominant:
         from llmcompressor_amd import ops

@@ -262,29 +262,40 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
             if key is not None:
                 sets.setdefault(key, []).append(m)
         rest = [m for m in jobs]
+        launched = []
         for members in sets.values():
             if len(members) < self.group_min_modules:
                 continue
             K = members[0].weight.shape[1]
             # bound the lock-step work buffers (factors + work matrices: about 10 K^2 bytes per problem)
             per_call = max(1, min(len(members), int(self.group_max_bytes // (10 * K * K))))
+            tallies = [self._num_samples.pop(m) for m in members]
+            if all(isinstance(t, torch.Tensor) and t.is_cuda for t in tallies):  # one transfer, not one per module
+                tallies = torch.stack([t.reshape(()) for t in tallies]).tolist()
+            tallies = [float(t) for t in tallies]
             for i in range(0, len(members), per_call):
                 part = members[i:i + per_call]
                 hs = [self._hessians.pop(m) for m in part]
-                counts = [float(self._num_samples.pop(m)) for m in part]
                 names = [self._module_names.get(m, m.__class__.__name__) for m in part]
                 logger.info(f"Quantizing {len(part)} modules in lock-step ({names[0]} .. {names[-1]})")
                 with torch.no_grad():
-                    results = quantize_weight_group(part, hs, counts, self.block_size, self.dampening_frac)
-                failed = torch.stack([r[2] for r in results]).tolist()
-                for m, name, (loss, q_param_dict, _), bad in zip(part, names, results, failed):
-                    if bad:
-                        logger.warning(f"Failed to invert hessian of {name} due to numerical instability. Falling "
-                                       "back to round-to-nearest for this module.")
-                    for attr, val in q_param_dict.items():
-                        update_offload_parameter(m, attr, val)
+                    results = quantize_weight_group(part, hs, tallies[i:i + per_call], self.block_size,
+                                                    self.dampening_frac)
+                launched.append((part, names, results))
             done = set(members)
             rest = [m for m in rest if m not in done]
+        if launched:
+            # the host waits for the device once, after every group has been enqueued
+            failed = torch.cat([torch.stack([r[2] for r in results]) for _, _, results in launched]).tolist()
+            at = 0
+            for part, names, results in launched:
+                for m, name, (loss, q_param_dict, _) in zip(part, names, results):
+                    if failed[at]:
+                        logger.warning(f"Failed to invert hessian of {name} due to numerical instability. Falling "
+                                       "back to round-to-nearest for this module.")
+                    at += 1
+                    for attr, val in q_param_dict.items():
+                        update_offload_parameter(m, attr, val)
         return rest
 
     def _compress_one(self, module, produced_on=None, consumed_on=None):
