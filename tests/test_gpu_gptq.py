@@ -316,3 +316,60 @@ def test_gptq_quantize_grouped_is_bit_identical_to_single_calls(R, K, n, fmt_cas
                                    global_scale=gs_arg[b] if gs_arg else None)
         assert torch.equal(outs[b], ob), b
         assert torch.equal(loss[b:b + 1], lb)
+
+
+@pytest.mark.parametrize("R,K", [(768, 2048), (2048, 768)])
+def test_gptq_grouped_at_moe_layer_size(R, K):
+    """128 expert Linears of one MoE layer (BASELINE config 5 shapes, Zipf-routed token counts, two experts
+    never routed) in one lock-step call: sampled problems equal the single-problem path bit for bit, every
+    output lies on its group's int4 grid, idle experts come out zeroed with zero loss, and every expert with at
+    least K tokens reports a positive finite loss."""
+    from llmcompressor_amd import ops
+
+    n, T, group = 128, 4096, 128
+    gen = torch.Generator(device="cuda").manual_seed(R)
+    logits = torch.randn(T, n, device="cuda", generator=gen) + torch.log(
+        1.0 / torch.arange(1, n + 1, device="cuda").float() ** 1.1)
+    logits[:, [17, 127]] = -1e9  # idle experts: no token, Hessian stays zero
+    idx = torch.topk(logits, 8, -1).indices
+    x_all = torch.randn(T, K, device="cuda", generator=gen).bfloat16()
+    Ws = [(torch.randn(R, K, device="cuda", generator=gen) * 0.02).bfloat16() for _ in range(n)]
+    Hs = [torch.zeros(K, K, device="cuda") for _ in range(n)]
+    xs = [x_all[(idx == e).any(-1)] for e in range(n)]
+    ops.hessian_accumulate_grouped_(Hs, xs, alpha=2.0)
+    counts = [int(x.shape[0]) for x in xs]
+    assert counts[17] == 0 and counts[127] == 0 and max(counts) > 8 * min(c for c in counts if c)
+    perms = torch.stack([torch.argsort(torch.diagonal(H), descending=True) for H in Hs]).to(torch.int32)
+    scales, gidx = [], []
+    base = torch.arange(K, dtype=torch.int32, device="cuda") // group
+    for b, W in enumerate(Ws):
+        mn, mx = ops.minmax_groups(W, group)
+        s, _, _ = ops.calculate_qparams(mn, mx, ops.FMT_INT, 4, True)
+        scales.append(s)
+        gidx.append(base[perms[b].long()])
+    U, dead, info = ops.gptq_hinv_grouped([H.clone() for H in Hs], perms, [1.0] * n, 0.01)
+    assert int(info.abs().sum()) == 0
+    outs, loss = ops.gptq_quantize_grouped(Ws, U, scales, None, ops.FMT_INT, 4, 1, K // group, g_idxs=gidx,
+                                           perms=perms, dead=dead)
+    torch.cuda.synchronize()
+    for b in (0, 17, 64, 126):
+        Ub, db, ib = ops.gptq_hinv_(Hs[b].clone(), perms[b], divisor=1.0)
+        assert torch.equal(Ub, U[b]) and torch.equal(db, dead[b])
+        ob, lb = ops.gptq_quantize(Ws[b], Ub, scales[b], None, ops.FMT_INT, 4, 1, K // group, g_idx=gidx[b],
+                                   perm=perms[b], dead=db)
+        assert torch.equal(outs[b], ob), b
+        assert torch.equal(loss[b:b + 1], lb)
+    assert torch.count_nonzero(outs[17]) == 0 and torch.count_nonzero(outs[127]) == 0
+    assert bool(dead[17].all()) and bool(dead[127].all())
+    for b in (0, 5, 64, 126):  # grid membership: out / scale is an integer code in [-8, 7]
+        s = scales[b].float().repeat_interleave(group, dim=1)
+        code = outs[b].float() / s
+        live = ~dead[b].bool()
+        # dequantised values are rounded to bf16 after code * scale: compare against the rounded grid
+        nearest = torch.round(code).clamp(-8, 7)
+        regrid = (nearest * s).bfloat16().float()
+        assert torch.equal(regrid[:, live], outs[b].float()[:, live]), b
+        assert torch.count_nonzero(outs[b][:, ~live]) == 0
+    assert torch.isfinite(loss).all() and float(loss[17]) == 0.0
+    routed = [b for b in range(n) if counts[b] >= K]
+    assert all(float(loss[b]) > 0 for b in routed)
