@@ -320,7 +320,7 @@ def test_gptq_quantize_grouped_is_bit_identical_to_single_calls(R, K, n, fmt_cas
 
 @pytest.mark.parametrize("R,K", [(768, 2048), (2048, 768)])
 def test_gptq_grouped_at_moe_layer_size(R, K):
-    """128 expert Linears of one MoE layer (BASELINE config 5 shapes, Zipf-routed token counts, two experts
+    """128 expert Linears of one MoE layer (Qwen3-30B-A3B expert shapes, Zipf-routed token counts, two experts
     never routed) in one lock-step call: sampled problems equal the single-problem path bit for bit, every
     output lies on its group's int4 grid, idle experts come out zeroed with zero loss, and every expert with at
     least K tokens reports a positive finite loss."""
