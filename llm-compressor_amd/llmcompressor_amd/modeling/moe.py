@@ -62,15 +62,39 @@ class LinearExperts2D(nn.ModuleList):
         return self
 
     def forward(self, hidden_states: torch.Tensor, top_k_index: torch.Tensor, top_k_weights: torch.Tensor):
-        """hidden_states [T,H]; top_k_index / top_k_weights [T,k]."""
-        final = torch.zeros_like(hidden_states)
-        onehot = torch.nn.functional.one_hot(top_k_index, num_classes=self.num_experts).permute(2, 1, 0)  # [E,k,T]
+        """hidden_states [T,H]; top_k_index / top_k_weights [T,k].
+
+        Same values as the reference's loop (``torch.where`` on a one-hot mask per expert, one ``index_add_`` per
+        expert, modeling/moe/linear_experts.py:235-268) with the routing done once for all experts: the
+        (slot, token) pairs are sorted by expert with a stable sort, which leaves each expert's pairs in the
+        slot-major order ``torch.where`` yields; the routed rows are gathered once and every expert's Linears are
+        called on a slice of that buffer (so their hooks fire as before, also for an expert with no token); the
+        weighted outputs are added per token in ascending expert order, one rounding to the output dtype per
+        addition, as the chain of ``index_add_`` calls does.  One host wait (the experts' token counts) per call
+        instead of one per expert."""
+        T, k = top_k_index.shape
+        E = self.num_experts
+        with torch.no_grad():
+            flat = top_k_index.t().reshape(-1)  # pair p = slot * T + token
+            order = torch.argsort(flat, stable=True)
+            counts = torch.bincount(flat, minlength=E).tolist()
+            slot_sorted = torch.div(order, T, rounding_mode="floor")
+            tok_sorted = order - slot_sorted * T
+            # position of each token's pairs in the sorted list, ascending = ascending expert
+            place = torch.empty_like(order)
+            place[order] = torch.arange(order.numel(), device=order.device)
+            place = place.view(k, T).sort(dim=0).values
+        routed = None if _CALIBRATE_ALL_EXPERTS else hidden_states[tok_sorted]
+        outs, at = [], 0
         for e, expert in enumerate(self):
-            slot, token_idx = torch.where(onehot[e])
+            n = counts[e]
             if _CALIBRATE_ALL_EXPERTS:
-                out = expert(hidden_states)[token_idx]
+                outs.append(expert(hidden_states)[tok_sorted[at:at + n]])
             else:
-                out = expert(hidden_states[token_idx])
-            if token_idx.numel() > 0:
-                final.index_add_(0, token_idx, (out * top_k_weights[token_idx, slot, None]).to(final.dtype))
+                outs.append(expert(routed[at:at + n]))
+            at += n
+        weighted = (torch.cat(outs) * top_k_weights[tok_sorted, slot_sorted, None]).to(hidden_states.dtype)
+        final = torch.zeros_like(hidden_states)
+        for j in range(k):
+            final = final + weighted[place[j]]
         return final

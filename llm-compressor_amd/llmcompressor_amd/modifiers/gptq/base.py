@@ -165,13 +165,15 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
         inp = args[0]
         if self.share_identical_inputs and self._follows_recent_input(module, inp):
             return
+        grouped = (self._group_pending is not None and isinstance(module, torch.nn.Linear) and inp.is_cuda
+                   and not self.offload_hessians and inp.dtype in (torch.bfloat16, torch.float16))
         if module not in self._num_samples:
             device = inp.device if inp.is_cuda else module.weight.device
             init_device = "cpu" if self.offload_hessians else device
             self._hessians[module] = make_empty_hessian(module, device=init_device)
-            self._num_samples[module] = torch.zeros(tuple(), device=device)
-        if (self._group_pending is not None and isinstance(module, torch.nn.Linear) and inp.is_cuda
-                and not self.offload_hessians and inp.dtype in (torch.bfloat16, torch.float16)):
+            # an expert's tally stays on the host: hundreds of one-element device additions per forward otherwise
+            self._num_samples[module] = 0.0 if grouped else torch.zeros(tuple(), device=device)
+        if grouped:
             self._group_pending.append((module, inp))
             return
         if self.hessian_batch_tokens > 0 and not self.offload_hessians and isinstance(module, torch.nn.Linear):

@@ -858,3 +858,38 @@ def test_moe_gptq_lock_step_groups_match_per_module_path(scheme):
     for n in p0:
         assert torch.equal(p0[n], p1[n]), n
     assert torch.count_nonzero(p1[f"layers.0.{E - 1}.down_proj.weight"]) == 0
+
+
+@pytest.mark.parametrize("all_experts", [False, True])
+def test_moe_forward_on_device_equals_the_per_expert_loop(all_experts):
+    """The single-pass routing of LinearExperts2D.forward against the reference's per-expert loop on the GPU
+    (bf16, 32 experts, top-4, skewed router with an idle expert): identical output, identical Hessian inputs."""
+    from llmcompressor_amd.modeling import LinearExperts2D, moe_calibration_context
+    from oracle.moe import experts_forward
+
+    torch.manual_seed(11)
+    E, H, I, T, k = 32, 256, 128, 1024, 4
+    experts = LinearExperts2D(E, H, I, torch.bfloat16, DEV)
+    for p in experts.parameters():
+        p.data.normal_(0, 0.05)
+    x = torch.randn(T, H, device=DEV).bfloat16()
+    logits = torch.randn(T, E, device=DEV) + torch.log(1.0 / torch.arange(1, E + 1, device=DEV).float() ** 1.1)
+    logits[:, 9] = -1e9
+    wts, idx = torch.topk(torch.softmax(logits, -1), k, -1)
+    wts = wts.bfloat16()
+    seen = []
+    for ex in experts:
+        ex.down_proj.register_forward_hook(lambda m, a, o: seen.append(a[0].detach().clone()))
+    with torch.no_grad():
+        if all_experts:
+            with moe_calibration_context():
+                got = experts(x, idx, wts)
+        else:
+            got = experts(x, idx, wts)
+        fast_inputs, seen[:] = list(seen), []
+        want = experts_forward(list(experts), x, idx, wts, calibrate_all_experts=all_experts)
+    assert torch.equal(got, want)
+    assert len(fast_inputs) == len(seen) == E
+    for a, b in zip(fast_inputs, seen):
+        assert a.shape == b.shape and torch.equal(a, b)
+    assert fast_inputs[9].shape[0] == (T if all_experts else 0)

@@ -389,3 +389,41 @@ def test_sparsegpt_modifier_fields_and_validation():
     """)
     (mod,) = recipe.modifiers
     assert isinstance(mod, SparseGPTModifier) and mod.ignore == ["re:.*lm_head"] and mod._prune_n == 2
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("all_experts", [False, True])
+def test_moe_forward_equals_the_per_expert_loop(dtype, all_experts):
+    """LinearExperts2D.forward routes once for all experts; its output equals the reference's per-expert loop
+    (oracle/moe.py) bit for bit, also with an idle expert and uneven counts, and the dense closed form in fp64."""
+    from llmcompressor_amd.modeling import LinearExperts2D, moe_calibration_context
+    from oracle.moe import experts_forward
+
+    torch.manual_seed(3)
+    E, H, I, T, k = 6, 16, 24, 40, 3
+    experts = LinearExperts2D.from_fused(torch.randn(E, 2 * I, H) * 0.3, torch.randn(E, H, I) * 0.3).to(dtype)
+    x = torch.randn(T, H).to(dtype)
+    logits = torch.randn(T, E)
+    logits[:, 4] = -1e9  # expert 4 idle
+    wts, idx = torch.topk(torch.softmax(logits, -1), k, -1)
+    wts = wts.to(dtype)
+    seen = {}
+    for e, ex in enumerate(experts):
+        ex.down_proj.register_forward_hook(lambda m, a, o, e=e: seen.__setitem__(e, a[0].shape[0]))
+    with torch.no_grad():
+        if all_experts:
+            with moe_calibration_context():
+                got = experts(x, idx, wts)
+        else:
+            got = experts(x, idx, wts)
+        want = experts_forward(list(experts), x, idx, wts, calibrate_all_experts=all_experts)
+    assert torch.equal(got, want)
+    assert seen[4] == (T if all_experts else 0) and len(seen) == E
+    dense = torch.zeros(T, H, dtype=torch.float64)
+    with torch.no_grad():
+        for t in range(T):
+            for j in range(k):
+                dense[t] += wts[t, j].double() * experts[int(idx[t, j])].double()(x[t].double())
+    experts.to(dtype)
+    tol = 1e-5 if dtype == torch.float32 else 5e-2
+    assert (got.double() - dense).abs().max() <= tol * dense.abs().max()
