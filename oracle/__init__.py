@@ -24,7 +24,9 @@ closed form or invariant says so here):
   (memoryless / static / moving average), MSE grid search (eight known-answer
   losses), ``flatten_for_calibration`` shape contract, ``accumulate_hessian``
   (fp64 closed form), ``quantize_weight`` (diagonal-Hessian == RTN, textbook
-  un-blocked GPTQ in fp64, block-size independence, grid membership).
+  un-blocked GPTQ in fp64, block-size independence, grid membership),
+  ``moe.experts_forward`` (the reference's routing counts for 4 experts / top-2,
+  the dense fp64 closed form).
 * parity unpinned (no reference-held vector exists; follows the public format
   specs): MXFP4 E8M0 scale generation, ``pack_to_int32`` / ``pack_fp4_to_uint8``
   byte layouts, fp8 storage, per-token dynamic FP8 scales, zero-scale epsilon
