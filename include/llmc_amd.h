@@ -50,7 +50,9 @@ int llmc_version(void);
  * (src/llmcompressor/modifiers/gptq/gptq_quantize.py:28-64):
  *     H[K,K] += alpha * X^T X,   X = [T,K] (tokens x in_features), alpha = 2.
  * bf16/f16 inputs are multiplied exactly and accumulated in fp32 on the MFMA
- * units.  Only the upper-triangular tiles are computed.  With
+ * units.  fp32 inputs (x_dtype = LLMC_F32; this entry point only, not the grouped
+ * and segmented forms) take the fp32 matrix-core GEMM over the full K x K matrix and
+ * ignore flags and workspace.  Only the upper-triangular tiles are computed.  With
  * LLMC_HESSIAN_ASSUME_SYMMETRIC the mirrored lower tiles are stored from the
  * upper results (H must be bitwise symmetric on entry, which holds for a
  * buffer that started as zeros and was only ever updated by this call);

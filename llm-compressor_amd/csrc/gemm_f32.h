@@ -5,8 +5,10 @@
 #include <stdint.h>
 
 struct GemmF32 {
-  // C[M,N] = alpha * A[M,Kc] * B' + beta * C,   all row-major
+  // C[M,N] = alpha * A' * B' + beta * C,   all row-major
   //   trans_b = 0: B' = B,  B stored [Kc,N];   trans_b = 1: B' = B^T, B stored [N,Kc]
+  //   trans_a = 0: A' = A,  A stored [M,Kc];   trans_a = 1: A' = A^T, A stored [Kc,M] (only with
+  //   trans_b = 0 and without the a_lower_tri hint)
   const float* A;
   int64_t lda;
   const float* B;
@@ -16,6 +18,7 @@ struct GemmF32 {
   int M, N, Kc;
   float alpha, beta;
   int trans_b;
+  int trans_a;
   // structure hints (tile-granular; operands must hold exact zeros where the structure says so)
   int c_lower;      // only tiles that touch the lower triangle of C are computed
   int a_lower_tri;  // A[m,k] = 0 for k > m : contraction stops at the tile's last row

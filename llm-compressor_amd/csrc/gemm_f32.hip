@@ -24,7 +24,7 @@ __device__ __forceinline__ float4 ld4(const float* p, int valid, bool vec) {
 
 // FAST: the tile lies fully inside C, the contraction range is a multiple of BK and all rows are
 // 16-byte aligned, so every load is an unconditional float4 and the main loop is one basic block.
-template <int BM, int BN, bool TRANS_B, bool FAST>
+template <int BM, int BN, bool TRANS_B, bool FAST, bool TRANS_A>
 __device__ __forceinline__ void gemm_tile(const GemmF32& g, const float* A, const float* B, float* C, int m0,
                                           int n0, int k_begin, int k_end, float* As, float* Bs) {
   constexpr int LDA_S = BM + 4, LDB_S = BN + 4;
@@ -47,6 +47,14 @@ __device__ __forceinline__ void gemm_tile(const GemmF32& g, const float* A, cons
 #pragma unroll
     for (int i = 0; i < A_LD; ++i) {
       const int f = tid + i * 256;
+      if (TRANS_A) {
+        const int k = k0 + f / (BM / 4), m = m0 + (f % (BM / 4)) * 4;
+        if (FAST)
+          ra[i] = *(const float4*)(A + (int64_t)k * g.lda + m);
+        else
+          ra[i] = (k < k_end) ? ld4(A + (int64_t)k * g.lda + m, g.M - m, false) : make_float4(0.f, 0.f, 0.f, 0.f);
+        continue;
+      }
       const int m = m0 + f / 4, k = k0 + (f % 4) * 4;
       if (FAST)
         ra[i] = *(const float4*)(A + (int64_t)m * g.lda + k);
@@ -75,6 +83,11 @@ __device__ __forceinline__ void gemm_tile(const GemmF32& g, const float* A, cons
 #pragma unroll
     for (int i = 0; i < A_LD; ++i) {
       const int f = tid + i * 256;
+      if (TRANS_A) {
+        const int k = f / (BM / 4), m = (f % (BM / 4)) * 4;
+        *(float4*)&As[k * LDA_S + m] = ra[i];
+        continue;
+      }
       const int m = f / 4, k = (f % 4) * 4;
       As[(k + 0) * LDA_S + m] = ra[i].x;
       As[(k + 1) * LDA_S + m] = ra[i].y;
@@ -190,7 +203,7 @@ __device__ __forceinline__ void gemm_tile(const GemmF32& g, const float* A, cons
 // ALL_FAST: the host has checked that every tile of the launch takes the unconditional path
 // (M, N multiples of the tile, contraction ranges multiples of BK, 16-byte aligned rows), so the
 // bounds-checked variant is not even instantiated: fewer registers, more waves per SIMD.
-template <int BM, int BN, bool TRANS_B, bool ALL_FAST>
+template <int BM, int BN, bool TRANS_B, bool ALL_FAST, bool TRANS_A = false>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32 g, int vec) {
   __shared__ float As[2 * BK * (BM + 4)];
   __shared__ float Bs[2 * BK * (BN + 4)];
@@ -204,13 +217,13 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32 g, int vec) {
   int k_end = g.Kc;
   if (g.a_lower_tri && m0 + BM < k_end) k_end = m0 + BM;
   if (ALL_FAST) {
-    gemm_tile<BM, BN, TRANS_B, true>(g, A, B, C, m0, n0, k_begin, k_end, As, Bs);
+    gemm_tile<BM, BN, TRANS_B, true, TRANS_A>(g, A, B, C, m0, n0, k_begin, k_end, As, Bs);
   } else {
     const bool fast = vec && m0 + BM <= g.M && n0 + BN <= g.N && ((k_end - k_begin) % BK) == 0;
     if (fast)
-      gemm_tile<BM, BN, TRANS_B, true>(g, A, B, C, m0, n0, k_begin, k_end, As, Bs);
+      gemm_tile<BM, BN, TRANS_B, true, TRANS_A>(g, A, B, C, m0, n0, k_begin, k_end, As, Bs);
     else
-      gemm_tile<BM, BN, TRANS_B, false>(g, A, B, C, m0, n0, k_begin, k_end, As, Bs);
+      gemm_tile<BM, BN, TRANS_B, false, TRANS_A>(g, A, B, C, m0, n0, k_begin, k_end, As, Bs);
   }
 }
 
@@ -218,6 +231,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32 g, int vec) {
 
 int llmc_gemm_f32(const GemmF32& g, hipStream_t st) {
   if (g.M <= 0 || g.N <= 0 || g.batch <= 0) return 0;
+  if (g.trans_a && (g.trans_b || g.a_lower_tri)) return 1000 + (int)hipErrorInvalidValue;
   const int nb2 = g.batch2 > 1 ? g.batch2 : 1;
   const int vec = ((g.lda & 3) == 0 && (g.ldb & 3) == 0 && (((uintptr_t)g.A | (uintptr_t)g.B) & 15) == 0 &&
                    (g.stride_a & 3) == 0 && (g.stride_b & 3) == 0 && (g.Kc & 3) == 0 &&
@@ -233,7 +247,12 @@ int llmc_gemm_f32(const GemmF32& g, hipStream_t st) {
   const bool all_fast = vec && g.M % bt == 0 && g.N % bt == 0 && g.Kc % BK == 0;
   dim3 grid((g.N + bt - 1) / bt, (g.M + bt - 1) / bt, g.batch * nb2);
 #define LLMC_GEMM(BT, TB, AF) hipLaunchKernelGGL((gemm_f32_kernel<BT, BT, TB, AF>), grid, dim3(256), 0, st, g, vec)
-  if (big) {
+  if (g.trans_a) {
+#define LLMC_GEMM_TA(BT, AF) hipLaunchKernelGGL((gemm_f32_kernel<BT, BT, false, AF, true>), grid, dim3(256), 0, st, g, vec)
+    if (big) { if (all_fast) LLMC_GEMM_TA(128, true); else LLMC_GEMM_TA(128, false); }
+    else { if (all_fast) LLMC_GEMM_TA(64, true); else LLMC_GEMM_TA(64, false); }
+#undef LLMC_GEMM_TA
+  } else if (big) {
     if (g.trans_b) { if (all_fast) LLMC_GEMM(128, true, true); else LLMC_GEMM(128, true, false); }
     else { if (all_fast) LLMC_GEMM(128, false, true); else LLMC_GEMM(128, false, false); }
   } else {

@@ -13,6 +13,7 @@
 #include <type_traits>
 
 #include "common.h"
+#include "gemm_f32.h"
 
 namespace {
 
@@ -747,10 +748,31 @@ extern "C" int llmc_hessian_accumulate(float* H, int64_t ldh, const void* X, int
   if (T == 0) return 0;
   LLMC_CHECK_ARG(X != nullptr, 3);
   LLMC_CHECK_ARG(ldx >= K, 4);
-  LLMC_CHECK_ARG(x_dtype == LLMC_BF16 || x_dtype == LLMC_F16, 7);
+  LLMC_CHECK_ARG(x_dtype == LLMC_BF16 || x_dtype == LLMC_F16 || x_dtype == LLMC_F32, 7);
   LLMC_CHECK_ARG(workspace_bytes >= 0 && (workspace_bytes == 0 || workspace != nullptr), 10);
   LLMC_CHECK_ARG((((uintptr_t)workspace) & 15) == 0, 10);
   hipStream_t st = (hipStream_t)stream;
+  if (x_dtype == LLMC_F32) {
+    // fp32 activations: the whole K x K product X^T X on the fp32 matrix-core GEMM (every element of H is
+    // read-modify-written; tile (i,j) and tile (j,i) form the same products in the same order, so a
+    // symmetric H stays bitwise symmetric)
+    LLMC_CHECK_ARG(K < (1ll << 31) - 256 && T < (1ll << 31) - 256, 5);
+    GemmF32 g = {};
+    g.A = (const float*)X;
+    g.lda = ldx;
+    g.trans_a = 1;
+    g.B = (const float*)X;
+    g.ldb = ldx;
+    g.C = H;
+    g.ldc = ldh;
+    g.M = (int)K;
+    g.N = (int)K;
+    g.Kc = (int)T;
+    g.alpha = alpha;
+    g.beta = 1.f;
+    g.batch = 1;
+    return llmc_gemm_f32(g, st);
+  }
   // 256-wide tiles need half the LDS traffic per matrix op of 128-wide ones; token chunks spread a
   // tile count that is not a multiple of the CU count over the whole chip
   // workspace layout: [pacing counters, PACE_BYTES][partial tiles of the token chunks]

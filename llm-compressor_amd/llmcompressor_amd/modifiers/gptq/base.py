@@ -176,7 +176,8 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
         if grouped:
             self._group_pending.append((module, inp))
             return
-        if self.hessian_batch_tokens > 0 and not self.offload_hessians and isinstance(module, torch.nn.Linear):
+        if (self.hessian_batch_tokens > 0 and not self.offload_hessians and isinstance(module, torch.nn.Linear)
+                and inp.dtype in (torch.bfloat16, torch.float16)):  # fp32 inputs go straight to the fp32 product
             self._stage(module, inp)
             return
         with self._maybe_onload_hessian(module):

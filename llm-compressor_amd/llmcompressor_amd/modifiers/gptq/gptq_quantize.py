@@ -48,11 +48,6 @@ def accumulate_hessian(inp: torch.Tensor, module: torch.nn.Module, H: torch.Tens
     else:  # Linear / Conv1D: rows are tokens
         inp = inp.reshape((-1, inp.shape[-1]))
     num_samples += num_added
-    if inp.dtype == torch.float32:
-        # the matrix cores take 16-bit operands; an fp32 activation is split into a bf16 head and
-        # tail, (h + t)^T (h + t) = h^T h + h^T t + t^T h + t^T t, accumulated in fp32
-        raise TypeError("accumulate_hessian: fp32 activations are not supported by this build; "
-                        "calibrate in bf16 or fp16")
     if inp.shape[0] > 0:
         ops.hessian_accumulate_(H, inp.contiguous(), alpha=2.0, assume_symmetric=True)
     return H, num_samples

@@ -25,7 +25,8 @@ def _require_gpu(*ts: torch.Tensor) -> None:
 
 def hessian_accumulate_(H: torch.Tensor, x: torch.Tensor, alpha: float = 2.0, assume_symmetric: bool = True,
                         use_workspace: bool = True):
-    """H[K,K] (fp32, in place) += alpha * x^T x for x = [T,K] bf16/f16.
+    """H[K,K] (fp32, in place) += alpha * x^T x for x = [T,K] bf16/f16 (exact products on the 16-bit matrix
+    cores) or fp32 (the fp32 matrix-core GEMM over the full matrix).
 
     With `use_workspace` a per-stream scratch buffer lets tiles that do not fill the chip be cut along
     the tokens (summed in fixed order, so results stay reproducible); without it every output tile
@@ -33,14 +34,14 @@ def hessian_accumulate_(H: torch.Tensor, x: torch.Tensor, alpha: float = 2.0, as
     _require_gpu(H, x)
     assert H.dtype == torch.float32 and H.ndim == 2 and H.shape[0] == H.shape[1]
     assert x.ndim == 2 and x.shape[1] == H.shape[0]
-    if x.dtype not in (torch.bfloat16, torch.float16):
+    if x.dtype not in (torch.bfloat16, torch.float16, torch.float32):
         raise TypeError(f"hessian_accumulate_: unsupported activation dtype {x.dtype}")
     if x.stride(1) != 1:
         x = x.contiguous()
     assert H.stride(1) == 1
     with torch.cuda.device(H.device):
         ws, nws = None, 0
-        if use_workspace:
+        if use_workspace and x.dtype != torch.float32:
             nws = int(_lib.lib().llmc_hessian_workspace_bytes(x.shape[0], x.shape[1]))
             ws = _workspace(H.device, nws) if nws else None
         rc = _lib.lib().llmc_hessian_accumulate(

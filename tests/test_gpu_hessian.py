@@ -230,3 +230,30 @@ def test_hessian_segments_full_size():
     rows = torch.tensor([0, 255, 256, 7000, 14335], device="cuda")
     ref = 2 * (cat[:, rows].double().t() @ cat.double())
     assert _rel(Hb[rows], ref) < TOL
+
+
+@pytest.mark.parametrize("T,K", [(64, 128), (100, 96), (37, 201), (1, 8), (300, 520), (2048, 1024), (513, 67)])
+def test_hessian_fp32_activations(T, K):
+    """fp32 activations (the reference's ``inp.float()`` path with nothing to cast, gptq_quantize.py:57-62)
+    take the fp32 matrix-core product: the oracle and the fp64 closed form within the Hessian tolerance, a
+    non-symmetric start is read-modify-written everywhere, a symmetric one stays bitwise symmetric, and a
+    row-strided view of the activations is accepted."""
+    from llmcompressor_amd import ops
+
+    torch.manual_seed(T * 7 + K)
+    wide = torch.randn(T, K + 5)
+    wide[:, K // 3] *= 20
+    x = wide[:, :K]
+    Hc, _ = G.accumulate_hessian(x.contiguous(), G.make_empty_hessian(K), torch.zeros(()))
+    Hc, _ = G.accumulate_hessian(x.flip(0).contiguous() * 0.5, Hc, torch.zeros(()))
+    Hg = torch.zeros(K, K, device="cuda")
+    ops.hessian_accumulate_(Hg, wide.cuda()[:, :K])
+    ops.hessian_accumulate_(Hg, (x.flip(0) * 0.5).cuda())
+    ref64 = 2 * x.double().t() @ x.double() * 1.25
+    assert _rel(Hg.cpu(), Hc) < TOL
+    assert _rel(Hg.cpu(), ref64) < TOL
+    assert torch.equal(Hg, Hg.t())
+    H0 = torch.randn(K, K)
+    Hn = H0.cuda()
+    ops.hessian_accumulate_(Hn, x.cuda().contiguous(), assume_symmetric=False)
+    assert _rel(Hn.cpu(), H0.double() + 2 * x.double().t() @ x.double()) < TOL

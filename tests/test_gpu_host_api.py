@@ -893,3 +893,46 @@ def test_moe_forward_on_device_equals_the_per_expert_loop(all_experts):
     for a, b in zip(fast_inputs, seen):
         assert a.shape == b.shape and torch.equal(a, b)
     assert fast_inputs[9].shape[0] == (T if all_experts else 0)
+
+
+def test_gptq_modifier_on_an_fp32_model():
+    """A model kept in fp32: the hooks receive fp32 activations (no staging, fp32 product) and the fp32 weights
+    are quantised; Hessian against the fp64 closed form and every weight on its group's int4 grid."""
+    from llmcompressor_amd.core import LifecycleCallbacks, active_session
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+
+    torch.manual_seed(2)
+
+    class Wrap(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.layers = torch.nn.ModuleList([torch.nn.Sequential(torch.nn.Linear(128, 256, bias=False),
+                                                                   torch.nn.Linear(256, 64, bias=False))])
+
+    model = Wrap().to(DEV)
+    W0 = model.layers[0][0].weight.detach().clone()
+    mod = GPTQModifier(targets="Linear", config_groups={"g": dict(targets=["Linear"], weights=dict(
+        num_bits=4, strategy="group", group_size=32))})
+    session = active_session()
+    session.reset()
+    session.initialize(model=model, recipe=mod)
+    LifecycleCallbacks.calibration_start()
+    xs = [torch.randn(2, 96, 128, device=DEV) for _ in range(3)]
+    with torch.no_grad():
+        for x in xs:
+            model.layers[0](x)
+    lin = model.layers[0][0]
+    flat = torch.cat([x.reshape(-1, 128) for x in xs]).double()
+    ref = 2 * flat.t() @ flat
+    H = mod._hessians[lin]
+    assert ((H.double() - ref).norm() / ref.norm()).item() < 1e-5
+    assert float(mod._num_samples[lin]) == 6.0
+    LifecycleCallbacks.sequential_epoch_end(modules=list(model.modules()))
+    LifecycleCallbacks.calibration_end()
+    session.finalize()
+    Q = lin.weight.detach()
+    assert Q.dtype == torch.float32 and not torch.equal(Q, W0)
+    s = lin.weight_scale.detach().float().repeat_interleave(32, dim=1)
+    code = Q / s
+    assert torch.all((code - code.round()).abs() < 1e-4) and code.round().min() >= -8 and code.round().max() <= 7
+    assert ((Q - W0).norm() / W0.norm()).item() < 0.2
