@@ -232,7 +232,21 @@ def forward_quantize(module: Module, value: torch.Tensor, base_name: str, args: 
     zp = getattr(module, f"{base_name}_zero_point", None)
     gs = getattr(module, f"{base_name}_global_scale", None)
     if args.dynamic in (True, DynamicType.LOCAL):
-        raise NotImplementedError("dynamic group / tensor activation quantization is not part of this build")
+        # scales of this call's values (compressed-tensors ``compute_dynamic_scales_and_zp``): one per run of
+        # group_size trailing elements, or one for the whole tensor; ``local`` keeps the calibrated global scale
+        x2, shape = _as_2d(value if value.is_contiguous() else value.contiguous())
+        rows, cols = x2.shape
+        if args.strategy in (QuantizationStrategy.GROUP, QuantizationStrategy.TENSOR_GROUP):
+            if cols % args.group_size != 0:
+                raise ValueError(f"dynamic group quantization: last dimension {cols} is not a multiple of the "
+                                 f"group size {args.group_size}")
+            mn, mx = ops.minmax_groups(x2, args.group_size)
+        elif args.strategy == QuantizationStrategy.TENSOR:
+            mn, mx = ops.minmax_strided(x2, rows, 1, cols, cols, cols)
+        else:
+            raise ValueError(f"dynamic quantization does not support {args.strategy}")
+        scale, zp = calculate_qparams(mn, mx, args, global_scale=gs)
+        return fake_quantize(x2, scale, zp, args, global_scale=gs).reshape(shape)
     g_idx = getattr(module, f"{base_name}_g_idx", None)
     if g_idx is not None and bool((g_idx < 0).any()):
         g_idx = None
@@ -309,7 +323,7 @@ def _wrapped_forward(module: Module):
             return original(self, *args, **kwargs)
         inp = args[0]
         if scheme.input_activations is not None and (
-            scheme.input_activations.dynamic is True or hasattr(self, "input_scale")
+            scheme.input_activations.dynamic in (True, DynamicType.LOCAL) or hasattr(self, "input_scale")
         ) and status in (QuantizationStatus.CALIBRATION, QuantizationStatus.FROZEN):
             inp = forward_quantize(self, inp, "input", scheme.input_activations)
         if scheme.weights is not None and status in (QuantizationStatus.CALIBRATION, QuantizationStatus.FROZEN):
@@ -321,7 +335,9 @@ def _wrapped_forward(module: Module):
                 self.weight.data = saved
         else:
             out = original(self, inp, *args[1:], **kwargs)
-        if scheme.output_activations is not None and hasattr(self, "output_scale") and status in (
+        if scheme.output_activations is not None and (
+            scheme.output_activations.dynamic in (True, DynamicType.LOCAL) or hasattr(self, "output_scale")
+        ) and status in (
             QuantizationStatus.CALIBRATION, QuantizationStatus.FROZEN
         ):
             out = forward_quantize(self, out, "output", scheme.output_activations)

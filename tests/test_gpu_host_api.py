@@ -936,3 +936,39 @@ def test_gptq_modifier_on_an_fp32_model():
     code = Q / s
     assert torch.all((code - code.round()).abs() < 1e-4) and code.round().min() >= -8 and code.round().max() <= 7
     assert ((Q - W0).norm() / W0.norm()).item() < 0.2
+
+
+def test_dynamic_local_nvfp4_activation_golden_through_hooks(golden):
+    # reference: test_lifecycle.py:168-273, second case (NVFP4 activations, dynamic="local", group 3): the
+    # calibrated global scale is kept, the group scales come from each call's values
+    L = _imports()
+    case = golden["lifecycle_activation"]["cases"][1]
+    args = _qargs(case["args"])
+    x = torch.arange(12, dtype=torch.bfloat16, device=DEV).reshape(1, 2, 6)
+    linear = torch.nn.Linear(6, 6, bias=False).to(DEV)
+    linear.weight.data = torch.eye(6, dtype=torch.bfloat16, device=DEV)
+    L["initialize_module_for_quantization"](linear, L["QuantizationScheme"](targets=[], input_activations=args))
+    L["initialize_observer"](linear, "input")
+    linear.input_observer(x)
+    L["update_qparams"](linear, "input")
+    assert linear.input_global_scale.item() == 244.0 and not hasattr(linear, "input_scale")
+    linear.quantization_status = L["QuantizationStatus"].FROZEN
+    out = linear(x)
+    assert torch.equal(out.cpu(), torch.tensor(case["quant"]).to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("spec", [dict(num_bits=8, strategy="group", group_size=32, dynamic=True),
+                                  dict(num_bits=8, strategy="tensor", dynamic=True, symmetric=False),
+                                  dict(num_bits=8, type="float", strategy="tensor", dynamic=True)])
+def test_dynamic_group_and_tensor_activations_match_oracle(spec):
+    """dynamic=True with group and tensor strategies: per-call scales, bit-exact against the oracle."""
+    L = _imports()
+    torch.manual_seed(9)
+    args = _qargs(spec)
+    x = (torch.randn(3, 40, 128) * 2).bfloat16()
+    x[1, 7, 5] = 31.0
+    linear = torch.nn.Linear(128, 128, bias=False).to(DEV).to(torch.bfloat16)
+    L["initialize_module_for_quantization"](linear, L["QuantizationScheme"](targets=[], input_activations=args))
+    got = L["forward_quantize"](linear, x.to(DEV), "input", args)
+    want, _ = F.forward_quantize_dynamic(x, F.QArgs(**spec))
+    assert got.shape == x.shape and torch.equal(got.cpu(), want)
