@@ -33,13 +33,17 @@ from ..quantization.calibration import observe, update_qparams
 from ..quantization.quantization import QuantizationMixin
 from ..utils.concurrent import run_on_streams
 from ..utils.hessian_staging import HessianStagingMixin
-from .gptq_quantize import accumulate_hessian, group_key, make_empty_hessian, quantize_weight, quantize_weight_group
+from .gptq_quantize import (accumulate_hessian, make_empty_hessian, quantize_weight, quantize_weight_group,
+                            width_key)
 
 logger = logging.getLogger("llmcompressor_amd")
 
 __all__ = ["GPTQModifier"]
 
 _GPTQ_Q_PARAMS = ["weight", "weight_scale", "weight_zero_point", "weight_g_idx"]
+
+
+_WIDE_SET = 16  # problems per lock-step set from which the set runs alone on the calling stream
 
 
 class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
@@ -61,9 +65,10 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
         them into a staging buffer, and hand the kernel the list of buffers.  Taken only for contiguous
         bf16/f16 inputs whose token count is a multiple of 64; anything else is copied.  An input that is
         modified in place before its batch is accumulated raises at the flush (tensor version check)
-    :param group_min_modules: when at least this many Linears of one ``compress_module_list`` call share shape,
-        dtype and scheme (the experts of an MoE layer), they are quantised together in lock-step grouped kernels
-        (0 = never); ``group_max_bytes`` bounds the work buffers of one such call
+    :param group_min_modules: when at least this many Linears of one ``compress_module_list`` call have the same
+        number of input features (the experts of an MoE layer; q/k/v/o/gate/up of a decoder layer), their
+        Cholesky chains run in lock-step in grouped kernels, and so do the column loops of those among them
+        that share shape and scheme (0 = never); ``group_max_bytes`` bounds the work buffers of one such job
     :param compress_concurrency: how many modules of one ``compress_module_list`` call are quantised at the
         same time, each on its own HIP stream (1 = one after the other, the reference's behaviour)
 
@@ -81,7 +86,7 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
     hessian_batch_tokens: int = 0
     share_identical_inputs: bool = False
     compress_concurrency: int = 4
-    group_min_modules: int = 8
+    group_min_modules: int = 3
     group_max_bytes: int = 8 << 30
     stage_by_reference: bool = True
 
@@ -239,67 +244,96 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
             self._flush(module)
             self._staged.pop(module, None)
             self._held.pop(module, None)
-        jobs = self._compress_groups(list(module_list))
+        jobs = self._plan_jobs(list(module_list))
+        # a set of many problems (the experts of an MoE layer) fills the chip by itself: such sets are enqueued one
+        # after the other on the calling stream, with one host wait for all of them
+        wide = [job for job in jobs if isinstance(job, list) and len(job) >= _WIDE_SET]
+        if wide:
+            self._finish_sets([self._launch_set(part) for part in wide])
+            jobs = [job for job in jobs if not (isinstance(job, list) and len(job) >= _WIDE_SET)]
         if not jobs:
             return
+        members = [m for job in jobs for m in (job if isinstance(job, list) else [job])]
         workers = min(int(self.compress_concurrency), len(jobs))
-        on_gpu = (all(m.weight.is_cuda and self._hessians[m].is_cuda for m in jobs)
-                  and len({m.weight.device for m in jobs}) == 1)  # one device per call
+        on_gpu = (all(m.weight.is_cuda and self._hessians[m].is_cuda for m in members)
+                  and len({m.weight.device for m in members}) == 1)  # one device per call
         if workers <= 1 or not on_gpu or self.offload_hessians:
-            for module in jobs:
-                self._compress_one(module)
+            for job in jobs:
+                self._compress_job(job)
             return
-        # several modules at once, one host thread and one HIP stream each, most expensive first so that the
+        # several jobs at once, one host thread and one HIP stream each, most expensive first so that the
         # widest module does not start last (see modifiers/utils/concurrent.py); results are unchanged
-        jobs.sort(key=lambda m: -(float(m.weight.shape[1]) ** 3 + float(m.weight.shape[0]) * m.weight.shape[1] ** 2))
-        run_on_streams(jobs, self._compress_one, workers, jobs[0].weight.device, self._streams)
 
-    def _compress_groups(self, jobs):
-        """Quantise sets of at least ``group_min_modules`` Linears of one shape and scheme (the experts of an MoE
-        layer) in lock-step and return the modules that are left for the per-module path."""
+        def cost(job):
+            return sum(float(m.weight.shape[1]) ** 3 + float(m.weight.shape[0]) * m.weight.shape[1] ** 2
+                       for m in (job if isinstance(job, list) else [job]))
+
+        jobs.sort(key=lambda job: -cost(job))
+        run_on_streams(jobs, self._compress_job, workers, members[0].weight.device, self._streams)
+
+    def _plan_jobs(self, modules):
+        """Split the modules of one call into jobs: a list = Linears of one width that share a lock-step
+        Cholesky chain (at least ``group_min_modules`` of them; the work buffers of one job stay within
+        ``group_max_bytes``), a module = the per-module path."""
         if self.group_min_modules <= 0 or self.offload_hessians:
-            return jobs
+            return modules
         sets = {}
-        for m in jobs:
-            key = group_key(m, getattr_chain(m, "quantization_scheme.weights"), self._hessians[m])
+        for m in modules:
+            key = width_key(m, getattr_chain(m, "quantization_scheme.weights"), self._hessians[m])
             if key is not None:
                 sets.setdefault(key, []).append(m)
-        rest = [m for m in jobs]
-        launched = []
+        planned, taken = [], set()
         for members in sets.values():
-            if len(members) < self.group_min_modules:
+            if len(members) < max(2, self.group_min_modules):
                 continue
             K = members[0].weight.shape[1]
-            # bound the lock-step work buffers (factors + work matrices: about 10 K^2 bytes per problem)
+            # factors + work matrices: about 10 K^2 bytes per problem
             per_call = max(1, min(len(members), int(self.group_max_bytes // (10 * K * K))))
-            tallies = [self._num_samples.pop(m) for m in members]
-            if all(isinstance(t, torch.Tensor) and t.is_cuda for t in tallies):  # one transfer, not one per module
-                tallies = torch.stack([t.reshape(()) for t in tallies]).tolist()
-            tallies = [float(t) for t in tallies]
             for i in range(0, len(members), per_call):
                 part = members[i:i + per_call]
-                hs = [self._hessians.pop(m) for m in part]
-                names = [self._module_names.get(m, m.__class__.__name__) for m in part]
-                logger.info(f"Quantizing {len(part)} modules in lock-step ({names[0]} .. {names[-1]})")
-                with torch.no_grad():
-                    results = quantize_weight_group(part, hs, tallies[i:i + per_call], self.block_size,
-                                                    self.dampening_frac)
-                launched.append((part, names, results))
-            done = set(members)
-            rest = [m for m in rest if m not in done]
-        if launched:
-            # the host waits for the device once, after every group has been enqueued
-            failed = torch.cat([torch.stack([r[2] for r in results]) for _, _, results in launched]).tolist()
-            at = 0
-            for part, names, results in launched:
-                for m, name, (loss, q_param_dict, _) in zip(part, names, results):
-                    if failed[at]:
-                        logger.warning(f"Failed to invert hessian of {name} due to numerical instability. Falling "
-                                       "back to round-to-nearest for this module.")
-                    at += 1
-                    for attr, val in q_param_dict.items():
-                        update_offload_parameter(m, attr, val)
-        return rest
+                planned.append(part if len(part) > 1 else part[0])
+            taken.update(members)
+        return planned + [m for m in modules if m not in taken]
+
+    def _compress_job(self, job, produced_on=None, consumed_on=None):
+        if isinstance(job, list):
+            self._compress_set(job, produced_on, consumed_on)
+        else:
+            self._compress_one(job, produced_on, consumed_on)
+
+    def _compress_set(self, part, produced_on=None, consumed_on=None):
+        """Linears of one width in lock-step (``quantize_weight_group``); parameters as on the per-module path."""
+        self._finish_sets([self._launch_set(part, produced_on)], consumed_on)
+
+    def _launch_set(self, part, produced_on=None):
+        hs = [self._hessians.pop(m) for m in part]
+        tallies = [self._num_samples.pop(m) for m in part]
+        if all(isinstance(t, torch.Tensor) and t.is_cuda for t in tallies):  # one transfer, not one per module
+            tallies = torch.stack([t.reshape(()) for t in tallies]).tolist()
+        tallies = [float(t) for t in tallies]
+        if produced_on is not None:  # allocated on the calibration stream, last read on this one
+            for h in hs:
+                h.record_stream(produced_on)
+        names = [self._module_names.get(m, m.__class__.__name__) for m in part]
+        logger.info(f"Quantizing {len(part)} modules in lock-step ({names[0]} .. {names[-1]})")
+        with torch.no_grad():
+            results = quantize_weight_group(part, hs, tallies, self.block_size, self.dampening_frac)
+        return part, names, results
+
+    def _finish_sets(self, launched, consumed_on=None):
+        # one host wait for everything enqueued so far
+        failed = torch.cat([torch.stack([r[2] for r in results]) for _, _, results in launched]).tolist()
+        at = 0
+        for part, names, results in launched:
+            for m, name, (loss, q_param_dict, _) in zip(part, names, results):
+                if failed[at]:
+                    logger.warning(f"Failed to invert hessian of {name} due to numerical instability. Falling "
+                                   "back to round-to-nearest for this module.")
+                at += 1
+                for attr, val in q_param_dict.items():
+                    if consumed_on is not None and val.is_cuda:  # allocated on a side stream, read by later forwards
+                        val.record_stream(consumed_on)
+                    update_offload_parameter(m, attr, val)
 
     def _compress_one(self, module, produced_on=None, consumed_on=None):
         name = self._module_names.get(module, module.__class__.__name__)

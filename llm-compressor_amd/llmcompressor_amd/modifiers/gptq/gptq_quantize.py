@@ -22,7 +22,7 @@ logger = logging.getLogger("llmcompressor_amd")
 GPTQ_PRECISION = torch.float32
 
 __all__ = ["make_empty_hessian", "accumulate_hessian", "quantize_weight", "quantize_weight_tensors",
-           "quantize_weight_group", "group_key"]
+           "quantize_weight_group", "group_key", "width_key"]
 
 
 def make_empty_hessian(module: torch.nn.Module, device: torch.device | None = None) -> torch.Tensor:
@@ -150,7 +150,7 @@ def quantize_weight(module: torch.nn.Module, quant_args: QuantizationArgs, hessi
 
 
 def group_key(module: torch.nn.Module, quant_args: QuantizationArgs, hessian: torch.Tensor):
-    """Modules with equal keys can go through ``quantize_weight_group`` together; None = not eligible."""
+    """Modules with equal keys share one lock-step column loop in ``quantize_weight_group``; None = not eligible."""
     w = module.weight
     if not isinstance(module, torch.nn.Linear) or w.ndim != 2 or not w.is_cuda or not hessian.is_cuda:
         return None
@@ -161,43 +161,82 @@ def group_key(module: torch.nn.Module, quant_args: QuantizationArgs, hessian: to
             quant_args.model_dump_json() if hasattr(quant_args, "model_dump_json") else repr(quant_args))
 
 
-def quantize_weight_group(modules, hessians, hessian_divisors, blocksize: int = 128, percdamp: float = 0.01):
-    """``quantize_weight`` for several Linears of one shape and scheme at once (the experts of an MoE layer):
-    one lock-step Cholesky chain and one lock-step column loop for all of them instead of a chain of tiny
-    kernels per module.  Same results as calling ``quantize_weight`` on each.  Returns a list of
-    (loss tensor, q_param_dict, info tensor)."""
-    n = len(modules)
-    quant_args = getattr(modules[0].quantization_scheme, "weights")
-    strategy, actorder = quant_args.strategy, quant_args.actorder
-    Ws = [m.weight.data if m.weight.data.is_contiguous() else m.weight.data.contiguous() for m in modules]
-    num_rows, num_columns = Ws[0].shape
-    final_dtype = Ws[0].dtype
-    if actorder == ActivationOrdering.GROUP and strategy not in (QuantizationStrategy.GROUP,
-                                                                 QuantizationStrategy.TENSOR_GROUP):
-        actorder = None
-    perms = None
-    if actorder:
-        perms = torch.stack([torch.argsort(torch.diagonal(H), descending=True) for H in hessians])
-    row_div, srow, divisor = _scale_layout(strategy, quant_args, num_rows, num_columns)
-    g_idxs = None
-    if divisor is not None:
-        base = torch.arange(num_columns, device=Ws[0].device, dtype=torch.int) // divisor
-        g_idxs = [base[perms[b]] if actorder == ActivationOrdering.WEIGHT else base for b in range(n)]
-    qps = [m.weight_observer.get_qparams() for m in modules]
-    fmt, bits = kernel_format(quant_args)
-    zps = None if quant_args.symmetric else [qp["zero_point"].to(torch.int8) for qp in qps]
-    kscales = [effective_scale(qp["scale"], quant_args, final_dtype) for qp in qps]
-    has_gs = qps[0]["global_scale"] is not None
-    gss = [qp["global_scale"] for qp in qps] if has_gs else None
+def width_key(module: torch.nn.Module, quant_args: QuantizationArgs, hessian: torch.Tensor):
+    """Modules with equal keys can share one lock-step Cholesky chain (``quantize_weight_group``): same number
+    of columns, device and Hessian layout, and all or none ordered by activation; None = not eligible."""
+    if group_key(module, quant_args, hessian) is None:
+        return None
+    return (module.weight.shape[1], module.weight.device, hessian.stride(0), bool(quant_args.actorder))
 
-    U, dead, info = ops.gptq_hinv_grouped(hessians, perms, hessian_divisors, percdamp)
-    outs, loss = ops.gptq_quantize_grouped(Ws, U, kscales, zps, fmt, bits, row_div, srow, g_idxs=g_idxs, perms=perms,
-                                           dead=dead, global_scales=gss, blocksize=blocksize)
-    results = []
-    for b, (m, qp) in enumerate(zip(modules, qps)):
+
+def quantize_weight_group(modules, hessians, hessian_divisors, blocksize: int = 128, percdamp: float = 0.01):
+    """``quantize_weight`` for several Linears of one width at once (the experts of an MoE layer, or the
+    projections of a decoder layer that read the hidden state): one lock-step Cholesky chain for all of them,
+    and one lock-step column loop per set of equal shape and scheme, instead of a chain of small kernels per
+    module.  Same results as calling ``quantize_weight`` on each.  Returns a list of
+    (loss tensor, q_param_dict, info tensor) in the order of ``modules``."""
+    n = len(modules)
+    keys = [group_key(m, m.quantization_scheme.weights, H) for m, H in zip(modules, hessians)]
+    # members of one column-loop set next to each other, so that their factors are one slice of the batch
+    order = sorted(range(n), key=lambda i: (keys.index(keys[i]), i))
+    mods = [modules[i] for i in order]
+    Hs = [hessians[i] for i in order]
+    divs = [hessian_divisors[i] for i in order]
+    keys = [keys[i] for i in order]
+    prep = []
+    for m, H in zip(mods, Hs):
+        quant_args = m.quantization_scheme.weights
+        strategy, actorder = quant_args.strategy, quant_args.actorder
+        W = m.weight.data if m.weight.data.is_contiguous() else m.weight.data.contiguous()
+        num_rows, num_columns = W.shape
+        perm = torch.argsort(torch.diagonal(H), descending=True) if actorder else None
+        row_div, srow, divisor = _scale_layout(strategy, quant_args, num_rows, num_columns)
+        g_idx = None
+        if divisor is not None:
+            g_idx = torch.arange(num_columns, device=W.device, dtype=torch.int) // divisor
+            if actorder == ActivationOrdering.WEIGHT:
+                g_idx = g_idx[perm]
+        qp = m.weight_observer.get_qparams()
+        prep.append(dict(args=quant_args, W=W, perm=perm, g_idx=g_idx, qp=qp, row_div=row_div, srow=srow,
+                         zp=None if quant_args.symmetric else qp["zero_point"].to(torch.int8),
+                         kscale=effective_scale(qp["scale"], quant_args, W.dtype)))
+    perms = torch.stack([p["perm"] for p in prep]) if prep[0]["perm"] is not None else None
+
+    U, dead, info = ops.gptq_hinv_grouped(Hs, perms, divs, percdamp)
+
+    outs, losses = [None] * n, [None] * n
+    at = 0
+    while at < n:
+        end = at + 1
+        while end < n and keys[end] == keys[at]:
+            end += 1
+        part = prep[at:end]
+        first = part[0]
+        fmt, bits = kernel_format(first["args"])
+        if end - at == 1:
+            outs[at], losses[at] = ops.gptq_quantize(
+                first["W"], U[at], first["kscale"], first["zp"], fmt, bits, first["row_div"], first["srow"],
+                g_idx=first["g_idx"], perm=first["perm"], dead=dead[at], global_scale=first["qp"]["global_scale"],
+                blocksize=blocksize)
+        else:
+            has_gs = first["qp"]["global_scale"] is not None
+            o, l = ops.gptq_quantize_grouped(
+                [p["W"] for p in part], U[at:end], [p["kscale"] for p in part],
+                None if first["zp"] is None else [p["zp"] for p in part], fmt, bits, first["row_div"], first["srow"],
+                g_idxs=None if first["g_idx"] is None else [p["g_idx"] for p in part],
+                perms=None if perms is None else perms[at:end], dead=dead[at:end],
+                global_scales=[p["qp"]["global_scale"] for p in part] if has_gs else None, blocksize=blocksize)
+            for b in range(end - at):
+                outs[at + b], losses[at + b] = o[b], l[b]
+        at = end
+
+    results = [None] * n
+    for j, (m, p) in enumerate(zip(mods, prep)):
+        quant_args, qp = p["args"], p["qp"]
+        final_dtype = p["W"].dtype
         scale, zero_point, global_scale = qp["scale"], qp["zero_point"], qp["global_scale"]
         q = {
-            "weight": outs[b].reshape(m.weight.shape),
+            "weight": outs[j].reshape(m.weight.shape),
             "weight_scale": scale if scale.dtype in (torch.uint8, torch.float8_e4m3fn) else scale.to(dtype=final_dtype),
             "weight_zero_point": zero_point.to(dtype=quant_args.zp_dtype),
         }
@@ -205,5 +244,5 @@ def quantize_weight_group(modules, hessians, hessian_divisors, blocksize: int = 
             q["weight_scale"] = scale
         if global_scale is not None:
             q["weight_global_scale"] = global_scale.to(dtype=final_dtype)
-        results.append((loss[b], q, info[b]))
+        results[order[j]] = (losses[j].reshape(()), q, info[j])
     return results

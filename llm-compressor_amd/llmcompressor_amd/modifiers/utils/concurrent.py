@@ -22,8 +22,13 @@ def run_on_streams(jobs: List, work: Callable, workers: int, device: torch.devic
     ``workers`` at a time.  The first exception stops the remaining jobs and is re-raised on the caller."""
     jobs = list(jobs)
     streams = stream_cache.setdefault(device, [])
-    while len(streams) < workers:
+    while len(streams) < max(workers, 4):
+        # the runtime binds a stream to one of its few hardware queues at the stream's first submission; two
+        # streams first used at the same moment from two threads have been seen to land on the same queue and
+        # then run strictly one after the other.  One tiny submission per new stream, in turn, spreads them.
         streams.append(torch.cuda.Stream(device=device))
+        with torch.cuda.stream(streams[-1]):
+            torch.zeros(1, device=device)
     main = torch.cuda.current_stream(device)
     ready = main.record_event()
     lock = threading.Lock()
