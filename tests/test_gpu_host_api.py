@@ -1033,3 +1033,60 @@ def test_gptq_same_width_linears_in_lock_step_match_per_module_path(actorder):
         for n in params:
             assert torch.equal(params[n], results[0][1][n]), n
     assert not torch.equal(results[0][1]["layers.0.q.weight"], init["layers.0.q.weight"])
+
+
+def test_oneshot_gptq_on_a_transformers_llama(tmp_path):
+    """A random-init transformers LlamaForCausalLM (2 layers, grouped-query attention) through oneshot with the
+    W4A16 preset: every decoder Linear ends on its group's int4 grid with the preset's parameters, lm_head is
+    left alone, the logits stay close to the dense model's, and the checkpoint holds the packed layout under
+    the model's own tensor names."""
+    transformers = pytest.importorskip("transformers")
+    from safetensors.torch import load_file
+
+    from llmcompressor_amd import oneshot
+    from llmcompressor_amd.compressors import decompress_weight
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+    from llmcompressor_amd.quantization import QuantizationArgs
+
+    torch.manual_seed(0)
+    cfg = transformers.LlamaConfig(hidden_size=128, intermediate_size=256, num_hidden_layers=2,
+                                   num_attention_heads=4, num_key_value_heads=2, vocab_size=256,
+                                   max_position_embeddings=128)
+    model = transformers.LlamaForCausalLM(cfg).to(torch.bfloat16).to(DEV)
+    dense = {n: p.detach().clone() for n, p in model.named_parameters()}
+    probe = torch.randint(0, 256, (2, 32), device=DEV)
+    with torch.no_grad():
+        logits0 = model(probe).logits.float()
+    data = [{"input_ids": torch.randint(0, 256, (1, 64))} for _ in range(8)]
+    out_dir = str(tmp_path / "llama")
+    oneshot(model=model, recipe=GPTQModifier(targets="Linear", scheme="W4A16", ignore=["lm_head"]), dataset=data,
+            output_dir=out_dir)
+    with torch.no_grad():
+        logits1 = model(probe).logits.float()
+    assert torch.isfinite(logits1).all()
+    assert ((logits1 - logits0).norm() / logits0.norm()).item() < 0.35
+    quantised = 0
+    for name, mod in model.named_modules():
+        if not isinstance(mod, torch.nn.Linear):
+            continue
+        if name == "lm_head":
+            assert not hasattr(mod, "weight_scale") and torch.equal(mod.weight, dense["lm_head.weight"])
+            continue
+        quantised += 1
+        assert mod.weight_scale.shape == (mod.out_features, mod.in_features // 128)
+        code = mod.weight.float() / mod.weight_scale.float().repeat_interleave(128, dim=1)
+        assert (code - code.round()).abs().max() <= 8 * 2.0 ** -8 and code.round().abs().max() <= 8
+        assert not torch.equal(mod.weight, dense[name + ".weight"])
+    assert quantised == 14
+    sd = load_file(os.path.join(out_dir, "model.safetensors"))
+    key = "model.layers.1.mlp.down_proj."
+    assert sd[key + "weight_packed"].dtype == torch.int32 and sd[key + "weight_packed"].shape == (128, 256 // 8)
+    assert sd[key + "weight_shape"].tolist() == [128, 256] and key + "weight" not in sd
+    assert "lm_head.weight" in sd and "model.embed_tokens.weight" in sd
+    deq = decompress_weight({k[len(key):]: v for k, v in sd.items() if k.startswith(key)},
+                            QuantizationArgs(num_bits=4, strategy="group", group_size=128), "pack-quantized")
+    assert torch.equal(deq.to(DEV), model.model.layers[1].mlp.down_proj.weight.data)
+    saved = json.load(open(os.path.join(out_dir, "config.json")))
+    assert saved["model_type"] == "llama" and saved["hidden_size"] == 128
+    q = saved["quantization_config"]
+    assert q["quant_method"] == "compressed-tensors" and q["format"] == "pack-quantized" and "lm_head" in q["ignore"]
