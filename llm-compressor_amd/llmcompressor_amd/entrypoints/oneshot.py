@@ -6,6 +6,7 @@ datasets by hub name needs network access and is not part of this build.
 """
 from __future__ import annotations
 
+import logging
 import os
 from typing import Optional
 
@@ -13,6 +14,8 @@ import torch
 
 from ..core import active_session
 from ..pipelines import CalibrationPipeline
+
+logger = logging.getLogger("llmcompressor_amd")
 
 __all__ = ["Oneshot", "oneshot"]
 
@@ -39,6 +42,12 @@ class Oneshot:
                                          moe_calibrate_all_experts=moe_calibrate_all_experts, **kwargs)
 
     def __call__(self):
+        from ..modeling.moe import get_non_linearized_moes, linearize_moe
+
+        if get_non_linearized_moes(self.model):  # reference: entrypoints/oneshot.py:237-243
+            logger.warning("Detected an MoE model whose experts are stored as fused 3-D tensors; replacing them "
+                           "by per-expert Linears so that they can be calibrated and quantized.")
+            linearize_moe(self.model)
         self.apply_recipe_modifiers(self.dataset)
         if self.output_dir is not None:
             from ..compressors import save_pretrained_compressed

@@ -81,15 +81,31 @@ class CalibrationPipeline:
 
 
 def find_decoder_layers(model: torch.nn.Module, sequential_targets=None) -> List[torch.nn.Module]:
-    """The modules that form the sequential partition: explicit class names, else the longest ModuleList."""
+    """The modules that form the sequential partition: explicit class names, else the model's own
+    ``_no_split_modules`` (what the reference infers for transformers models), else the longest ModuleList
+    that is not nested inside an element of another one (an experts list inside a decoder layer is not the
+    layer list)."""
     if sequential_targets:
         names = [sequential_targets] if isinstance(sequential_targets, str) else list(sequential_targets)
         layers = [m for m in model.modules() if m.__class__.__name__ in names]
         if layers:
             return layers
+    no_split = getattr(model, "_no_split_modules", None)
+    if no_split:
+        layers = [m for m in model.modules() if m.__class__.__name__ in set(no_split)]
+        # nested matches (a no-split block inside another) would run twice: keep the outermost
+        inner = {id(x) for l in layers for x in l.modules() if x is not l}
+        layers = [l for l in layers if id(l) not in inner]
+        if layers:
+            return layers
+    lists = [m for m in model.modules() if isinstance(m, torch.nn.ModuleList) and len(m) > 0]
+    nested = set()
+    for outer in lists:
+        for element in outer:
+            nested.update(id(x) for x in element.modules() if isinstance(x, torch.nn.ModuleList))
     best = None
-    for m in model.modules():
-        if isinstance(m, torch.nn.ModuleList) and len(m) > 0 and (best is None or len(m) > len(best)):
+    for m in lists:
+        if id(m) not in nested and (best is None or len(m) > len(best)):
             best = m
     if best is None:
         raise ValueError("could not infer sequential targets: the model has no ModuleList of layers")

@@ -1090,3 +1090,53 @@ def test_oneshot_gptq_on_a_transformers_llama(tmp_path):
     assert saved["model_type"] == "llama" and saved["hidden_size"] == 128
     q = saved["quantization_config"]
     assert q["quant_method"] == "compressed-tensors" and q["format"] == "pack-quantized" and "lm_head" in q["ignore"]
+
+
+def test_oneshot_gptq_on_a_transformers_qwen3_moe(tmp_path):
+    """A random-init transformers Qwen3MoeForCausalLM (fused 3-D expert tensors): oneshot replaces the fused
+    experts by per-expert Linears (same logits bit for bit), partitions by decoder layer (not by the experts
+    list), quantises attention and expert Linears with routed calibration, leaves the router alone, and writes
+    the per-expert tensor names."""
+    transformers = pytest.importorskip("transformers")
+    import copy
+
+    from safetensors.torch import load_file
+
+    from llmcompressor_amd import oneshot
+    from llmcompressor_amd.modeling import LinearExperts2D, get_non_linearized_moes, linearize_moe
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+
+    torch.manual_seed(0)
+    cfg = transformers.Qwen3MoeConfig(hidden_size=128, intermediate_size=256, moe_intermediate_size=128,
+                                      num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2,
+                                      head_dim=32, vocab_size=256, max_position_embeddings=128, num_experts=8,
+                                      num_experts_per_tok=2)
+    model = transformers.Qwen3MoeForCausalLM(cfg).to(torch.bfloat16).to(DEV)
+    probe = torch.randint(0, 256, (2, 32), device=DEV)
+    with torch.no_grad():
+        logits0 = model(probe).logits.float()
+        assert len(get_non_linearized_moes(model)) == 2
+        twin = linearize_moe(copy.deepcopy(model))
+        assert get_non_linearized_moes(twin) == [] and isinstance(twin.model.layers[0].mlp.experts, LinearExperts2D)
+        assert torch.equal(twin(probe).logits.float(), logits0)
+    del twin
+    router0 = model.model.layers[0].mlp.gate.weight.detach().clone()
+    data = [{"input_ids": torch.randint(0, 256, (1, 64))} for _ in range(8)]
+    out_dir = str(tmp_path / "moe")
+    oneshot(model=model, recipe=GPTQModifier(targets="Linear", scheme="W4A16", ignore=["lm_head", "re:.*mlp.gate$"]),
+            dataset=data, output_dir=out_dir, moe_calibrate_all_experts=False)
+    with torch.no_grad():
+        logits1 = model(probe).logits.float()
+    assert torch.isfinite(logits1).all() and ((logits1 - logits0).norm() / logits0.norm()).item() < 0.4
+    assert torch.equal(model.model.layers[0].mlp.gate.weight, router0)
+    experts = model.model.layers[1].mlp.experts
+    assert isinstance(experts, LinearExperts2D) and len(experts) == 8
+    for lin in (experts[3].gate_proj, experts[5].down_proj, model.model.layers[1].self_attn.o_proj):
+        code = lin.weight.float() / lin.weight_scale.float().repeat_interleave(128, dim=1)
+        assert (code - code.round()).abs().max() <= 8 * 2.0 ** -8 and code.round().abs().max() <= 8
+    sd = load_file(os.path.join(out_dir, "model.safetensors"))
+    for e in range(8):
+        for proj, shape in (("gate_proj", [128, 128]), ("up_proj", [128, 128]), ("down_proj", [128, 128])):
+            key = f"model.layers.0.mlp.experts.{e}.{proj}."
+            assert sd[key + "weight_packed"].dtype == torch.int32 and sd[key + "weight_shape"].tolist() == shape
+    assert "model.layers.0.mlp.gate.weight" in sd and "model.layers.0.mlp.experts.gate_up_proj" not in sd

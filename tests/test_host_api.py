@@ -427,3 +427,78 @@ def test_moe_forward_equals_the_per_expert_loop(dtype, all_experts):
     experts.to(dtype)
     tol = 1e-5 if dtype == torch.float32 else 5e-2
     assert (got.double() - dense).abs().max() <= tol * dense.abs().max()
+
+
+def test_sequential_partition_prefers_decoder_layers_over_nested_lists():
+    """The layer list is the model's ``_no_split_modules`` classes when it names them, else the longest
+    ModuleList that is not nested inside another list's element (an experts list is not the layer list)."""
+    from llmcompressor_amd.pipelines import find_decoder_layers
+
+    class Layer(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.experts = torch.nn.ModuleList([torch.nn.Linear(4, 4) for _ in range(8)])
+
+    class Model(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.layers = torch.nn.ModuleList([Layer() for _ in range(2)])
+
+    m = Model()
+    assert find_decoder_layers(m, None) == list(m.layers)
+    m._no_split_modules = ["Layer"]
+    assert find_decoder_layers(m, None) == list(m.layers)
+    assert find_decoder_layers(m, ["Linear"]) == [x for x in m.modules() if isinstance(x, torch.nn.Linear)]
+
+
+@pytest.mark.parametrize("transposed,bias", [(False, False), (True, False), (False, True)])
+def test_linearize_moe_keeps_the_function(transposed, bias):
+    """A fused experts module (standard layout, transposed layout, with biases) and its per-expert replacement
+    compute the same function (reference: modeling/moe/linear_experts.py:186-208, linearize.py:97-125)."""
+    from llmcompressor_amd.modeling import LinearExperts2D, get_non_linearized_moes, linearize_moe
+
+    E, H, I, T, k = 4, 8, 12, 10, 2
+    torch.manual_seed(5)
+
+    class Fused(torch.nn.Module):
+        is_transposed = transposed
+
+        def __init__(self):
+            super().__init__()
+            gu, dn = torch.randn(E, 2 * I, H), torch.randn(E, H, I)
+            self.gate_up_proj = torch.nn.Parameter(gu.transpose(1, 2).contiguous() if transposed else gu)
+            self.down_proj = torch.nn.Parameter(dn.transpose(1, 2).contiguous() if transposed else dn)
+            if bias:
+                self.gate_up_proj_bias = torch.nn.Parameter(torch.randn(E, 2 * I))
+                self.down_proj_bias = torch.nn.Parameter(torch.randn(E, H))
+            self.act_fn = torch.nn.GELU()
+
+        def forward(self, x, idx, w):
+            out = torch.zeros_like(x)
+            for t in range(x.shape[0]):
+                for j in range(idx.shape[1]):
+                    e = int(idx[t, j])
+                    gu = self.gate_up_proj[e].t() if transposed else self.gate_up_proj[e]
+                    dn = self.down_proj[e].t() if transposed else self.down_proj[e]
+                    h = gu @ x[t] + (self.gate_up_proj_bias[e] if bias else 0)
+                    h = self.act_fn(h[:I]) * h[I:]
+                    out[t] += w[t, j] * (dn @ h + (self.down_proj_bias[e] if bias else 0))
+            return out
+
+    class Model(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.block = torch.nn.ModuleDict({"experts": Fused()})
+
+    model = Model()
+    x = torch.randn(T, H)
+    w, idx = torch.topk(torch.softmax(torch.randn(T, E), -1), k, -1)
+    with torch.no_grad():
+        want = model.block["experts"](x, idx, w)
+        assert [n for n, _ in get_non_linearized_moes(model)] == ["block.experts"]
+        linearize_moe(model)
+        lin = model.block["experts"]
+        assert isinstance(lin, LinearExperts2D) and get_non_linearized_moes(model) == []
+        assert isinstance(lin[0].act_fn, torch.nn.GELU) and (lin[0].gate_proj.bias is not None) == bias
+        got = lin(x, idx, w)
+    assert torch.allclose(got, want, atol=1e-4, rtol=1e-4)
