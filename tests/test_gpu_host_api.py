@@ -1140,3 +1140,35 @@ def test_oneshot_gptq_on_a_transformers_qwen3_moe(tmp_path):
             key = f"model.layers.0.mlp.experts.{e}.{proj}."
             assert sd[key + "weight_packed"].dtype == torch.int32 and sd[key + "weight_shape"].tolist() == shape
     assert "model.layers.0.mlp.gate.weight" in sd and "model.layers.0.mlp.experts.gate_up_proj" not in sd
+
+
+@pytest.mark.parametrize("scheme", ["FP8_DYNAMIC", "NVFP4A16", "W4A16"])
+def test_model_free_ptq_equals_oneshot_rtn_on_a_transformers_checkpoint(tmp_path, scheme):
+    """model_free_ptq on the safetensors checkpoint of a transformers Llama writes, tensor for tensor and byte
+    for byte, what oneshot with a data-free QuantizationModifier writes for the loaded model (the NVFP4
+    global scales fused over q/k/v and gate/up included)."""
+    transformers = pytest.importorskip("transformers")
+    from safetensors.torch import load_file
+
+    from llmcompressor_amd import model_free_ptq, oneshot
+    from llmcompressor_amd.modifiers.quantization import QuantizationModifier
+
+    torch.manual_seed(0)
+    cfg = transformers.LlamaConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=2,
+                                   num_attention_heads=4, num_key_value_heads=2, vocab_size=256,
+                                   max_position_embeddings=128)
+    model = transformers.LlamaForCausalLM(cfg).to(torch.bfloat16).to(DEV)
+    src, dst, out = str(tmp_path / "src"), str(tmp_path / "dst"), str(tmp_path / "out")
+    model.save_pretrained(src, safe_serialization=True)
+    model_free_ptq(model_stub=src, save_directory=dst, scheme=scheme,
+                   ignore=["lm_head", "re:.*embed.*", "re:.*norm.*"], device="cuda:0")
+    oneshot(model=model, recipe=QuantizationModifier(targets="Linear", scheme=scheme, ignore=["lm_head"]),
+            output_dir=out)
+    a, b = load_file(os.path.join(dst, "model.safetensors")), load_file(os.path.join(out, "model.safetensors"))
+    assert sorted(a) == sorted(b)
+    for k in b:
+        assert a[k].dtype == b[k].dtype and a[k].shape == b[k].shape, k
+        assert torch.equal(a[k].contiguous().view(torch.uint8), b[k].contiguous().view(torch.uint8)), k
+    qa = json.load(open(os.path.join(dst, "config.json")))["quantization_config"]
+    qb = json.load(open(os.path.join(out, "config.json")))["quantization_config"]
+    assert qa["format"] == qb["format"] and qa["quant_method"] == qb["quant_method"] == "compressed-tensors"
