@@ -55,7 +55,9 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
     :param actorder: column order; defaults to "static" (quantise in descending diag(H) order, no g_idx)
     :param offload_hessians: keep Hessians on the CPU between hook calls
     :param hessian_batch_tokens: stage activations and launch the Hessian kernel once this many tokens
-        are pending (0 = one launch per hook call, the reference's behaviour)
+        are pending (0 = one launch per hook call, the reference's behaviour).  The [K,K] accumulator is read
+        and written once per launch, so for wide Linears many hook calls per launch are what keeps the kernel
+        on the matrix cores instead of on memory
 
     :param share_identical_inputs: Linears that are fed the very same tensor on every call (q/k/v, gate/up)
         have the same Hessian; accumulate it once and hand each of them a copy when it is compressed.
@@ -83,7 +85,7 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
     dampening_frac: float | None = 0.01
     actorder: ActivationOrdering | Sentinel | None = Sentinel("static")
     offload_hessians: bool = False
-    hessian_batch_tokens: int = 0
+    hessian_batch_tokens: int = 65536
     share_identical_inputs: bool = False
     compress_concurrency: int = 4
     group_min_modules: int = 3

@@ -560,7 +560,8 @@ def test_gptq_shared_input_hessians_are_identical():
         raw = ops.hessian_accumulate_
         ops.hessian_accumulate_ = lambda H, x, **kw: (calls.append(1), raw(H, x, **kw))[1]
         try:
-            mod = GPTQModifier(targets="Linear", share_identical_inputs=share, config_groups={"g": dict(
+            mod = GPTQModifier(targets="Linear", share_identical_inputs=share, hessian_batch_tokens=0,
+                               config_groups={"g": dict(
                 targets=["Linear"], weights=dict(num_bits=4, strategy="group", group_size=32))})
             session = active_session()
             session.reset()
