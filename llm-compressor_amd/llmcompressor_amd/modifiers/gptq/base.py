@@ -67,6 +67,8 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
         them into a staging buffer, and hand the kernel the list of buffers.  Taken only for contiguous
         bf16/f16 inputs whose token count is a multiple of 64; anything else is copied.  An input that is
         modified in place before its batch is accumulated raises at the flush (tensor version check)
+    :param stage_max_bytes: bound on the activations held by reference over all modules; beyond it everything
+        pending is accumulated at once (matters when a pipeline runs the whole model per batch)
     :param group_min_modules: when at least this many Linears of one ``compress_module_list`` call have the same
         number of input features (the experts of an MoE layer; q/k/v/o/gate/up of a decoder layer), their
         Cholesky chains run in lock-step in grouped kernels, and so do the column loops of those among them
@@ -91,12 +93,14 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
     group_min_modules: int = 3
     group_max_bytes: int = 8 << 30
     stage_by_reference: bool = True
+    stage_max_bytes: int = 16 << 30
 
     _module_names: dict = PrivateAttr(default_factory=dict)
     _hessians: dict = PrivateAttr(default_factory=dict)
     _num_samples: dict = PrivateAttr(default_factory=dict)
     _staged: dict = PrivateAttr(default_factory=dict)
     _held: dict = PrivateAttr(default_factory=dict)
+    _held_bytes: int = PrivateAttr(default=0)
     _group_pending: list | None = PrivateAttr(default=None)
     _leader: dict = PrivateAttr(default_factory=dict)  # follower module -> module whose Hessian it shares
     _recent_input: tuple | None = PrivateAttr(default=None)  # (tensor kept alive, its version, leader)
@@ -370,6 +374,7 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
         self._num_samples = dict()
         self._staged = dict()
         self._held = dict()
+        self._held_bytes = 0
         self._leader = dict()
         self._recent_input = None
         return True

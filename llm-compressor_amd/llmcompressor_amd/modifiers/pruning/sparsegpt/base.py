@@ -44,12 +44,14 @@ class SparseGPTModifier(SparsityModifierBase, HessianStagingMixin):
     offload_hessians: bool = False
     hessian_batch_tokens: int = 0
     stage_by_reference: bool = True
+    stage_max_bytes: int = 16 << 30
     compress_concurrency: int = 4
 
     _num_samples: dict = PrivateAttr(default_factory=dict)
     _hessians: dict = PrivateAttr(default_factory=dict)
     _staged: dict = PrivateAttr(default_factory=dict)
     _held: dict = PrivateAttr(default_factory=dict)
+    _held_bytes: int = PrivateAttr(default=0)
     _streams: dict = PrivateAttr(default_factory=dict)
 
     def calibrate_module(self, module: torch.nn.Module, args: tuple[torch.Tensor, ...], _output: torch.Tensor):
@@ -122,6 +124,7 @@ class SparseGPTModifier(SparsityModifierBase, HessianStagingMixin):
         self._num_samples = dict()
         self._staged = dict()
         self._held = dict()
+        self._held_bytes = 0
         self._module_names = dict()
         self._module_sparsities = dict()
         return True

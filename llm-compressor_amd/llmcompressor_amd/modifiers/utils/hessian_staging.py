@@ -5,7 +5,8 @@ modifiers/pruning/sparsegpt/base.py:88-117 in the reference).
 The ``[K,K]`` accumulator is read and written once per launch, so several hook calls are accumulated by one
 launch: either by reference (the hook's input tensors are held and handed to the kernel as a list of buffers)
 or through a staging buffer.  A class using the mixin provides ``_hessians``, ``_num_samples``, ``_staged``,
-``_held`` (dicts keyed by module) and the fields ``hessian_batch_tokens`` and ``stage_by_reference``.
+``_held`` (dicts keyed by module), ``_held_bytes`` and the fields ``hessian_batch_tokens``, ``stage_by_reference``
+and ``stage_max_bytes`` (bound on the activations held by reference over all modules).
 """
 from __future__ import annotations
 
@@ -37,8 +38,14 @@ class HessianStagingMixin:
                 held[0].append(x)
                 held[1].append((inp, inp._version))
                 held[2] += samples
+                self._held_bytes = getattr(self, "_held_bytes", 0) + x.numel() * x.element_size()
                 if len(held[0]) * n >= self.hessian_batch_tokens or len(held[0]) >= ops.SEGMENTS_MAX:
                     self._flush(module)
+                elif self._held_bytes > getattr(self, "stage_max_bytes", 1 << 62):
+                    # many modules holding batches at once (a pipeline that runs the whole model per batch):
+                    # accumulate everything pending rather than keep more activations alive
+                    for other in [m for m, h in self._held.items() if h[0]]:
+                        self._flush(other)
                 return
             if held is not None and held[0]:
                 self._flush(module)
@@ -68,6 +75,7 @@ class HessianStagingMixin:
                         "after the forward hook saw it; set stage_by_reference=False for this model")
             ops.hessian_accumulate_segments_(self._hessians[module], held[0], alpha=2.0, assume_symmetric=True)
             self._num_samples[module] += held[2]
+            self._held_bytes = getattr(self, "_held_bytes", 0) - sum(x.numel() * x.element_size() for x in held[0])
             self._held[module] = [[], [], 0]
         st = self._staged.get(module)
         if st is None or st[1] == 0:

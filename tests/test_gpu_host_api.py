@@ -1173,3 +1173,56 @@ def test_model_free_ptq_equals_oneshot_rtn_on_a_transformers_checkpoint(tmp_path
     qa = json.load(open(os.path.join(dst, "config.json")))["quantization_config"]
     qb = json.load(open(os.path.join(out, "config.json")))["quantization_config"]
     assert qa["format"] == qb["format"] and qa["quant_method"] == qb["quant_method"] == "compressed-tensors"
+
+
+def test_gptq_held_activations_are_bounded():
+    """stage_max_bytes: with a tiny bound the batches held by reference are accumulated early (more launches,
+    never more than the bound alive); Hessians and sample counts equal the unbounded run's."""
+    from llmcompressor_amd import ops
+    from llmcompressor_amd.core import LifecycleCallbacks, active_session
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+
+    class Wrap(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.layers = torch.nn.ModuleList([torch.nn.Sequential(*[torch.nn.Linear(128, 128, bias=False)
+                                                                      for _ in range(4)])])
+
+    torch.manual_seed(8)
+    init = Wrap().to(DEV).to(torch.bfloat16).state_dict()
+    xs = [torch.randn(1, 64, 128, device=DEV).bfloat16() for _ in range(6)]
+    got = []
+    for cap in (16 << 30, 3 * 64 * 128 * 2):
+        model = Wrap().to(DEV).to(torch.bfloat16)
+        model.load_state_dict(init)
+        launches, peak = [], [0]
+        raw = ops.hessian_accumulate_segments_
+        ops.hessian_accumulate_segments_ = lambda H, views, **kw: (launches.append(len(views)), raw(H, views, **kw))[1]
+        try:
+            mod = GPTQModifier(targets="Linear", stage_max_bytes=cap, config_groups={"g": dict(
+                targets=["Linear"], weights=dict(num_bits=4, strategy="group", group_size=32))})
+            session = active_session()
+            session.reset()
+            session.initialize(model=model, recipe=mod)
+            LifecycleCallbacks.calibration_start()
+            with torch.no_grad():
+                for x in xs:
+                    model.layers[0](x)
+                    peak[0] = max(peak[0], mod._held_bytes)
+            assert mod._held_bytes <= cap
+            for m in list(mod._num_samples):
+                mod._flush(m)
+            assert mod._held_bytes == 0
+            got.append((list(launches), peak[0], {m: mod._hessians[m].clone() for m in mod._hessians},
+                        [float(v) for v in mod._num_samples.values()]))
+            LifecycleCallbacks.sequential_epoch_end(modules=list(model.modules()))
+            LifecycleCallbacks.calibration_end()
+            session.finalize()
+        finally:
+            ops.hessian_accumulate_segments_ = raw
+    (l0, p0, h0, n0), (l1, p1, h1, n1) = got
+    assert l0 == [6] * 4 and len(l1) > 4 and sum(l1) == 24 and max(l1) < 6
+    assert p1 <= 3 * 64 * 128 * 2 + 64 * 128 * 2 < p0
+    assert n0 == n1 == [6.0] * 4
+    for a, b in zip(h0.values(), h1.values()):
+        assert ((a.double() - b.double()).norm() / a.double().norm()).item() < 1e-6
