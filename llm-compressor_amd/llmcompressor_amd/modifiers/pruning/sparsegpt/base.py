@@ -42,7 +42,7 @@ class SparseGPTModifier(SparsityModifierBase, HessianStagingMixin):
     dampening_frac: float | None = 0.01
     preserve_sparsity_mask: bool = False
     offload_hessians: bool = False
-    hessian_batch_tokens: int = 0
+    hessian_batch_tokens: int = 65536
     stage_by_reference: bool = True
     stage_max_bytes: int = 16 << 30
     compress_concurrency: int = 4
