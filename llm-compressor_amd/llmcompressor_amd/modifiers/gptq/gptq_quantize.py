@@ -92,9 +92,11 @@ def quantize_weight_tensors(weight: torch.Tensor, observer, quant_args: Quantiza
     if actorder:
         perm = torch.argsort(torch.diagonal(H), descending=True)
     if actorder == ActivationOrdering.GROUP:
-        # re-observe the permuted weight so that groups are runs of the permuted columns
+        # re-observe the permuted weight so that groups are runs of the permuted columns.  The reference observes
+        # its fp32 work copy here (gptq_quantize.py:88,111-114), so these statistics and the scales the column
+        # loop divides by are fp32, not rounded to the weight's dtype as on the other paths
         observer.delete_statistics(check_fused=False)
-        observer(W2[:, perm].contiguous())
+        observer(W2[:, perm].to(GPTQ_PRECISION).contiguous())
 
     row_div, srow, divisor = _scale_layout(strategy, quant_args, num_rows, num_columns)
     g_idx = None

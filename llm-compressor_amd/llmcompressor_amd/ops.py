@@ -214,6 +214,13 @@ def minmax_strided(x: torch.Tensor, n0: int, n1: int, group: int, s0: int, s1: i
     return mn, mx
 
 
+def _gs32(global_scale):
+    """The kernels read the global scale as one fp32 value."""
+    if global_scale is None:
+        return None
+    return global_scale.to(torch.float32).contiguous()
+
+
 def global_scale_from_stats(stats):
     """NVFP4 global scale from the (min, max) arrays of every observer of a fused group -> fp32 [1]."""
     mn0 = stats[0][0]
@@ -234,6 +241,7 @@ def global_scale_from_stats(stats):
 def calculate_qparams(mn, mx, fmt: int, bits: int, symmetric: bool, scale_mode: int = SCALE_PLAIN,
                       global_scale=None, want_codes: bool = False):
     """(min,max) -> (scale, zero_point int8, scale_code uint8|None); shapes follow `mn`."""
+    global_scale = _gs32(global_scale)
     _require_gpu(mn, mx)
     mn, mx = mn.contiguous(), mx.contiguous()
     sdt = torch.float32 if scale_mode == SCALE_NVFP4 else mn.dtype
@@ -252,6 +260,7 @@ def calculate_qparams(mn, mx, fmt: int, bits: int, symmetric: bool, scale_mode: 
 def quantize(x, scale, zero_point, fmt: int, bits: int, row_div: int, scale_row_stride: int, col_div: int,
              out_mode: int = OUT_FAKEQUANT, g_idx=None, global_scale=None, out_dtype=None):
     """Element-wise quantise of x [R,K]; see llmc_quantize in include/llmc_amd.h for the scale indexing."""
+    global_scale = _gs32(global_scale)
     _require_gpu(x, scale)
     assert x.ndim == 2 and x.stride(1) == 1
     R, K = x.shape
@@ -363,6 +372,7 @@ def gptq_hinv_grouped(Hs, perms=None, divisors=None, percdamp: float = 0.01):
 def gptq_quantize(weight, U, scale, zero_point, fmt: int, bits: int, row_div: int, scale_row_stride: int,
                   g_idx=None, perm=None, dead=None, global_scale=None, blocksize: int = 128):
     """The GPTQ column loop.  Returns (quantised-dequantised weight in weight.dtype, loss fp32 [1])."""
+    global_scale = _gs32(global_scale)
     _require_gpu(weight, U, scale)
     assert weight.ndim == 2 and weight.stride(1) == 1 and U.stride(1) == 1
     R, K = weight.shape
@@ -425,7 +435,7 @@ def gptq_quantize_grouped(weights, U, scales, zero_points, fmt: int, bits: int, 
     wp = (ctypes.c_void_p * n)(*[w.data_ptr() for w in weights])
     op = (ctypes.c_void_p * n)(*[o.data_ptr() for o in outs])
     sp, zp = ptrs(scales), ptrs(zero_points)
-    gp, ip = ptrs(global_scales), ptrs(g_idxs, torch.int32)
+    gp, ip = ptrs(global_scales, torch.float32), ptrs(g_idxs, torch.int32)
     with torch.cuda.device(w0.device):
         rc = _lib.lib().llmc_gptq_quantize_grouped(
             wp, _dt(w0), n, R, K, w0.stride(0), U.data_ptr(), K, K * K, _ptr(perms), _ptr(dead), sp, _dt(keep[0]),
