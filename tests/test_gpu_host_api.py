@@ -808,7 +808,11 @@ def test_sparsegpt_modifier_matches_oracle(structure, staging):
 @pytest.mark.parametrize("scheme", [dict(num_bits=4, strategy="group", group_size=32),
                                     dict(num_bits=4, strategy="channel", symmetric=False, actorder="weight"),
                                     dict(num_bits=4, type="float", strategy="tensor_group", group_size=16,
-                                         scale_dtype=torch.float8_e4m3fn)])
+                                         scale_dtype=torch.float8_e4m3fn),
+                                    dict(num_bits=4, type="float", strategy="group", group_size=32,
+                                         scale_dtype=torch.uint8),
+                                    dict(num_bits=8, strategy="tensor", symmetric=False),
+                                    dict(num_bits=8, type="float", strategy="block", block_structure=[32, 32])])
 def test_moe_gptq_lock_step_groups_match_per_module_path(scheme):
     """The experts of a LinearExperts2D block quantised in lock-step (grouped Cholesky chain and column loop)
     end up with exactly the parameters of the per-module path, a never-routed expert included."""
