@@ -180,8 +180,9 @@ int llmc_imatrix_observe_blocks(const void* x, int32_t dtype, int64_t R, int64_t
  * llmc_absmax_accumulate + llmc_generate_gparam replace Observer.get_global_scale()
  * (src/llmcompressor/observers/base.py:78-96; CT generate_gparam): absmax_inout
  * (fp32, caller zero-initialised) takes max(absmax, -min, max) over the arrays of
- * every observer of a fused group, one call each; gparam = 448*6/absmax divided in
- * the statistics' dtype, returned as fp32 [1].
+ * every observer of a fused group, one call each; gparam = 448*6/absmax evaluated as
+ * torch evaluates `float / Tensor` (reciprocal in the statistics' dtype, then the
+ * product, rounded again), returned as fp32 [1].
  * llmc_calculate_qparams replaces CT calculate_qparams as called from
  * observers/base.py:114-119: n (min,max) pairs -> scale (scale_out_dtype; fp32
  * e4m3-grid values for LLMC_SCALE_NVFP4), int8 zero points (NULL when symmetric),

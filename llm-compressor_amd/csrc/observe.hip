@@ -203,8 +203,11 @@ __global__ __launch_bounds__(256) void absmax_kernel(const void* __restrict__ mn
 }
 
 __global__ void gparam_kernel(const float* absmax, int sd, float* out) {
-  // 448*6/absmax, divided in the statistics' dtype, then widened to fp32
-  out[0] = round_rt(2688.0f / round_rt(absmax[0], sd), sd);
+  // The reference forms `448 * 6 / absmax` with a Python float on the left, which torch evaluates as
+  // absmax.reciprocal() * 2688: the reciprocal is rounded to the statistics' dtype before the product, and
+  // the product is rounded again (2688/40 gives 67.5 in bf16 this way, not the 67.0 of a single division).
+  const float r = round_rt(__fdiv_rn(1.0f, round_rt(absmax[0], sd)), sd);
+  out[0] = round_rt(__fmul_rn(r, 2688.0f), sd);
 }
 
 __global__ __launch_bounds__(256) void qparams_kernel(const void* __restrict__ mn, const void* __restrict__ mx,

@@ -165,7 +165,10 @@ def calculate_qparams(min_vals, max_vals, args: QArgs, global_scale=None):
 
 
 def generate_gparam(min_val, max_val, dtype=torch.float32):
-    """NVFP4 global scale 448*6/absmax, divided in the statistics' dtype."""
+    """NVFP4 global scale ``448 * 6 / absmax`` as compressed-tensors writes it: a Python float divided by a
+    tensor, which torch evaluates as ``absmax.reciprocal() * 2688.0`` (``Tensor.__rtruediv__``) -- for bf16
+    statistics the reciprocal is rounded to bf16 before the product (2688/40 -> 67.5, a single division would
+    give 67.0).  The reference's golden vectors (2688/23 -> 117.0, 2688/11 -> 244.0) hold either way."""
     mn = torch.min(min_val, torch.zeros_like(min_val))
     mx = torch.max(max_val, torch.zeros_like(max_val))
     absmax = torch.max(torch.abs(mn), torch.abs(mx))

@@ -1295,3 +1295,36 @@ def test_quantize_weight_seam_matches_oracle_on_correlated_hessians(spec):
                                  global_scale=q.get("weight_global_scale"))
         e_rtn = ((w0.float() - rtn.cpu().float()) @ xf.t()).norm()
         assert e_got < e_rtn
+
+
+@pytest.mark.parametrize("name", ["minmax", "static_minmax", "memoryless_minmax", "mse", "memoryless_mse"])
+@pytest.mark.parametrize("spec", [
+    dict(num_bits=8, type="float", strategy="tensor"),
+    dict(num_bits=8, strategy="tensor", symmetric=False),
+    dict(num_bits=8, strategy="group", group_size=64),
+    dict(num_bits=4, type="float", strategy="tensor_group", group_size=16, scale_dtype="float8_e4m3fn"),
+], ids=["fp8_tensor", "int8_tensor_asym", "int8_group", "nvfp4"])
+def test_activation_observers_over_batches_match_oracle(name, spec):
+    """Input-activation observers from the registry over five bf16 batches [2, 96, 256] with outliers: the
+    running statistics after every batch and the final qparams equal the CPU oracle's bit for bit (moving
+    average in the activations' dtype, static running min/max, memoryless replacement, MSE searches)."""
+    from llmcompressor_amd.observers import Observer
+
+    torch.manual_seed(23)
+    ospec = dict(spec)
+    if "scale_dtype" in ospec:
+        ospec["scale_dtype"] = getattr(torch, ospec["scale_dtype"])
+    oobs = O.Observer(name, "input", F.QArgs(**ospec))
+    gobs = Observer.load_from_registry(name, base_name="input", args=_qargs(spec))
+    for step in range(5):
+        x = (torch.randn(2, 96, 256) * (1 + step)).bfloat16()
+        x[step % 2, 5 * step, 17] = 40.0 + step
+        oobs(x)
+        gobs(x.to(DEV))
+        assert torch.equal(gobs.min_vals.cpu().float().reshape(-1), oobs.min_vals.float().reshape(-1)), step
+        assert torch.equal(gobs.max_vals.cpu().float().reshape(-1), oobs.max_vals.float().reshape(-1)), step
+    oq, gq = oobs.get_qparams(), gobs.get_qparams()
+    assert torch.equal(gq["scale"].cpu().float().reshape(-1), oq["scale"].float().reshape(-1))
+    assert torch.equal(gq["zero_point"].cpu().float().reshape(-1), oq["zero_point"].float().reshape(-1))
+    if oq["global_scale"] is not None:
+        assert torch.equal(gq["global_scale"].cpu().float(), oq["global_scale"].float())

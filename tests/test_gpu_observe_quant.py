@@ -334,3 +334,22 @@ def test_full_size_microscale_and_mse_properties():
         return (f.float() - w.float()).abs().pow(2.4).sum().item()
 
     assert qerr(mmn, mmx) <= 1.0001 * qerr(mn, mx)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_global_scale_matches_oracle_for_many_absmax_values(dtype):
+    """The NVFP4 global scale for 600 absmax values per statistics dtype, bit for bit against the oracle
+    (reciprocal rounded to the dtype, then the product rounded again)."""
+    from llmcompressor_amd import ops
+
+    torch.manual_seed(4)
+    vals = torch.cat([torch.rand(300) * 60 + 0.01, torch.rand(200) * 2.0 ** -6, torch.tensor([40.0, 23.0, 11.0]),
+                      torch.rand(97) * 3000]).to(dtype)
+    bad = []
+    for v in vals:
+        t = v.reshape(1)
+        want = F.generate_gparam(-t, t).item()
+        got = ops.global_scale_from_stats([(-t.cuda(), t.cuda())]).item()
+        if got != want:
+            bad.append((v.item(), got, want))
+    assert not bad, bad[:5]

@@ -223,3 +223,14 @@ def test_cast_to_fp4_matches_torch_e2m1_table():
     exp = torch.where(tie, cand, near)
     assert torch.equal(got.abs(), exp)
     assert torch.equal(torch.signbit(got), (xs < 0))
+
+
+def test_generate_gparam_is_reciprocal_then_product():
+    """``float / Tensor`` is ``Tensor.reciprocal() * float`` in torch, so the global scale of bf16 statistics
+    carries two roundings; a single correctly rounded division differs for some absmax values (40.0)."""
+    for v, want in ((40.0, 67.5), (23.0, 117.0), (11.0, 244.0)):
+        t = torch.tensor([v], dtype=torch.bfloat16)
+        gs = F.generate_gparam(-t, t)
+        assert gs.dtype == torch.float32 and gs.item() == want
+        assert gs.item() == (t.reciprocal() * 2688.0).float().item()
+    assert (torch.tensor([2688.0]).bfloat16() / torch.tensor([40.0]).bfloat16()).item() == 67.0
