@@ -24,14 +24,47 @@ from ...utils.hooks import HooksMixin
 from ..calibration import (
     apply_calibration_status,
     calibrate_input_hook,
+    calibrate_key_hook,
     calibrate_output_hook,
+    calibrate_value_hook,
     freeze_module_quantization,
     initialize_observer,
     reset_quantization_status,
 )
 from ..group_size_validation import validate_group_size_divisibility
 
-__all__ = ["QuantizationMixin"]
+__all__ = ["QuantizationMixin", "KV_CACHE_TARGETS"]
+
+# attention modules are found by name, as in the reference (compressed-tensors KV_CACHE_TARGETS)
+KV_CACHE_TARGETS = ["re:.*self_attn$"]
+
+
+class _ObservedKVCache:
+    """Stands in for the attention module's ``past_key_values`` during calibration: ``update`` shows the key
+    and value states (keys after the rotary embedding, as they would enter the cache) to the module's
+    observers, then defers to the real cache, or hands the states back when there is none."""
+
+    def __init__(self, module, inner):
+        self._module, self._inner = module, inner
+
+    def update(self, key_states, value_states, *args, **kwargs):
+        calibrate_key_hook(self._module, key_states)
+        calibrate_value_hook(self._module, value_states)
+        if self._inner is not None:
+            return self._inner.update(key_states, value_states, *args, **kwargs)
+        return key_states, value_states
+
+    def __getattr__(self, name):
+        return getattr(self._inner, name)
+
+
+def _kv_cache_pre_hook(module, args, kwargs):
+    for name in ("past_key_values", "past_key_value"):
+        if name in kwargs:
+            kwargs[name] = _ObservedKVCache(module, kwargs[name])
+            return args, kwargs
+    kwargs["past_key_values"] = _ObservedKVCache(module, None)
+    return args, kwargs
 
 
 class QuantizationMixin(HooksMixin):
@@ -90,12 +123,15 @@ class QuantizationMixin(HooksMixin):
         targets = set()
         for group in self.resolved_config.config_groups.values():
             targets.update(group.targets)
+        if self.resolved_config.kv_cache_scheme is not None:
+            targets.update(KV_CACHE_TARGETS)
         return targets
 
     def initialize_quantization(self, model: torch.nn.Module):
         for _, module in match_named_modules(model, self.resolved_targets, self.ignore):
             reset_quantization_status(module)
         apply_quantization_config(model, self.resolved_config)
+        self._initialize_kv_cache(model)
         if not self.bypass_divisibility_checks:
             validate_group_size_divisibility(model, self.resolved_targets, self.ignore)
         model.apply(disable_quantization)
@@ -184,10 +220,39 @@ class QuantizationMixin(HooksMixin):
                 setattr(scheme, attr, QuantizationArgs.model_validate(d))
         return scheme
 
+    def _initialize_kv_cache(self, model: torch.nn.Module):
+        """Attention modules get a scheme whose input arguments are the kv-cache arguments and ``k_scale`` /
+        ``v_scale`` parameters (reference: mixin.py:216-218,342-383; compressed-tensors initialises the
+        parameters from the observed shape (kv heads, head dim)).  Their forward is not wrapped: the scales are
+        calibrated for the serving engine's cache, the calibration forward itself stays unquantised."""
+        kv_args = self.resolved_config.kv_cache_scheme
+        if kv_args is None:
+            return
+        from ....quantization.lifecycle import initialize_qparams
+
+        for _, module in match_named_modules(model, KV_CACHE_TARGETS, self.ignore):
+            config = getattr(module, "config", None)
+            heads = getattr(config, "num_key_value_heads", None) or getattr(config, "num_attention_heads", None)
+            head_dim = getattr(module, "head_dim", None)
+            if heads is None or head_dim is None:
+                raise ValueError("kv_cache_scheme: attention modules need `config.num_key_value_heads` and "
+                                 f"`head_dim` (found {type(module).__name__})")
+            module.quantization_scheme = QuantizationScheme(targets=list(KV_CACHE_TARGETS), input_activations=kv_args)
+            module.quantization_status = QuantizationStatus.INITIALIZED
+            module._llmc_kv_cache = True
+            dtype = next(module.parameters()).dtype
+            for base in ("k", "v"):
+                initialize_qparams(module, base, kv_args, (heads, head_dim), dtype, force_zero_point=False)
+
     def _initialize_observers(self, module: torch.nn.Module):
         if not hasattr(module, "quantization_scheme"):
             return
         scheme: QuantizationScheme = module.quantization_scheme
+        if getattr(module, "_llmc_kv_cache", False):
+            if scheme.input_activations.dynamic in (False, DynamicType.LOCAL):
+                initialize_observer(module, base_name="k")
+                initialize_observer(module, base_name="v")
+            return
         inp = scheme.input_activations and scheme.input_activations.dynamic in (False, DynamicType.LOCAL)
         out = scheme.output_activations and not scheme.output_activations.dynamic
         if inp:
@@ -204,6 +269,10 @@ class QuantizationMixin(HooksMixin):
         scheme: QuantizationScheme = module.quantization_scheme
         inp = scheme.input_activations and scheme.input_activations.dynamic in (False, DynamicType.LOCAL)
         out = scheme.output_activations and not scheme.output_activations.dynamic
+        if getattr(module, "_llmc_kv_cache", False):
+            if inp:
+                hooks.add(self.register_hook(module, _kv_cache_pre_hook, "forward_pre", with_kwargs=True))
+            return hooks
         if inp:
             hooks.add(self.register_hook(module, calibrate_input_hook, "forward_pre"))
         if out:

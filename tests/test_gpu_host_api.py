@@ -1328,3 +1328,62 @@ def test_activation_observers_over_batches_match_oracle(name, spec):
     assert torch.equal(gq["zero_point"].cpu().float().reshape(-1), oq["zero_point"].float().reshape(-1))
     if oq["global_scale"] is not None:
         assert torch.equal(gq["global_scale"].cpu().float(), oq["global_scale"].float())
+
+
+@pytest.mark.parametrize("strategy", ["tensor", "attn_head"])
+def test_kv_cache_scheme_calibrates_k_and_v_scales_on_a_transformers_llama(tmp_path, strategy):
+    """kv_cache_scheme (FP8, static): every ``self_attn`` module gets ``k_scale`` / ``v_scale`` from the key
+    states after the rotary embedding and the value states, over all calibration batches (moving-average
+    min-max observer, as for other static activations); equal to the oracle's observer run on the states
+    captured from an unquantised twin, and written to the checkpoint under the attention module's name."""
+    transformers = pytest.importorskip("transformers")
+    from safetensors.torch import load_file
+
+    from llmcompressor_amd import oneshot
+    from llmcompressor_amd.modifiers.quantization import QuantizationModifier
+
+    torch.manual_seed(0)
+    cfg = transformers.LlamaConfig(hidden_size=128, intermediate_size=256, num_hidden_layers=2,
+                                   num_attention_heads=4, num_key_value_heads=2, vocab_size=256,
+                                   max_position_embeddings=128)
+    model = transformers.LlamaForCausalLM(cfg).to(torch.bfloat16).to(DEV)
+    data = [{"input_ids": torch.randint(0, 256, (1, 64))} for _ in range(4)]
+    kv = dict(num_bits=8, type="float", strategy=strategy, dynamic=False, symmetric=True)
+
+    # layer-0 key / value states as the cache would see them, from the untouched model
+    seen = {"k": [], "v": []}
+
+    class Spy:
+        def update(self, k, v, *a, **kw):
+            seen["k"].append(k.detach().cpu())
+            seen["v"].append(v.detach().cpu())
+            return k, v
+
+    attn0 = model.model.layers[0].self_attn
+    handle = attn0.register_forward_pre_hook(
+        lambda m, a, kw: (a, {**kw, "past_key_values": Spy()}), with_kwargs=True)
+    with torch.no_grad():
+        for d in data:
+            model(d["input_ids"].to(DEV), use_cache=False)
+    handle.remove()
+    assert len(seen["k"]) == 4 and seen["k"][0].shape == (1, 2, 64, 32)
+
+    out_dir = str(tmp_path / "kv")
+    oneshot(model=model, dataset=data, output_dir=out_dir, recipe=QuantizationModifier(
+        targets="Linear", scheme="FP8_DYNAMIC", ignore=["lm_head"], kv_cache_scheme=kv))
+    for base in ("k", "v"):
+        oobs = O.Observer("minmax", base, F.QArgs(**kv))
+        for t in seen[base]:
+            oobs(t)
+        want = oobs.get_qparams()["scale"]
+        got = getattr(attn0, f"{base}_scale").detach().cpu()
+        assert got.shape == ((1,) if strategy == "tensor" else (2, 1, 1))
+        assert torch.equal(got.float().reshape(-1), want.float().reshape(-1)), base
+        assert not hasattr(attn0, f"{base}_observer")
+    sd = load_file(os.path.join(out_dir, "model.safetensors"))
+    for layer in range(2):
+        for base in ("k", "v"):
+            assert f"model.layers.{layer}.self_attn.{base}_scale" in sd
+    q = json.load(open(os.path.join(out_dir, "config.json")))["quantization_config"]
+    assert q["kv_cache_scheme"]["strategy"] == strategy and q["kv_cache_scheme"]["num_bits"] == 8
+    assert "model.layers.0.self_attn.q_proj.weight_scale" in sd
