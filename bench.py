@@ -279,6 +279,55 @@ def probe_moe():
         print(f"| {label} | {best[0] * 1e3:.1f} | {best[1] * 1e3:.1f} | {best[1] * 1e3 / (3 * E):.2f} |")
 
 
+def probe_oneshot(batches, tokens):
+    """oneshot() on a transformers LlamaForCausalLM with two Llama-3-8B-shaped decoder layers (random weights,
+    vocabulary cut to 32000), GPTQ W4A16 with the modifier's defaults, `batches` x `tokens` calibration tokens:
+    wall time per layer with both passes of the sequential pipeline, staged and unstaged Hessian launches, and the
+    model's own forward for comparison.  Prints a table."""
+    import torch
+    from transformers import LlamaConfig, LlamaForCausalLM
+
+    from llmcompressor_amd import oneshot
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+
+    layers = 2
+    cfg = LlamaConfig(hidden_size=HIDDEN, intermediate_size=INTER, num_hidden_layers=layers, num_attention_heads=32,
+                      num_key_value_heads=8, vocab_size=32000, max_position_embeddings=max(4096, tokens))
+    torch.manual_seed(0)
+    data = [{"input_ids": torch.randint(0, 32000, (1, tokens))} for _ in range(batches)]
+
+    def make():
+        with torch.device("cuda"):
+            return LlamaForCausalLM(cfg).to(torch.bfloat16)
+
+    model = make()
+    with torch.no_grad():
+        for rep in range(2):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for d in data:
+                model(d["input_ids"].cuda(), use_cache=False)
+            torch.cuda.synchronize()
+            fwd = time.perf_counter() - t0
+    del model
+    print(f"| oneshot GPTQ W4A16, {layers} layers of 4096/14336, {batches} x {tokens} tokens | s | ms per layer |")
+    print("|---|---|---|")
+    print(f"| model forward alone, one pass over the data (embedding and lm_head included) | {fwd:.2f} | {fwd / layers * 1e3:.0f} |")
+    for label, stage in (("Hessian launches of 65536 staged tokens (default)", 65536), ("one Hessian launch per hook call", 0)):
+        best = None
+        for rep in range(2):
+            model = make()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            oneshot(model=model, dataset=data, recipe=GPTQModifier(targets="Linear", scheme="W4A16", ignore=["lm_head"],
+                                                                     hessian_batch_tokens=stage))
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+            del model
+        print(f"| {label} | {best:.2f} | {best / layers * 1e3:.0f} |")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -296,6 +345,9 @@ def main():
                     help="print achieved GB/s of the observer / quantize / pack kernels instead of the bench line")
     ap.add_argument("--probe-sparsegpt", action="store_true",
                     help="print SparseGPT timings per Linear shape instead of the bench line")
+    ap.add_argument("--probe-oneshot", action="store_true",
+                    help="print end-to-end oneshot timings on a transformers Llama with two 8B-shaped layers "
+                    "(--batches x --tokens calibration tokens) instead of the bench line")
     ap.add_argument("--probe-moe", action="store_true",
                     help="print the timings of one 128-expert MoE layer through GPTQModifier instead of the bench line")
     a = ap.parse_args()
@@ -320,6 +372,9 @@ def main():
         return
     if a.probe_moe:
         probe_moe()
+        return
+    if a.probe_oneshot:
+        probe_oneshot(a.batches, a.tokens)
         return
     if a.probe_dominant:
         from llmcompressor_amd import ops
