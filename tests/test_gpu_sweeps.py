@@ -1,0 +1,168 @@
+"""GPU parity sweeps: randomised shapes, dtypes, strategies and value distributions through the product's
+seams (Observer registry -> get_qparams -> fake_quantize, and quantize_weight) against the CPU oracle.  Seeds are
+fixed, so the cases are the same on every run."""
+import random
+
+import pytest
+import torch
+
+from oracle import gptq as G
+from oracle import observers as O
+from oracle import qformat as F
+
+pytestmark = pytest.mark.gpu
+
+
+def test_rtn_seam_sweep_is_bit_exact():
+    """220 random round-to-nearest cases (int 2-8 bit group / channel / tensor / block, symmetric and not, FP8,
+    NVFP4, MXFP4
+    bf16 / f16 / f32 weights
+    zero rows, outliers, tiny and large magnitudes): scales, zero points
+    and fake-quantised weights equal the oracle's bit for bit."""
+    from llmcompressor_amd.observers import Observer
+    from llmcompressor_amd.quantization import QuantizationArgs, fake_quantize
+
+    random.seed(0)
+    torch.manual_seed(0)
+
+    def same(a, b):
+        a, b = a.cpu(), b.cpu()
+        if a.dtype == torch.uint8 or b.dtype == torch.uint8:
+            return a.shape == b.shape and torch.equal(a.view(torch.uint8) if a.dtype != torch.uint8 else a, b.view(torch.uint8) if b.dtype != torch.uint8 else b)
+        return a.reshape(-1).shape == b.reshape(-1).shape and torch.equal(a.float().reshape(-1).nan_to_num(7e7), b.float().reshape(-1).nan_to_num(7e7))
+    bad = 0
+    n = 0
+    for trial in range(220):
+        dtype = random.choice([torch.bfloat16, torch.bfloat16, torch.float16, torch.float32])
+        kind = random.choice(["int_group", "int_channel", "int_tensor", "int_block", "fp8_channel", "fp8_tensor", "fp8_block", "nvfp4", "mxfp4", "int_group_asym", "int_channel_asym", "int_tensor_asym"])
+        R = random.choice([1, 3, 8, 33, 64, 100, 256])
+        g = random.choice([8, 16, 32, 64, 128])
+        K = g * random.choice([1, 2, 3, 5, 8])
+        bits = random.choice([2, 3, 4, 5, 6, 8])
+        spec = dict(num_bits=bits)
+        if kind.startswith("int_group"): spec.update(strategy="group", group_size=g)
+        elif kind.startswith("int_channel"): spec.update(strategy="channel")
+        elif kind.startswith("int_tensor"): spec.update(strategy="tensor")
+        elif kind == "int_block": spec.update(strategy="block", block_structure=[random.choice([2, 16, 128]), random.choice([8, 64, 128])])
+        elif kind == "fp8_channel": spec.update(num_bits=8, type="float", strategy="channel")
+        elif kind == "fp8_tensor": spec.update(num_bits=8, type="float", strategy="tensor")
+        elif kind == "fp8_block": spec.update(num_bits=8, type="float", strategy="block", block_structure=[random.choice([16, 128]), random.choice([32, 128])])
+        elif kind == "nvfp4":
+            spec.update(num_bits=4, type="float", strategy="tensor_group", group_size=16, scale_dtype="float8_e4m3fn")
+            K = 16 * random.choice([1, 3, 8, 20])
+        elif kind == "mxfp4":
+            spec.update(num_bits=4, type="float", strategy="group", group_size=32, scale_dtype="uint8")
+            K = 32 * random.choice([1, 3, 8])
+            dtype = torch.bfloat16
+        if kind.endswith("asym"): spec["symmetric"] = False
+        dist = random.choice(["normal", "small", "large", "zeros_rows", "positive", "outliers"])
+        w = torch.randn(R, K)
+        if dist == "small": w *= 1e-4
+        if dist == "large": w *= 300
+        if dist == "positive": w = w.abs() + 0.1
+        if dist == "zeros_rows": w[::2] = 0
+        if dist == "outliers": w[torch.rand(R, K) < 0.01] *= 50
+        w = (w * 0.05).to(dtype)
+        ospec = dict(spec)
+        if "scale_dtype" in ospec: ospec["scale_dtype"] = getattr(torch, ospec["scale_dtype"])
+        try:
+            oargs = F.QArgs(**ospec)
+            oobs = O.Observer("memoryless_minmax", "weight", oargs)
+            oobs(w)
+            oq = oobs.get_qparams()
+            ofq = F.fake_quantize(w, oq["scale"], oq["zero_point"], oargs, global_scale=oq["global_scale"])
+        except Exception as e:
+            print("oracle error", kind, spec, type(e).__name__, str(e)[:100])
+            continue
+        n += 1
+        try:
+            args = QuantizationArgs(**spec)
+            gobs = Observer.load_from_registry("memoryless_minmax", base_name="weight", args=args)
+            gobs(w.cuda())
+            gq = gobs.get_qparams()
+            gfq = fake_quantize(w.cuda(), gq["scale"], gq["zero_point"], args, global_scale=gq["global_scale"])
+            es = oq["scale"]
+            gsx = gq["scale"]
+            if gsx.dtype == torch.uint8: es = (torch.log2(es.float()) + 127).to(torch.uint8)
+            ok_s = same(gsx, es)
+            ok_z = True if args.symmetric else same(gq["zero_point"].float(), oq["zero_point"].float())
+            ok_f = same(gfq, ofq.to(dtype))
+            if not (ok_s and ok_z and ok_f):
+                bad += 1
+                print("MISMATCH", kind, spec, dtype, (R, K), dist, "scale", ok_s, "zp", ok_z, "fq", ok_f, flush=True)
+        except Exception as e:
+            bad += 1
+            print("PRODUCT ERROR", kind, spec, dtype, (R, K), dist, type(e).__name__, str(e)[:160], flush=True)
+    assert n >= 200 and bad == 0
+
+
+
+def test_gptq_seam_sweep_matches_oracle():
+    """70 random GPTQ cases through quantize_weight (all strategies and formats of the column loop, activation
+    ordering none / weight / group, block sizes 32 / 48 / 128, dead columns, rank-deficient Hessians, two
+    dampening fractions): at least 99.9 % identical weights in every case."""
+    from llmcompressor_amd.modifiers.gptq import quantize_weight
+    from llmcompressor_amd.modifiers.quantization.calibration import initialize_observer, observe
+    from llmcompressor_amd.quantization import QuantizationArgs, QuantizationScheme
+
+    random.seed(1)
+    torch.manual_seed(1)
+    worst = 1.0
+    bad = 0
+    for trial in range(70):
+        kind = random.choice(["int_group", "int_group_asym", "int_channel", "int_tensor", "int_block", "fp8_channel", "nvfp4", "mxfp4"])
+        actorder = random.choice([None, "weight", "weight", "group"])
+        g = random.choice([16, 32, 64, 128])
+        K = g * random.choice([1, 2, 3, 5])
+        R = random.choice([1, 7, 32, 100, 130])
+        bits = random.choice([3, 4, 8])
+        spec = dict(num_bits=bits)
+        if kind.startswith("int_group"): spec.update(strategy="group", group_size=g)
+        elif kind == "int_channel": spec.update(strategy="channel")
+        elif kind == "int_tensor": spec.update(strategy="tensor")
+        elif kind == "int_block": spec.update(strategy="block", block_structure=[random.choice([2, 16]), g])
+        elif kind == "fp8_channel": spec.update(num_bits=8, type="float", strategy="channel")
+        elif kind == "nvfp4":
+            spec.update(num_bits=4, type="float", strategy="tensor_group", group_size=16, scale_dtype="float8_e4m3fn")
+            K = 16 * random.choice([2, 5, 12])
+        elif kind == "mxfp4":
+            spec.update(num_bits=4, type="float", strategy="group", group_size=32, scale_dtype="uint8")
+            K = 32 * random.choice([1, 3, 6])
+        if kind.endswith("asym"): spec["symmetric"] = False
+        if actorder: spec["actorder"] = actorder
+        blocksize = random.choice([128, 128, 32, 48])
+        T = random.choice([K // 2, 2 * K, 4 * K])
+        mix = torch.randn(K, K) * 0.3 + torch.eye(K)
+        x = (torch.randn(T, K) @ mix).bfloat16()
+        ndead = random.choice([0, 0, 1, 3])
+        if ndead: x[:, torch.randperm(K)[:ndead]] = 0
+        w0 = (torch.randn(R, K) * 0.05).bfloat16()
+        ospec = dict(spec)
+        if "scale_dtype" in ospec: ospec["scale_dtype"] = getattr(torch, ospec["scale_dtype"])
+        oargs = F.QArgs(**ospec)
+        oobs = O.Observer("memoryless_minmax", "weight", oargs)
+        oobs(w0)
+        Ho, n = G.make_empty_hessian(K), torch.zeros(())
+        Ho, n = G.accumulate_hessian(x.unsqueeze(0), Ho, n)
+        Hn = (Ho / n).clone()
+        percdamp = random.choice([0.01, 0.1])
+        _, exp, info = G.quantize_weight(w0, oobs, oargs, Hn.clone(), blocksize=blocksize, percdamp=percdamp)
+        module = torch.nn.Linear(K, R, bias=False).cuda().to(torch.bfloat16)
+        module.weight.data = w0.cuda()
+        args = QuantizationArgs(**spec)
+        module.quantization_scheme = QuantizationScheme(targets=["Linear"], weights=args)
+        initialize_observer(module, "weight")
+        observe(module, "weight")
+        try:
+            loss, q = quantize_weight(module=module, quant_args=args, hessian=Hn.clone().cuda(), blocksize=blocksize, percdamp=percdamp)
+        except Exception as e:
+            bad += 1
+            print("PRODUCT ERROR", spec, (R, K, T), type(e).__name__, str(e)[:200], flush=True)
+            continue
+        agree = (q["weight"].cpu() == exp["weight"]).float().mean().item()
+        worst = min(worst, agree)
+        if agree < 0.999 or not info["ok"]:
+            bad += (agree < 0.999)
+            print(f"agree {agree:.4f} ok={info['ok']}", spec, (R, K, T), "blocksize", blocksize, "dead", ndead, "damp", percdamp, flush=True)
+    assert bad == 0 and worst >= 0.999
+
