@@ -38,6 +38,15 @@ struct MseParams {
 
 __device__ __forceinline__ float step_factor(int i, double grid) { return (float)(1.0 - (double)i / grid); }
 
+// a^norm (a >= 0) as the eager pow forms it in dtype dt: exponents 2, 3 and 0.5 have closed forms (a*a,
+// (a*a)*a with the inner product rounded to dt as well, sqrt), anything else is one pow rounded to dt
+__device__ __forceinline__ float pow_eager(float a, float norm, int dt) {
+  if (norm == 2.0f) return round_rt(__fmul_rn(a, a), dt);
+  if (norm == 3.0f) return round_rt(__fmul_rn(round_rt(__fmul_rn(a, a), dt), a), dt);
+  if (norm == 0.5f) return round_rt(__fsqrt_rn(a), dt);
+  return round_rt(powf(a, norm), dt);
+}
+
 // |fq(x) - x|^norm with every intermediate rounded to dt
 __device__ __forceinline__ float elem_error(float x, float s, float zp, bool has_zp, int dt, const QFormat& f,
                                             float norm) {
@@ -45,8 +54,7 @@ __device__ __forceinline__ float elem_error(float x, float s, float zp, bool has
   const float dq = dequantize_value(q, s, zp, has_zp, dt);
   const float a = fabsf(round_rt(dq - x, dt));
   // `norm` arrives already rounded to dt: the eager pow converts its scalar exponent to the tensor dtype
-  const float pw = norm == 2.0f ? a * a : powf(a, norm);
-  return round_rt(pw, dt);
+  return pow_eager(a, norm, dt);
 }
 
 // fp32 error of the importance-weighted search: fq(x) in dt, then (fq - x), abs, pow in fp32; the
@@ -58,6 +66,7 @@ __device__ __forceinline__ float elem_error32(float x, float s, float zp, bool h
   const float a = fabsf(__fsub_rn(dq, x));
   if (norm == 2.0f) return __fmul_rn(a, a);
   if (norm == 3.0f) return __fmul_rn(__fmul_rn(a, a), a);
+  if (norm == 0.5f) return __fsqrt_rn(a);
   return powf(a, norm);
 }
 
@@ -232,7 +241,7 @@ __device__ __forceinline__ float chunk_error(const float (&x)[8], float s, float
       const float q = quantize_value(x[j], s, zp, HAS_ZP, DT, f);
       const float dq = dequantize_value(q, s, zp, HAS_ZP, DT);
       const float a = fabsf(round_rt(dq - x[j], DT));
-      err += round_rt(norm == 2.0f ? a * a : powf(a, norm), DT);
+      err += pow_eager(a, norm, DT);
     }
     return err;
   }
@@ -265,7 +274,14 @@ __device__ __forceinline__ float chunk_error(const float (&x)[8], float s, float
     if (HAS_ZP) dq = round16_finite<DT>(dq - zp);
     dq = round16_finite<DT>(dq * s);
     const float a = fabsf(round16_finite<DT>(dq - x[j]));
-    err += norm == 2.0f ? round16_finite<DT>(a * a) : pow_round16<DT>(a, norm);
+    if (norm == 2.0f)
+      err += round16_finite<DT>(a * a);
+    else if (norm == 3.0f)
+      err += round16_finite<DT>(round16_finite<DT>(a * a) * a);
+    else if (norm == 0.5f)
+      err += round16_finite<DT>(__fsqrt_rn(a));
+    else
+      err += pow_round16<DT>(a, norm);
   }
   return err;
 }

@@ -111,6 +111,15 @@ def fuse_weight_observers(model: Module):
 
 
 def lerp(start: torch.Tensor, end: torch.Tensor, weight: float) -> torch.Tensor:
+    """``start * (1 - weight) + end * weight`` with each of the three operations rounded to the tensors' dtype
+    (reference: observers/helpers.py:218-220).  For 16-bit tensors every operation is spelled out as an fp32
+    operation followed by a cast: the device compiler may otherwise fuse a product with its conversion to f16
+    into one instruction with a single rounding, which differs from the eager result on near-ties."""
+    if start.dtype in (torch.float16, torch.bfloat16):
+        dt = start.dtype
+        a = (start.float() * (1.0 - weight)).to(dt)
+        b = (end.float() * weight).to(dt)
+        return (a.float() + b.float()).to(dt)
     return (start * (1.0 - weight)) + (end * weight)
 
 

@@ -166,3 +166,68 @@ def test_gptq_seam_sweep_matches_oracle():
             print(f"agree {agree:.4f} ok={info['ok']}", spec, (R, K, T), "blocksize", blocksize, "dead", ndead, "damp", percdamp, flush=True)
     assert bad == 0 and worst >= 0.999
 
+
+
+def test_mse_observer_seam_sweep_is_bit_exact():
+    """60 random MSE-observer cases from the registry (weights and multi-batch activations; int / FP8 / NVFP4 /
+    MXFP4; bf16 / f16 / f32; search settings including the error exponents 2, 3, 0.5 and 1 for which the eager pow
+    has closed forms with their own roundings): min / max of every group equal the oracle's."""
+    from llmcompressor_amd.observers import Observer
+    from llmcompressor_amd.quantization import QuantizationArgs
+
+    random.seed(2)
+    torch.manual_seed(2)
+    bad = 0
+    worst = 1.0
+    for trial in range(60):
+        dtype = random.choice([torch.bfloat16, torch.bfloat16, torch.float32, torch.float16])
+        kind = random.choice(["int_group", "int_channel", "int_tensor", "int_block", "fp8_channel", "nvfp4", "mxfp4", "int_group_asym", "int_tensor_asym", "fp4_tg_noscale"])
+        R = random.choice([1, 5, 32, 64])
+        g = random.choice([16, 32, 128])
+        K = g * random.choice([1, 2, 4])
+        bits = random.choice([3, 4, 8])
+        spec = dict(num_bits=bits)
+        if kind.startswith("int_group"): spec.update(strategy="group", group_size=g)
+        elif kind == "int_channel": spec.update(strategy="channel")
+        elif kind.startswith("int_tensor"): spec.update(strategy="tensor")
+        elif kind == "int_block": spec.update(strategy="block", block_structure=[random.choice([2, 16]), g])
+        elif kind == "fp8_channel": spec.update(num_bits=8, type="float", strategy="channel")
+        elif kind == "nvfp4":
+            spec.update(num_bits=4, type="float", strategy="tensor_group", group_size=16, scale_dtype="float8_e4m3fn")
+            K = 16 * random.choice([2, 8])
+        elif kind == "fp4_tg_noscale":
+            spec.update(num_bits=4, type="float", strategy="tensor_group", group_size=16)
+            K = 16 * random.choice([2, 8])
+        elif kind == "mxfp4":
+            spec.update(num_bits=4, type="float", strategy="group", group_size=32, scale_dtype="uint8")
+            K = 32 * random.choice([1, 4])
+            dtype = torch.bfloat16
+        if kind.endswith("asym"): spec["symmetric"] = False
+        kw = random.choice([{}, {}, dict(maxshrink=0.8, patience=100), dict(norm=2.0), dict(grid=50.0, maxshrink=0.5, patience=3),
+                            dict(norm=3.0, patience=1), dict(norm=0.5), dict(norm=1.0, maxshrink=0.4)])
+        base = random.choice(["weight", "input"])
+        name = "memoryless_mse" if base == "weight" else random.choice(["mse", "memoryless_mse"])
+        if base == "input" and spec.get("strategy") in ("channel", "block"): base, name = "weight", "memoryless_mse"
+        spec["observer_kwargs"] = dict(kw)
+        ospec = dict(spec)
+        if "scale_dtype" in ospec: ospec["scale_dtype"] = getattr(torch, ospec["scale_dtype"])
+        oobs = O.Observer(name, base, F.QArgs(**ospec))
+        gobs = Observer.load_from_registry(name, base_name=base, args=QuantizationArgs(**spec))
+        ok = True
+        frac = 1.0
+        for step in range(1 if base == "weight" else 3):
+            w = torch.randn(R, K) * random.choice([0.02, 1.0, 30.0])
+            w[torch.rand(R, K) < 0.02] *= 8
+            w = w.to(dtype)
+            if base == "input": w = w.reshape(1, R, K)
+            oobs(w)
+            gobs(w.cuda())
+            a, b = gobs.min_vals.cpu().float().reshape(-1), oobs.min_vals.float().reshape(-1)
+            c, d = gobs.max_vals.cpu().float().reshape(-1), oobs.max_vals.float().reshape(-1)
+            frac = min(frac, ((a == b) & (c == d)).float().mean().item())
+        worst = min(worst, frac)
+        if frac < 1.0:
+            bad += 1
+            print(f"identical groups {frac:.4f}", name, base, spec, dtype, (R, K), flush=True)
+    assert bad == 0 and worst == 1.0
+
