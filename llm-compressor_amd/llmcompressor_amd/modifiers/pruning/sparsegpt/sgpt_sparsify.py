@@ -57,7 +57,9 @@ def sparsify_weight_tensors(weight: torch.Tensor, hessian: torch.Tensor, sparsit
     ``num_samples`` samples.  Returns (loss tensor [1], pruned weight in weight.dtype, info tensor)."""
     W = weight if weight.is_contiguous() else weight.contiguous()
     if preserve_sparsity_mask:
-        current = (W == 0).sum() / W.numel()
+        # the reference counts after zeroing the dead columns (sgpt_sparsify.py:103-106,127-133)
+        dead_cols = torch.diagonal(hessian) == 0
+        current = ((W == 0) | dead_cols.to(W.device)[None, :]).sum() / W.numel()
         if float(current) > sparsity:
             raise ValueError("The target sparsity is lower than the sparsity of the base model. Please retry "
                              "after turning preserve_sparsity_mask=False")
