@@ -14,6 +14,8 @@ import json
 import os
 from typing import Dict, Optional
 
+import math
+
 import torch
 
 from .. import ops
@@ -93,7 +95,10 @@ def compress_module(module: torch.nn.Module, fmt: Optional[str] = None) -> Dict[
         out["weight_packed"] = _run(weight, scale, zp, args, ops.OUT_PACKED, g_idx)
         out["weight_shape"] = torch.tensor(list(weight.shape), dtype=torch.int64, device=weight.device)
         out["weight_scale"] = scale
-        if not args.symmetric and zp is not None:
+        if not args.symmetric and zp is not None and args.strategy not in (QuantizationStrategy.GROUP,
+                                                                           QuantizationStrategy.CHANNEL):
+            out["weight_zero_point"] = zp  # only group / channel zero points are packed
+        elif not args.symmetric and zp is not None:
             # zero points are packed along the row dimension like the weights along the columns
             z = (zp.to(torch.int32) + (1 << (args.num_bits - 1))).to(torch.int32)
             pf = 32 // args.num_bits
@@ -131,24 +136,52 @@ def compress_module(module: torch.nn.Module, fmt: Optional[str] = None) -> Dict[
 _E2M1 = (0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0)
 
 
+def _expand_qparam(param: torch.Tensor, args: QuantizationArgs, R: int, K: int, g_idx=None) -> torch.Tensor:
+    """A scale / zero-point array broadcast to the weight's [R, K] layout for its strategy."""
+    s = args.strategy
+    if param.numel() == 1:
+        return param.reshape(1, 1)
+    if s in (QuantizationStrategy.GROUP, QuantizationStrategy.TENSOR_GROUP):
+        param = param.reshape(R, -1)
+        if g_idx is not None:
+            return param[:, g_idx.long()]
+        return param.repeat_interleave(args.group_size, dim=1)[:, :K]
+    if s == QuantizationStrategy.BLOCK:
+        bh, bw = args.block_structure
+        return param.repeat_interleave(bh, dim=0)[:R].repeat_interleave(bw, dim=1)[:, :K]
+    return param.reshape(R, 1)  # channel
+
+
+def _unpack_int32(packed: torch.Tensor, num_bits: int, count: int) -> torch.Tensor:
+    """Fields of `num_bits` bits from int32 words along the last dimension, lowest bits first, offset removed."""
+    pf = 32 // num_bits
+    shifts = torch.arange(pf, device=packed.device, dtype=torch.int32) * num_bits
+    fields = (packed.unsqueeze(-1) >> shifts) & ((1 << num_bits) - 1)
+    return fields.reshape(*packed.shape[:-1], -1)[..., :count] - (1 << (num_bits - 1))
+
+
 def decompress_weight(tensors: Dict[str, torch.Tensor], args: QuantizationArgs, fmt: str, dtype=torch.bfloat16):
-    """Inverse of compress_module for checks and reloads (plain tensor ops on the stored codes)."""
-    if fmt == CompressionFormat.pack_quantized:
-        packed = tensors["weight_packed"]
-        R, K = [int(v) for v in tensors["weight_shape"].tolist()]
-        pf = 32 // args.num_bits
-        shifts = torch.arange(pf, device=packed.device, dtype=torch.int32) * args.num_bits
-        codes = ((packed.unsqueeze(-1) >> shifts) & ((1 << args.num_bits) - 1)).reshape(R, -1)[:, :K]
-        codes = (codes - (1 << (args.num_bits - 1))).to(dtype)
-        scale = tensors["weight_scale"].to(dtype)
-        g = args.group_size if args.strategy in (QuantizationStrategy.GROUP, QuantizationStrategy.TENSOR_GROUP) else K
-        if "weight_g_idx" in tensors:
-            s = scale[:, tensors["weight_g_idx"].long()]
+    """Inverse of compress_module for checks and reloads (plain tensor ops on the stored codes): every
+    strategy, symmetric or with (packed) zero points."""
+    if fmt in (CompressionFormat.pack_quantized, CompressionFormat.float_quantized, CompressionFormat.int_quantized,
+               CompressionFormat.naive_quantized):
+        if fmt == CompressionFormat.pack_quantized:
+            R, K = [int(v) for v in tensors["weight_shape"].tolist()]
+            codes = _unpack_int32(tensors["weight_packed"], args.num_bits, K).to(torch.float32)
         else:
-            s = scale.repeat_interleave(g, dim=1)[:, :K] if scale.ndim == 2 and scale.shape[1] > 1 else scale
-        return codes * s
-    if fmt in (CompressionFormat.float_quantized, CompressionFormat.int_quantized, CompressionFormat.naive_quantized):
-        return tensors["weight"].to(dtype) * tensors["weight_scale"].to(dtype)
+            codes = tensors["weight"].to(torch.float32)
+            R, K = codes.shape
+        g_idx = tensors.get("weight_g_idx")
+        zp = tensors.get("weight_zero_point")
+        if zp is not None and not args.symmetric:
+            if fmt == CompressionFormat.pack_quantized and zp.dtype == torch.int32:
+                # packed along the rows: [ceil(rows / pack_factor), columns of the zero-point array]
+                rows = 1 if args.strategy == QuantizationStrategy.TENSOR else (
+                    math.ceil(R / args.block_structure[0]) if args.strategy == QuantizationStrategy.BLOCK else R)
+                zp = _unpack_int32(zp.t().contiguous(), args.num_bits, rows).t()
+            codes = codes - _expand_qparam(zp.to(torch.float32), args, R, K, g_idx)
+        scale = _expand_qparam(tensors["weight_scale"].to(dtype), args, R, K, g_idx)
+        return codes.to(dtype) * scale
     packed = tensors["weight_packed"]
     grid = torch.tensor(_E2M1 + tuple(-v for v in _E2M1), dtype=torch.float32, device=packed.device)
     vals = torch.stack([grid[(packed & 0xF).long()], grid[(packed >> 4).long()]], dim=-1).reshape(packed.shape[0], -1)

@@ -226,8 +226,14 @@ def forward_quantize(module: Module, value: torch.Tensor, base_name: str, args: 
     if args.dynamic is True and args.strategy == QuantizationStrategy.TOKEN:
         fmt, bits = kernel_format(args)
         x2, shape = _as_2d(value)
-        out, _ = ops.dynamic_per_token_quantize(x2.contiguous(), fmt, bits)
-        return out.reshape(shape)
+        x2 = x2.contiguous()
+        if args.symmetric and bits == 8:  # the fused kernel: row absmax, scale and fake-quant in one pass
+            out, _ = ops.dynamic_per_token_quantize(x2, fmt, bits)
+            return out.reshape(shape)
+        # other widths and asymmetric ranges: row min/max, qparams and fake-quant as separate kernels
+        mn, mx = ops.minmax_groups(x2, x2.shape[1])
+        scale, zp = calculate_qparams(mn, mx, args)
+        return fake_quantize(x2, scale, zp, args).reshape(shape)
     scale = getattr(module, f"{base_name}_scale", None)
     zp = getattr(module, f"{base_name}_zero_point", None)
     gs = getattr(module, f"{base_name}_global_scale", None)

