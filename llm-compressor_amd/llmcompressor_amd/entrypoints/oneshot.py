@@ -48,6 +48,11 @@ class Oneshot:
             logger.warning("Detected an MoE model whose experts are stored as fused 3-D tensors; replacing them "
                            "by per-expert Linears so that they can be calibrated and quantized.")
             linearize_moe(self.model)
+        left = [name for name, m in self.model.named_modules()
+                if isinstance(getattr(m, "down_proj", None), torch.nn.Parameter) and m.down_proj.ndim == 3]
+        if left:
+            logger.warning(f"{len(left)} fused expert modules have a layout or forward signature that is not "
+                           f"recognised ({left[0]}, ...); they stay as they are and their weights are not quantized.")
         self.apply_recipe_modifiers(self.dataset)
         if self.output_dir is not None:
             from ..compressors import save_pretrained_compressed

@@ -30,33 +30,56 @@ def moe_calibration_context(calibrate_all_experts: bool = True):
         _CALIBRATE_ALL_EXPERTS = prev
 
 
+def _default_apply_gate(self, gate_up: torch.Tensor) -> torch.Tensor:
+    gate, up = gate_up.chunk(2, dim=-1)
+    return self.act_fn(gate) * up
+
+
 class ExpertMLP(nn.Module):
+    """One expert as plain Linears.  ``forward`` is ``down(apply_gate(cat[gate(x), up(x)]))`` as in the reference
+    (modeling/moe/linear_experts.py:26-87): "gate" and "up" name the first and second half of the fused
+    projection's output columns, and ``apply_gate`` is the fused module's own gating function (by default
+    ``act_fn(first half) * second half``), so an interleaved layout or a clamped activation keeps its meaning."""
+
     def __init__(self, hidden: int, intermediate: int, dtype=torch.bfloat16, device=None, act_fn=None,
-                 bias: bool = False):
+                 bias: bool = False, apply_gate=None):
         super().__init__()
         self.gate_proj = nn.Linear(hidden, intermediate, bias=bias, dtype=dtype, device=device)
         self.up_proj = nn.Linear(hidden, intermediate, bias=bias, dtype=dtype, device=device)
         self.down_proj = nn.Linear(intermediate, hidden, bias=bias, dtype=dtype, device=device)
         self.act_fn = act_fn if act_fn is not None else nn.SiLU()
+        self._gate_fn = apply_gate  # a plain callable (bound to the experts list), not a submodule
 
     def forward(self, x):
-        return self.down_proj(self.act_fn(self.gate_proj(x)) * self.up_proj(x))
+        if self._gate_fn is None:
+            return self.down_proj(self.act_fn(self.gate_proj(x)) * self.up_proj(x))
+        return self.down_proj(self._gate_fn(torch.cat([self.gate_proj(x), self.up_proj(x)], dim=-1)))
 
 
 class LinearExperts2D(nn.ModuleList):
     """Experts as a list of ExpertMLP; ``from_fused`` splits [E, 2I, H] gate_up and [E, H, I] down tensors."""
 
     def __init__(self, num_experts: int, hidden: int, intermediate: int, dtype=torch.bfloat16, device=None,
-                 act_fn=None, bias: bool = False):
-        super().__init__([ExpertMLP(hidden, intermediate, dtype, device, act_fn, bias) for _ in range(num_experts)])
+                 act_fn=None, bias: bool = False, apply_gate=None, gate_attributes=None):
+        nn.Module.__init__(self)
+        # what a fused module's own gating function reads from `self` (activation, clamp limits, ...)
+        for key, value in (gate_attributes or {}).items():
+            object.__setattr__(self, key, value)
+        bound = None
+        if apply_gate is not None:
+            import types
+
+            bound = types.MethodType(apply_gate, self)
+        self.extend([ExpertMLP(hidden, intermediate, dtype, device, act_fn, bias, bound) for _ in range(num_experts)])
         self.num_experts = num_experts
 
     @classmethod
     def from_fused(cls, gate_up_proj: torch.Tensor, down_proj: torch.Tensor, act_fn=None, gate_up_bias=None,
-                   down_bias=None) -> "LinearExperts2D":
+                   down_bias=None, apply_gate=None, gate_attributes=None) -> "LinearExperts2D":
         E, two_i, H = gate_up_proj.shape
         inter = two_i // 2
-        self = cls(E, H, inter, gate_up_proj.dtype, gate_up_proj.device, act_fn, bias=gate_up_bias is not None)
+        self = cls(E, H, inter, gate_up_proj.dtype, gate_up_proj.device, act_fn, bias=gate_up_bias is not None,
+                   apply_gate=apply_gate, gate_attributes=gate_attributes)
         with torch.no_grad():
             for e, expert in enumerate(self):
                 expert.gate_proj.weight.copy_(gate_up_proj[e, :inter])
@@ -72,13 +95,21 @@ class LinearExperts2D(nn.ModuleList):
     def from_experts_module(cls, experts: nn.Module) -> "LinearExperts2D":
         """From a fused experts module in the standard transformers layout (reference:
         modeling/moe/linear_experts.py:186-208): ``gate_up_proj`` [E, 2I, H] and ``down_proj`` [E, H, I]
-        parameters (``is_transposed``: [E, H, 2I] and [E, I, H]), optional ``*_bias`` parameters, ``act_fn``."""
+        parameters (``is_transposed``: [E, H, 2I] and [E, I, H]), optional ``*_bias`` parameters, ``act_fn``, and
+        the class's own ``_apply_gate`` when it defines one."""
         gate_up, down = experts.gate_up_proj.data, experts.down_proj.data
         if getattr(experts, "is_transposed", False):
             gate_up, down = gate_up.transpose(1, 2), down.transpose(1, 2)
         gub, db = getattr(experts, "gate_up_proj_bias", None), getattr(experts, "down_proj_bias", None)
-        return cls.from_fused(gate_up, down, getattr(experts, "act_fn", None),
-                              None if gub is None else gub.data, None if db is None else db.data)
+        apply_gate = getattr(type(experts), "_apply_gate", None)
+        attributes = {k: v for k, v in vars(experts).items()
+                      if not k.startswith("_") and isinstance(v, (int, float, bool)) and k != "training"}
+        act_fn = getattr(experts, "act_fn", None)
+        if act_fn is not None:
+            attributes["act_fn"] = act_fn  # a plain attribute of the list, so that its length stays the expert count
+        return cls.from_fused(gate_up, down, act_fn if isinstance(act_fn, nn.Module) else None,
+                              None if gub is None else gub.data, None if db is None else db.data,
+                              apply_gate=apply_gate, gate_attributes=attributes)
 
     def forward(self, hidden_states: torch.Tensor, top_k_index: torch.Tensor, top_k_weights: torch.Tensor):
         """hidden_states [T,H]; top_k_index / top_k_weights [T,k].
@@ -119,6 +150,20 @@ class LinearExperts2D(nn.ModuleList):
         return final
 
 
+def _takes_routing_arguments(module: nn.Module) -> bool:
+    """forward(hidden_states, top_k_index, top_k_weights): the call LinearExperts2D.forward answers."""
+    import inspect
+
+    try:
+        params = [p for p in inspect.signature(module.forward).parameters.values()
+                  if p.kind in (p.POSITIONAL_ONLY, p.POSITIONAL_OR_KEYWORD)]
+    except (TypeError, ValueError):
+        return False
+    if any(p.kind == p.VAR_POSITIONAL for p in inspect.signature(module.forward).parameters.values()):
+        return True  # a dispatching wrapper (*args, **kwargs)
+    return len(params) == 3
+
+
 def get_non_linearized_moes(model: nn.Module):
     """(name, module) of every fused experts module: 3-D ``gate_up_proj`` and ``down_proj`` parameters whose
     shapes fit each other (reference: modeling/moe/linearize.py:128-147)."""
@@ -134,7 +179,7 @@ def get_non_linearized_moes(model: nn.Module):
             fits = gu.shape[2] == 2 * dn.shape[1] and gu.shape[1] == dn.shape[2]
         else:
             fits = gu.shape[1] == 2 * dn.shape[2] and gu.shape[2] == dn.shape[1]
-        if fits:
+        if fits and _takes_routing_arguments(module):
             found.append((name, module))
     return found
 

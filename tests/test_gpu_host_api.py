@@ -1423,3 +1423,38 @@ def test_gptq_beats_round_to_nearest_end_to_end_on_a_transformers_llama():
         with torch.no_grad():
             errs[name] = ((m(held).logits.float() - dense).norm() / dense.norm()).item()
     assert errs["gptq"] < 0.9 * errs["rtn"], errs
+
+
+@pytest.mark.parametrize("family", ["mixtral", "gpt_oss"])
+def test_linearize_moe_keeps_the_logits_of_transformers_moe_families(family):
+    """Fused experts of other transformers families keep their function when replaced by per-expert Linears:
+    Mixtral (standard layout); GPT-OSS (transposed weights, biases, interleaved gate / up columns
+    and a clamped gate, all inside the class's own ``_apply_gate``) up to the rounding of the fused bias add."""
+    transformers = pytest.importorskip("transformers")
+    import copy
+
+    from llmcompressor_amd.modeling import LinearExperts2D, get_non_linearized_moes, linearize_moe
+
+    torch.manual_seed(0)
+    common = dict(hidden_size=128, num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2, vocab_size=256,
+                  max_position_embeddings=128, num_local_experts=4, num_experts_per_tok=2)
+    if family == "mixtral":
+        model = transformers.MixtralForCausalLM(transformers.MixtralConfig(intermediate_size=256, **common))
+    else:
+        model = transformers.GptOssForCausalLM(transformers.GptOssConfig(intermediate_size=128, head_dim=32,
+                                                                         sliding_window=32, **common))
+    model = model.to(torch.bfloat16).to(DEV)
+    for p in model.parameters():  # biases and experts start at zero or empty in some families
+        if p.ndim >= 1 and float(p.detach().float().abs().sum()) == 0:
+            p.data.normal_(0, 0.05)
+    probe = torch.randint(0, 256, (2, 32), device=DEV)
+    with torch.no_grad():
+        want = model(probe).logits.float()
+        assert len(get_non_linearized_moes(model)) == 2
+        twin = linearize_moe(copy.deepcopy(model))
+        assert get_non_linearized_moes(twin) == []
+        assert sum(isinstance(m, LinearExperts2D) for m in twin.modules()) == 2
+        got = twin(probe).logits.float()
+    # the fused module runs one product for gate and up together, the replacement one each: the library may sum
+    # them in a different order, so equality holds only up to bf16 rounding
+    assert ((got - want).norm() / want.norm()).item() < (5e-3 if family == "mixtral" else 2e-2)
