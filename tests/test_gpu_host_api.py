@@ -1458,3 +1458,41 @@ def test_linearize_moe_keeps_the_logits_of_transformers_moe_families(family):
     # the fused module runs one product for gate and up together, the replacement one each: the library may sum
     # them in a different order, so equality holds only up to bf16 rounding
     assert ((got - want).norm() / want.norm()).item() < (5e-3 if family == "mixtral" else 2e-2)
+
+
+def test_scheduling_options_do_not_change_gptq_results_on_a_transformers_llama():
+    """The scheduling fields of GPTQModifier (lock-step sets, stream concurrency, staging by reference or by
+    copy, shared Hessians for identical inputs) leave every quantised parameter bit-identical; one Hessian launch
+    per hook call instead of staged launches changes the summation order only (>= 99.9 % identical weights)."""
+    transformers = pytest.importorskip("transformers")
+
+    from llmcompressor_amd import oneshot
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+
+    cfg = transformers.LlamaConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=2,
+                                   num_attention_heads=4, num_key_value_heads=2, vocab_size=256,
+                                   max_position_embeddings=128)
+    torch.manual_seed(3)
+    data = [{"input_ids": torch.randint(0, 256, (1, 128))} for _ in range(6)]
+
+    def run(**kw):
+        torch.manual_seed(0)
+        model = transformers.LlamaForCausalLM(cfg).to(torch.bfloat16).to(DEV)
+        oneshot(model=model, dataset=data, recipe=GPTQModifier(targets="Linear", scheme="W4A16", ignore=["lm_head"],
+                                                               **kw))
+        return {n: p.detach().clone() for n, p in model.named_parameters()}
+
+    base = run()
+    for kw in (dict(group_min_modules=0), dict(compress_concurrency=1), dict(group_min_modules=0, compress_concurrency=1),
+               dict(stage_by_reference=False), dict(share_identical_inputs=True), dict(stage_max_bytes=1 << 16)):
+        other = run(**kw)
+        assert other.keys() == base.keys()
+        same_everywhere = all(torch.equal(base[n], other[n]) for n in base)
+        if "stage_max_bytes" in kw:  # early flushes regroup the token sums
+            agree = min((base[n] == other[n]).float().mean().item() for n in base if n.endswith("proj.weight"))
+            assert agree >= 0.999, (kw, agree)
+        else:
+            assert same_everywhere, kw
+    unstaged = run(hessian_batch_tokens=0)
+    agree = min((base[n] == unstaged[n]).float().mean().item() for n in base if n.endswith("proj.weight"))
+    assert agree >= 0.999, agree
