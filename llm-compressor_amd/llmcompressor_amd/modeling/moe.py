@@ -10,6 +10,8 @@ weights of the tokens actually routed to it.
 from __future__ import annotations
 
 import contextlib
+import inspect
+import types
 
 import torch
 from torch import nn
@@ -28,11 +30,6 @@ def moe_calibration_context(calibrate_all_experts: bool = True):
         yield
     finally:
         _CALIBRATE_ALL_EXPERTS = prev
-
-
-def _default_apply_gate(self, gate_up: torch.Tensor) -> torch.Tensor:
-    gate, up = gate_up.chunk(2, dim=-1)
-    return self.act_fn(gate) * up
 
 
 class ExpertMLP(nn.Module):
@@ -61,15 +58,11 @@ class LinearExperts2D(nn.ModuleList):
 
     def __init__(self, num_experts: int, hidden: int, intermediate: int, dtype=torch.bfloat16, device=None,
                  act_fn=None, bias: bool = False, apply_gate=None, gate_attributes=None):
-        nn.Module.__init__(self)
+        super().__init__()
         # what a fused module's own gating function reads from `self` (activation, clamp limits, ...)
         for key, value in (gate_attributes or {}).items():
             object.__setattr__(self, key, value)
-        bound = None
-        if apply_gate is not None:
-            import types
-
-            bound = types.MethodType(apply_gate, self)
+        bound = types.MethodType(apply_gate, self) if apply_gate is not None else None
         self.extend([ExpertMLP(hidden, intermediate, dtype, device, act_fn, bias, bound) for _ in range(num_experts)])
         self.num_experts = num_experts
 
@@ -152,8 +145,6 @@ class LinearExperts2D(nn.ModuleList):
 
 def _takes_routing_arguments(module: nn.Module) -> bool:
     """forward(hidden_states, top_k_index, top_k_weights): the call LinearExperts2D.forward answers."""
-    import inspect
-
     try:
         params = [p for p in inspect.signature(module.forward).parameters.values()
                   if p.kind in (p.POSITIONAL_ONLY, p.POSITIONAL_OR_KEYWORD)]
