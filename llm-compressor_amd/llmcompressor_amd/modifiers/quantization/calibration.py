@@ -1,10 +1,12 @@
-"""Observer attachment and qparam updates (reference: modifiers/quantization/calibration.py:36-231)."""
+"""Observer attachment and qparam updates (reference: modifiers/quantization/calibration.py:36-231).
+
+The public names and their behaviour are the reference's; the observers they attach run the HIP min-max / MSE
+kernels (``llmcompressor_amd.observers``).
+"""
 from __future__ import annotations
 
 import logging
-from collections.abc import Iterable
-from itertools import product
-from typing import Any
+from typing import Any, Iterable, Iterator
 
 import torch
 from torch.nn import Module
@@ -35,6 +37,13 @@ __all__ = [
     "calibrate_value_hook",
 ]
 
+# which part of a scheme describes an observed value; q / k / v of an attention module share the input arguments
+_SCHEME_FIELD = {"weight": "weights", "output": "output_activations", "input": "input_activations",
+                 "q": "input_activations", "k": "input_activations", "v": "input_activations"}
+# weight observers never need history: a weight is observed once, so the running variants only cost memory
+_MEMORYLESS = {"static_minmax": "memoryless_minmax", "minmax": "memoryless_minmax", "mse": "memoryless_mse"}
+_OBSERVED = tuple(_SCHEME_FIELD)
+
 _warned = set()
 
 
@@ -44,46 +53,45 @@ def _warn_once(msg):
         logger.warning(msg)
 
 
+def _modules_of(target) -> Iterator[Module]:
+    """One module, or every module of an iterable (an ``nn.ModuleList`` counts as one module)."""
+    if isinstance(target, Module):
+        yield target
+    else:
+        yield from target
+
+
 def initialize_observer(module: Module, base_name: str):
-    """Attach ``<base_name>_observer``; weights always get the memoryless variants."""
-    if base_name == "weight":
-        arg_name = "weights"
-    elif base_name == "output":
-        arg_name = "output_activations"
-    else:  # input, q, k, v
-        arg_name = "input_activations"
-    args: QuantizationArgs = getattr_chain(module, f"quantization_scheme.{arg_name}", None)
-    observer = args.observer
-    if base_name == "weight" and args.observer in ("static_minmax", "minmax"):
-        observer = "memoryless_minmax"
-        _warn_once(f"Overriding weight observer for lower memory usage ({args.observer} -> {observer})")
-    if base_name == "weight" and args.observer in ("mse",):
-        observer = "memoryless_mse"
-        _warn_once(f"Overriding weight observer for lower memory usage ({args.observer} -> {observer})")
-    if args is not None and args.dynamic is not True:
-        observer = Observer.load_from_registry(observer, base_name=base_name, args=args)
-        module.register_module(f"{base_name}_observer", observer)
-        observer.attach(module)
+    """Attach ``<base_name>_observer`` as the scheme asks; nothing for fully dynamic arguments."""
+    args: QuantizationArgs = getattr_chain(module, f"quantization_scheme.{_SCHEME_FIELD[base_name]}", None)
+    name = args.observer
+    if base_name == "weight" and name in _MEMORYLESS:
+        name = _MEMORYLESS[name]
+        _warn_once(f"Overriding weight observer for lower memory usage ({args.observer} -> {name})")
+    if args.dynamic is True:
+        return
+    observer = Observer.load_from_registry(name, base_name=base_name, args=args)
+    module.register_module(f"{base_name}_observer", observer)
+    observer.attach(module)
 
 
 def observe(module: Module | Iterable[Module], base_name: str):
-    if isinstance(module, Iterable) and not isinstance(module, Module):
-        for m in module:
-            observe(m, base_name)
-        return
-    observer = getattr(module, f"{base_name}_observer", None)
-    if observer is None:
-        return
-    observer(getattr(module, base_name))
+    """Show ``module.<base_name>`` (normally the weight) to its observer, for one module or many."""
+    for m in _modules_of(module):
+        observer = getattr(m, f"{base_name}_observer", None)
+        if observer is not None:
+            observer(getattr(m, base_name))
 
 
 def update_qparams(module: Module | Iterable[Module], base_name: str | Iterable[str], only_update_onload: bool = False):
-    if (isinstance(module, Iterable) and not isinstance(module, Module)) or not isinstance(base_name, str):
-        modules = [module] if isinstance(module, Module) else module
-        base_names = [base_name] if isinstance(base_name, str) else base_name
-        for m, b in product(list(modules), list(base_names)):
-            update_qparams(m, b, only_update_onload=only_update_onload)
-        return
+    """Turn the observers' statistics into ``<base_name>_scale`` / ``_zero_point`` / ``_global_scale``."""
+    names = (base_name,) if isinstance(base_name, str) else tuple(base_name)
+    for m in list(_modules_of(module)):
+        for name in names:
+            _update_one(m, name, only_update_onload)
+
+
+def _update_one(module: Module, base_name: str, only_update_onload: bool):
     observer = getattr(module, f"{base_name}_observer", None)
     if observer is None:
         return
@@ -93,25 +101,20 @@ def update_qparams(module: Module | Iterable[Module], base_name: str | Iterable[
             "calibration setup, such as not using `moe_calibrate_all_experts` or selecting the wrong calibration "
             "pipeline.")
         return
-    args = observer.args
-    is_dynamic = getattr(args, "dynamic", False) in (True, DynamicType.LOCAL)
-    qparams = observer.get_qparams()
-    for param_name, param_val in qparams.items():
-        if param_val is None:
+    # dynamic and local arguments keep only the global scale: their scales come from each call's values
+    keep_only_global = getattr(observer.args, "dynamic", False) in (True, DynamicType.LOCAL)
+    for key, value in observer.get_qparams().items():
+        target = f"{base_name}_{key}"
+        if value is None or (keep_only_global and key != "global_scale") or not hasattr(module, target):
             continue
-        if is_dynamic and param_name in ("scale", "zero_point"):
-            continue
-        full = f"{base_name}_{param_name}"
-        if hasattr(module, full):
-            if not only_update_onload:
-                update_offload_parameter(module, full, param_val)
-            else:
-                getattr(module, full).data = param_val
+        if only_update_onload:
+            getattr(module, target).data = value
+        else:
+            update_offload_parameter(module, target, value)
 
 
 def calibrate_input_hook(module: Module, args: Any):
-    args = args[0] if isinstance(args, tuple) else args
-    module.input_observer(args)
+    module.input_observer(args[0] if isinstance(args, tuple) else args)
 
 
 def calibrate_output_hook(module: Module, _args: Any, output: torch.Tensor):
@@ -133,21 +136,20 @@ def calibrate_value_hook(module: Module, value_states: torch.Tensor):
 
 
 def apply_calibration_status(module: Module):
-    if not getattr(module, "quantization_scheme", None):
-        return
-    module.quantization_status = QuantizationStatus.CALIBRATION
+    if getattr(module, "quantization_scheme", None):
+        module.quantization_status = QuantizationStatus.CALIBRATION
 
 
 def freeze_module_quantization(module: Module):
-    if not getattr(module, "quantization_scheme", None):
+    """Drop the observers and mark the module frozen (idempotent)."""
+    if not getattr(module, "quantization_scheme", None) or module.quantization_status == QuantizationStatus.FROZEN:
         return
-    if module.quantization_status == QuantizationStatus.FROZEN:
-        return
-    for name in ("input", "weight", "output", "q", "k", "v"):
-        obs_name = f"{name}_observer"
-        if hasattr(module, obs_name):
-            getattr(module, obs_name).detach(module)
-            delattr(module, obs_name)
+    for base_name in _OBSERVED:
+        attr = f"{base_name}_observer"
+        observer = getattr(module, attr, None)
+        if observer is not None:
+            observer.detach(module)
+            delattr(module, attr)
     module.quantization_status = QuantizationStatus.FROZEN
 
 
