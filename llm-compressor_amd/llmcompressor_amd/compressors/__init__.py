@@ -126,8 +126,13 @@ def compress_module(module: torch.nn.Module, fmt: Optional[str] = None) -> Dict[
         raise ValueError(f"unsupported compression format {fmt}")
     for name in ("input_scale", "input_zero_point", "input_global_scale", "output_scale", "output_zero_point"):
         t = getattr(module, name, None)
-        if t is not None:
-            out[name] = t.data
+        if t is None:
+            continue
+        if name.endswith("zero_point"):  # zero points of symmetric arguments are all zero and are not stored
+            act = scheme.input_activations if name.startswith("input") else scheme.output_activations
+            if act is None or act.symmetric:
+                continue
+        out[name] = t.data
     if getattr(module, "bias", None) is not None:
         out["bias"] = module.bias.data
     return out

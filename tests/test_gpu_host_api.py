@@ -1496,3 +1496,26 @@ def test_scheduling_options_do_not_change_gptq_results_on_a_transformers_llama()
     unstaged = run(hessian_batch_tokens=0)
     agree = min((base[n] == unstaged[n]).float().mean().item() for n in base if n.endswith("proj.weight"))
     assert agree >= 0.999, agree
+
+
+def test_checkpoint_omits_zero_points_of_symmetric_activations(tmp_path):
+    """Static activation quantisation: ``input_scale`` is written; ``input_zero_point`` only when the activation
+    arguments are asymmetric (symmetric zero points are all zero and are not stored)."""
+    from safetensors.torch import load_file
+
+    from llmcompressor_amd import oneshot
+    from llmcompressor_amd.modifiers.quantization import QuantizationModifier
+
+    torch.manual_seed(1)
+    data = [{"input_ids": torch.randint(0, 100, (1, 48))} for _ in range(4)]
+    for symmetric in (True, False):
+        model = _tiny(3).to(DEV)
+        out_dir = str(tmp_path / f"sym{symmetric}")
+        recipe = QuantizationModifier(targets="Linear", ignore=["lm_head"], config_groups={"g": dict(
+            targets=["Linear"], weights=dict(num_bits=8, strategy="channel"),
+            input_activations=dict(num_bits=8, strategy="tensor", dynamic=False, symmetric=symmetric))})
+        oneshot(model=model, recipe=recipe, dataset=data, output_dir=out_dir)
+        sd = load_file(os.path.join(out_dir, "model.safetensors"))
+        key = "layers.0.q_proj."
+        assert key + "input_scale" in sd and key + "weight_scale" in sd and key + "weight_zero_point" not in sd
+        assert (key + "input_zero_point" in sd) == (not symmetric)
