@@ -1,2 +1,2 @@
-from .moe import (ExpertMLP, LinearExperts2D, get_non_linearized_moes, linearize_moe,  # noqa: F401
-                  moe_calibration_context)
+from .moe import (ExpertMLP, LinearExperts2D, Llama4LinearExperts, get_non_linearized_moes,  # noqa: F401
+                  linearize_moe, moe_calibration_context)

@@ -16,7 +16,8 @@ import types
 import torch
 from torch import nn
 
-__all__ = ["ExpertMLP", "LinearExperts2D", "moe_calibration_context", "get_non_linearized_moes", "linearize_moe"]
+__all__ = ["ExpertMLP", "LinearExperts2D", "Llama4LinearExperts", "moe_calibration_context",
+           "get_non_linearized_moes", "linearize_moe"]
 
 _CALIBRATE_ALL_EXPERTS = False
 
@@ -143,6 +144,32 @@ class LinearExperts2D(nn.ModuleList):
         return final
 
 
+class Llama4LinearExperts(LinearExperts2D):
+    """Per-expert Linears for ``Llama4TextExperts`` (reference: modeling/moe/llama4.py:15-110).  That module is
+    called with the tokens already laid out per expert, ``[E * T, H]`` (every expert sees every token; the router's
+    scores were applied upstream), stores ``gate_up_proj`` as [E, H, 2I] and ``down_proj`` as [E, I, H], and
+    returns ``[E * T, H]``."""
+
+    @classmethod
+    def from_experts_module(cls, experts: nn.Module) -> "Llama4LinearExperts":
+        gate_up, down = experts.gate_up_proj.data.transpose(1, 2), experts.down_proj.data.transpose(1, 2)
+        return cls.from_fused(gate_up, down, getattr(experts, "act_fn", None))
+
+    def forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
+        per_expert = hidden_states.view(self.num_experts, -1, hidden_states.shape[-1])
+        outs = []
+        for e, expert in enumerate(self):
+            if _CALIBRATE_ALL_EXPERTS:
+                outs.append(expert(hidden_states).view(self.num_experts, -1, hidden_states.shape[-1])[e])
+            else:
+                outs.append(expert(per_expert[e]))
+        return torch.cat(outs, dim=0)
+
+
+# fused modules whose call convention differs from (hidden_states, top_k_index, top_k_weights), by class name
+_SPECIAL_EXPERTS = {"Llama4TextExperts": Llama4LinearExperts}
+
+
 def _takes_routing_arguments(module: nn.Module) -> bool:
     """forward(hidden_states, top_k_index, top_k_weights): the call LinearExperts2D.forward answers."""
     try:
@@ -162,6 +189,9 @@ def get_non_linearized_moes(model: nn.Module):
     for name, module in model.named_modules():
         if isinstance(module, LinearExperts2D):
             continue
+        if type(module).__name__ in _SPECIAL_EXPERTS:
+            found.append((name, module))
+            continue
         gu, dn = getattr(module, "gate_up_proj", None), getattr(module, "down_proj", None)
         if not (isinstance(gu, torch.Tensor) and isinstance(dn, torch.Tensor) and gu.ndim == 3 and dn.ndim == 3
                 and gu.shape[0] == dn.shape[0]):
@@ -179,5 +209,6 @@ def linearize_moe(model: nn.Module) -> nn.Module:
     """Replace every fused experts module by a ``LinearExperts2D`` of plain Linears, so that per-expert
     weights can be calibrated and quantised (reference: modeling/moe/linearize.py:97-125)."""
     for name, module in get_non_linearized_moes(model):
-        model.set_submodule(name, LinearExperts2D.from_experts_module(module))
+        cls = _SPECIAL_EXPERTS.get(type(module).__name__, LinearExperts2D)
+        model.set_submodule(name, cls.from_experts_module(module))
     return model

@@ -1425,10 +1425,10 @@ def test_gptq_beats_round_to_nearest_end_to_end_on_a_transformers_llama():
     assert errs["gptq"] < 0.9 * errs["rtn"], errs
 
 
-@pytest.mark.parametrize("family", ["mixtral", "gpt_oss"])
+@pytest.mark.parametrize("family", ["mixtral", "gpt_oss", "llama4"])
 def test_linearize_moe_keeps_the_logits_of_transformers_moe_families(family):
     """Fused experts of other transformers families keep their function when replaced by per-expert Linears:
-    Mixtral (standard layout); GPT-OSS (transposed weights, biases, interleaved gate / up columns
+    Mixtral (standard layout); Llama-4 (tokens laid out per expert, transposed weights; its own list class); GPT-OSS (transposed weights, biases, interleaved gate / up columns
     and a clamped gate, all inside the class's own ``_apply_gate``) up to the rounding of the fused bias add."""
     transformers = pytest.importorskip("transformers")
     import copy
@@ -1440,6 +1440,10 @@ def test_linearize_moe_keeps_the_logits_of_transformers_moe_families(family):
                   max_position_embeddings=128, num_local_experts=4, num_experts_per_tok=2)
     if family == "mixtral":
         model = transformers.MixtralForCausalLM(transformers.MixtralConfig(intermediate_size=256, **common))
+    elif family == "llama4":  # its experts module is called with the tokens laid out per expert
+        common["num_experts_per_tok"] = 1
+        model = transformers.Llama4ForCausalLM(transformers.Llama4TextConfig(
+            intermediate_size=256, intermediate_size_mlp=256, head_dim=32, interleave_moe_layer_step=1, **common))
     else:
         model = transformers.GptOssForCausalLM(transformers.GptOssConfig(intermediate_size=128, head_dim=32,
                                                                          sliding_window=32, **common))
