@@ -502,3 +502,115 @@ def test_linearize_moe_keeps_the_function(transposed, bias):
         assert isinstance(lin[0].act_fn, torch.nn.GELU) and (lin[0].gate_proj.bias is not None) == bias
         got = lin(x, idx, w)
     assert torch.allclose(got, want, atol=1e-4, rtol=1e-4)
+
+
+def test_gptq_job_planning():
+    """compress_module_list plans lock-step sets by input width: at least ``group_min_modules`` Linears of one width
+    form a set (split so that a set's work buffers stay within ``group_max_bytes``), the rest go one by one."""
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+    from llmcompressor_amd.quantization import QuantizationArgs, QuantizationScheme
+
+    class FakeCuda(torch.Tensor):
+        """A CPU tensor that claims to live on the GPU, enough for the planner's eligibility checks."""
+
+        @property
+        def is_cuda(self):
+            return True
+
+    def lin(i, o):
+        m = torch.nn.Linear(i, o, bias=False)
+        m.weight = torch.nn.Parameter(torch.Tensor._make_subclass(FakeCuda, m.weight.data), requires_grad=False)
+        m.quantization_scheme = QuantizationScheme(targets=["Linear"], weights=QuantizationArgs(
+            num_bits=4, strategy="group", group_size=32))
+        return m
+
+    mods = [lin(64, 64), lin(64, 16), lin(64, 16), lin(64, 128), lin(128, 64), lin(96, 32), lin(96, 32)]
+    mod = GPTQModifier(targets="Linear", scheme="W4A16")
+    for m in mods:
+        mod._hessians[m] = torch.Tensor._make_subclass(FakeCuda, torch.zeros(m.in_features, m.in_features))
+    plan = mod._plan_jobs(list(mods))
+    sets = [j for j in plan if isinstance(j, list)]
+    singles = [j for j in plan if not isinstance(j, list)]
+    assert len(sets) == 1 and sets[0] == mods[:4]            # four Linears of width 64
+    assert singles == mods[4:]                               # width 128 alone; two of width 96 are below the minimum
+    mod.group_min_modules = 2
+    plan = mod._plan_jobs(list(mods))
+    assert [len(j) for j in plan if isinstance(j, list)] == [4, 2]
+    mod.group_max_bytes = 10 * 64 * 64 * 3                   # room for three width-64 problems per job
+    plan = mod._plan_jobs(list(mods))
+    assert [len(j) if isinstance(j, list) else 1 for j in plan][:2] == [3, 1]
+    mod.group_min_modules = 0
+    assert mod._plan_jobs(list(mods)) == mods
+
+
+def test_observed_kv_cache_stand_in():
+    """The stand-in for ``past_key_values`` shows keys and values to the module's observers and defers to the
+    real cache when there is one."""
+    from llmcompressor_amd.modifiers.quantization.quantization.mixin import _kv_cache_pre_hook, _ObservedKVCache
+
+    seen = []
+
+    class Attn(torch.nn.Module):
+        def k_observer(self, x):
+            seen.append(("k", x.shape))
+
+        def v_observer(self, x):
+            seen.append(("v", x.shape))
+
+    class Real:
+        marker = 7
+
+        def update(self, k, v, layer_idx, cache_kwargs=None):
+            return k + 1, v + 1
+
+    attn = Attn()
+    k, v = torch.zeros(1, 2, 5, 4), torch.ones(1, 2, 5, 4)
+    _, kwargs = _kv_cache_pre_hook(attn, (), {"past_key_values": None, "x": 1})
+    k2, v2 = kwargs["past_key_values"].update(k, v, 0)
+    assert k2 is k and v2 is v and seen == [("k", k.shape), ("v", v.shape)] and kwargs["x"] == 1
+    wrapped = _ObservedKVCache(attn, Real())
+    k3, v3 = wrapped.update(k, v, 0, cache_kwargs={})
+    assert torch.equal(k3, k + 1) and torch.equal(v3, v + 1) and wrapped.marker == 7 and len(seen) == 4
+    _, kwargs = _kv_cache_pre_hook(attn, (), {})
+    assert isinstance(kwargs["past_key_values"], _ObservedKVCache)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_lerp_equals_the_eager_expression_on_cpu(dtype):
+    """The step-by-step lerp of the activation observers equals ``start * (1 - w) + end * w`` as eager CPU ops
+    evaluate it (reference: observers/helpers.py:218-220)."""
+    from llmcompressor_amd.observers.helpers import lerp
+
+    torch.manual_seed(0)
+    a, b = (torch.randn(50000) * 3).to(dtype), (torch.randn(50000) * 3).to(dtype)
+    for w in (0.01, 0.1, 0.5):
+        assert torch.equal(lerp(a, b, w), (a * (1.0 - w)) + (b * w))
+
+
+def test_checkpoint_unpacking_helpers_match_the_oracle_pack():
+    """_unpack_int32 inverts the oracle's pack_to_int32 for 2 to 8 bit fields and ragged widths; _expand_qparam lays
+    scales out per strategy."""
+    from oracle import pack as P
+
+    from llmcompressor_amd.compressors import _expand_qparam, _unpack_int32
+    from llmcompressor_amd.quantization import QuantizationArgs
+
+    torch.manual_seed(0)
+    for bits in (2, 3, 4, 8):
+        for K in (1, 7, 32, 45):
+            lo, hi = -(1 << (bits - 1)), (1 << (bits - 1)) - 1
+            codes = torch.randint(lo, hi + 1, (5, K), dtype=torch.int8)
+            packed = P.pack_to_int32(codes, bits)
+            assert torch.equal(_unpack_int32(packed, bits, K).to(torch.int8), codes)
+    s = torch.arange(6, dtype=torch.float32).reshape(2, 3)
+    g = _expand_qparam(s, QuantizationArgs(num_bits=4, strategy="group", group_size=2), 2, 6)
+    assert g.tolist() == [[0, 0, 1, 1, 2, 2], [3, 3, 4, 4, 5, 5]]
+    b = _expand_qparam(s, QuantizationArgs(num_bits=4, strategy="block", block_structure=[2, 2]), 3, 5)
+    assert b.shape == (3, 5) and b[2].tolist() == [3, 3, 4, 4, 5] and b[0].tolist() == [0, 0, 1, 1, 2]
+    c = _expand_qparam(torch.tensor([[2.0], [3.0]]), QuantizationArgs(num_bits=8, strategy="channel"), 2, 4)
+    assert c.shape == (2, 1)
+    t = _expand_qparam(torch.tensor([5.0]), QuantizationArgs(num_bits=8, strategy="tensor"), 2, 4)
+    assert t.shape == (1, 1)
+    perm = torch.tensor([2, 0, 1, 1, 0, 2])
+    gi = _expand_qparam(s, QuantizationArgs(num_bits=4, strategy="group", group_size=2), 2, 6, g_idx=perm)
+    assert gi[0].tolist() == [2, 0, 1, 1, 0, 2]
