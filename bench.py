@@ -216,7 +216,7 @@ def probe_sparsegpt():
           f"{(time.perf_counter() - t0) * 1e3:.0f} ms")
 
 
-def probe_moe():
+def probe_moe(mode="both"):
     """One MoE expert layer (128 experts, hidden 2048, intermediate 768, top-8 routing of 4096 tokens: 384 expert
     Linears) through GPTQModifier W4A16: time of the calibration forward (grouped Hessian launches from the hooks)
     and of the quantisation of the 384 Linears, with lock-step groups and with the per-module path.  Prints a table."""
@@ -249,7 +249,10 @@ def probe_moe():
     w, idx = torch.topk(torch.softmax(logits, -1), TOPK, -1)
     print("| quantisation of the 384 expert Linears | forward + Hessians ms per batch | quantise ms | ms per Linear |")
     print("|---|---|---|---|")
-    for label, gmin in (("lock-step groups (default)", 8), ("one module at a time, 4 streams", 0)):
+    variants = (("lock-step groups (default)", 8, "lockstep"), ("one module at a time, 4 streams", 0, "permodule"))
+    for label, gmin, key in variants:
+        if mode not in ("both", key):
+            continue
         best = None
         for _ in range(3):
             for p in model.parameters():
@@ -345,6 +348,8 @@ def main():
                     help="print achieved GB/s of the observer / quantize / pack kernels instead of the bench line")
     ap.add_argument("--probe-sparsegpt", action="store_true",
                     help="print SparseGPT timings per Linear shape instead of the bench line")
+    ap.add_argument("--moe-mode", choices=("both", "lockstep", "permodule"), default="both",
+                    help="which quantisation path --probe-moe runs (one path alone gives a clean kernel profile)")
     ap.add_argument("--probe-oneshot", action="store_true",
                     help="print end-to-end oneshot timings on a transformers Llama with two 8B-shaped layers "
                     "(--batches x --tokens calibration tokens) instead of the bench line")
@@ -371,7 +376,7 @@ def main():
         probe_sparsegpt()
         return
     if a.probe_moe:
-        probe_moe()
+        probe_moe(a.moe_mode)
         return
     if a.probe_oneshot:
         probe_oneshot(a.batches, a.tokens)
