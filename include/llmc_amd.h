@@ -157,6 +157,17 @@ int llmc_mse_observe_blocks(const void* x, int32_t dtype, int64_t R, int64_t K, 
 int64_t llmc_sumsq_workspace_bytes(int64_t K);
 int llmc_sumsq_accumulate(const void* x, int32_t dtype, int64_t T, int64_t K, int64_t ldx, float* sum,
                           void* workspace, int64_t workspace_bytes, void* stream);
+/* llmc_sumsq_accumulate for callers that cannot allocate (code under HIP graph capture, tight loops,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same result as
+ * llmc_sumsq_accumulate bit for bit, but the partial sums go to a 4 MiB device array that the library
+ * itself holds on every GPU it runs on (until the process ends) instead of a caller's workspace, and the
+ * call allocates and frees nothing.  K above LLMC_SUMSQ_NOALLOC_MAX_K is rejected (-4).  The first call
+ * on a device looks up that device's copy of the array (make it before a capture begins).  All calls on
+ * one GPU share the array: calls that overlap in time on one GPU (two streams, two threads) race; calls
+ * on one stream, or ordered by events, do not. */
+#define LLMC_SUMSQ_NOALLOC_MAX_K 16384
+int llmc_sumsq_accumulate_noalloc(const void* x, int32_t dtype, int64_t T, int64_t K, int64_t ldx, float* sum,
+                                  void* stream);
 int llmc_imatrix_observe_groups(const void* x, int32_t dtype, int64_t R, int64_t K, int64_t ldw,
                                 int64_t group, int32_t fmt, int32_t num_bits, int32_t symmetric,
                                 int32_t scale_mode, int32_t steps, double grid, int32_t patience,

@@ -11,6 +11,8 @@
 // weight is read from HBM once.
 #include <string.h>
 
+#include <mutex>
+
 #include "qformat.h"
 
 namespace {
@@ -759,6 +761,24 @@ __global__ __launch_bounds__(256) void sumsq_partial16_kernel(const uint16_t* __
 
 extern "C" int64_t llmc_sumsq_workspace_bytes(int64_t K) { return align256(K * SUMSQ_SLICES * 4); }
 
+// both entry points: partial sums of the token slices into `partial` ([slices, K] fp32), then sum += their total
+static int sumsq_launch(const void* x, int32_t dtype, int64_t T, int64_t K, int64_t ldx, float* sum, float* partial,
+                        hipStream_t st) {
+  const int slices = T < SUMSQ_SLICES ? (int)T : SUMSQ_SLICES;
+  const bool wide = dtype != LLMC_F32 && K % 8 == 0 && ldx % 8 == 0 && (((uintptr_t)x) & 15) == 0;
+  if (wide)
+    hipLaunchKernelGGL(sumsq_partial16_kernel, dim3((unsigned)((K + 255) / 256), (unsigned)slices), dim3(256), 0, st,
+                       (const uint16_t*)x, dtype, T, K, ldx, slices, partial);
+  else
+    hipLaunchKernelGGL(sumsq_partial_kernel, dim3((unsigned)((K + 255) / 256), (unsigned)slices), dim3(256), 0, st, x,
+                       dtype, T, K, ldx, slices, partial);
+  LLMC_LAUNCH_STATUS();
+  hipLaunchKernelGGL(sumsq_finish_kernel, dim3((unsigned)((K + 255) / 256)), dim3(256), 0, st,
+                     (const float*)partial, K, slices, sum);
+  LLMC_LAUNCH_STATUS();
+  return 0;
+}
+
 extern "C" int llmc_sumsq_accumulate(const void* x, int32_t dtype, int64_t T, int64_t K, int64_t ldx, float* sum,
                                      void* workspace, int64_t workspace_bytes, void* stream) {
   LLMC_CHECK_ARG(dtype >= 0 && dtype <= 2, 2);
@@ -766,20 +786,55 @@ extern "C" int llmc_sumsq_accumulate(const void* x, int32_t dtype, int64_t T, in
   if (T == 0) return 0;
   LLMC_CHECK_ARG(x != nullptr && sum != nullptr, 1);
   LLMC_CHECK_ARG(workspace && (((uintptr_t)workspace) & 255) == 0 && workspace_bytes >= llmc_sumsq_workspace_bytes(K), 7);
-  hipStream_t st = (hipStream_t)stream;
-  const int slices = T < SUMSQ_SLICES ? (int)T : SUMSQ_SLICES;
-  const bool wide = dtype != LLMC_F32 && K % 8 == 0 && ldx % 8 == 0 && (((uintptr_t)x) & 15) == 0;
-  if (wide)
-    hipLaunchKernelGGL(sumsq_partial16_kernel, dim3((unsigned)((K + 255) / 256), (unsigned)slices), dim3(256), 0, st,
-                       (const uint16_t*)x, dtype, T, K, ldx, slices, (float*)workspace);
-  else
-    hipLaunchKernelGGL(sumsq_partial_kernel, dim3((unsigned)((K + 255) / 256), (unsigned)slices), dim3(256), 0, st, x,
-                       dtype, T, K, ldx, slices, (float*)workspace);
-  LLMC_LAUNCH_STATUS();
-  hipLaunchKernelGGL(sumsq_finish_kernel, dim3((unsigned)((K + 255) / 256)), dim3(256), 0, st,
-                     (const float*)workspace, K, slices, sum);
-  LLMC_LAUNCH_STATUS();
+  return sumsq_launch(x, dtype, T, K, ldx, sum, (float*)workspace, (hipStream_t)stream);
+}
+
+// ---- the same accumulation for callers that cannot allocate ---------------------------------------
+// The partial sums live in a device array of this library instead of a caller's workspace.  Every GPU
+// that loads the library holds its own copy of the array (4 MiB) at its own address until the process
+// ends; host code never uses the array's name as an address, only the pointer hipGetSymbolAddress
+// returned for the device that is current.
+constexpr int64_t SUMSQ_NOALLOC_MAX_K = LLMC_SUMSQ_NOALLOC_MAX_K;
+static __device__ __align__(256) float scratch[SUMSQ_SLICES * SUMSQ_NOALLOC_MAX_K];
+
+namespace {
+constexpr int NOALLOC_MAX_DEVICES = 64;
+std::mutex g_scratch_mutex;
+float* g_scratch_ptr[NOALLOC_MAX_DEVICES] = {};
+
+// the address of `scratch` on the current device, looked up once per device
+int scratch_for_current_device(float** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return 1000 + (int)e;
+  if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) return 2000;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return 1000 + (int)e;
+    if (!p) return 2001;
+    g_scratch_ptr[dev] = (float*)p;
+  }
+  *out = g_scratch_ptr[dev];
   return 0;
+}
+}  // namespace
+
+extern "C" int llmc_sumsq_accumulate_noalloc(const void* x, int32_t dtype, int64_t T, int64_t K, int64_t ldx,
+                                             float* sum, void* stream) {
+  LLMC_CHECK_ARG(dtype >= 0 && dtype <= 2, 2);
+  LLMC_CHECK_ARG(T >= 0 && ldx >= K, 3);
+  // widths beyond the array's capacity are refused, never truncated
+  LLMC_CHECK_ARG(K > 0 && K <= SUMSQ_NOALLOC_MAX_K, 4);
+  if (T == 0) return 0;
+  LLMC_CHECK_ARG(x != nullptr && sum != nullptr, 1);
+  float* partial = nullptr;
+  const int rc = scratch_for_current_device(&partial);
+  if (rc) return rc;
+  // every partial row that the finishing kernel reads is written by this call's first kernel, so the
+  // contents that an earlier (possibly wider or longer) call left behind need no clearing
+  return sumsq_launch(x, dtype, T, K, ldx, sum, partial, (hipStream_t)stream);
 }
 
 extern "C" int llmc_imatrix_observe_groups(const void* x, int32_t dtype, int64_t R, int64_t K, int64_t ldw,

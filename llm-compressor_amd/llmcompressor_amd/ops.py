@@ -512,6 +512,27 @@ def sumsq_accumulate_(total: torch.Tensor, x: torch.Tensor):
     return total
 
 
+SUMSQ_NOALLOC_MAX_K = 16384  # LLMC_SUMSQ_NOALLOC_MAX_K
+
+
+def sumsq_accumulate_noalloc_(total: torch.Tensor, x: torch.Tensor):
+    """sumsq_accumulate_ without any allocation: the partial sums use a device array inside the library.
+    x must already be [T, K] with unit column stride and K <= SUMSQ_NOALLOC_MAX_K; calls on one GPU must not
+    overlap in time."""
+    _require_gpu(total, x)
+    assert total.dtype == torch.float32 and total.ndim == 1 and x.ndim == 2 and x.shape[1] == total.shape[0]
+    if x.stride(1) != 1:
+        raise ValueError("sumsq_accumulate_noalloc_: x needs unit column stride (making it contiguous would allocate)")
+    if x.shape[1] > SUMSQ_NOALLOC_MAX_K:
+        raise ValueError(f"sumsq_accumulate_noalloc_: K={x.shape[1]} exceeds the library's device array "
+                         f"(K <= {SUMSQ_NOALLOC_MAX_K}); use sumsq_accumulate_ with a workspace")
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().llmc_sumsq_accumulate_noalloc(x.data_ptr(), _dt(x), x.shape[0], x.shape[1], x.stride(0),
+                                                      total.data_ptr(), _stream(x))
+    _lib.check(rc, "llmc_sumsq_accumulate_noalloc")
+    return total
+
+
 def imatrix_observe_groups(w, group: int, fmt: int, bits: int, symmetric: bool, scale_mode: int = SCALE_PLAIN,
                            importance=None, maxshrink=0.95, patience=5, grid=20, norm=3.0, expand=1.0):
     """Importance-weighted grid search per run of `group` columns of w [R,K] -> (min, max) [R, K/group]."""
