@@ -423,9 +423,10 @@ extern "C" int llmc_gptq_hinv_grouped(const float* const* H, int64_t ldh, int32_
     host[b].div = divisors[b];
     host[b].pad = 0;
   }
-  // pageable source: the copy has read `host` when the call returns
-  hipError_t me = hipMemcpyAsync(items, host.data(), n * sizeof(HinvItem), hipMemcpyHostToDevice, st);
-  if (me != hipSuccess) return 1000 + (int)me;
+  {
+    const int urc = upload_items(host.data(), n, (HinvItem*)items, st);
+    if (urc) return urc;
+  }
 
   hipLaunchKernelGGL(hinv_stats_kernel, dim3(n), dim3(256), 0, st, (const float*)nullptr, ldh, (int)K,
                      (const int32_t*)nullptr, 1.f, percdamp, (uint8_t*)nullptr, sc, (const HinvItem*)items);

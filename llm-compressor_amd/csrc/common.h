@@ -95,3 +95,30 @@ __device__ __forceinline__ float wave_sum(float v) {
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
   return v;
 }
+
+// Host tables of per-problem pointers reach the device as kernel arguments (copied when the launch is
+// enqueued), 32 entries per launch: the host array may be released as soon as the call returns, nothing
+// depends on how the runtime stages copies from pageable memory, and the upload is an ordinary kernel
+// node for a caller that captures the stream.
+template <typename T>
+struct ItemChunk {
+  T v[32];
+};
+template <typename T>
+__global__ void upload_items_kernel(ItemChunk<T> c, int count, T* __restrict__ dst) {
+  const int i = threadIdx.x;
+  if (i < count) dst[i] = c.v[i];
+}
+template <typename T>
+inline int upload_items(const T* host, int n, T* dev, hipStream_t st) {
+  static_assert(sizeof(ItemChunk<T>) <= 3072, "chunk must fit the kernel argument buffer");
+  for (int at = 0; at < n; at += 32) {
+    ItemChunk<T> c = {};
+    const int count = n - at < 32 ? n - at : 32;
+    for (int i = 0; i < count; ++i) c.v[i] = host[at + i];
+    hipLaunchKernelGGL((upload_items_kernel<T>), dim3(1), dim3(32), 0, st, c, count, dev + at);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return 1000 + (int)e;
+  }
+  return 0;
+}

@@ -750,8 +750,10 @@ extern "C" int llmc_gptq_quantize_grouped(const void* const* weight, int32_t w_d
     host[b].g_idx = g_idx ? g_idx[b] : nullptr;
     host[b].out = out_weight[b];
   }
-  hipError_t me = hipMemcpyAsync(items, host.data(), n * sizeof(GptqItem), hipMemcpyHostToDevice, st);
-  if (me != hipSuccess) return 1000 + (int)me;
+  {
+    const int urc = upload_items(host.data(), n, (GptqItem*)items, st);
+    if (urc) return urc;
+  }
 
   dim3 grid3((unsigned)((K + 255) / 256), (unsigned)R, (unsigned)n);
 #define LLMC_PREP(DT)                                                                                         \
