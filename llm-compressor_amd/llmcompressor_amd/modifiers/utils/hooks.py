@@ -15,6 +15,7 @@ __all__ = ["HooksMixin"]
 class HooksMixin(BaseModel):
     _HOOKS_DISABLED: ClassVar[bool] = False
     _HOOKS_KEEP_ENABLED: ClassVar[set] = set()
+    _ALL_HANDLES: ClassVar[set] = set()  # every live handle of every modifier (for `keep` by module)
 
     _hooks: set = PrivateAttr(default_factory=set)
 
@@ -44,6 +45,7 @@ class HooksMixin(BaseModel):
         register = getattr(target, name)
         handle = register(wrapped_hook, **kwargs)
         self._hooks.add(handle)
+        HooksMixin._ALL_HANDLES.add(handle)
         return handle
 
     def remove_hooks(self, handles: set | None = None):
@@ -51,4 +53,5 @@ class HooksMixin(BaseModel):
             handles = self._hooks
         for h in list(handles):
             h.remove()
+        HooksMixin._ALL_HANDLES.difference_update(handles)
         self._hooks -= set(handles)

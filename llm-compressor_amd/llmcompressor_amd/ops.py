@@ -154,7 +154,14 @@ _ws_cache = {}
 
 
 def _workspace(device, nbytes: int) -> torch.Tensor:
-    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    """Scratch memory for one C call, cached per (device, stream, host thread).
+
+    Several entry points issue more than one launch over their workspace, and ctypes releases the GIL during
+    a call, so two host threads on one stream could interleave their launches: each thread therefore owns its
+    buffer (work of one thread on one stream is ordered by the stream)."""
+    import threading
+
+    key = (device, torch.cuda.current_stream(device).cuda_stream, threading.get_ident())
     ws = _ws_cache.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(max(nbytes, 1 << 16), dtype=torch.uint8, device=device)

@@ -134,6 +134,10 @@ class SequentialPipeline(CalibrationPipeline):
                 captured.append((args, kwargs))
                 raise _StopForward()
 
+            inside = {id(x) for l in layers for x in l.modules()}
+            rest = [m for m in model.modules() if id(m) not in inside]
+            before = set()  # modules that run ahead of the first layer (their hooks fire in this capture pass)
+            trackers = [m.register_forward_pre_hook(lambda mod, args: before.add(id(mod))) for m in rest]
             handle = layers[0].register_forward_pre_hook(grab, with_kwargs=True)
             try:
                 for batch in dataloader:
@@ -142,14 +146,20 @@ class SequentialPipeline(CalibrationPipeline):
                         model(**batch) if isinstance(batch, dict) else model(batch)
                     except _StopForward:
                         pass
+                    for t in trackers:
+                        t.remove()
+                    trackers = []
             finally:
                 handle.remove()
+                for t in trackers:
+                    t.remove()
             # the activations between layers live in a device-resident cache (no CPU offload)
             offload = getattr(dataset_args, "sequential_offload_device", None) if dataset_args is not None else None
             cache = IntermediatesCache.empty(len(captured), offload_device=offload)
             for i, (args, kwargs) in enumerate(captured):
                 cache.update(i, {"args": tuple(args), "kwargs": dict(kwargs)})
             del captured
+            returns_tuple = False
             for idx, layer in enumerate(layers):
                 # pass 1: calibrate (hooks fire: Hessians / activation observers)
                 for inputs in cache.iter_prefetch():
@@ -160,12 +170,67 @@ class SequentialPipeline(CalibrationPipeline):
                     for i in range(len(cache)):
                         inputs = cache.fetch(i)
                         out = layer(*inputs["args"], **inputs["kwargs"])
-                        hidden = out[0] if isinstance(out, (tuple, list)) else out
+                        returns_tuple = isinstance(out, (tuple, list))
+                        hidden = out[0] if returns_tuple else out
                         cache.update(i, {"args": (hidden,) + tuple(inputs["args"][1:])})
-            # modules outside the layer list (e.g. lm_head) that modifiers may target
-            rest = [m for m in model.modules() if not any(m is x for l in layers for x in l.modules())]
+            # what follows the last layer (final norm, lm_head): the reference's last traced subgraph holds it
+            # (pipelines/sequential/pipeline.py:136-181), so a module there that a modifier hooked is calibrated too
+            tail = [m for m in rest if id(m) not in before and _has_calibration_hooks(m)]
+            if tail:
+                _calibrate_tail(model, layers, tail, dataloader, cache, device, returns_tuple)
             LifecycleCallbacks.sequential_epoch_end(modules=rest)
         LifecycleCallbacks.calibration_end()
+
+
+def _has_calibration_hooks(module: torch.nn.Module) -> bool:
+    """Did a modifier register a forward (pre-)hook on this very module?"""
+    return bool(module._forward_hooks) or bool(module._forward_pre_hooks)
+
+
+def _calibrate_tail(model, layers, tail, dataloader, cache, device, returns_tuple: bool) -> None:
+    """Run what follows the last sequential layer on every cached hidden state, with the hooks of `tail` on.
+
+    The model is called on the original batches while every sequential layer is short-circuited: the last one
+    returns the cached output of the propagation pass, the others hand their input through.  What precedes
+    the layers (embeddings, rotary tables) is recomputed, which is cheap; its hooks fired in the capture pass
+    already, so only the handles registered on the `tail` modules are kept enabled."""
+    keep = set()
+    for m in tail:
+        keep.update(_handles_of(m))
+    current = {}
+
+    def hand_through(*args, **kwargs):
+        hidden_states = args[0] if args else kwargs["hidden_states"]
+        return (hidden_states,) if returns_tuple else hidden_states
+
+    def cached_output(*args, **kwargs):
+        return (current["hidden"],) if returns_tuple else current["hidden"]
+
+    patched = []
+    try:
+        for layer in layers[:-1]:
+            layer.forward = hand_through
+            patched.append(layer)
+        layers[-1].forward = cached_output
+        patched.append(layers[-1])
+        with HooksMixin.disable_hooks(keep=keep):
+            for i, batch in enumerate(dataloader):
+                if i >= len(cache):
+                    break
+                current["hidden"] = cache.fetch(i)["args"][0]
+                batch = _to_device(batch, device)
+                model(**batch) if isinstance(batch, dict) else model(batch)
+    finally:
+        for layer in patched:
+            del layer.forward  # back to the class's method
+
+
+def _handles_of(module: torch.nn.Module):
+    """The RemovableHandle objects of the hooks registered on `module`, as HooksMixin keeps them."""
+    from torch.utils.hooks import RemovableHandle
+
+    ids = set(module._forward_hooks) | set(module._forward_pre_hooks)
+    return {h for h in HooksMixin._ALL_HANDLES if isinstance(h, RemovableHandle) and h.id in ids}
 
 
 @CalibrationPipeline.register("datafree")

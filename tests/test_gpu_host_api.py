@@ -242,9 +242,6 @@ def test_oneshot_gptq_sequential_matches_oracle_layer0(tmp_path, staging):
     model = _tiny().to(DEV)
     torch.manual_seed(1)
     data = [torch.randint(0, 100, (1, 48)) for _ in range(12)]
-    recipe = GPTQModifier(targets="Linear", scheme={"W4A16": ["Linear"]}, ignore=["lm_head"], actorder="static",
-                          hessian_batch_tokens=staging,
-                          config_groups=None)
     recipe = GPTQModifier(targets="Linear", ignore=["lm_head"], hessian_batch_tokens=staging, config_groups={
         "g": dict(targets=["Linear"], weights=dict(num_bits=4, strategy="group", group_size=32))})
     out_dir = str(tmp_path / "out")
@@ -286,6 +283,47 @@ def test_oneshot_gptq_sequential_matches_oracle_layer0(tmp_path, staging):
     deq = decompress_weight({k[len(key):]: v for k, v in sd.items() if k.startswith(key)},
                             QuantizationArgs(num_bits=4, strategy="group", group_size=32), "pack-quantized")
     assert torch.equal(deq, got)
+
+
+def test_oneshot_gptq_calibrates_a_targeted_lm_head():
+    """A Linear after the last decoder layer (lm_head not ignored) gets its Hessian from the hidden states that
+    leave the last compressed layer, like the reference's last subgraph: its weight is the oracle's GPTQ
+    result on that Hessian, not a round-to-nearest one, and the embedding's hooks do not fire twice."""
+    from llmcompressor_amd import oneshot
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+
+    ref = _tiny()
+    model = _tiny().to(DEV)
+    torch.manual_seed(2)
+    data = [torch.randint(0, 100, (1, 40)) for _ in range(10)]
+    recipe = GPTQModifier(targets="Linear", actorder=None, config_groups={
+        "g": dict(targets=["Linear"], weights=dict(num_bits=4, strategy="group", group_size=32))})
+    oneshot(model=model, recipe=recipe, dataset=[{"input_ids": d} for d in data])
+    assert hasattr(model.lm_head, "weight_scale")
+    with torch.no_grad():
+        xs = []
+        for d in data:
+            h = model.embed(d.to(DEV))
+            for layer in model.layers:
+                h = layer(h)
+            xs.append(h.cpu())
+    H, n = G.make_empty_hessian(64), torch.zeros(())
+    for x in xs:
+        H, n = G.accumulate_hessian(x, H, n)
+    oargs = F.QArgs(num_bits=4, strategy="group", group_size=32)
+    w0 = ref.lm_head.weight.data
+    oobs = O.Observer("memoryless_minmax", "weight", oargs)
+    oobs(w0)
+    _, exp, info = G.quantize_weight(w0, oobs, oargs, H / n)
+    assert info["ok"]
+    got = model.lm_head.weight.data.cpu()
+    assert (got == exp["weight"]).float().mean().item() >= 0.999
+    oobs2 = O.Observer("memoryless_minmax", "weight", oargs)
+    oobs2(w0)
+    rtn = F.fake_quantize(w0, *F.calculate_qparams(oobs2.min_vals, oobs2.max_vals, oargs), oargs)
+    assert (got == rtn).float().mean().item() < 0.99  # error feedback moved some weights off the RTN choice
+    # the layers are back on their own forward
+    assert all("forward" not in vars(layer) for layer in model.layers)
 
 
 @pytest.mark.parametrize("scheme,fmt", [("FP8_DYNAMIC", "float-quantized"), ("NVFP4A16", "nvfp4-pack-quantized"),
@@ -525,6 +563,59 @@ def test_model_free_ptq_rejects_indivisible_groups(tmp_path):
     with pytest.raises(ValueError, match="Unable to quantize tensor"):
         model_free_ptq(src, str(tmp_path / "dst"), scheme="W4A16", ignore=["model.embed_tokens", "lm_head"],
                        device="cuda:0")
+
+
+def test_model_free_ptq_worker_threads_do_not_share_scratch(tmp_path):
+    """max_workers > 1: shards are quantised by several host threads on one stream.  Per-tensor statistics of
+    large weights go through a two-launch reduction over scratch memory, which every thread must own: the
+    checkpoint written by three workers is byte-identical to the one written by a single worker."""
+    import json
+    import os
+
+    from safetensors import safe_open
+    from safetensors.torch import save_file
+
+    from llmcompressor_amd import model_free_ptq
+    from llmcompressor_amd.quantization import QuantizationArgs, QuantizationScheme
+
+    src = str(tmp_path / "src")
+    os.makedirs(src)
+    g = torch.Generator().manual_seed(5)
+    wm = {}
+    for shard in range(6):
+        fn = f"model-{shard + 1:05d}-of-00006.safetensors"
+        tensors = {}
+        for j in range(4):
+            name = f"model.layers.{shard}.mlp.proj{j}.weight"
+            # a different magnitude per tensor, so that a borrowed partial result changes the scale
+            tensors[name] = (torch.randn(256, 512, generator=g) * 0.01 * (1 + shard * 4 + j)).bfloat16()
+            wm[name] = fn
+        save_file(tensors, os.path.join(src, fn))
+    json.dump({"metadata": {}, "weight_map": wm}, open(os.path.join(src, "model.safetensors.index.json"), "w"))
+    json.dump({"model_type": "toy"}, open(os.path.join(src, "config.json"), "w"))
+    sch = QuantizationScheme(targets=["Linear"], weights=QuantizationArgs(num_bits=8, strategy="tensor"))
+    outs = []
+    for workers in (1, 3):
+        dst = str(tmp_path / f"dst{workers}")
+        _, wmap = model_free_ptq(src, dst, scheme=sch, max_workers=workers, device="cuda:0")
+        got = {}
+        for fn in sorted(set(wmap.values())):
+            with safe_open(f"{dst}/{fn}", framework="pt") as f:
+                for k in f.keys():
+                    got[k] = f.get_tensor(k)
+        outs.append(got)
+    assert set(outs[0]) == set(outs[1]) and len(outs[0]) >= 48
+    for k in outs[0]:
+        assert torch.equal(outs[0][k].view(torch.uint8), outs[1][k].view(torch.uint8)), k
+    for name in wm:  # and the single-worker scales are the per-tensor absmax / 127.5 of the source
+        base = name[: -len(".weight")]
+        w = None
+        with safe_open(os.path.join(src, wm[name]), framework="pt") as f:
+            w = f.get_tensor(name)
+        args = F.QArgs(num_bits=8, strategy="tensor")
+        obs = O.Observer("memoryless_minmax", "weight", args)
+        obs(w)
+        assert torch.equal(outs[1][base + ".weight_scale"].reshape(-1), obs.get_qparams()["scale"].reshape(-1)), name
 
 
 def test_gptq_shared_input_hessians_are_identical():
