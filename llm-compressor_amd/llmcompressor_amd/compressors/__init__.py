@@ -19,6 +19,7 @@ import math
 import torch
 
 from .. import ops
+from ..torch_ops import llmc
 from ..quantization import (
     QuantizationArgs,
     QuantizationConfig,
@@ -73,8 +74,7 @@ def _run(weight, scale, zp, args: QuantizationArgs, mode, g_idx=None, global_sca
     zpa = None if args.symmetric or zp is None else zp.to(torch.int8)
     if g_idx is not None and bool((g_idx < 0).any()):
         g_idx = None
-    return ops.quantize(weight.contiguous(), es, zpa, fmt, bits, row_div, srow, col_div, out_mode=mode, g_idx=g_idx,
-                        global_scale=global_scale)
+    return llmc.quant_pack(weight.contiguous(), es, zpa, fmt, bits, row_div, srow, col_div, mode, g_idx, global_scale)
 
 
 def compress_module(module: torch.nn.Module, fmt: Optional[str] = None) -> Dict[str, torch.Tensor]:

@@ -13,7 +13,8 @@ import logging
 import torch
 from pydantic import PrivateAttr
 
-from ... import ops
+from ... import ops  # noqa: F401
+from ...torch_ops import llmc
 from ...core import Event, State
 from ...observers import ACTIVATION_OBS
 from ...quantization import (
@@ -231,8 +232,7 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
             x = inp.reshape(-1, inp.shape[-1])
             by_width.setdefault((x.shape[1], x.dtype), []).append((self._hessians[module], x))
         for group in by_width.values():
-            ops.hessian_accumulate_grouped_([h for h, _ in group], [x for _, x in group], alpha=2.0,
-                                            assume_symmetric=True)
+            llmc.hessian_accum_grouped_([h for h, _ in group], [x for _, x in group], 2.0, True)
 
     def compress_modules(self):
         self.compress_module_list(list(self._num_samples.keys()))

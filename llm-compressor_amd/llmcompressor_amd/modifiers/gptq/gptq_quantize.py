@@ -13,7 +13,8 @@ import math
 
 import torch
 
-from ... import ops
+from ... import ops  # noqa: F401  (format constants)
+from ...torch_ops import llmc
 from ...quantization import ActivationOrdering, QuantizationArgs, QuantizationStrategy
 from ...quantization.lifecycle import effective_scale, kernel_format
 
@@ -49,7 +50,7 @@ def accumulate_hessian(inp: torch.Tensor, module: torch.nn.Module, H: torch.Tens
         inp = inp.reshape((-1, inp.shape[-1]))
     num_samples += num_added
     if inp.shape[0] > 0:
-        ops.hessian_accumulate_(H, inp.contiguous(), alpha=2.0, assume_symmetric=True)
+        llmc.hessian_accum_(H, inp.contiguous(), 2.0, True)
     return H, num_samples
 
 
@@ -90,7 +91,9 @@ def quantize_weight_tensors(weight: torch.Tensor, observer, quant_args: Quantiza
 
     perm = None
     if actorder:
-        perm = torch.argsort(torch.diagonal(H), descending=True)
+        # stable: equal diagonal entries keep their column order, so that the column order (and with it the
+        # result) is reproducible; torch leaves the order of ties unspecified otherwise
+        perm = torch.argsort(torch.diagonal(H), descending=True, stable=True)
     if actorder == ActivationOrdering.GROUP:
         # re-observe the permuted weight so that groups are runs of the permuted columns.  The reference observes
         # its fp32 work copy here (gptq_quantize.py:88,111-114), so these statistics and the scales the column
@@ -109,13 +112,14 @@ def quantize_weight_tensors(weight: torch.Tensor, observer, quant_args: Quantiza
     scale, zero_point, global_scale = qparams["scale"], qparams["zero_point"], qparams["global_scale"]
 
     # dead columns, damping, Cholesky -> inverse -> upper factor; identity on failure
-    U, dead, info = ops.gptq_hinv_(H, perm, divisor=float(hessian_divisor), percdamp=percdamp)
+    dead, info = llmc.gptq_prepare_hinv_(H, perm, float(hessian_divisor), float(percdamp))
+    U = H  # overwritten in place by the upper factor
 
     fmt, bits = kernel_format(quant_args)
     zp = None if quant_args.symmetric else zero_point.to(torch.int8)
     kscale = effective_scale(scale, quant_args, final_dtype)
-    Wq, loss = ops.gptq_quantize(W2, U, kscale, zp, fmt, bits, row_div, srow, g_idx=g_idx, perm=perm, dead=dead,
-                                 global_scale=global_scale, blocksize=blocksize)
+    Wq, loss = llmc.gptq_quantize(W2, U, kscale, zp, fmt, bits, row_div, srow, g_idx=g_idx, perm=perm, dead=dead,
+                                  global_scale=global_scale, blocksize=blocksize)
     if int(info.item()) != 0:
         logger.warning("Failed to invert hessian due to numerical instability. Consider increasing "
                        "GPTQModifier.dampening_frac, increasing the number of calibration samples, or shuffling "
@@ -191,7 +195,7 @@ def quantize_weight_group(modules, hessians, hessian_divisors, blocksize: int = 
         strategy, actorder = quant_args.strategy, quant_args.actorder
         W = m.weight.data if m.weight.data.is_contiguous() else m.weight.data.contiguous()
         num_rows, num_columns = W.shape
-        perm = torch.argsort(torch.diagonal(H), descending=True) if actorder else None
+        perm = torch.argsort(torch.diagonal(H), descending=True, stable=True) if actorder else None
         row_div, srow, divisor = _scale_layout(strategy, quant_args, num_rows, num_columns)
         g_idx = None
         if divisor is not None:
@@ -204,7 +208,7 @@ def quantize_weight_group(modules, hessians, hessian_divisors, blocksize: int = 
                          kscale=effective_scale(qp["scale"], quant_args, W.dtype)))
     perms = torch.stack([p["perm"] for p in prep]) if prep[0]["perm"] is not None else None
 
-    U, dead, info = ops.gptq_hinv_grouped(Hs, perms, divs, percdamp)
+    U, dead, info = llmc.gptq_prepare_hinv_grouped(Hs, perms, [float(d) for d in divs], float(percdamp))
 
     outs, losses = [None] * n, [None] * n
     at = 0
@@ -216,13 +220,13 @@ def quantize_weight_group(modules, hessians, hessian_divisors, blocksize: int = 
         first = part[0]
         fmt, bits = kernel_format(first["args"])
         if end - at == 1:
-            outs[at], losses[at] = ops.gptq_quantize(
+            outs[at], losses[at] = llmc.gptq_quantize(
                 first["W"], U[at], first["kscale"], first["zp"], fmt, bits, first["row_div"], first["srow"],
                 g_idx=first["g_idx"], perm=first["perm"], dead=dead[at], global_scale=first["qp"]["global_scale"],
                 blocksize=blocksize)
         else:
             has_gs = first["qp"]["global_scale"] is not None
-            o, l = ops.gptq_quantize_grouped(
+            o, l = llmc.gptq_quantize_grouped(
                 [p["W"] for p in part], U[at:end], [p["kscale"] for p in part],
                 None if first["zp"] is None else [p["zp"] for p in part], fmt, bits, first["row_div"], first["srow"],
                 g_idxs=None if first["g_idx"] is None else [p["g_idx"] for p in part],

@@ -13,6 +13,7 @@ from __future__ import annotations
 import torch
 
 from ... import ops
+from ...torch_ops import llmc
 
 __all__ = ["HessianStagingMixin"]
 
@@ -73,14 +74,14 @@ class HessianStagingMixin:
                     raise RuntimeError(
                         "an activation that was held for Hessian accumulation was modified in place "
                         "after the forward hook saw it; set stage_by_reference=False for this model")
-            ops.hessian_accumulate_segments_(self._hessians[module], held[0], alpha=2.0, assume_symmetric=True)
+            llmc.hessian_accum_segments_(self._hessians[module], held[0], 2.0, True)
             self._num_samples[module] += held[2]
             self._held_bytes = getattr(self, "_held_bytes", 0) - sum(x.numel() * x.element_size() for x in held[0])
             self._held[module] = [[], [], 0]
         st = self._staged.get(module)
         if st is None or st[1] == 0:
             return
-        ops.hessian_accumulate_(self._hessians[module], st[0].narrow(0, 0, st[1]), alpha=2.0, assume_symmetric=True)
+        llmc.hessian_accum_(self._hessians[module], st[0].narrow(0, 0, st[1]), 2.0, True)
         self._num_samples[module] += st[2]
         st[1] = 0
         st[2] = 0

@@ -13,6 +13,7 @@ from typing import Dict, List, Optional, Tuple, TypedDict
 import torch
 
 from .. import ops
+from ..torch_ops import llmc
 from ..quantization import QuantizationArgs, QuantizationStrategy, calculate_qparams, generate_gparam
 from .fusion import FusionHandler
 from .helpers import flatten_for_calibration
@@ -130,11 +131,11 @@ class Observer(torch.nn.Module):
         """min/max over dims (0,-1) of the calibration view of ``value``; subclasses may search instead."""
         (kind, t, p), shape = _observed_layout(value, self.base_name, self.args)
         if kind == "groups":
-            mn, mx = ops.minmax_groups(t, p)
+            mn, mx = llmc.minmax_observe(t, p)
         elif kind == "blocks":
-            mn, mx = ops.minmax_blocks(t, *p)
+            mn, mx = llmc.minmax_observe_blocks(t, *p)
         else:
-            mn, mx = ops.minmax_strided(t, *p)
+            mn, mx = llmc.minmax_observe_strided(t, *p)
         return mn.reshape(shape), mx.reshape(shape)
 
     def compute_min_max(self, value: torch.Tensor) -> MinMaxTuple:
@@ -158,11 +159,11 @@ class Observer(torch.nn.Module):
         self.update_statistics(mn.reshape(qshape), mx.reshape(qshape))
 
     def _rows(self, rows2d):
-        mn, mx = ops.minmax_groups(rows2d, rows2d.shape[1])
+        mn, mx = llmc.minmax_observe(rows2d, rows2d.shape[1])
         return mn, mx
 
     def _strided(self, flat, n0, n1, G):
-        return ops.minmax_strided(flat, n0, n1, G, n1 * G, G)
+        return llmc.minmax_observe_strided(flat, n0, n1, G, n1 * G, G)
 
     def get_global_scale(self) -> Optional[torch.Tensor]:
         if self.args.strategy != QuantizationStrategy.TENSOR_GROUP:

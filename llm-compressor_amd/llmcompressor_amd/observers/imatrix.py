@@ -12,6 +12,7 @@ from typing import Optional
 import torch
 
 from .. import ops
+from ..torch_ops import llmc
 from ..quantization import QuantizationStrategy
 from ..quantization.lifecycle import kernel_format
 from .base import Observer, _observed_layout
@@ -82,7 +83,7 @@ class IMatrixMSEObserver(Observer):
             n_tokens = math.prod(x.shape[:-1])
             self._imatrix_sum = self._imatrix_sum.to(x.device)
             self._imatrix_count = self._imatrix_count.to(x.device)
-            ops.sumsq_accumulate_(self._imatrix_sum, x.reshape(-1, x.shape[-1]))
+            llmc.sumsq_accum_(self._imatrix_sum, x.reshape(-1, x.shape[-1]))
             self._imatrix_count += n_tokens
 
         self._imatrix_hook = module.register_forward_pre_hook(_hook)
@@ -104,11 +105,11 @@ class IMatrixMSEObserver(Observer):
         kw = dict(maxshrink=self.maxshrink, patience=self.patience, grid=self.grid, norm=self.norm,
                   expand=self.expand)
         if kind == "groups":
-            mn, mx = ops.imatrix_observe_groups(t, p, fmt, bits, self.args.symmetric, mode, importance=imp, **kw)
+            mn, mx = llmc.imatrix_observe(t, p, fmt, bits, self.args.symmetric, mode, importance=imp, **kw)
         elif kind == "blocks":  # no importance here: _validated_importance sent block-wise weights to the fall-back
-            mn, mx = ops.imatrix_observe_blocks(t, p[0], p[1], fmt, bits, self.args.symmetric, mode, **kw)
+            mn, mx = llmc.imatrix_observe_blocks(t, p[0], p[1], fmt, bits, self.args.symmetric, mode, **kw)
         else:
-            mn, mx = ops.imatrix_observe_strided(t, *p, fmt, bits, self.args.symmetric, mode, **kw)
+            mn, mx = llmc.imatrix_observe_strided(t, *p, fmt, bits, self.args.symmetric, mode, **kw)
         return mn.reshape(shape), mx.reshape(shape)
 
     def _fallback(self, exc_type, msg: str):

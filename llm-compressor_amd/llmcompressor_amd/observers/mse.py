@@ -2,6 +2,7 @@
 import torch
 
 from .. import ops
+from ..torch_ops import llmc
 from ..quantization import QuantizationStrategy
 from ..quantization.lifecycle import kernel_format
 from .base import Observer, _observed_layout
@@ -42,24 +43,23 @@ class MemorylessMSEObserver(Observer):
         mode = ops.SCALE_MXFP4 if self.args.is_mx else ops.SCALE_PLAIN
         kw = self._search_kwargs()
         if kind == "groups":
-            mn, mx = ops.mse_observe_groups(t, p, fmt, bits, self.args.symmetric, mode, **kw)
+            mn, mx = llmc.mse_observe(t, p, fmt, bits, self.args.symmetric, mode, **kw)
         elif kind == "blocks":
-            mn, mx = ops.mse_observe_blocks(t, p[0], p[1], fmt, bits, self.args.symmetric, mode, **kw)
+            mn, mx = llmc.mse_observe_blocks(t, p[0], p[1], fmt, bits, self.args.symmetric, mode, **kw)
         else:
-            mn, mx = ops.mse_observe_strided(t, *p, fmt, bits, self.args.symmetric, mode, **kw)
+            mn, mx = llmc.mse_observe_strided(t, *p, fmt, bits, self.args.symmetric, mode, **kw)
         return mn.reshape(shape), mx.reshape(shape)
 
     def _rows(self, rows2d):
         fmt, bits = kernel_format(self.args)
         mode = ops.SCALE_MXFP4 if self.args.is_mx else ops.SCALE_PLAIN
-        return ops.mse_observe_groups(rows2d, rows2d.shape[1], fmt, bits, self.args.symmetric, mode,
-                                      **self._search_kwargs())
+        return llmc.mse_observe(rows2d, rows2d.shape[1], fmt, bits, self.args.symmetric, mode, **self._search_kwargs())
 
     def _strided(self, flat, n0, n1, G):
         fmt, bits = kernel_format(self.args)
         mode = ops.SCALE_MXFP4 if self.args.is_mx else ops.SCALE_PLAIN
-        return ops.mse_observe_strided(flat, n0, n1, G, n1 * G, G, fmt, bits, self.args.symmetric, mode,
-                                       **self._search_kwargs())
+        return llmc.mse_observe_strided(flat, n0, n1, G, n1 * G, G, fmt, bits, self.args.symmetric, mode,
+                                        **self._search_kwargs())
 
 
 @Observer.register("mse")

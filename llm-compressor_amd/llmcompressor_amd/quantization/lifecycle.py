@@ -19,6 +19,7 @@ import torch
 from torch.nn import Module, Parameter
 
 from .. import ops
+from ..torch_ops import llmc
 from .quant_args import (
     ActivationOrdering,
     DynamicType,
@@ -165,9 +166,9 @@ def calculate_qparams(min_vals, max_vals, quantization_args: QuantizationArgs, g
     """-> (scale, zero_point).  NVFP4: scale holds e4m3-grid values in fp32; MXFP4: E8M0 codes (uint8)."""
     fmt, bits = kernel_format(quantization_args)
     mode = scale_mode(quantization_args, global_scale is not None)
-    scale, zp, codes = ops.calculate_qparams(
-        min_vals, max_vals, fmt, bits, quantization_args.symmetric, mode,
-        global_scale if mode == ops.SCALE_NVFP4 else None, want_codes=(mode == ops.SCALE_MXFP4))
+    scale, zp, codes = llmc.qparams(
+        min_vals, max_vals, fmt, bits, bool(quantization_args.symmetric), mode,
+        global_scale if mode == ops.SCALE_NVFP4 else None, mode == ops.SCALE_MXFP4)
     if mode == ops.SCALE_MXFP4:
         scale = codes
     if scale.ndim == 0:
@@ -180,7 +181,7 @@ def calculate_qparams(min_vals, max_vals, quantization_args: QuantizationArgs, g
 
 def generate_gparam(stats) -> torch.Tensor:
     """stats: list of (min_vals, max_vals) over a fused group -> fp32 [1] global scale."""
-    return ops.global_scale_from_stats(stats)
+    return llmc.global_scale([mn for mn, _ in stats], [mx for _, mx in stats])
 
 
 def _as_2d(x: torch.Tensor):
@@ -202,8 +203,7 @@ def _run_quantize(x, scale, zero_point, args: QuantizationArgs, out_mode, g_idx=
     zp = None
     if zero_point is not None and not args.symmetric:
         zp = zero_point.to(torch.int8)
-    out = ops.quantize(x2, es, zp, fmt, bits, row_div, srow, col_div, out_mode=out_mode, g_idx=g_idx,
-                       global_scale=global_scale)
+    out = llmc.quant_pack(x2, es, zp, fmt, bits, row_div, srow, col_div, out_mode, g_idx, global_scale)
     if out_mode == ops.OUT_PACKED:
         return out
     return out.reshape(shape)
@@ -228,10 +228,10 @@ def forward_quantize(module: Module, value: torch.Tensor, base_name: str, args: 
         x2, shape = _as_2d(value)
         x2 = x2.contiguous()
         if args.symmetric and bits == 8:  # the fused kernel: row absmax, scale and fake-quant in one pass
-            out, _ = ops.dynamic_per_token_quantize(x2, fmt, bits)
+            out, _ = llmc.fp8_dynamic_per_token(x2, fmt, bits)
             return out.reshape(shape)
         # other widths and asymmetric ranges: row min/max, qparams and fake-quant as separate kernels
-        mn, mx = ops.minmax_groups(x2, x2.shape[1])
+        mn, mx = llmc.minmax_observe(x2, x2.shape[1])
         scale, zp = calculate_qparams(mn, mx, args)
         return fake_quantize(x2, scale, zp, args).reshape(shape)
     scale = getattr(module, f"{base_name}_scale", None)
@@ -246,9 +246,11 @@ def forward_quantize(module: Module, value: torch.Tensor, base_name: str, args: 
             if cols % args.group_size != 0:
                 raise ValueError(f"dynamic group quantization: last dimension {cols} is not a multiple of the "
                                  f"group size {args.group_size}")
-            mn, mx = ops.minmax_groups(x2, args.group_size)
+            mn, mx = llmc.minmax_observe(x2, args.group_size)
         elif args.strategy == QuantizationStrategy.TENSOR:
-            mn, mx = ops.minmax_strided(x2, rows, 1, cols, cols, cols)
+            # one group holding every element: the split reduction of the row kernels fills the chip
+            mn, mx = llmc.minmax_observe(x2.reshape(1, -1), rows * cols)
+            mn, mx = mn.reshape(1), mx.reshape(1)
         else:
             raise ValueError(f"dynamic quantization does not support {args.strategy}")
         scale, zp = calculate_qparams(mn, mx, args, global_scale=gs)

@@ -1,0 +1,64 @@
+"""The reference's import paths resolve to this package (no GPU needed: nothing is computed).
+
+Reference: src/llmcompressor/__init__.py:23-29, modifiers/quantization/__init__.py,
+modifiers/quantization/gptq/__init__.py (deprecated re-export)."""
+import importlib
+import sys
+import warnings
+
+import pytest
+
+
+def test_llmcompressor_root_is_an_alias_of_this_package():
+    import llmcompressor
+    import llmcompressor_amd
+    from llmcompressor import model_free_ptq, oneshot
+    from llmcompressor.modifiers.gptq import GPTQModifier
+    from llmcompressor.modifiers.quantization import GPTQModifier as G2
+    from llmcompressor.modifiers.quantization import QuantizationModifier
+    from llmcompressor.observers import Observer
+
+    import llmcompressor_amd.modifiers.gptq as real_gptq
+    import llmcompressor_amd.observers as real_obs
+
+    assert oneshot is llmcompressor_amd.oneshot and model_free_ptq is llmcompressor_amd.model_free_ptq
+    assert GPTQModifier is real_gptq.GPTQModifier is G2
+    assert Observer is real_obs.Observer  # one registry, whichever root was imported
+    assert sys.modules["llmcompressor.modifiers.gptq"] is sys.modules["llmcompressor_amd.modifiers.gptq"]
+    assert QuantizationModifier.__name__ == "QuantizationModifier"
+    assert llmcompressor.__version__ == llmcompressor_amd.__version__
+    from llmcompressor import active_session
+
+    assert active_session() is llmcompressor_amd.active_session()
+    with pytest.raises(ModuleNotFoundError):
+        importlib.import_module("llmcompressor.no_such_module")
+
+
+@pytest.mark.parametrize("root", ["llmcompressor", "llmcompressor_amd"])
+def test_deprecated_gptq_location_warns_and_reexports(root):
+    import llmcompressor  # noqa: F401  (installs the alias finder)
+
+    for name in (f"{root}.modifiers.quantization.gptq", "llmcompressor_amd.modifiers.quantization.gptq",
+                 "llmcompressor.modifiers.quantization.gptq"):
+        sys.modules.pop(name, None)
+    with warnings.catch_warnings(record=True) as caught:
+        warnings.simplefilter("always")
+        mod = importlib.import_module(f"{root}.modifiers.quantization.gptq")
+    assert any(issubclass(w.category, DeprecationWarning) and "deprecated" in str(w.message) for w in caught)
+    real = importlib.import_module("llmcompressor_amd.modifiers.gptq")
+    assert mod.GPTQModifier is real.GPTQModifier
+    assert mod.quantize_weight is real.quantize_weight and mod.accumulate_hessian is real.accumulate_hessian
+
+
+def test_torch_ops_are_registered_without_a_cpu_implementation():
+    import torch
+
+    from llmcompressor_amd import torch_ops
+
+    for name in ("hessian_accum_", "gptq_prepare_hinv_", "gptq_quantize", "minmax_observe", "mse_observe", "qparams",
+                 "quant_pack", "fp8_dynamic_per_token", "hessian_accum_grouped_", "gptq_quantize_grouped"):
+        assert name in torch_ops.OP_NAMES and hasattr(torch.ops.llmc, name)
+    with pytest.raises((NotImplementedError, RuntimeError), match="CPU"):
+        torch.ops.llmc.hessian_accum_(torch.zeros(8, 8), torch.zeros(4, 8, dtype=torch.bfloat16))
+    with pytest.raises((NotImplementedError, RuntimeError), match="CPU"):
+        torch.ops.llmc.minmax_observe(torch.zeros(4, 8), 8)
