@@ -90,80 +90,109 @@ def cpu_baseline(tokens: int):
     }
 
 
-def probe_bandwidth():
-    """Observer / quantize / pack kernels on a 14336 x 4096 bf16 weight (the gate/up projection) and the
-    per-token activation kernel on 8192 x 4096: algorithmic bytes (one read of the input plus one write of
-    the output) over the event-timed launch, against the 8 TB/s HBM peak.  Prints a table."""
+def probe_bandwidth(rows_filter=None, reps=20, stack=8):
+    """Observer / quantize / pack kernels on a 114688 x 4096 bf16 weight (eight gate/up projections stacked,
+    0.94 GB) and the per-token activation kernel on 65536 x 4096 inputs (0.54 GB): algorithmic bytes (one read
+    of the input plus one write of the output) over the event-timed launch, against the 8 TB/s HBM peak.
+
+    Cold cache: one launch streams several times the 256 MB last-level cache, consecutive launches read a
+    different one of 3 distinct inputs and write an output buffer of their own (the last 3 results are kept
+    alive), and a launch lasts 150 us or more, so the host's launch overhead hides behind the queue.
+    `rows_filter` (substrings) selects rows, so that a counter run can hold one row per kernel name.
+    `stack` = 1 runs the single-Linear size instead (14336 x 4096 weights, 8192 x 4096 activations, 12 distinct
+    inputs in rotation): launches of 20-40 us whose event timing includes the host's launch overhead, so their
+    durations are read from a kernel trace.  Prints a table."""
     import torch
 
     from llmcompressor_amd import ops
 
-    def timed(fn, n=20):
-        for _ in range(3):
-            fn()
+    NW = 3 if stack > 1 else 12
+
+    def timed(fn, n=reps):
+        keep = [None] * NW
+        for i in range(3):
+            keep[i % NW] = fn(i % NW)
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        for _ in range(n):
-            fn()
+        for i in range(n):
+            keep[i % NW] = fn((i + 3) % NW)
         e1.record()
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / n * 1e-3
 
-    R, K = INTER, HIDDEN
+    R, K = stack * INTER, HIDDEN
     n = R * K
-    w = (torch.randn(R, K, device="cuda") * 0.02).bfloat16()
+    NT = 8192 * stack
+    ws = [(torch.randn(R, K, device="cuda") * 0.02).bfloat16() for _ in range(NW)]
+    xs = [torch.randn(NT, HIDDEN, device="cuda").bfloat16() for _ in range(NW)]
+    nx = xs[0].numel()
     rows = []
 
-    def rep(name, t, nbytes):
-        rows.append((name, t * 1e6, nbytes / t / 1e9, nbytes / t / 8e12))
+    def want(name):
+        return not rows_filter or any(f in name for f in rows_filter)
 
-    dst = torch.empty_like(w)
-    rep("copy (reference), 4 B/elem", timed(lambda: dst.copy_(w)), 4 * n)
+    def rep(name, fn, nbytes, n_launch=reps, note=None):
+        if not want(name):
+            return
+        t = timed(fn, n_launch)
+        rows.append((name if note is None else name + note(t), t * 1e6, nbytes / t / 1e9, nbytes / t / 8e12))
+
+    dsts = [torch.empty_like(ws[0]) for _ in range(NW)]
+    rep("copy (reference), 4 B/elem", lambda i: dsts[i].copy_(ws[i]), 4 * n)
     for g in (16, 32, 128, K):
-        rep(f"min-max observer g={g}, 2 B/elem", timed(lambda: ops.minmax_groups(w, g)), 2 * n)
-    mn, mx = ops.minmax_groups(w, 128)
-    sc, _, _ = ops.calculate_qparams(mn, mx, ops.FMT_INT, 4, True)
+        rep(f"min-max observer g={g}, 2 B/elem", lambda i, g=g: ops.minmax_groups(ws[i], g), 2 * n)
+
+    def scales(g, fmt, bits, mode=ops.SCALE_PLAIN, with_gs=False):
+        out = []
+        for w in ws:
+            mn, mx = ops.minmax_groups(w, g)
+            gs = ops.global_scale_from_stats([(mn, mx)]) if with_gs else None
+            sc, _, codes = ops.calculate_qparams(mn, mx, fmt, bits, True, mode, gs, want_codes=mode == ops.SCALE_MXFP4)
+            out.append((sc, gs))
+        return out
+
     grp = (1, K // 128, 128)
-    rep("int4 g128 -> packed int32, 2.5 B/elem",
-        timed(lambda: ops.quantize(w, sc, None, ops.FMT_INT, 4, *grp, out_mode=ops.OUT_PACKED)), 2.5 * n)
-    rep("int4 g128 fake-quant, 4 B/elem", timed(lambda: ops.quantize(w, sc, None, ops.FMT_INT, 4, *grp)), 4 * n)
-    mn, mx = ops.minmax_groups(w, K)
-    s8, _, _ = ops.calculate_qparams(mn, mx, ops.FMT_FP8, 8, True)
-    rep("fp8 e4m3 per-channel -> bytes, 3 B/elem",
-        timed(lambda: ops.quantize(w, s8, None, ops.FMT_FP8, 8, 1, 1, 1 << 40, out_mode=ops.OUT_PACKED)), 3 * n)
-    mn, mx = ops.minmax_groups(w, 16)
-    gs = ops.global_scale_from_stats([(mn, mx)])
-    s4, _, _ = ops.calculate_qparams(mn, mx, ops.FMT_FP4, 4, True, ops.SCALE_NVFP4, gs)
-    rep("nvfp4 g16 -> packed nibbles, 2.5 B/elem",
-        timed(lambda: ops.quantize(w, s4, None, ops.FMT_FP4, 4, 1, K // 16, 16, out_mode=ops.OUT_PACKED, global_scale=gs)),
-        2.5 * n)
-    mn, mx = ops.minmax_groups(w, 32)
-    sm, _, _ = ops.calculate_qparams(mn, mx, ops.FMT_FP4, 4, True, ops.SCALE_MXFP4, want_codes=True)
-    rep("mxfp4 g32 -> packed nibbles, 2.5 B/elem",
-        timed(lambda: ops.quantize(w, sm, None, ops.FMT_FP4, 4, 1, K // 32, 32, out_mode=ops.OUT_PACKED)), 2.5 * n)
-    x = torch.randn(8192, HIDDEN, device="cuda").bfloat16()
-    rep("fp8 dynamic per-token fake-quant [8192x4096], 4 B/elem", timed(lambda: ops.dynamic_per_token_quantize(x)),
-        4 * x.numel())
-    rep("fp8 dynamic per-token -> bytes [8192x4096], 3 B/elem",
-        timed(lambda: ops.dynamic_per_token_quantize(x, out_mode=ops.OUT_CODES)), 3 * x.numel())
+    if want("int4 g128"):
+        sc = scales(128, ops.FMT_INT, 4)
+        rep("int4 g128 -> packed int32, 2.5 B/elem",
+            lambda i: ops.quantize(ws[i], sc[i][0], None, ops.FMT_INT, 4, *grp, out_mode=ops.OUT_PACKED), 2.5 * n)
+        rep("int4 g128 fake-quant, 4 B/elem", lambda i: ops.quantize(ws[i], sc[i][0], None, ops.FMT_INT, 4, *grp), 4 * n)
+    if want("fp8 e4m3 per-channel"):
+        s8 = scales(K, ops.FMT_FP8, 8)
+        rep("fp8 e4m3 per-channel -> bytes, 3 B/elem",
+            lambda i: ops.quantize(ws[i], s8[i][0], None, ops.FMT_FP8, 8, 1, 1, 1 << 40, out_mode=ops.OUT_PACKED), 3 * n)
+    if want("nvfp4 g16"):
+        s4 = scales(16, ops.FMT_FP4, 4, ops.SCALE_NVFP4, with_gs=True)
+        rep("nvfp4 g16 -> packed nibbles, 2.5625 B/elem",
+            lambda i: ops.quantize(ws[i], s4[i][0], None, ops.FMT_FP4, 4, 1, K // 16, 16, out_mode=ops.OUT_PACKED,
+                                   global_scale=s4[i][1]), 2.5625 * n)
+    if want("mxfp4 g32"):
+        sm = scales(32, ops.FMT_FP4, 4, ops.SCALE_MXFP4)
+        rep("mxfp4 g32 -> packed nibbles, 2.53125 B/elem",
+            lambda i: ops.quantize(ws[i], sm[i][0], None, ops.FMT_FP4, 4, 1, K // 32, 32, out_mode=ops.OUT_PACKED),
+            2.53125 * n)
+    rep(f"fp8 dynamic per-token fake-quant [{NT}x4096], 4 B/elem", lambda i: ops.dynamic_per_token_quantize(xs[i]), 4 * nx)
+    rep(f"fp8 dynamic per-token -> bytes [{NT}x4096], 3 B/elem",
+        lambda i: ops.dynamic_per_token_quantize(xs[i], out_mode=ops.OUT_CODES), 3 * nx)
     # the MSE grid search is arithmetic-bound (every candidate scale re-quantises the group): its figure
     # of merit is candidate evaluations per second; the GB/s column is its one read of the weight
     for name, kw, fmt, bits, g in (("mse observer int4 g128, 20 candidates", {}, ops.FMT_INT, 4, 128),
                                    ("mse observer fp4 g16, 20 candidates", {}, ops.FMT_FP4, 4, 16),
                                    ("mse observer fp4 g16, 80 candidates (maxshrink 0.8, no early stop)",
                                     dict(maxshrink=0.8, patience=100), ops.FMT_FP4, 4, 16)):
-        t = timed(lambda: ops.mse_observe_groups(w, g, fmt, bits, True, ops.SCALE_PLAIN, **kw), n=5)
         cands = 80 if kw else 20
-        rep(f"{name}: {n * cands / t / 1e12:.2f} T element-candidates/s", t, 2 * n)
+        rep(name, lambda i, g=g, fmt=fmt, bits=bits, kw=kw: ops.mse_observe_groups(ws[i], g, fmt, bits, True,
+                                                                                   ops.SCALE_PLAIN, **kw),
+            2 * n, n_launch=5, note=lambda t, c=cands: f": {n * c / t / 1e12:.2f} T element-candidates/s")
     tot = torch.zeros(HIDDEN, dtype=torch.float32, device="cuda")
-    rep("imatrix hook: sum of squares per channel [8192x4096], 2 B/elem", timed(lambda: ops.sumsq_accumulate_(tot, x)),
-        2 * x.numel())
+    rep(f"imatrix hook: sum of squares per channel [{NT}x4096], 2 B/elem", lambda i: ops.sumsq_accumulate_(tot, xs[i]),
+        2 * nx)
     imp = torch.rand(K, device="cuda") + 0.1
-    t = timed(lambda: ops.imatrix_observe_groups(w, 128, ops.FMT_INT, 4, True, importance=imp), n=5)
-    rep(f"imatrix observer int4 g128, 20 candidates, fp32 weighted error: {n * 20 / t / 1e12:.2f} T element-candidates/s",
-        t, 2 * n)
-    print("| kernel (14336 x 4096 bf16 unless noted) | us | GB/s | of 8 TB/s |")
+    rep("imatrix observer int4 g128, 20 candidates, fp32 weighted error",
+        lambda i: ops.imatrix_observe_groups(ws[i], 128, ops.FMT_INT, 4, True, importance=imp), 2 * n, n_launch=5,
+        note=lambda t: f": {n * 20 / t / 1e12:.2f} T element-candidates/s")
+    print(f"| kernel ({R} x {K} bf16 unless noted), cold cache | us | GB/s | of 8 TB/s |")
     print("|---|---|---|---|")
     for name, us, gbs, frac in rows:
         print(f"| {name} | {us:.1f} | {gbs:.0f} | {frac * 100:.1f}% |")
@@ -346,6 +375,10 @@ def main():
                     "tokens) and N plain copies of a 1 GiB buffer (the known-size kernel the HBM counters are scaled by)")
     ap.add_argument("--probe-bandwidth", action="store_true",
                     help="print achieved GB/s of the observer / quantize / pack kernels instead of the bench line")
+    ap.add_argument("--probe-rows", default="", help="comma-separated substrings: the rows --probe-bandwidth runs")
+    ap.add_argument("--probe-reps", type=int, default=20, help="timed launches per row of --probe-bandwidth")
+    ap.add_argument("--probe-stack", type=int, default=8,
+                    help="--probe-bandwidth: gate/up projections stacked into one weight (1 = the single-Linear size)")
     ap.add_argument("--probe-sparsegpt", action="store_true",
                     help="print SparseGPT timings per Linear shape instead of the bench line")
     ap.add_argument("--moe-mode", choices=("both", "lockstep", "permodule"), default="both",
@@ -370,7 +403,7 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     if a.probe_bandwidth:
-        probe_bandwidth()
+        probe_bandwidth([r for r in a.probe_rows.split(",") if r], a.probe_reps, a.probe_stack)
         return
     if a.probe_sparsegpt:
         probe_sparsegpt()

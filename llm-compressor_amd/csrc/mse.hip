@@ -711,12 +711,22 @@ __global__ __launch_bounds__(256) void sumsq_partial_kernel(const void* __restri
   partial[(int64_t)s * K + c] = acc;
 }
 
-__global__ __launch_bounds__(256) void sumsq_finish_kernel(const float* __restrict__ partial, int64_t K, int slices,
-                                                           float* __restrict__ sum) {
-  const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+__global__ __launch_bounds__(64) void sumsq_finish_kernel(const float* __restrict__ partial, int64_t K, int slices,
+                                                          float* __restrict__ sum) {
+  const int64_t c = (int64_t)blockIdx.x * 64 + threadIdx.x;
   if (c >= K) return;
+  // the loads of 16 slices are issued together (one memory round trip per batch); the additions keep
+  // the order s = 0, 1, 2, ...
   float acc = 0.f;
-  for (int s = 0; s < slices; ++s) acc += partial[(int64_t)s * K + c];
+  int s = 0;
+  for (; s + 16 <= slices; s += 16) {
+    float v[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) v[j] = partial[(int64_t)(s + j) * K + c];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc += v[j];
+  }
+  for (; s < slices; ++s) acc += partial[(int64_t)s * K + c];
   sum[c] += acc;
 }
 
@@ -773,7 +783,7 @@ static int sumsq_launch(const void* x, int32_t dtype, int64_t T, int64_t K, int6
     hipLaunchKernelGGL(sumsq_partial_kernel, dim3((unsigned)((K + 255) / 256), (unsigned)slices), dim3(256), 0, st, x,
                        dtype, T, K, ldx, slices, partial);
   LLMC_LAUNCH_STATUS();
-  hipLaunchKernelGGL(sumsq_finish_kernel, dim3((unsigned)((K + 255) / 256)), dim3(256), 0, st,
+  hipLaunchKernelGGL(sumsq_finish_kernel, dim3((unsigned)((K + 63) / 64)), dim3(64), 0, st,
                      (const float*)partial, K, slices, sum);
   LLMC_LAUNCH_STATUS();
   return 0;

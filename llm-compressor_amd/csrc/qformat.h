@@ -160,6 +160,42 @@ __device__ __forceinline__ float fastdiv(float x, const FastDiv& d) {
 __device__ __forceinline__ bool fastdiv_big_ok(float q) { return fabsf(q) < 0x1p100f; }
 __device__ __forceinline__ bool fastdiv_small(float q) { return fabsf(q) < 0x1p-40f; }
 
+// ---- bf16 / bf16 quotient rounded to bf16, with one multiply.  For x and s both bf16 (8-bit
+// significands X, S in [128, 255]) the exact quotient X/S is never a rounding midpoint of bf16 (a midpoint
+// has a 9-bit odd significand M, and M*S' = X*2^k has no solution with M >= 257 > X), and it lies at
+// least 2^-16 (relative) away from the nearest one: |256 X - M S| >= 1 over 256 S.  x * y with y the
+// reciprocal of make_fastdiv() is within 2^-22 of the quotient, so bf16(x * y) == bf16(x / s) whenever the
+// quotient is a normal bf16 number and nothing overflows.  bf16_inputs_plain() bounds that from the inputs:
+// every nonzero |x| lies in [2^-96, 2^96) (which also excludes inf and NaN), and bf16_scale_plain() asks
+// |s| in (2^-30, 2^30), so |x / s| lies in (2^-126, 2^126).  A zero dividend gives an exact zero.
+typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
+struct Bf16Range {
+  u16x2_t mx, mn;
+};
+__device__ __forceinline__ Bf16Range bf16_range_init() {
+  Bf16Range r;
+  r.mx = (u16x2_t){0, 0};
+  r.mn = (u16x2_t){0xffff, 0xffff};
+  return r;
+}
+// fold the two bf16 values of one 32-bit word into the running magnitude range (zeros do not lower it)
+__device__ __forceinline__ void bf16_range_add(Bf16Range& r, uint32_t w) {
+  const uint32_t a = w & 0x7fff7fffu;
+  u16x2_t m;
+  __builtin_memcpy(&m, &a, 4);
+  r.mx = __builtin_elementwise_max(r.mx, m);
+  r.mn = __builtin_elementwise_min(r.mn, (u16x2_t)(m - (u16x2_t){1, 1}));
+}
+__device__ __forceinline__ bool bf16_inputs_plain(const Bf16Range& r) {
+  constexpr uint32_t LO = (127u - 96u) << 7, HI = (127u + 96u) << 7;  // bit patterns of 2^-96 and 2^96
+  const uint32_t mx = max((uint32_t)r.mx.x, (uint32_t)r.mx.y), mn = min((uint32_t)r.mn.x, (uint32_t)r.mn.y);
+  return mx < HI && mn >= LO - 1u;
+}
+__device__ __forceinline__ bool bf16_scale_plain(float s) {
+  const float a = fabsf(s);
+  return a > 0x1p-30f && a < 0x1p30f;
+}
+
 struct QFormat {
   int fmt;   // LLMC_FMT_*
   float qmin, qmax;

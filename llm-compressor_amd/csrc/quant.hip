@@ -224,17 +224,28 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(QuantParams p, int c
     unpack8<XDT>(raw0, x);
     unpack8<XDT>(raw1, x + 8);
     const FastDiv d = make_fastdiv(s);
-    bool big = false, small = false;
+    bool redo;
+    if (XDT == LLMC_BF16 && SM == 0) {
+      // bf16 values over a bf16 scale: the rounded quotient is one multiply away (see qformat.h)
+      Bf16Range rg = bf16_range_init();
+      bf16_range_add(rg, raw0.x); bf16_range_add(rg, raw0.y); bf16_range_add(rg, raw0.z); bf16_range_add(rg, raw0.w);
+      bf16_range_add(rg, raw1.x); bf16_range_add(rg, raw1.y); bf16_range_add(rg, raw1.z); bf16_range_add(rg, raw1.w);
+      redo = !(bf16_inputs_plain(rg) & bf16_scale_plain(s));
 #pragma unroll
-    for (int j = 0; j < E; ++j) {
-      v[j] = fastdiv(x[j], d);
-      big = big | !fastdiv_big_ok(v[j]);
-      small = small | fastdiv_small(v[j]);
-    }
-    bool redo = big | !d.ok;
-    if (small) {
+      for (int j = 0; j < E; ++j) v[j] = x[j] * d.y;
+    } else {
+      bool big = false, small = false;
 #pragma unroll
-      for (int j = 0; j < E; ++j) redo = redo | (fastdiv_small(v[j]) & (x[j] != 0.f));
+      for (int j = 0; j < E; ++j) {
+        v[j] = fastdiv(x[j], d);
+        big = big | !fastdiv_big_ok(v[j]);
+        small = small | fastdiv_small(v[j]);
+      }
+      redo = big | !d.ok;
+      if (small) {
+#pragma unroll
+        for (int j = 0; j < E; ++j) redo = redo | (fastdiv_small(v[j]) & (x[j] != 0.f));
+      }
     }
     if (redo) {
       // out-of-range divisor or quotient, NaN: the plain division, then the same tail
@@ -503,7 +514,6 @@ __global__ __launch_bounds__(256) void dynamic_token_wave_kernel(const void* __r
   const uint16_t* xr = (const uint16_t*)x + r * ldx;
   const int nchunk = K >> 3;
   uint4 raw[NC];
-  typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
   u16x2_t m = {0, 0};  // packed max of 15-bit magnitudes (magnitude bits order like the values)
 #pragma unroll
   for (int i = 0; i < NC; ++i) {
@@ -530,6 +540,9 @@ __global__ __launch_bounds__(256) void dynamic_token_wave_kernel(const void* __r
   if (s == 0.f) s = dtype_eps(DT);
   if (lane == 0) store_from_f32<DT>(scale_out, r, s);
   const FastDiv d = make_fastdiv(s);
+  // bf16 rows: the scale is a bf16 value too, so the rounded quotient is one multiply away (see qformat.h);
+  // the row's largest magnitude is known, only values far below it need the guard
+  const bool plain_scale = DT == LLMC_BF16 && bf16_scale_plain(s) && mm < ((127u + 96u) << 7);
 
 #pragma unroll
   for (int i = 0; i < NC; ++i) {
@@ -537,17 +550,26 @@ __global__ __launch_bounds__(256) void dynamic_token_wave_kernel(const void* __r
     if (c >= nchunk) break;
     float xv[8], v[8];
     unpack8<DT>(raw[i], xv);
-    bool big = false, small = false;
+    bool redo;
+    if (DT == LLMC_BF16) {
+      Bf16Range rg = bf16_range_init();
+      bf16_range_add(rg, raw[i].x); bf16_range_add(rg, raw[i].y); bf16_range_add(rg, raw[i].z); bf16_range_add(rg, raw[i].w);
+      redo = !(bf16_inputs_plain(rg) & plain_scale);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      v[j] = fastdiv(xv[j], d);
-      big = big | !fastdiv_big_ok(v[j]);
-      small = small | fastdiv_small(v[j]);
-    }
-    bool redo = big | !d.ok;
-    if (small) {
+      for (int j = 0; j < 8; ++j) v[j] = xv[j] * d.y;
+    } else {
+      bool big = false, small = false;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) redo = redo | (fastdiv_small(v[j]) & (xv[j] != 0.f));
+      for (int j = 0; j < 8; ++j) {
+        v[j] = fastdiv(xv[j], d);
+        big = big | !fastdiv_big_ok(v[j]);
+        small = small | fastdiv_small(v[j]);
+      }
+      redo = big | !d.ok;
+      if (small) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) redo = redo | (fastdiv_small(v[j]) & (xv[j] != 0.f));
+      }
     }
     if (redo) {
 #pragma unroll

@@ -57,12 +57,13 @@ def infer_format(scheme: QuantizationScheme) -> str:
         if w.type == QuantizationType.INT and w.num_bits in (4, 8):
             return CompressionFormat.pack_quantized
         return CompressionFormat.naive_quantized
+    # weights and activations quantised: 8-bit floats are stored as fp8, every integer width one code per byte
+    # (compressed-tensors' branch order; the reference's own table, tests/.../test_compress_tensor_utils.py:289-325,
+    # holds W8A8 rows only, so the W4A8 row is not pinned by a reference-held vector)
     if w.type == QuantizationType.FLOAT and w.num_bits == 8:
         return CompressionFormat.float_quantized
-    if w.type == QuantizationType.INT and w.num_bits == 8:
+    if w.type == QuantizationType.INT:
         return CompressionFormat.int_quantized
-    if w.type == QuantizationType.INT and w.num_bits == 4:
-        return CompressionFormat.pack_quantized
     return CompressionFormat.naive_quantized
 
 

@@ -4,10 +4,6 @@ from __future__ import annotations
 import logging
 import warnings
 from abc import abstractmethod
-from collections import defaultdict
-from functools import partial
-
-import numpy
 import torch
 from pydantic import Field, PrivateAttr, field_validator, model_validator
 
@@ -15,7 +11,6 @@ from ....core import Event, State
 from ....quantization import match_named_modules
 from ....quantization.lifecycle import _match_one
 from ...modifier import Modifier
-from ...utils.hooks import HooksMixin
 
 logger = logging.getLogger("llmcompressor_amd")
 
@@ -97,27 +92,32 @@ class SparsityModifierBase(Modifier):
                              f"values, but model has {len(layers)} target layers")
         return True
 
-    def on_calibration_start(self, state: State, event: Event, **kwargs):
+    def _sparsity_of_layer(self, index: int, layer_name: str):
+        if isinstance(self.sparsity, dict):
+            return self.sparsity[layer_name]
+        if isinstance(self.sparsity, list):
+            return self.sparsity[index]
+        return self.sparsity
+
+    def _prunable_modules(self):
+        """(qualified name, module, sparsity of its layer) of every module this modifier prunes."""
         for index, (layer_name, layer) in enumerate(self._target_layers.items()):
-            if isinstance(self.sparsity, list):
-                layer_sparsity = self.sparsity[index]
-            elif isinstance(self.sparsity, dict):
-                layer_sparsity = self.sparsity[layer_name]
-            else:
-                layer_sparsity = self.sparsity
-            for name, module in match_named_modules(layer, PRUNABLE_LAYER_TYPES):
-                name = f"{layer_name}.{name}" if name else layer_name
-                if any(_match_one(name, module, i) for i in self.ignore):
+            target = self._sparsity_of_layer(index, layer_name)
+            for local, module in match_named_modules(layer, PRUNABLE_LAYER_TYPES):
+                qualified = ".".join(part for part in (layer_name, local) if part)
+                if isinstance(module, torch.nn.Embedding) or any(_match_one(qualified, module, i) for i in self.ignore):
                     continue
-                if isinstance(module, torch.nn.Embedding):
-                    continue
-                if name.endswith("lm_head"):
-                    logger.warning("`lm_head` was previously auto-ignored by SparseGPT and Wanda modifiers and is "
-                                   "not advised. Please add `re:.*lm_head` to your ignore list if this was "
-                                   "unintentional")
-                self._module_names[module] = name
-                self._module_sparsities[module] = layer_sparsity
-                self.register_hook(module, self.calibrate_module, "forward")
+                yield qualified, module, target
+
+    def on_calibration_start(self, state: State, event: Event, **kwargs):
+        for qualified, module, target in self._prunable_modules():
+            if qualified.endswith("lm_head"):
+                logger.warning("`lm_head` was previously auto-ignored by SparseGPT and Wanda modifiers and is "
+                               "not advised. Please add `re:.*lm_head` to your ignore list if this was "
+                               "unintentional")
+            self._module_names[module] = qualified
+            self._module_sparsities[module] = target
+            self.register_hook(module, self.calibrate_module, "forward")
 
     def on_sequential_epoch_end(self, state: State, event: Event, **kwargs):
         self.compress_modules()
@@ -125,48 +125,29 @@ class SparsityModifierBase(Modifier):
     def on_calibration_end(self, state: State, event: Event, **kwargs):
         self.remove_hooks()
 
-    # -- Outlier Weighed Layerwise sparsity (https://arxiv.org/pdf/2310.05175)
+    # -- Outlier Weighed Layerwise sparsity (Yin et al. 2023, arXiv 2310.05175)
     def _infer_owl_layer_sparsity(self, model, layers, dataloader) -> dict:
-        activations = self._get_activations(model, dataloader)
-        groups = {}
-        for name, layer in layers.items():
-            prunable = dict(match_named_modules(layer, PRUNABLE_LAYER_TYPES))
-            z = [m.weight.abs() * activations[f"{name}.{n}"].unsqueeze(0) for n, m in prunable.items()]
-            groups[name] = torch.cat([item.flatten().cpu() for item in z])
-        del activations
-        ratios = {}
-        for g, values in groups.items():
-            threshold = torch.mean(values) * self.owl_m
-            ratios[g] = 100 * (values > threshold).sum().item() / values.numel()
-        arr = numpy.array(list(ratios.values()))
-        for g in ratios:
-            ratios[g] = (ratios[g] - arr.min()) * (1 / (arr.max() - arr.min()) * self.owl_lmbda * 2)
-        arr = numpy.array(list(ratios.values()))
-        sparsities = {g: 1 - (ratios[g] - numpy.mean(arr) + (1 - float(self.sparsity))) for g in ratios}
-        logger.info(f"OWL sparsities for sp={self.sparsity} are:")
-        for g, sp in sparsities.items():
-            logger.info(f"Sparsity for {g}: {sp}")
+        """Per-layer sparsities from the layers' outlier ratios: D_l = percentage of the layer's scores
+        |W_ij| * a_j above ``owl_m`` times their mean, with a_j the input-channel norm summed over the
+        calibration batches; the ratios are stretched to [0, 2 * owl_lmbda], centred, and subtracted from
+        the global target.  Everything stays on the weights' device: two reductions per layer, no
+        concatenated copy of the scores."""
+        from .owl import channel_norms, outlier_percentage
+
+        norms = channel_norms(self, model, dataloader)
+        percent = {}
+        for layer_name, layer in layers.items():
+            members = [(m.weight, norms[f"{layer_name}.{n}" if n else layer_name])
+                       for n, m in match_named_modules(layer, PRUNABLE_LAYER_TYPES)
+                       if (f"{layer_name}.{n}" if n else layer_name) in norms]
+            percent[layer_name] = outlier_percentage(members, float(self.owl_m))
+        d = torch.tensor(list(percent.values()), dtype=torch.float64)
+        spread = d.max() - d.min()
+        stretched = (d - d.min()) * (2.0 * float(self.owl_lmbda) / spread)
+        keep = stretched - stretched.mean() + (1.0 - float(self.sparsity))
+        sparsities = {name: float(1.0 - k) for name, k in zip(percent, keep)}
+        logger.info(f"OWL sparsities for sp={self.sparsity}: " + ", ".join(f"{n}={v:.4f}" for n, v in sparsities.items()))
         return sparsities
-
-    def _get_activations(self, model, dataloader, nsamples=128) -> dict:
-        acts = defaultdict(int)
-
-        def save_acts(_module, inputs, name: str):
-            x = inputs[0] if isinstance(inputs, tuple) else inputs
-            acts[name] += 1.0 / nsamples * x.pow(2).sum(dim=(0, 1)).sqrt()
-
-        hooks = set(self.register_hook(mod, partial(save_acts, name=name), "forward_pre")
-                    for name, mod in model.named_modules()
-                    if isinstance(mod, torch.nn.Linear) and "lm_head" not in name)
-        device = next(model.parameters()).device
-        with HooksMixin.disable_hooks(keep=hooks), torch.no_grad():
-            for batch in dataloader or ():
-                if isinstance(batch, dict):
-                    model(**{k: (v.to(device) if torch.is_tensor(v) else v) for k, v in batch.items()})
-                else:
-                    model(batch.to(device) if torch.is_tensor(batch) else batch)
-        self.remove_hooks(hooks)
-        return acts
 
     def _split_mask_structure(self, mask_structure: str) -> tuple[int, int]:
         n, m = mask_structure.split(":")

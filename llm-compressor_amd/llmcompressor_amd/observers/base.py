@@ -66,6 +66,8 @@ def _observed_layout(value: torch.Tensor, base_name: str, args: QuantizationArgs
             return ("strided", x3, (x3.shape[0], x3.shape[1], K, x3.shape[1] * K, K)), (x3.shape[1],)
         if s in (S.GROUP, S.TENSOR_GROUP):
             g = args.group_size
+            if K % g != 0:  # the reference's unflatten into (K // g, g) raises here as well
+                raise ValueError(f"activation width {K} is not divisible by group_size {g}")
             n0 = x.numel() // K
             return ("strided", x, (n0, K // g, g, K, g)), (K // g,)
         flatten_for_calibration(value, base_name, args)

@@ -166,6 +166,11 @@ def calculate_qparams(min_vals, max_vals, quantization_args: QuantizationArgs, g
     """-> (scale, zero_point).  NVFP4: scale holds e4m3-grid values in fp32; MXFP4: E8M0 codes (uint8)."""
     fmt, bits = kernel_format(quantization_args)
     mode = scale_mode(quantization_args, global_scale is not None)
+    if mode == ops.SCALE_MXFP4 and min_vals.dtype != torch.bfloat16:
+        # the shared exponent is read off the bf16 bit pattern of the group maximum; for statistics of another
+        # dtype the rule is undefined (compressed-tensors asserts bf16 there), so nothing is guessed
+        raise TypeError(f"MXFP4 scales are defined on bfloat16 statistics; got {min_vals.dtype}. Cast the weights "
+                        "to bfloat16 or choose another scheme.")
     scale, zp, codes = llmc.qparams(
         min_vals, max_vals, fmt, bits, bool(quantization_args.symmetric), mode,
         global_scale if mode == ops.SCALE_NVFP4 else None, mode == ops.SCALE_MXFP4)

@@ -125,7 +125,15 @@ def _gpu_pipeline(w, args, dtype):
 def test_rtn_pipeline_bit_exact(name, dtype):
     args = F.QArgs(**SCHEMES[name])
     if args.is_mx and dtype != torch.bfloat16:
-        pytest.skip("MXFP4 scale generation is defined on bf16 statistics")
+        # the exponent rule reads the bf16 bit pattern of the group maximum: other dtypes are refused, not guessed
+        from llmcompressor_amd.quantization import QuantizationArgs
+        from llmcompressor_amd.quantization.lifecycle import calculate_qparams
+
+        stats = torch.ones(4, 2, dtype=dtype, device="cuda")
+        qa = QuantizationArgs(num_bits=4, type="float", strategy="group", group_size=32, scale_dtype="uint8")
+        with pytest.raises(TypeError, match="bfloat16 statistics"):
+            calculate_qparams(-stats, stats, qa)
+        return
     w = _w(256, 512, dtype, seed=len(name), std=0.05)
     w[7, 100] = 3.0  # outlier
     got = _gpu_pipeline(w, args, dtype)

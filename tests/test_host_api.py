@@ -614,3 +614,21 @@ def test_checkpoint_unpacking_helpers_match_the_oracle_pack():
     perm = torch.tensor([2, 0, 1, 1, 0, 2])
     gi = _expand_qparam(s, QuantizationArgs(num_bits=4, strategy="group", group_size=2), 2, 6, g_idx=perm)
     assert gi[0].tolist() == [2, 0, 1, 1, 0, 2]
+
+
+def test_owl_outlier_percentage_and_sparsity_mapping():
+    """The OWL profile's layer statistic against a brute-force count, and the mapping of the ratios to per-layer
+    sparsities: mean of (1 - sparsity) equals the global keep ratio, spread equals 2 * lambda."""
+    from llmcompressor_amd.modifiers.pruning.sparsegpt.owl import outlier_percentage
+
+    torch.manual_seed(0)
+    members = [(torch.randn(12, 16), torch.rand(16) + 0.1), (torch.randn(5, 16) * 3, torch.rand(16))]
+    scores = torch.cat([(w.abs() * a[None, :]).flatten() for w, a in members])
+    want = 100.0 * (scores > 3.0 * scores.mean()).sum().item() / scores.numel()
+    assert abs(outlier_percentage(members, 3.0) - want) < 1e-9
+    assert outlier_percentage([], 3.0) == 0.0
+    d = torch.tensor([1.0, 4.0, 2.5], dtype=torch.float64)
+    lmbda, target = 0.08, 0.6
+    stretched = (d - d.min()) * (2 * lmbda / (d.max() - d.min()))
+    keep = stretched - stretched.mean() + (1 - target)
+    assert abs(keep.mean().item() - (1 - target)) < 1e-12 and abs((keep.max() - keep.min()).item() - 2 * lmbda) < 1e-12

@@ -234,3 +234,71 @@ def test_generate_gparam_is_reciprocal_then_product():
         assert gs.dtype == torch.float32 and gs.item() == want
         assert gs.item() == (t.reciprocal() * 2688.0).float().item()
     assert (torch.tensor([2688.0]).bfloat16() / torch.tensor([40.0]).bfloat16()).item() == 67.0
+
+
+# ---- what mathematics and the installed libraries can still say about the unpinned format rules -----------------
+
+def _all_positive_normal_bf16():
+    # exponent fields 3..253: every normal bf16 for which neither rule leaves the E8M0 range
+    bits = torch.arange(3 << 7, 254 << 7, dtype=torch.int32).to(torch.int16)
+    return bits.view(torch.bfloat16)
+
+
+def test_mxfp4_exponent_rule_against_the_ocp_mx_definition_over_every_bf16_maximum():
+    """OCP Microscaling v1.0 (section 6.3): shared exponent = floor(log2(max|x|)) - emax(e2m1) with emax = 2.
+    The oracle follows the bf16 bit-pattern rule of compressed-tensors (a rounding bump of 0x20 before the mantissa
+    is dropped).  Brute force over every positive normal bf16 maximum (exponent fields 3..253): the two rules agree whenever the three
+    leading mantissa bits are below 0b110; for mantissas >= 1.75 the bump carries into the exponent and the
+    bit-pattern rule gives one more -- exactly those, nothing else.  (Which rule compressed-tensors' release
+    applies cannot be confirmed without the package: the function stays parity unpinned.)"""
+    amax = _all_positive_normal_bf16()
+    got = F.mxfp4_scale_exponent(amax).to(torch.int32)
+    ocp = (torch.floor(torch.log2(amax.double())) - 2 + 127).to(torch.int32)
+    mant = amax.view(torch.int16).to(torch.int32) & 0x7F
+    carries = mant >= 0x60  # 1.75 and above
+    assert torch.equal(got[~carries], ocp[~carries])
+    assert torch.equal(got[carries], ocp[carries] + 1)
+    assert 0.24 < carries.float().mean().item() < 0.26
+    # either way the scaled maximum amax / 2^(e-127) stays inside what e2m1 can round to 6 without clipping more
+    # than its top step: OCP gives [4, 8), the bump rule [3.5, 7)
+    ratio_bump = amax.double() / torch.pow(2.0, got.double() - 127)
+    ratio_ocp = amax.double() / torch.pow(2.0, ocp.double() - 127)
+    assert ratio_ocp.min() >= 4 and ratio_ocp.max() < 8
+    assert ratio_bump.min() >= 3.5 and ratio_bump.max() < 7
+
+
+def test_e8m0_code_is_the_byte_of_torch_float8_e8m0fnu():
+    """The stored MXFP4 scale byte e stands for 2^(e-127): the same byte torch's float8_e8m0fnu cast produces
+    for that power of two, for every exponent the rule can emit."""
+    e = torch.arange(1, 255, dtype=torch.int32)
+    value = torch.pow(2.0, (e - 127).double()).to(torch.float32)
+    as_e8m0 = value.to(torch.float8_e8m0fnu).view(torch.uint8).to(torch.int32)
+    assert torch.equal(as_e8m0, e)
+    back = F.mxfp4_scale_from_exponent(e.float(), dtype=torch.float32)
+    assert torch.equal(back, value)
+
+
+def test_per_token_dynamic_fp8_against_the_consumer_side_definition():
+    """Cross-check, not the oracle: an HF-side consumer of FP8 activations quantises per row with fp32 scales,
+    scale = where(rowmax > 0, rowmax, 1) / 448, q = clamp(x / scale, +-448).to(e4m3)
+    (transformers/integrations/compressed_tensors.py, the per-row FP8 helper).  The calibration-time path keeps the scale in
+    the activation dtype (bf16).  On N(0,1) rows with outliers the two agree on the reduce dimension (one scale
+    per token: the bf16 scale is the fp32 one rounded to bf16, row by row) and on >= 95 % of the code bytes; every
+    differing byte is one e4m3 step away.  The remaining per-token rule (keepdim shape, dtype of the scale) is
+    still parity unpinned."""
+    torch.manual_seed(4)
+    x = torch.randn(64, 512)
+    x[::7, ::31] *= 15
+    x = x.bfloat16()
+    args = F.QArgs(num_bits=8, type="float", strategy="token", dynamic=True)
+    scale, zp = F.compute_dynamic_scales_and_zp(x.unsqueeze(0), args)
+    assert scale.shape == (1, 64, 1) and scale.dtype == torch.bfloat16
+    rowmax = x.float().abs().amax(dim=-1, keepdim=True)
+    s32 = torch.where(rowmax > 0, rowmax, torch.ones_like(rowmax)) / 448.0
+    assert torch.equal(scale.reshape(-1), s32.to(torch.bfloat16).reshape(-1))
+    q_consumer = torch.clamp(x.float() / s32, -448, 448).to(torch.float8_e4m3fn)
+    q_oracle = F.quantize(x.unsqueeze(0), scale, zp, args, dtype=torch.float8_e4m3fn)[0]
+    a, b = q_consumer.view(torch.uint8).to(torch.int32), q_oracle.view(torch.uint8).to(torch.int32)
+    same = (a == b).float().mean().item()
+    assert same >= 0.95
+    assert ((a - b).abs() <= 1).all()
