@@ -311,22 +311,24 @@ def probe_moe(mode="both"):
         print(f"| {label} | {best[0] * 1e3:.1f} | {best[1] * 1e3:.1f} | {best[1] * 1e3 / (3 * E):.2f} |")
 
 
-def probe_oneshot(batches, tokens):
-    """oneshot() on a transformers LlamaForCausalLM with two Llama-3-8B-shaped decoder layers (random weights,
-    vocabulary cut to 32000), GPTQ W4A16 with the modifier's defaults, `batches` x `tokens` calibration tokens:
-    wall time per layer with both passes of the sequential pipeline, staged and unstaged Hessian launches, and the
-    model's own forward for comparison.  Prints a table."""
+def probe_oneshot(batches, tokens, layers=2, vocab=32000):
+    """oneshot() on a transformers LlamaForCausalLM with `layers` Llama-3-8B-shaped decoder layers (random
+    weights), GPTQ W4A16 with the modifier's defaults, `batches` x `tokens` calibration tokens: wall time per layer
+    with both passes of the sequential pipeline, the time inside the epoch-end events (observers + quantize_weight),
+    peak device memory, and the model's own forward for comparison.  With more than 4 layers (the whole-model run:
+    --layers 32 --vocab 128256) only the default configuration runs, once.  Prints a table."""
     import torch
     from transformers import LlamaConfig, LlamaForCausalLM
 
     from llmcompressor_amd import oneshot
+    from llmcompressor_amd.core import LifecycleCallbacks
     from llmcompressor_amd.modifiers.gptq import GPTQModifier
 
-    layers = 2
+    whole = layers > 4
     cfg = LlamaConfig(hidden_size=HIDDEN, intermediate_size=INTER, num_hidden_layers=layers, num_attention_heads=32,
-                      num_key_value_heads=8, vocab_size=32000, max_position_embeddings=max(4096, tokens))
+                      num_key_value_heads=8, vocab_size=vocab, max_position_embeddings=max(4096, tokens))
     torch.manual_seed(0)
-    data = [{"input_ids": torch.randint(0, 32000, (1, tokens))} for _ in range(batches)]
+    data = [{"input_ids": torch.randint(0, vocab, (1, tokens))} for _ in range(batches)]
 
     def make():
         with torch.device("cuda"):
@@ -334,30 +336,55 @@ def probe_oneshot(batches, tokens):
 
     model = make()
     with torch.no_grad():
-        for rep in range(2):
+        for rep in range(1 if whole else 2):
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             for d in data:
-                model(d["input_ids"].cuda(), use_cache=False)
+                model(d["input_ids"].cuda(), use_cache=False, logits_to_keep=1)
             torch.cuda.synchronize()
             fwd = time.perf_counter() - t0
     del model
-    print(f"| oneshot GPTQ W4A16, {layers} layers of 4096/14336, {batches} x {tokens} tokens | s | ms per layer |")
-    print("|---|---|---|")
-    print(f"| model forward alone, one pass over the data (embedding and lm_head included) | {fwd:.2f} | {fwd / layers * 1e3:.0f} |")
-    for label, stage in (("Hessian launches of 65536 staged tokens (default)", 65536), ("one Hessian launch per hook call", 0)):
+    torch.cuda.empty_cache()
+    print(f"| oneshot GPTQ W4A16, {layers} layers of 4096/14336, vocabulary {vocab}, {batches} x {tokens} tokens | s | "
+          "ms per layer | s inside epoch-end events | peak GiB |")
+    print("|---|---|---|---|---|")
+    print(f"| model forward alone, one pass over the data (embedding included, lm_head on the last token) | {fwd:.2f} | "
+          f"{fwd / layers * 1e3:.0f} | | |")
+    variants = [("Hessian launches of 65536 staged tokens (default)", 65536)]
+    if not whole:
+        variants.append(("one Hessian launch per hook call", 0))
+    raw_end = LifecycleCallbacks.sequential_epoch_end
+    for label, stage in variants:
         best = None
-        for rep in range(2):
+        for rep in range(1 if whole else 2):
             model = make()
+            spent = [0.0]
+
+            def timed_end(*args, **kw):
+                torch.cuda.synchronize()
+                t = time.perf_counter()
+                out = raw_end(*args, **kw)
+                torch.cuda.synchronize()
+                spent[0] += time.perf_counter() - t
+                return out
+
+            LifecycleCallbacks.sequential_epoch_end = staticmethod(timed_end)
+            torch.cuda.reset_peak_memory_stats()
             torch.cuda.synchronize()
             t0 = time.perf_counter()
-            oneshot(model=model, dataset=data, recipe=GPTQModifier(targets="Linear", scheme="W4A16", ignore=["lm_head"],
-                                                                     hessian_batch_tokens=stage))
+            try:
+                oneshot(model=model, dataset=data, recipe=GPTQModifier(targets="Linear", scheme="W4A16", ignore=["lm_head"],
+                                                                         hessian_batch_tokens=stage))
+            finally:
+                LifecycleCallbacks.sequential_epoch_end = raw_end
             torch.cuda.synchronize()
             dt = time.perf_counter() - t0
-            best = dt if best is None else min(best, dt)
+            peak = torch.cuda.max_memory_allocated() / 2 ** 30
+            if best is None or dt < best[0]:
+                best = (dt, spent[0], peak)
             del model
-        print(f"| {label} | {best:.2f} | {best / layers * 1e3:.0f} |")
+            torch.cuda.empty_cache()
+        print(f"| {label} | {best[0]:.2f} | {best[0] / layers * 1e3:.0f} | {best[1]:.2f} | {best[2]:.1f} |")
 
 
 def main():
@@ -386,6 +413,8 @@ def main():
     ap.add_argument("--probe-oneshot", action="store_true",
                     help="print end-to-end oneshot timings on a transformers Llama with two 8B-shaped layers "
                     "(--batches x --tokens calibration tokens) instead of the bench line")
+    ap.add_argument("--layers", type=int, default=2, help="--probe-oneshot: decoder layers of the model (config: 32)")
+    ap.add_argument("--vocab", type=int, default=32000, help="--probe-oneshot: vocabulary size (config: 128256)")
     ap.add_argument("--probe-moe", action="store_true",
                     help="print the timings of one 128-expert MoE layer through GPTQModifier instead of the bench line")
     a = ap.parse_args()
@@ -412,7 +441,7 @@ def main():
         probe_moe(a.moe_mode)
         return
     if a.probe_oneshot:
-        probe_oneshot(a.batches, a.tokens)
+        probe_oneshot(a.batches, a.tokens, a.layers, a.vocab)
         return
     if a.probe_dominant:
         from llmcompressor_amd import ops
