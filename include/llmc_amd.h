@@ -306,6 +306,23 @@ int llmc_gptq_quantize_grouped(const void* const* weight, int32_t w_dtype, int32
                                int32_t blocksize, void* const* out_weight, int64_t ldo, float* loss_out,
                                void* workspace, int64_t workspace_bytes, void* stream);
 
+/* ---- fp32 product of the lazy trailing updates ----------------------------------------------------
+ * Replaces the matmul of W[:, i2:] -= Err1.matmul(Hinv[i1:i2, i2:]) (gptq_quantize.py:245) and the products
+ * inside torch.linalg.cholesky / cholesky_inverse of gptq_quantize.py:153-155:
+ *     C[M,N] = alpha * A[M,Kc] * B' + beta * C,  B' = B[Kc,N] (trans_b = 0) or B[N,Kc]^T (trans_b = 1),
+ * all row-major fp32.  Products whose shape is a whole number of 128- or 256-wide tiles run on the 16-bit
+ * matrix cores with every operand split into three bf16 terms (six partial products, the dropped ones below
+ * the rounding of an fp32 product); other shapes, and every shape with LLMC_SGEMM_FP32_MFMA, use the fp32
+ * matrix instruction.  Structure flags are tile-granular promises about exact zeros in the operands. */
+enum {
+  LLMC_SGEMM_C_LOWER = 1,      /* only tiles touching the lower triangle of C are computed and written     */
+  LLMC_SGEMM_A_LOWER_TRI = 2,  /* A[m,k] == 0 for k > m                                                    */
+  LLMC_SGEMM_B_LOWER_TRI = 4,  /* B'[k,n] == 0 for k < n                                                   */
+  LLMC_SGEMM_FP32_MFMA = 8     /* never split: v_mfma_f32_32x32x2_f32 only                                 */
+};
+int llmc_sgemm(const float* A, int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc, int64_t M,
+               int64_t N, int64_t Kc, float alpha, float beta, int32_t trans_b, int32_t flags, void* stream);
+
 /* ---- SparseGPT (a "next" row: the same Hessian / Cholesky / column-loop skeleton) ----------
  * Replaces the loop of sparsify_weight (src/llmcompressor/modifiers/pruning/sparsegpt/
  * sgpt_sparsify.py:125-213); the factor U comes from llmc_gptq_hinv (:97-118 are the same

@@ -448,7 +448,7 @@ extern "C" int llmc_gptq_hinv_grouped(const float* const* H, int64_t ldh, int32_
       GemmF32 g = {};
       g.A = A21; g.lda = Kp; g.B = A + (int64_t)c0 * Kp + c0; g.ldb = Kp; g.C = A21; g.ldc = Kp;
       g.M = M; g.N = NB; g.Kc = NB; g.alpha = 1.f; g.beta = 0.f; g.trans_b = 1;
-      g.batch = n; g.stride_a = mat; g.stride_b = mat; g.stride_c = mat;
+      g.batch = 1; g.batch2 = n; g.stride2_a = mat; g.stride2_b = mat; g.stride2_c = mat;
       int rc = llmc_gemm_f32(g, st);
       if (rc) return rc;
       const int nrem = k0 + pw - (c0 + NB);
@@ -456,7 +456,7 @@ extern "C" int llmc_gptq_hinv_grouped(const float* const* H, int64_t ldh, int32_
         GemmF32 u = {};
         u.A = A21; u.lda = Kp; u.B = A21; u.ldb = Kp; u.C = A + (int64_t)(c0 + NB) * Kp + c0 + NB; u.ldc = Kp;
         u.M = M; u.N = nrem; u.Kc = NB; u.alpha = -1.f; u.beta = 1.f; u.trans_b = 1; u.c_lower = 1;
-        u.batch = n; u.stride_a = mat; u.stride_b = mat; u.stride_c = mat;
+        u.batch = 1; u.batch2 = n; u.stride2_a = mat; u.stride2_b = mat; u.stride2_c = mat;
         rc = llmc_gemm_f32(u, st);
         if (rc) return rc;
       }
@@ -467,7 +467,7 @@ extern "C" int llmc_gptq_hinv_grouped(const float* const* H, int64_t ldh, int32_
       GemmF32 t = {};
       t.A = P; t.lda = Kp; t.B = P; t.ldb = Kp; t.C = A + (int64_t)(k0 + pw) * ((int64_t)Kp + 1); t.ldc = Kp;
       t.M = M2; t.N = M2; t.Kc = pw; t.alpha = -1.f; t.beta = 1.f; t.trans_b = 1; t.c_lower = 1;
-      t.batch = n; t.stride_a = mat; t.stride_b = mat; t.stride_c = mat;
+      t.batch = 1; t.batch2 = n; t.stride2_a = mat; t.stride2_b = mat; t.stride2_c = mat;
       const int rc = llmc_gemm_f32(t, st);
       if (rc) return rc;
     }

@@ -34,3 +34,10 @@ struct GemmF32 {
 
 // enqueue on `st`; returns 0 or 1000 + hipError_t
 int llmc_gemm_f32(const GemmF32& g, hipStream_t st);
+
+// The same product on the 16-bit matrix cores (every operand split into three bf16 planes, six partial
+// products; see gemm_x3.hip): taken when the shape is a whole number of 128- or 256-wide tiles and big enough
+// to fill the chip.  Returns -1 when the product is left to the fp32 matrix instruction.
+int llmc_gemm_x3(const GemmF32& g, hipStream_t st);
+// 0 = never use the split product, 1 = whenever it applies (default)
+void llmc_gemm_x3_set_mode(int mode);

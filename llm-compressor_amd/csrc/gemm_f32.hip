@@ -229,9 +229,39 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32 g, int vec) {
 
 }  // namespace
 
+static int gemm_f32_mfma(const GemmF32& g, hipStream_t st);
+
 int llmc_gemm_f32(const GemmF32& g, hipStream_t st) {
   if (g.M <= 0 || g.N <= 0 || g.batch <= 0) return 0;
   if (g.trans_a && (g.trans_b || g.a_lower_tri)) return 1000 + (int)hipErrorInvalidValue;
+  const int rc = llmc_gemm_x3(g, st);
+  if (rc >= 0) return rc;
+  return gemm_f32_mfma(g, st);
+}
+
+// C[M,N] = alpha * A * B' + beta * C for callers outside the library (the product of the lazy trailing
+// update, W[:, i2:] -= Err1 @ Hinv[i1:i2, i2:]); flags: 1 = only the lower triangle of C, 2 = A lower
+// triangular, 4 = B' zero above... (see include/llmc_amd.h), 8 = force the fp32 matrix instruction
+extern "C" int llmc_sgemm(const float* A, int64_t lda, const float* B, int64_t ldb, float* C, int64_t ldc, int64_t M,
+                          int64_t N, int64_t Kc, float alpha, float beta, int32_t trans_b, int32_t flags,
+                          void* stream) {
+  LLMC_CHECK_ARG(A != nullptr && lda > 0, 1);
+  LLMC_CHECK_ARG(B != nullptr && ldb > 0, 3);
+  LLMC_CHECK_ARG(C != nullptr && ldc >= N, 5);
+  LLMC_CHECK_ARG(M >= 0 && N >= 0 && Kc >= 0 && M < (1 << 30) && N < (1 << 30) && Kc < (1 << 30), 7);
+  LLMC_CHECK_ARG(lda >= Kc && ldb >= (trans_b ? Kc : N), 2);
+  LLMC_CHECK_ARG(flags >= 0 && flags < 16, 13);
+  GemmF32 g = {};
+  g.A = A; g.lda = lda; g.B = B; g.ldb = ldb; g.C = C; g.ldc = ldc;
+  g.M = (int)M; g.N = (int)N; g.Kc = (int)Kc; g.alpha = alpha; g.beta = beta; g.trans_b = trans_b ? 1 : 0;
+  g.c_lower = flags & 1; g.a_lower_tri = (flags >> 1) & 1; g.b_lower_tri = (flags >> 2) & 1; g.batch = 1;
+  if (g.M == 0 || g.N == 0) return 0;
+  hipStream_t st = (hipStream_t)stream;
+  if (flags & 8) return gemm_f32_mfma(g, st);
+  return llmc_gemm_f32(g, st);
+}
+
+static int gemm_f32_mfma(const GemmF32& g, hipStream_t st) {
   const int nb2 = g.batch2 > 1 ? g.batch2 : 1;
   const int vec = ((g.lda & 3) == 0 && (g.ldb & 3) == 0 && (((uintptr_t)g.A | (uintptr_t)g.B) & 15) == 0 &&
                    (g.stride_a & 3) == 0 && (g.stride_b & 3) == 0 && (g.Kc & 3) == 0 &&

@@ -811,7 +811,7 @@ extern "C" int llmc_gptq_quantize_grouped(const void* const* weight, int32_t w_d
         GemmF32 g = {};
         g.A = p.E; g.lda = ldE; g.B = U + i1 * ldu + i2; g.ldb = ldu; g.C = Wf + i2; g.ldc = K;
         g.M = (int)R; g.N = (int)(gend - i2); g.Kc = count; g.alpha = -1.f; g.beta = 1.f;
-        g.batch = n; g.stride_a = R * (int64_t)ldE; g.stride_b = u_stride; g.stride_c = R * K;
+        g.batch = 1; g.batch2 = n; g.stride2_a = R * (int64_t)ldE; g.stride2_b = u_stride; g.stride2_c = R * K;
         const int rc = llmc_gemm_f32(g, st);
         if (rc) return rc;
       }
@@ -820,7 +820,7 @@ extern "C" int llmc_gptq_quantize_grouped(const void* const* weight, int32_t w_d
       GemmF32 g = {};
       g.A = E; g.lda = ldE; g.B = U + g0 * ldu + gend; g.ldb = ldu; g.C = Wf + gend; g.ldc = K;
       g.M = (int)R; g.N = (int)(K - gend); g.Kc = (int)(gend - g0); g.alpha = -1.f; g.beta = 1.f;
-      g.batch = n; g.stride_a = R * (int64_t)ldE; g.stride_b = u_stride; g.stride_c = R * K;
+      g.batch = 1; g.batch2 = n; g.stride2_a = R * (int64_t)ldE; g.stride2_b = u_stride; g.stride2_c = R * K;
       const int rc = llmc_gemm_f32(g, st);
       if (rc) return rc;
     }

@@ -85,6 +85,7 @@ SIGNATURES.update({
     "llmc_mse_observe_groups": [_P, _I32, _I64, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _F64, _I32, _F32,
                                 _F32, _P, _P, _P, _I64, _P],
     "llmc_sumsq_workspace_bytes": [_I64],
+    "llmc_sgemm": [_P, _I64, _P, _I64, _P, _I64, _I64, _I64, _I64, _F32, _F32, _I32, _I32, _P],
     "llmc_sumsq_accumulate": [_P, _I32, _I64, _I64, _I64, _P, _P, _I64, _P],
     "llmc_sumsq_accumulate_noalloc": [_P, _I32, _I64, _I64, _I64, _P, _P],
     "llmc_imatrix_observe_groups": [_P, _I32, _I64, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _F64, _I32, _F32,

@@ -638,3 +638,22 @@ def imatrix_observe_blocks(w, bh: int, bw: int, fmt: int, bits: int, symmetric: 
             mx.data_ptr(), ws.data_ptr(), ws.numel(), _stream(w))
     _lib.check(rc, "llmc_imatrix_observe_blocks")
     return mn, mx
+
+
+SGEMM_C_LOWER, SGEMM_A_LOWER_TRI, SGEMM_B_LOWER_TRI, SGEMM_FP32_MFMA = 1, 2, 4, 8
+
+
+def sgemm_(C: torch.Tensor, A: torch.Tensor, B: torch.Tensor, alpha: float = 1.0, beta: float = 0.0,
+           trans_b: bool = False, flags: int = 0):
+    """C (fp32 [M,N], in place) = alpha * A @ (B.T if trans_b else B) + beta * C on the matrix cores."""
+    _require_gpu(C, A, B)
+    for t in (C, A, B):
+        assert t.dtype == torch.float32 and t.ndim == 2 and t.stride(1) == 1
+    M, Kc = A.shape
+    N = B.shape[0] if trans_b else B.shape[1]
+    assert C.shape == (M, N) and (B.shape[1] if trans_b else B.shape[0]) == Kc
+    with torch.cuda.device(C.device):
+        rc = _lib.lib().llmc_sgemm(A.data_ptr(), A.stride(0), B.data_ptr(), B.stride(0), C.data_ptr(), C.stride(0),
+                                   M, N, Kc, float(alpha), float(beta), 1 if trans_b else 0, int(flags), _stream(C))
+    _lib.check(rc, "llmc_sgemm")
+    return C
