@@ -45,47 +45,71 @@ LINEARS = [  # name, out_features, in_features
 ]
 GROUP = 128
 MFMA_BF16_PEAK_TFLOPS = 2500.0
-# HBM bytes per launch of the dominant kernel from FETCH_SIZE / WRITE_SIZE counter runs scaled by a
-# 1 GiB copy (profiles/hessian_syrk_k14336_t65536_hbm_traffic.md), keyed by tokens per launch
-DOMINANT_TRAFFIC_BYTES = {65536: 30.3e9}
+
+
+def dominant_traffic_bytes(tokens_per_launch: int):
+    """HBM bytes per launch of the dominant kernel, from the FETCH_SIZE / WRITE_SIZE counter runs whose raw
+    averages and calibration are kept next to their summary (profiles/hessian_syrk_k14336_t65536_hbm_traffic.json);
+    None when no counter run exists for this launch size."""
+    path = os.path.join(ROOT, "profiles", "hessian_syrk_k14336_t65536_hbm_traffic.json")
+    try:
+        with open(path) as f:
+            rec = json.load(f)
+    except OSError:
+        return None
+    if int(rec.get("tokens_per_launch", -1)) != int(tokens_per_launch) or int(rec.get("K", -1)) != INTER:
+        return None
+    return float(rec["FETCH_SIZE_avg_per_dispatch"]) * rec["FETCH_SIZE_unit_bytes"] + \
+        float(rec["WRITE_SIZE_avg_per_dispatch"]) * rec["WRITE_SIZE_unit_bytes"]
 
 
 def cpu_baseline(tokens: int):
-    """The oracle (a port of the reference's torch CPU path) on a bounded sample of the same workload."""
+    """The oracle (a port of the reference's torch CPU path) on a bounded sample of the same workload: one
+    warm-up, then the median of three timings for each half of the metric.  Threads: the host's CPU count,
+    capped at the 16 cores one GPU's share of the box provides."""
+    import statistics
+
     import torch
 
     from oracle import gptq as G
     from oracle import observers as O
     from oracle import qformat as F
 
-    cores = os.cpu_count() or 1
-    cores = min(cores, 16)
+    host_cpus = os.cpu_count() or 1
+    cores = min(host_cpus, 16)
     torch.set_num_threads(cores)
     torch.manual_seed(0)
     K = HIDDEN
-    calls = 8
+    calls = 4
     x = torch.randn(calls, 1, tokens, K).bfloat16()
     H = G.make_empty_hessian(K)
     n = torch.zeros(())
     G.accumulate_hessian(x[0], H, n)  # warm-up
-    t0 = time.perf_counter()
-    for i in range(calls):
-        G.accumulate_hessian(x[i], H, n)
-    t_h = (time.perf_counter() - t0) / calls
+    t_hs = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        for i in range(calls):
+            G.accumulate_hessian(x[i], H, n)
+        t_hs.append((time.perf_counter() - t0) / calls)
+    t_h = statistics.median(t_hs)
     w = (torch.randn(HIDDEN, K) * 0.02).bfloat16()
     args = F.QArgs(num_bits=4, strategy="group", group_size=GROUP, actorder="weight")
-    obs = O.Observer("memoryless_minmax", "weight", args)
-    t0 = time.perf_counter()
-    obs(w)
-    G.quantize_weight(w, obs, args, H / n)
-    t_q = time.perf_counter() - t0
+    t_qs = []
+    for rep in range(4):  # the first one is the warm-up
+        obs = O.Observer("memoryless_minmax", "weight", args)
+        t0 = time.perf_counter()
+        obs(w)
+        G.quantize_weight(w, obs, args, H / n)
+        t_qs.append(time.perf_counter() - t0)
+    t_q = statistics.median(t_qs[1:])
     return {
         "value": round(2.0 * tokens * K * K / t_h / 1e12, 4),
         "unit": "TFLOP/s",
         "cores": cores,
+        "host_cpus": host_cpus,
         "kind": "port",
-        "sample": f"{calls} accumulate_hessian calls of [1,{tokens},{K}] bf16 (fp32 GEMM) + 1 quantize_weight of a "
-        f"{HIDDEN}x{K} Linear (W4A16 g128, actorder static)",
+        "sample": f"median of 3 x ({calls} accumulate_hessian calls of [1,{tokens},{K}] bf16, fp32 GEMM) and median of 3 "
+        f"quantize_weight of a {HIDDEN}x{K} Linear (W4A16 g128, actorder static), one warm-up each, {cores} torch threads",
         "quantize_weight_ms_per_linear": round(t_q * 1e3, 1),
     }
 
@@ -617,7 +641,7 @@ def main():
             # cores actually do per launch, next to the algorithmic figure of the reference's full GEMM
             "executed_tflops": round(dom_exec_flop / (dom_ms * 1e-3) / 1e12, 2),
             "executed_frac": round(dom_exec_flop / (dom_ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
-            "traffic": DOMINANT_TRAFFIC_BYTES.get(int(dom_T)),
+            "traffic": dominant_traffic_bytes(int(dom_T)),
             "algorithmic_hbm_bytes": 2.0 * dom_T * INTER + 8.0 * INTER * INTER,
             "avg_launch_ms": round(dom_ms, 4),
             "launches_timed": len(dom_events),
