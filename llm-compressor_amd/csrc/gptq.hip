@@ -6,7 +6,8 @@
 // lane, held in registers.  The block's 128x128 slice of U sits in LDS.  Per
 // column: the owning lane's value is broadcast inside the team, every lane
 // quantises it, forms err = (w - q)/U[i][i] and subtracts err * U[i][c] from its
-// own 8 columns (U is zero below the diagonal, so no masking is needed).
+// own 8 columns (U is zero below the diagonal, so no masking is needed).  That is the layout of the
+// SparseGPT kernel below; the quantiser's kernel spreads a row over 4 lanes and is described at its constants.
 // After the block, W[:, i2:] -= Err * U[i1:i2, i2:] runs as an fp32 MFMA GEMM.
 #include <vector>
 
@@ -53,6 +54,49 @@ __global__ __launch_bounds__(256) void gptq_prepare_w_kernel(const void* __restr
   Wf[(int64_t)r * K + c] = v;
 }
 
+// The block's [GB][GB] slice of U into LDS, zero outside the upper triangle and past `count`.  Addresses are
+// clamped into the block instead of predicated, so the loads of a batch are all in flight together.
+__device__ __forceinline__ void load_u_block(float* __restrict__ Hs, const float* __restrict__ U, int64_t ldu,
+                                             int i1, int count, int tid) {
+  const float* base = U + (int64_t)i1 * ldu + i1;
+  if (count == GB && (ldu & 3) == 0 && (i1 & 3) == 0 && ((uintptr_t)U & 15) == 0) {
+    // full block, rows 16-byte aligned: one batch of 16 four-wide loads per thread
+    constexpr int PER = GB * GB / 4 / 256;
+    const int c4 = (tid % (GB / 4)) * 4, r0 = tid / (GB / 4);
+    float4 v[PER];
+#pragma unroll
+    for (int b = 0; b < PER; ++b) v[b] = *(const float4*)&base[(int64_t)(b * (1024 / GB) + r0) * ldu + c4];
+#pragma unroll
+    for (int b = 0; b < PER; ++b) {
+      const int i = b * (1024 / GB) + r0;
+      float4 o;
+      o.x = c4 + 0 >= i ? v[b].x : 0.f;
+      o.y = c4 + 1 >= i ? v[b].y : 0.f;
+      o.z = c4 + 2 >= i ? v[b].z : 0.f;
+      o.w = c4 + 3 >= i ? v[b].w : 0.f;
+      *(float4*)&Hs[i * GB + c4] = o;
+    }
+    return;
+  }
+  const int c = tid % GB;
+  const int cc = c < count ? c : count - 1;
+  constexpr int BATCH = 16;
+  for (int it0 = 0; it0 < GB * GB / 256; it0 += BATCH) {
+    float v[BATCH];
+#pragma unroll
+    for (int b = 0; b < BATCH; ++b) {
+      const int i = (it0 + b) * (256 / GB) + tid / GB;
+      const int ic = i < count ? i : count - 1;
+      v[b] = base[(int64_t)ic * ldu + cc];
+    }
+#pragma unroll
+    for (int b = 0; b < BATCH; ++b) {
+      const int i = (it0 + b) * (256 / GB) + tid / GB;
+      Hs[(it0 + b) * 256 + tid] = (c >= i && c < count) ? v[b] : 0.f;
+    }
+  }
+}
+
 struct GptqBlockParams {
   float* Wf;        // [R,K] fp32 work copy (permuted columns)
   int R, K;
@@ -76,9 +120,212 @@ struct GptqBlockParams {
   int64_t u_stride;
 };
 
+// Layout of the quantiser's block kernel: a row is spread over a team of QTEAM lanes (one DPP quad), each
+// holding QCPL columns of the block in registers as QNCH runs of QG neighbouring columns; run j of lane t
+// covers columns j*QCW + t*QG .. +QG-1.  The lane that owns a run quantises its QG columns by itself (the
+// serial chain of a row never crosses lanes inside a run), then the QG scaled errors are broadcast to the team
+// once and every lane applies them, in column order, to the runs that are still open.
+constexpr int QTEAM = 4;
+constexpr int QCPL = GB / QTEAM;   // 32 columns per lane
+constexpr int QG = 4;              // neighbouring columns per run
+constexpr int QNCH = QCPL / QG;    // 8 runs per lane
+constexpr int QCW = QTEAM * QG;    // 16 columns per round of the team
+constexpr int Q_ROWS_PER_WG = 256 / QTEAM;
+
+// ---- divisions of the column loop.  x / s goes through the hoisted reciprocal y of s (see make_fastdiv():
+// the steps of the correctly rounded division with the divisor's part taken out).  The short form gives the
+// IEEE quotient while |q| stays in [2^-40, 2^100) or both x and q are zero; `worst` collects, without a
+// branch, how far outside that window any quotient of a run fell, and the caller redoes the run with plain
+// divisions when it did.  A divisor outside make_fastdiv()'s range has a NaN reciprocal, which lands outside
+// the window as well.
+constexpr uint32_t QDIV_LO = 0x2b800000u;  // bits of 2^-40
+constexpr uint32_t QDIV_SPAN = 0x71800000u - QDIV_LO;  // up to 2^100
+__device__ __forceinline__ float shared_reciprocal(float s) {
+  const FastDiv d = make_fastdiv(s);
+  return d.ok ? d.y : __builtin_nanf("");
+}
+template <bool EXACT>
+__device__ __forceinline__ float run_div(float x, float s, float y, uint32_t& worst) {
+  if (EXACT) return x / s;
+  float q = x * y;
+  float r = fmaf(-s, q, x);
+  q = fmaf(r, y, q);
+  r = fmaf(-s, q, x);
+  q = fmaf(r, y, q);
+  const uint32_t qb = __float_as_uint(q) & 0x7fffffffu, xb = __float_as_uint(x) & 0x7fffffffu;
+  const uint32_t t = (qb | xb) == 0u ? QDIV_LO : qb;
+  worst = max(worst, t - QDIV_LO);
+  return q;
+}
+
+template <int SD>
+__device__ __forceinline__ float round_sd(float x) {
+  if (SD == LLMC_BF16) return round16_finite<LLMC_BF16>(x);
+  if (SD == LLMC_F16) return round16_finite<LLMC_F16>(x);
+  return x;
+}
+
+struct QRun {
+  float4 q, e;  // dequantised values and scaled errors of the run's QG columns
+};
+
+// One run of QG neighbouring columns of one row, start to finish inside a lane: column m is quantised, its
+// scaled error err = (w - q) / d is applied to the columns of the run behind it (one fused multiply-subtract
+// per element; the reference rounds the outer product before it subtracts, the fused form keeps the product
+// exact), and so on.  u0..u2 are rows 0..2 of the run's QG x QG diagonal block of U.
+template <int FMT, int SD, bool HAS_ZP, bool EXACT>
+__device__ __forceinline__ QRun gptq_run(float4 w, float4 s, float4 y, float4 z, float4 d, float4 dy,
+                                         float4 u0, float4 u1, float4 u2, const QFormat& f, uint32_t& worst) {
+  QRun o;
+  auto column = [&](float wv, float sc, float yc, float zp, float dc, float dyc, float& q, float& err) {
+    // quantize_value() with the quotient formed by run_div()
+    float v = run_div<EXACT>(wv, sc, yc, worst);
+    v = HAS_ZP ? v + zp : v + 0.0f;
+    const float qc = round_to_grid(v, f);
+    float dq = qc;
+    if (HAS_ZP) dq = round_sd<SD>(dq - zp);
+    q = round_sd<SD>(dq * sc);
+    err = run_div<EXACT>(__fsub_rn(wv, q), dc, dyc, worst);
+  };
+  column(w.x, s.x, y.x, z.x, d.x, dy.x, o.q.x, o.e.x);
+  w.y = fmaf(-o.e.x, u0.y, w.y);
+  w.z = fmaf(-o.e.x, u0.z, w.z);
+  w.w = fmaf(-o.e.x, u0.w, w.w);
+  column(w.y, s.y, y.y, z.y, d.y, dy.y, o.q.y, o.e.y);
+  w.z = fmaf(-o.e.y, u1.z, w.z);
+  w.w = fmaf(-o.e.y, u1.w, w.w);
+  column(w.z, s.z, y.z, z.z, d.z, dy.z, o.q.z, o.e.z);
+  w.w = fmaf(-o.e.z, u2.w, w.w);
+  column(w.w, s.w, y.w, z.w, d.w, dy.w, o.q.w, o.e.w);
+  return o;
+}
+static_assert(QG == 4, "gptq_run() is written out for runs of four columns");
+
+// the rare way round: plain divisions, kept out of line
+template <int FMT, int SD, bool HAS_ZP>
+__device__ __noinline__ QRun gptq_run_exact(float4 w, float4 s, float4 z, float4 d, float4 u0, float4 u1,
+                                            float4 u2, int bits) {
+  const QFormat f = make_qformat(FMT, bits);
+  uint32_t unused = 0;
+  return gptq_run<FMT, SD, HAS_ZP, true>(w, s, s, z, d, d, u0, u1, u2, f, unused);
+}
+
+// the registers of one lane: QCPL columns of one row, their scales, the scales' reciprocals, zero points
+template <bool HAS_ZP>
+struct QLane {
+  float4 w[QNCH], sv[QNCH], yv[QNCH], zv[HAS_ZP ? QNCH : 1];
+};
+
+// Round J of the team: for each lane in turn, its run J is quantised and the errors applied to everything
+// that is still open.  Columns at or past `count` hold w = 0, scale 1, d = 1 and zero rows of U: they
+// quantise to zero with zero error, so only the stores look at `count`.
+template <int J, int FMT, int SD, bool HAS_ZP>
+__device__ __forceinline__ void gptq_round(QLane<HAS_ZP>& r, const float* __restrict__ Hs,
+                                           const float* __restrict__ Dd, const float* __restrict__ Dy, int tl,
+                                           int count, bool live, float* __restrict__ wrow,
+                                           float* __restrict__ erow, const QFormat& f, int bits, float& loss) {
+#pragma unroll 1
+  for (int li = 0; li < QTEAM; ++li) {
+    const int i0 = J * QCW + li * QG;  // first column of this run
+    if (i0 >= count) break;            // uniform across the workgroup
+    const float* diag = Hs + i0 * GB + i0;
+    const float4 d = *(const float4*)&Dd[i0], dy = *(const float4*)&Dy[i0];
+    const float4 u0 = *(const float4*)&diag[0], u1 = *(const float4*)&diag[GB], u2 = *(const float4*)&diag[2 * GB];
+    const float4 z = r.zv[HAS_ZP ? J : 0];
+    const bool own = tl == li;
+    // every lane runs the chain on its own run J; only the owner's is due, the others' results are dropped
+    uint32_t worst = 0;
+    QRun o = gptq_run<FMT, SD, HAS_ZP, false>(r.w[J], r.sv[J], r.yv[J], z, d, dy, u0, u1, u2, f, worst);
+    if (own && worst >= QDIV_SPAN) o = gptq_run_exact<FMT, SD, HAS_ZP>(r.w[J], r.sv[J], z, d, u0, u1, u2, bits);
+    if (own && live) {
+      if (i0 + 0 < count) wrow[i0 + 0] = o.q.x;
+      if (i0 + 1 < count) wrow[i0 + 1] = o.q.y;
+      if (i0 + 2 < count) wrow[i0 + 2] = o.q.z;
+      if (i0 + 3 < count) wrow[i0 + 3] = o.q.w;
+      erow[i0 + 0] = o.e.x;
+      erow[i0 + 1] = o.e.y;
+      erow[i0 + 2] = o.e.z;
+      erow[i0 + 3] = o.e.w;
+    }
+    const float eb[QG] = {__shfl(o.e.x, li, QTEAM), __shfl(o.e.y, li, QTEAM), __shfl(o.e.z, li, QTEAM),
+                          __shfl(o.e.w, li, QTEAM)};
+#pragma unroll
+    for (int m = 0; m < QG; ++m) {
+      loss += eb[m] * eb[m];  // (w-q)^2 / d^2
+      // this round's run: lanes before the owner see zeros of U, the owner is already done
+      const float eff = own ? 0.f : eb[m];
+      const float* hrow = Hs + (i0 + m) * GB + tl * QG;
+      const float4 h = *(const float4*)&hrow[J * QCW];
+      r.w[J].x = fmaf(-eff, h.x, r.w[J].x);
+      r.w[J].y = fmaf(-eff, h.y, r.w[J].y);
+      r.w[J].z = fmaf(-eff, h.z, r.w[J].z);
+      r.w[J].w = fmaf(-eff, h.w, r.w[J].w);
+#pragma unroll
+      for (int j2 = J + 1; j2 < QNCH; ++j2) {
+        const float4 g = *(const float4*)&hrow[j2 * QCW];
+        r.w[j2].x = fmaf(-eb[m], g.x, r.w[j2].x);
+        r.w[j2].y = fmaf(-eb[m], g.y, r.w[j2].y);
+        r.w[j2].z = fmaf(-eb[m], g.z, r.w[j2].z);
+        r.w[j2].w = fmaf(-eb[m], g.w, r.w[j2].w);
+      }
+    }
+  }
+}
+
+// the block's weights, scales and zero points of one lane; SDT = dtype of the stored scales
+template <int SDT, bool HAS_ZP>
+__device__ __forceinline__ void gptq_load_lane(QLane<HAS_ZP>& r, const GptqBlockParams& p, int row, int tl,
+                                               bool live) {
+  const int rowc = live ? row : p.R - 1;  // every load stays inside the arrays; dead lanes are blanked below
+  const float* wsrc = p.Wf + (int64_t)rowc * p.K + p.i1;
+  const int64_t sbase = ((int64_t)rowc / p.row_div) * p.srow;
+  const float gs = p.gscale ? p.gscale[0] : 1.f;
+  float w[QCPL], s[QCPL], zp[QCPL];
+  int gi[QCPL];
+  // three sweeps, each with all its loads in flight: group numbers, then what they index
+#pragma unroll
+  for (int e = 0; e < QCPL; ++e) gi[e] = 0;
+  if (p.g_idx) {
+#pragma unroll
+    for (int e = 0; e < QCPL; ++e) {
+      const int cb = (e / QG) * QCW + tl * QG + (e % QG);
+      gi[e] = p.g_idx[p.i1 + (cb < p.count ? cb : p.count - 1)];
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < QCPL; ++e) {
+    const int cb = (e / QG) * QCW + tl * QG + (e % QG);
+    w[e] = wsrc[cb < p.count ? cb : p.count - 1];
+    s[e] = load_as_f32<SDT>(p.scale, sbase + gi[e]);
+    zp[e] = HAS_ZP ? (float)p.zp[sbase + gi[e]] : 0.f;
+  }
+#pragma unroll
+  for (int e = 0; e < QCPL; ++e) {
+    const int cb = (e / QG) * QCW + tl * QG + (e % QG);
+    if (p.gscale) s[e] = s[e] / gs;
+    if (!live || cb >= p.count) {
+      w[e] = 0.f;
+      s[e] = 1.f;
+      zp[e] = 0.f;
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < QNCH; ++j) {
+    r.w[j] = make_float4(w[j * QG], w[j * QG + 1], w[j * QG + 2], w[j * QG + 3]);
+    r.sv[j] = make_float4(s[j * QG], s[j * QG + 1], s[j * QG + 2], s[j * QG + 3]);
+    r.yv[j] = make_float4(shared_reciprocal(s[j * QG]), shared_reciprocal(s[j * QG + 1]),
+                          shared_reciprocal(s[j * QG + 2]), shared_reciprocal(s[j * QG + 3]));
+    if (HAS_ZP) r.zv[j] = make_float4(zp[j * QG], zp[j * QG + 1], zp[j * QG + 2], zp[j * QG + 3]);
+  }
+  if (!HAS_ZP) r.zv[0] = make_float4(0.f, 0.f, 0.f, 0.f);
+}
+
 template <int FMT, int SD, bool HAS_ZP>
 __global__ __launch_bounds__(256) void gptq_block_kernel(GptqBlockParams p) {
-  extern __shared__ __attribute__((aligned(16))) float Hs[];  // [GB][GB], zero outside the upper triangle
+  // [GB][GB] slice of U, zero outside the upper triangle; then its diagonal and the diagonal's reciprocals
+  extern __shared__ __attribute__((aligned(16))) float Hs[];
+  float* Dd = Hs + GB * GB;
+  float* Dy = Dd + GB;
   if (p.items) {
     const GptqItem it = p.items[blockIdx.y];
     p.scale = it.scale; p.zp = it.zp; p.gscale = it.gscale; p.g_idx = it.g_idx;
@@ -88,79 +335,45 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(GptqBlockParams p) {
     p.loss_rows += (int64_t)blockIdx.y * p.R;
   }
   const int tid = threadIdx.x;
-  for (int e = tid; e < GB * GB; e += 256) {
-    const int i = e / GB, c = e % GB;
-    Hs[e] = (c >= i && c < p.count) ? p.U[(int64_t)(p.i1 + i) * p.ldu + p.i1 + c] : 0.f;
+  const int count = p.count;
+  load_u_block(Hs, p.U, p.ldu, p.i1, count, tid);
+  if (tid < GB) {
+    const float d = tid < count ? p.U[(int64_t)(p.i1 + tid) * p.ldu + p.i1 + tid] : 1.f;
+    Dd[tid] = d;
+    Dy[tid] = shared_reciprocal(d);
   }
-  const int tl = tid % TEAM;
-  const int row = blockIdx.x * ROWS_PER_WG + tid / TEAM;
+  const int tl = tid % QTEAM;
+  const int row = blockIdx.x * Q_ROWS_PER_WG + tid / QTEAM;
   const bool live = row < p.R;
   const QFormat f = make_qformat(FMT, p.bits);  // the format is a compile-time constant here
-  constexpr bool has_zp = HAS_ZP;
-  const float gs = p.gscale ? p.gscale[0] : 1.f;
+  float* wrow = p.Wf + (int64_t)row * p.K + p.i1;
+  float* erow = p.E + (int64_t)row * p.ldE;
 
-  float w[CPL], sv[CPL], zv[CPL], qv[CPL], ev[CPL];
-#pragma unroll
-  for (int e = 0; e < CPL; ++e) {
-    const int cb = tl * CPL + e;
-    const int c = p.i1 + cb;
-    w[e] = 0.f;
-    sv[e] = 1.f;
-    zv[e] = 0.f;
-    qv[e] = 0.f;
-    ev[e] = 0.f;
-    if (live && cb < p.count) {
-      w[e] = p.Wf[(int64_t)row * p.K + c];
-      const int64_t si = ((int64_t)row / p.row_div) * p.srow + (p.g_idx ? (int64_t)p.g_idx[c] : 0);
-      float s = load_rt(p.scale, si, p.scale_dt);
-      if (p.gscale) s = s / gs;
-      sv[e] = s;
-      if (has_zp) zv[e] = (float)p.zp[si];
-    }
-  }
+  QLane<HAS_ZP> r;
+  if (p.scale_dt == LLMC_BF16)
+    gptq_load_lane<LLMC_BF16, HAS_ZP>(r, p, row, tl, live);
+  else if (p.scale_dt == LLMC_F16)
+    gptq_load_lane<LLMC_F16, HAS_ZP>(r, p, row, tl, live);
+  else
+    gptq_load_lane<LLMC_F32, HAS_ZP>(r, p, row, tl, live);
   __syncthreads();
 
   float loss = 0.f;
-  for (int li = 0; li < TEAM; ++li) {
-    if (li * CPL >= p.count) break;
-#pragma unroll
-    for (int e = 0; e < CPL; ++e) {
-      const int i = li * CPL + e;
-      if (i < p.count) {  // uniform across the workgroup
-        const float wv = __shfl(w[e], li, TEAM);
-        const float s = __shfl(sv[e], li, TEAM);
-        const float zp = has_zp ? __shfl(zv[e], li, TEAM) : 0.f;
-        const float qc = quantize_value(wv, s, zp, has_zp, LLMC_F32, f);
-        const float q = dequantize_value(qc, s, zp, has_zp, SD);
-        const float d = Hs[i * GB + i];
-        const float diff = __fsub_rn(wv, q);
-        const float err = diff / d;
-        loss += err * err;  // (w-q)^2 / d^2
-        const float4 h0 = *(const float4*)&Hs[i * GB + tl * CPL];
-        const float4 h1 = *(const float4*)&Hs[i * GB + tl * CPL + 4];
-        // product rounded, then subtracted: the reference forms the outer product first
-        w[0] = __fsub_rn(w[0], __fmul_rn(err, h0.x));
-        w[1] = __fsub_rn(w[1], __fmul_rn(err, h0.y));
-        w[2] = __fsub_rn(w[2], __fmul_rn(err, h0.z));
-        w[3] = __fsub_rn(w[3], __fmul_rn(err, h0.w));
-        w[4] = __fsub_rn(w[4], __fmul_rn(err, h1.x));
-        w[5] = __fsub_rn(w[5], __fmul_rn(err, h1.y));
-        w[6] = __fsub_rn(w[6], __fmul_rn(err, h1.z));
-        w[7] = __fsub_rn(w[7], __fmul_rn(err, h1.w));
-        if (tl == li) {
-          qv[e] = q;
-          ev[e] = err;
-        }
-      }
-    }
-  }
+#define LLMC_ROUND(J) \
+  if (J * QCW < count) gptq_round<J, FMT, SD, HAS_ZP>(r, Hs, Dd, Dy, tl, count, live, wrow, erow, f, p.bits, loss);
+  LLMC_ROUND(0) LLMC_ROUND(1) LLMC_ROUND(2) LLMC_ROUND(3)
+  LLMC_ROUND(4) LLMC_ROUND(5) LLMC_ROUND(6) LLMC_ROUND(7)
+#undef LLMC_ROUND
+  static_assert(QNCH == 8, "one LLMC_ROUND per run of a lane");
 
   if (live) {
+    // the runs that were never reached carry no error into the trailing products
 #pragma unroll
-    for (int e = 0; e < CPL; ++e) {
-      const int cb = tl * CPL + e;
-      if (cb < p.count) p.Wf[(int64_t)row * p.K + p.i1 + cb] = qv[e];
-      p.E[(int64_t)row * p.ldE + cb] = ev[e];
+    for (int j = 0; j < QNCH; ++j) {
+      if (j * QCW >= count) {
+#pragma unroll
+        for (int m = 0; m < QG; ++m) erow[j * QCW + tl * QG + m] = 0.f;
+      }
     }
     if (tl == 0) p.loss_rows[row] += loss * 0.5f;
   }
@@ -312,10 +525,7 @@ __global__ __launch_bounds__(256) void sgpt_block_kernel(SgptParams p) {
   extern __shared__ __attribute__((aligned(16))) float Hs[];  // [GB][GB], zero outside the upper triangle
   __shared__ unsigned scratch[258];
   const int tid = threadIdx.x;
-  for (int e = tid; e < GB * GB; e += 256) {
-    const int i = e / GB, c = e % GB;
-    Hs[e] = (c >= i && c < p.count) ? p.U[(int64_t)(p.i1 + i) * p.ldu + p.i1 + c] : 0.f;
-  }
+  load_u_block(Hs, p.U, p.ldu, p.i1, p.count, tid);
   // unstructured: the block's threshold from its three histograms
   float thresh = 0.f;
   bool use_thresh = false;
@@ -631,7 +841,7 @@ extern "C" int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R
   p.E = E; p.loss_rows = loss_rows;
   p.items = nullptr; p.u_stride = 0;
 
-  const int smem = GB * GB * 4;
+  const int smem = (GB * GB + 2 * GB) * 4;
   void (*kern)(GptqBlockParams) = nullptr;
   const bool hz = zero_point != nullptr;
 #define LLMC_PICK(F, S)                                                         \
@@ -649,7 +859,7 @@ extern "C" int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R
   if (kern == nullptr) return -17;
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
   if (e != hipSuccess) return 1000 + (int)e;
-  const unsigned wgs = (unsigned)((R + ROWS_PER_WG - 1) / ROWS_PER_WG);
+  const unsigned wgs = (unsigned)((R + Q_ROWS_PER_WG - 1) / Q_ROWS_PER_WG);
   // Lazy updates on two levels.  After a block is quantised its scaled errors E_b update only the
   // columns left in its group of GROUP blocks (what the next block needs); the columns beyond the
   // group get the whole group's errors in one rank-(GROUP*bs) product.  Same sums as updating
@@ -776,7 +986,7 @@ extern "C" int llmc_gptq_quantize_grouped(const void* const* weight, int32_t w_d
   p.E = E; p.loss_rows = loss_rows;
   p.items = items; p.u_stride = u_stride;
 
-  const int smem = GB * GB * 4;
+  const int smem = (GB * GB + 2 * GB) * 4;
   void (*kern)(GptqBlockParams) = nullptr;
   const bool hz = zero_point != nullptr;
 #define LLMC_PICK(F, S)                                                         \
@@ -794,7 +1004,7 @@ extern "C" int llmc_gptq_quantize_grouped(const void* const* weight, int32_t w_d
   if (kern == nullptr) return -19;
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
   if (e != hipSuccess) return 1000 + (int)e;
-  const unsigned wgs = (unsigned)((R + ROWS_PER_WG - 1) / ROWS_PER_WG);
+  const unsigned wgs = (unsigned)((R + Q_ROWS_PER_WG - 1) / Q_ROWS_PER_WG);
   const int ldE = GROUP * GB;
   p.ldE = ldE;
   for (int64_t g0 = 0; g0 < K; g0 += (int64_t)GROUP * bs) {

@@ -161,6 +161,35 @@ def test_gptq_diagonal_hessian_is_rtn_bit_exact():
     assert loss.item() >= 0
 
 
+def test_gptq_extreme_magnitudes_take_the_plain_division_route():
+    """The column loop divides through hoisted reciprocals and falls back to plain divisions when a scale or a
+    quotient leaves the range in which the short form is exact.  Tiny weights beside ordinary ones, whole
+    groups of tiny weights (scale below 2^-60) and exact zeros force that route; with a diagonal Hessian the
+    result must still be round-to-nearest bit for bit."""
+    from llmcompressor_amd import ops
+
+    torch.manual_seed(3)
+    R, K, g = 24, 256, 32
+    w = torch.randn(R, K)
+    mag = torch.ones(R, K)
+    mag[:, 32:64] = 1e-30                      # a whole group far below the reciprocal's range
+    mag[:, 64:96:3] = 1e-20                    # tiny values beside ordinary ones: quotients below 2^-40
+    mag[:, 130:140] = 0.0                      # exact zeros: zero dividends
+    mag[5] = 1e-25
+    w = (w * mag).bfloat16()
+    args = F.QArgs(num_bits=4, strategy="group", group_size=g)
+    obs = O.Observer("memoryless_minmax", "weight", args)
+    obs(w)
+    scale, zp = F.calculate_qparams(obs.min_vals, obs.max_vals, args)
+    H = torch.diag(torch.linspace(1.0, 3.0, K))
+    U, dead, info = ops.gptq_hinv_(H.cuda())
+    g_idx = torch.arange(K, dtype=torch.int32) // g
+    wq, loss = ops.gptq_quantize(w.cuda(), U, scale.cuda(), None, ops.FMT_INT, 4, 1, K // g, g_idx=g_idx.cuda(), dead=dead)
+    rtn = F.fake_quantize(w.float(), scale, zp, args).to(torch.bfloat16)
+    assert torch.isfinite(wq.float()).all() and torch.isfinite(loss).all()
+    assert torch.equal(wq.cpu(), rtn)
+
+
 def test_gptq_zero_hessian_zeroes_weight_and_failure_is_rtn():
     from llmcompressor_amd import ops
 
