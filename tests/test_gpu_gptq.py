@@ -299,10 +299,13 @@ def test_hinv_grouped_is_bit_identical_to_single_calls(K, n, actorder):
 
 
 @pytest.mark.parametrize("R,K,n,fmt_case", [(96, 768, 5, "int4_sym"), (64, 512, 4, "int4_asym_actorder"),
-                                            (48, 256, 3, "nvfp4")])
+                                            (48, 256, 3, "nvfp4"), (1024, 4096, 2, "int4_sym"),
+                                            (1024, 4608, 2, "int4_asym_actorder")])
 def test_gptq_quantize_grouped_is_bit_identical_to_single_calls(R, K, n, fmt_case):
     """llmc_gptq_quantize_grouped on the factors of llmc_gptq_hinv_grouped: identical weights and losses to n
-    single calls (int4 symmetric g128, int4 asymmetric g64 with activation ordering, NVFP4 with global scales)."""
+    single calls (int4 symmetric g128, int4 asymmetric g64 with activation ordering, NVFP4 with global scales).
+    The two larger cases reach the split-bf16 products of the trailing updates (the small ones stay on the fp32
+    matrix instructions), whose choice must not depend on how many problems a call carries."""
     from llmcompressor_amd import ops
 
     torch.manual_seed(R + K)
