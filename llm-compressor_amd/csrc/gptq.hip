@@ -1,14 +1,14 @@
 // GPTQ quantize_weight: blocked column loop with error feedback.
 //
-// Rows of W are independent given the inverse-Hessian factor U, so a workgroup
-// owns 16 rows and never synchronises with another one inside a block of
-// columns.  A row is spread over a team of 16 lanes, 8 columns of the block per
-// lane, held in registers.  The block's 128x128 slice of U sits in LDS.  Per
-// column: the owning lane's value is broadcast inside the team, every lane
-// quantises it, forms err = (w - q)/U[i][i] and subtracts err * U[i][c] from its
-// own 8 columns (U is zero below the diagonal, so no masking is needed).  That is the layout of the
-// SparseGPT kernel below; the quantiser's kernel spreads a row over 4 lanes and is described at its constants.
-// After the block, W[:, i2:] -= Err * U[i1:i2, i2:] runs as an fp32 MFMA GEMM.
+// Rows of W are independent given the inverse-Hessian factor U, so a workgroup owns a set of rows and never
+// synchronises with another one inside a block of columns.  The block's 128x128 slice of U sits in LDS, a
+// row's columns of the block in registers.  Per column: quantise, form err = (w - q)/U[i][i] and subtract
+// err * U[i][c] from the columns behind it (U is zero below the diagonal, so no masking is needed).
+//   * quantiser (gptq_block_kernel): 4 lanes per row, 32 columns per lane as 8 runs of 4 neighbouring
+//     columns; a run is quantised start to finish inside its lane (layout described at the Q* constants).
+//   * SparseGPT (sgpt_block_kernel): 16 lanes per row, 8 columns per lane; the column's value and prune flag
+//     are broadcast inside the team and every lane forms the error.
+// After the block, W[:, i2:] -= Err * U[i1:i2, i2:] runs as a matrix-core GEMM (llmc_gemm_f32).
 #include <vector>
 
 #include "gemm_f32.h"
@@ -608,14 +608,15 @@ __global__ __launch_bounds__(256) void sgpt_block_kernel(SgptParams p) {
         loss += err * err;  // (w-q)^2 / d^2
         const float4 h0 = *(const float4*)&Hs[i * GB + tl * CPL];
         const float4 h1 = *(const float4*)&Hs[i * GB + tl * CPL + 4];
-        w[0] = __fsub_rn(w[0], __fmul_rn(err, h0.x));
-        w[1] = __fsub_rn(w[1], __fmul_rn(err, h0.y));
-        w[2] = __fsub_rn(w[2], __fmul_rn(err, h0.z));
-        w[3] = __fsub_rn(w[3], __fmul_rn(err, h0.w));
-        w[4] = __fsub_rn(w[4], __fmul_rn(err, h1.x));
-        w[5] = __fsub_rn(w[5], __fmul_rn(err, h1.y));
-        w[6] = __fsub_rn(w[6], __fmul_rn(err, h1.z));
-        w[7] = __fsub_rn(w[7], __fmul_rn(err, h1.w));
+        // one fused multiply-subtract per element, as in the quantiser's kernel
+        w[0] = fmaf(-err, h0.x, w[0]);
+        w[1] = fmaf(-err, h0.y, w[1]);
+        w[2] = fmaf(-err, h0.z, w[2]);
+        w[3] = fmaf(-err, h0.w, w[3]);
+        w[4] = fmaf(-err, h1.x, w[4]);
+        w[5] = fmaf(-err, h1.y, w[5]);
+        w[6] = fmaf(-err, h1.z, w[6]);
+        w[7] = fmaf(-err, h1.w, w[7]);
         if (tl == li) {
           qv[e] = q;
           ev[e] = err;

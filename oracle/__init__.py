@@ -30,7 +30,14 @@ closed form or invariant says so here):
 * parity unpinned (no reference-held vector exists; follows the public format
   specs): MXFP4 E8M0 scale generation, ``pack_to_int32`` / ``pack_fp4_to_uint8``
   byte layouts, fp8 storage, per-token dynamic FP8 scales, zero-scale epsilon
-  substitution.
+  substitution, the BLOCK strategy inside the GPTQ column loop, the checkpoint
+  format name of int weights with quantised activations.  Cross-checks that do
+  not lift the status (``tests/test_oracle_golden.py``): the MXFP4 exponent rule
+  against the OCP Microscaling definition over every bf16 maximum (equal, or one
+  more where the rounding bump carries, mantissas >= 1.75); the E8M0 byte against
+  ``torch.float8_e8m0fnu``; per-token FP8 against the per-row helper a consumer
+  of such checkpoints applies (same reduce dimension, scales equal after rounding
+  to bf16, >= 95 % equal bytes, the rest one e4m3 step away).
 * parity unpinned by reference vectors, pinned by mathematics only:
   ``sparsegpt.accumulate_hessian`` / ``sparsegpt.sparsify_weight`` (the
   reference's SparseGPT tests need hub models; see ``tests/test_oracle_sparsegpt.py``:
