@@ -138,8 +138,10 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) __attribute__((amdgpu_waves
   // Workgroup ids are dealt round-robin to the 8 XCDs.  XCD x takes the tile rows x, 15 - x, 16 + x, 31 - x, ...
   // (a row's tiles share the A panel in that XCD's L2; the back-and-forth order balances the XCDs when the
   // work of a row grows with its index, as it does for triangular operands), longest rows first.
+  // With fewer than 8 tile rows left in a group of 8, some XCDs get no row of this problem; the slot is rotated
+  // by the problem index so that over a batch every XCD is given the same share.
   const int id = blockIdx.x;
-  const int x = id & 7, j = id >> 3;
+  const int x = (id + (int)blockIdx.z) & 7, j = id >> 3;
   const int i = j / tiles_x, tx = j - i * tiles_x;
   const int rrow = 8 * i + ((i & 1) ? 7 - x : x);
   if (rrow >= tiles_y) return;
