@@ -101,6 +101,58 @@ __global__ __launch_bounds__(256) void hinv_copyin_kernel(const float* __restric
   A[(int64_t)i * Kp + j] = v;
 }
 
+// hinv_copyin_kernel for a permuted order, one workgroup per row of A: row perm[K-1-i] of H is read whole and
+// coalesced into LDS and the permuted columns are picked there (element-wise the gather costs one cache line
+// per value).  Rows of up to COPYIN_STAGE_MAX values.
+constexpr int COPYIN_STAGE_MAX = 16384;
+__global__ __launch_bounds__(256) void hinv_copyin_rows_kernel(const float* __restrict__ H, int64_t ldh, int K,
+                                                               int Kp, const int32_t* __restrict__ perm, float div,
+                                                               const HinvScalars* __restrict__ sc,
+                                                               float* __restrict__ A,
+                                                               const HinvItem* __restrict__ items) {
+  extern __shared__ float rowbuf[];
+  if (items) {
+    const HinvItem it = items[blockIdx.y];
+    H = it.H; perm = it.perm; div = it.div;
+    sc += blockIdx.y;
+    A += (int64_t)blockIdx.y * Kp * Kp;
+  }
+  const int i = blockIdx.x, tid = threadIdx.x;
+  float* out = A + (int64_t)i * Kp;
+  if (i >= K) {  // identity padding
+    for (int j = tid; j < Kp; j += 256) out[j] = (i == j) ? 1.f : 0.f;
+    return;
+  }
+  const float* src = H + (int64_t)perm[K - 1 - i] * ldh;
+  constexpr int BATCH = 8;
+  for (int c0 = 0; c0 < K; c0 += 256 * BATCH) {
+    float v[BATCH];
+#pragma unroll
+    for (int b = 0; b < BATCH; ++b) {
+      const int c = c0 + b * 256 + tid;
+      v[b] = src[c < K ? c : K - 1];
+    }
+#pragma unroll
+    for (int b = 0; b < BATCH; ++b) {
+      const int c = c0 + b * 256 + tid;
+      if (c < K) rowbuf[c] = v[b];
+    }
+  }
+  __syncthreads();
+  const float damp = sc->damp;
+  for (int j = tid; j < Kp; j += 256) {
+    float v = 0.f;
+    if (j <= i) {
+      v = rowbuf[perm[K - 1 - j]] / div;
+      if (i == j) {
+        if (v == 0.f) v = 1.f;
+        v += damp;
+      }
+    }
+    out[j] = v;
+  }
+}
+
 // Factor the 64x64 diagonal block at (k0,k0) and replace it by the inverse of its factor.
 // The block and the growing inverse X = L^-1 live in registers: thread (ty, tx) of a 16 x 16 grid
 // owns the 4x4 sub-blocks L[4ty.., 4tx..] and X[4ty.., 4tx..].  Right-looking in steps of four
@@ -296,8 +348,18 @@ extern "C" int llmc_gptq_hinv(float* H, int64_t ldh, int64_t K, const int32_t* p
   hipLaunchKernelGGL(hinv_stats_kernel, dim3(1), dim3(256), 0, st, H, ldh, (int)K, perm, divisor, percdamp,
                      dead_out, sc, (const HinvItem*)nullptr);
   LLMC_LAUNCH_STATUS();
-  hipLaunchKernelGGL(hinv_copyin_kernel, dim3((Kp + 255) / 256, Kp), dim3(256), 0, st, H, ldh, (int)K, Kp, perm,
-                     divisor, sc, A, (const HinvItem*)nullptr);
+  if (perm != nullptr && K <= COPYIN_STAGE_MAX) {
+    if (K * 4 > 48 * 1024) {
+      const hipError_t e = hipFuncSetAttribute((const void*)hinv_copyin_rows_kernel,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)K * 4);
+      if (e != hipSuccess) return 1000 + (int)e;
+    }
+    hipLaunchKernelGGL(hinv_copyin_rows_kernel, dim3(Kp), dim3(256), (size_t)K * 4, st, H, ldh, (int)K, Kp, perm,
+                       divisor, sc, A, (const HinvItem*)nullptr);
+  } else {
+    hipLaunchKernelGGL(hinv_copyin_kernel, dim3((Kp + 255) / 256, Kp), dim3(256), 0, st, H, ldh, (int)K, Kp, perm,
+                       divisor, sc, A, (const HinvItem*)nullptr);
+  }
   LLMC_LAUNCH_STATUS();
 
   // Blocked Cholesky, two levels: inside a 256-wide outer panel the 64-wide steps (diagonal block
@@ -431,8 +493,20 @@ extern "C" int llmc_gptq_hinv_grouped(const float* const* H, int64_t ldh, int32_
   hipLaunchKernelGGL(hinv_stats_kernel, dim3(n), dim3(256), 0, st, (const float*)nullptr, ldh, (int)K,
                      (const int32_t*)nullptr, 1.f, percdamp, (uint8_t*)nullptr, sc, (const HinvItem*)items);
   LLMC_LAUNCH_STATUS();
-  hipLaunchKernelGGL(hinv_copyin_kernel, dim3((Kp + 255) / 256, Kp, n), dim3(256), 0, st, (const float*)nullptr, ldh,
-                     (int)K, Kp, (const int32_t*)nullptr, 1.f, sc, A, (const HinvItem*)items);
+  bool all_perm = perm != nullptr;
+  for (int b = 0; b < n && all_perm; ++b) all_perm = perm[b] != nullptr;
+  if (all_perm && K <= COPYIN_STAGE_MAX) {
+    if (K * 4 > 48 * 1024) {
+      const hipError_t e = hipFuncSetAttribute((const void*)hinv_copyin_rows_kernel,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)K * 4);
+      if (e != hipSuccess) return 1000 + (int)e;
+    }
+    hipLaunchKernelGGL(hinv_copyin_rows_kernel, dim3(Kp, n), dim3(256), (size_t)K * 4, st, (const float*)nullptr, ldh,
+                       (int)K, Kp, (const int32_t*)nullptr, 1.f, sc, A, (const HinvItem*)items);
+  } else {
+    hipLaunchKernelGGL(hinv_copyin_kernel, dim3((Kp + 255) / 256, Kp, n), dim3(256), 0, st, (const float*)nullptr, ldh,
+                       (int)K, Kp, (const int32_t*)nullptr, 1.f, sc, A, (const HinvItem*)items);
+  }
   LLMC_LAUNCH_STATUS();
 
   const int NBO = Kp >= 8192 ? 512 : 256;

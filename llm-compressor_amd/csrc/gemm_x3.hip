@@ -139,9 +139,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) __attribute__((amdgpu_waves
   // (a row's tiles share the A panel in that XCD's L2; the back-and-forth order balances the XCDs when the
   // work of a row grows with its index, as it does for triangular operands), longest rows first.
   // With fewer than 8 tile rows left in a group of 8, some XCDs get no row of this problem; the slot is rotated
-  // by the problem index so that over a batch every XCD is given the same share.
+  // by the problem index times that remainder, so that the rows of successive problems fill the XCDs in turn.
   const int id = blockIdx.x;
-  const int x = (id + (int)blockIdx.z) & 7, j = id >> 3;
+  const int x = (id + (int)blockIdx.z * (tiles_y & 7)) & 7, j = id >> 3;
   const int i = j / tiles_x, tx = j - i * tiles_x;
   const int rrow = 8 * i + ((i & 1) ? 7 - x : x);
   if (rrow >= tiles_y) return;

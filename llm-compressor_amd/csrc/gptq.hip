@@ -54,6 +54,88 @@ __global__ __launch_bounds__(256) void gptq_prepare_w_kernel(const void* __restr
   Wf[(int64_t)r * K + c] = v;
 }
 
+// Row-at-a-time forms of the column gather / scatter for a permuted column order (activation ordering): one
+// workgroup moves one row through LDS, so global memory sees whole rows and the random accesses stay on chip.
+// Rows of up to ROW_STAGE_MAX fp32 values fit; wider ones keep the element-wise kernels.
+constexpr int ROW_STAGE_MAX = 16384;
+
+template <int WDT>
+__global__ __launch_bounds__(256) void gptq_prepare_w_rows_kernel(const void* __restrict__ w, int64_t ldw, int R,
+                                                                  int K, const int32_t* __restrict__ perm,
+                                                                  const uint8_t* __restrict__ dead,
+                                                                  float* __restrict__ Wf,
+                                                                  const GptqItem* __restrict__ items) {
+  extern __shared__ float rowbuf[];
+  if (items) {
+    w = items[blockIdx.y].weight;
+    perm += (int64_t)blockIdx.y * K;
+    if (dead) dead += (int64_t)blockIdx.y * K;
+    Wf += (int64_t)blockIdx.y * R * K;
+  }
+  const int r = blockIdx.x, tid = threadIdx.x;
+  constexpr int BATCH = 8;
+  for (int c0 = 0; c0 < K; c0 += 256 * BATCH) {
+    float v[BATCH];
+#pragma unroll
+    for (int b = 0; b < BATCH; ++b) {
+      const int c = c0 + b * 256 + tid;
+      v[b] = load_as_f32<WDT>(w, (int64_t)r * ldw + (c < K ? c : K - 1));
+    }
+#pragma unroll
+    for (int b = 0; b < BATCH; ++b) {
+      const int c = c0 + b * 256 + tid;
+      if (c < K) rowbuf[c] = v[b];
+    }
+  }
+  __syncthreads();
+  for (int c = tid; c < K; c += 256) {
+    float v = rowbuf[perm[c]];
+    if (dead && dead[c]) v = 0.f;
+    Wf[(int64_t)r * K + c] = v;
+  }
+}
+
+template <int WDT>
+__global__ __launch_bounds__(256) void gptq_finalize_rows_kernel(const float* __restrict__ Wf, int R, int K,
+                                                                 const int32_t* __restrict__ perm,
+                                                                 void* __restrict__ out, int64_t ldo,
+                                                                 const GptqItem* __restrict__ items) {
+  extern __shared__ float rowbuf[];
+  if (items) {
+    out = items[blockIdx.y].out;
+    perm += (int64_t)blockIdx.y * K;
+    Wf += (int64_t)blockIdx.y * R * K;
+  }
+  const int r = blockIdx.x, tid = threadIdx.x;
+  constexpr int BATCH = 8;
+  for (int c0 = 0; c0 < K; c0 += 256 * BATCH) {
+    float v[BATCH];
+    int dst[BATCH];
+#pragma unroll
+    for (int b = 0; b < BATCH; ++b) {
+      const int c = c0 + b * 256 + tid;
+      const int cc = c < K ? c : K - 1;
+      v[b] = Wf[(int64_t)r * K + cc];
+      dst[b] = perm[cc];
+    }
+#pragma unroll
+    for (int b = 0; b < BATCH; ++b) {
+      const int c = c0 + b * 256 + tid;
+      if (c < K) rowbuf[dst[b]] = v[b];
+    }
+  }
+  __syncthreads();
+  for (int c = tid; c < K; c += 256) store_from_f32<WDT>(out, (int64_t)r * ldo + c, rowbuf[c]);
+}
+
+// dynamic LDS above 48 KB has to be asked for once per kernel
+template <typename KernT>
+inline int allow_row_stage(KernT kern, int K) {
+  if ((size_t)K * 4 <= 48 * 1024) return 0;
+  const hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, K * 4);
+  return e == hipSuccess ? 0 : 1000 + (int)e;
+}
+
 // The block's [GB][GB] slice of U into LDS, zero outside the upper triangle and past `count`.  Addresses are
 // clamped into the block instead of predicated, so the loads of a batch are all in flight together.
 __device__ __forceinline__ void load_u_block(float* __restrict__ Hs, const float* __restrict__ U, int64_t ldu,
@@ -823,11 +905,20 @@ extern "C" int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R
   float* loss_rows = (float*)((char*)E + align256(R * GROUP * GB * 4));
 
   dim3 grid2((unsigned)((K + 255) / 256), (unsigned)R);
-#define LLMC_PREP(DT) \
-  hipLaunchKernelGGL((gptq_prepare_w_kernel<DT>), grid2, dim3(256), 0, st, weight, ldw, (int)R, (int)K, perm, dead, Wf)
-  if (w_dtype == LLMC_BF16) LLMC_PREP(LLMC_BF16);
-  else if (w_dtype == LLMC_F16) LLMC_PREP(LLMC_F16);
-  else LLMC_PREP(LLMC_F32);
+  const bool by_rows = perm != nullptr && K <= ROW_STAGE_MAX;  // permuted columns: gather and scatter a row in LDS
+#define LLMC_PREP(DT)                                                                                               \
+  if (by_rows) {                                                                                                    \
+    const int arc = allow_row_stage(gptq_prepare_w_rows_kernel<DT>, (int)K);                                        \
+    if (arc) return arc;                                                                                            \
+    hipLaunchKernelGGL((gptq_prepare_w_rows_kernel<DT>), dim3((unsigned)R), dim3(256), (size_t)K * 4, st, weight, ldw, \
+                       (int)R, (int)K, perm, dead, Wf, (const GptqItem*)nullptr);                                   \
+  } else {                                                                                                          \
+    hipLaunchKernelGGL((gptq_prepare_w_kernel<DT>), grid2, dim3(256), 0, st, weight, ldw, (int)R, (int)K, perm, dead, \
+                       Wf);                                                                                         \
+  }
+  if (w_dtype == LLMC_BF16) LLMC_PREP(LLMC_BF16)
+  else if (w_dtype == LLMC_F16) LLMC_PREP(LLMC_F16)
+  else LLMC_PREP(LLMC_F32)
 #undef LLMC_PREP
   LLMC_LAUNCH_STATUS();
   hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((R + 255) / 256)), dim3(256), 0, st, loss_rows, R);
@@ -895,11 +986,18 @@ extern "C" int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R
     }
   }
 
-#define LLMC_FIN(DT) \
-  hipLaunchKernelGGL((gptq_finalize_kernel<DT>), grid2, dim3(256), 0, st, Wf, (int)R, (int)K, perm, out_weight, ldo)
-  if (w_dtype == LLMC_BF16) LLMC_FIN(LLMC_BF16);
-  else if (w_dtype == LLMC_F16) LLMC_FIN(LLMC_F16);
-  else LLMC_FIN(LLMC_F32);
+#define LLMC_FIN(DT)                                                                                                \
+  if (by_rows) {                                                                                                    \
+    const int arc = allow_row_stage(gptq_finalize_rows_kernel<DT>, (int)K);                                         \
+    if (arc) return arc;                                                                                            \
+    hipLaunchKernelGGL((gptq_finalize_rows_kernel<DT>), dim3((unsigned)R), dim3(256), (size_t)K * 4, st, Wf, (int)R,   \
+                       (int)K, perm, out_weight, ldo, (const GptqItem*)nullptr);                                    \
+  } else {                                                                                                          \
+    hipLaunchKernelGGL((gptq_finalize_kernel<DT>), grid2, dim3(256), 0, st, Wf, (int)R, (int)K, perm, out_weight, ldo); \
+  }
+  if (w_dtype == LLMC_BF16) LLMC_FIN(LLMC_BF16)
+  else if (w_dtype == LLMC_F16) LLMC_FIN(LLMC_F16)
+  else LLMC_FIN(LLMC_F32)
 #undef LLMC_FIN
   LLMC_LAUNCH_STATUS();
   if (loss_out) {
@@ -967,12 +1065,20 @@ extern "C" int llmc_gptq_quantize_grouped(const void* const* weight, int32_t w_d
   }
 
   dim3 grid3((unsigned)((K + 255) / 256), (unsigned)R, (unsigned)n);
-#define LLMC_PREP(DT)                                                                                         \
-  hipLaunchKernelGGL((gptq_prepare_w_kernel<DT>), grid3, dim3(256), 0, st, (const void*)nullptr, ldw, (int)R, \
-                     (int)K, perm, dead, Wf, (const GptqItem*)items)
-  if (w_dtype == LLMC_BF16) LLMC_PREP(LLMC_BF16);
-  else if (w_dtype == LLMC_F16) LLMC_PREP(LLMC_F16);
-  else LLMC_PREP(LLMC_F32);
+  const bool by_rows = perm != nullptr && K <= ROW_STAGE_MAX;  // as in the single-problem call
+#define LLMC_PREP(DT)                                                                                           \
+  if (by_rows) {                                                                                                \
+    const int arc = allow_row_stage(gptq_prepare_w_rows_kernel<DT>, (int)K);                                    \
+    if (arc) return arc;                                                                                        \
+    hipLaunchKernelGGL((gptq_prepare_w_rows_kernel<DT>), dim3((unsigned)R, (unsigned)n), dim3(256), (size_t)K * 4, \
+                       st, (const void*)nullptr, ldw, (int)R, (int)K, perm, dead, Wf, (const GptqItem*)items);  \
+  } else {                                                                                                      \
+    hipLaunchKernelGGL((gptq_prepare_w_kernel<DT>), grid3, dim3(256), 0, st, (const void*)nullptr, ldw, (int)R, \
+                       (int)K, perm, dead, Wf, (const GptqItem*)items);                                         \
+  }
+  if (w_dtype == LLMC_BF16) LLMC_PREP(LLMC_BF16)
+  else if (w_dtype == LLMC_F16) LLMC_PREP(LLMC_F16)
+  else LLMC_PREP(LLMC_F32)
 #undef LLMC_PREP
   LLMC_LAUNCH_STATUS();
   hipLaunchKernelGGL(zero_f32_kernel, dim3((unsigned)((n * R + 255) / 256)), dim3(256), 0, st, loss_rows, n * R);
@@ -1037,12 +1143,19 @@ extern "C" int llmc_gptq_quantize_grouped(const void* const* weight, int32_t w_d
     }
   }
 
-#define LLMC_FIN(DT)                                                                                          \
-  hipLaunchKernelGGL((gptq_finalize_kernel<DT>), grid3, dim3(256), 0, st, Wf, (int)R, (int)K, perm, (void*)nullptr, \
-                     ldo, (const GptqItem*)items)
-  if (w_dtype == LLMC_BF16) LLMC_FIN(LLMC_BF16);
-  else if (w_dtype == LLMC_F16) LLMC_FIN(LLMC_F16);
-  else LLMC_FIN(LLMC_F32);
+#define LLMC_FIN(DT)                                                                                            \
+  if (by_rows) {                                                                                                \
+    const int arc = allow_row_stage(gptq_finalize_rows_kernel<DT>, (int)K);                                     \
+    if (arc) return arc;                                                                                        \
+    hipLaunchKernelGGL((gptq_finalize_rows_kernel<DT>), dim3((unsigned)R, (unsigned)n), dim3(256), (size_t)K * 4,  \
+                       st, Wf, (int)R, (int)K, perm, (void*)nullptr, ldo, (const GptqItem*)items);              \
+  } else {                                                                                                      \
+    hipLaunchKernelGGL((gptq_finalize_kernel<DT>), grid3, dim3(256), 0, st, Wf, (int)R, (int)K, perm,           \
+                       (void*)nullptr, ldo, (const GptqItem*)items);                                            \
+  }
+  if (w_dtype == LLMC_BF16) LLMC_FIN(LLMC_BF16)
+  else if (w_dtype == LLMC_F16) LLMC_FIN(LLMC_F16)
+  else LLMC_FIN(LLMC_F32)
 #undef LLMC_FIN
   LLMC_LAUNCH_STATUS();
   if (loss_out) {
