@@ -190,6 +190,37 @@ def test_gptq_extreme_magnitudes_take_the_plain_division_route():
     assert torch.equal(wq.cpu(), rtn)
 
 
+@pytest.mark.parametrize("K", [2048, 16640])
+def test_gptq_permuted_columns_on_a_diagonal_hessian_are_rtn(K):
+    """Activation ordering with a diagonal Hessian of distinct entries: the column loop runs in the permuted
+    order, nothing propagates, and the result written back through the inverse permutation must be
+    round-to-nearest bit for bit.  K = 2048 takes the gather / scatter kernels that move whole rows through
+    LDS, K = 16640 is wider than they stage and takes the element-wise ones."""
+    from llmcompressor_amd import ops
+
+    torch.manual_seed(K)
+    R, g = 8, 128
+    w = (torch.randn(R, K) * 0.05).bfloat16()
+    args = F.QArgs(num_bits=4, strategy="group", group_size=g)
+    obs = O.Observer("memoryless_minmax", "weight", args)
+    obs(w)
+    scale, zp = F.calculate_qparams(obs.min_vals, obs.max_vals, args)
+    d = torch.rand(K) + 0.5
+    perm = torch.argsort(d, descending=True).to(torch.int32)
+    U, dead, info = ops.gptq_hinv_(torch.diag(d).cuda(), perm.cuda())
+    assert info.item() == 0
+    g_idx = (torch.arange(K, dtype=torch.int32) // g)[perm.long()]
+    wq, loss = ops.gptq_quantize(w.cuda(), U, scale.cuda(), None, ops.FMT_INT, 4, 1, K // g, g_idx=g_idx.cuda(),
+                                 perm=perm.cuda(), dead=dead)
+    rtn = F.fake_quantize(w.float(), scale, zp, args).to(torch.bfloat16)
+    assert torch.equal(wq.cpu(), rtn)
+    # the factor of a diagonal matrix in the permuted order: 1 / sqrt(d + damp) on the diagonal
+    damp = 0.01 * d.mean()
+    expect = 1.0 / torch.sqrt(d[perm.long()] + damp)
+    assert torch.allclose(torch.diagonal(U).cpu(), expect, rtol=1e-5)
+    assert torch.count_nonzero(U.cpu() - torch.diag(torch.diagonal(U).cpu())) == 0
+
+
 def test_gptq_zero_hessian_zeroes_weight_and_failure_is_rtn():
     from llmcompressor_amd import ops
 
