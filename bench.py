@@ -269,6 +269,75 @@ def probe_sparsegpt():
           f"{(time.perf_counter() - t0) * 1e3:.0f} ms")
 
 
+def probe_chain():
+    """The quantize phase's pieces run alone, event-timed: the damped Cholesky chain and the column loop for the
+    layer's three Linear shapes (W4A16 g128, static activation ordering), and the fp32 products they are made
+    of, through `llmc_sgemm`, at the shapes the K = 14336 chain and the down_proj loop use.  Prints two tables."""
+    import torch
+
+    from llmcompressor_amd import ops
+
+    def timed(fn, n=5):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n
+
+    print("| Linear (rows x columns) | Cholesky chain ms | column loop ms |")
+    print("|---|---|---|")
+    for R, K in ((HIDDEN, HIDDEN), (INTER, HIDDEN), (HIDDEN, INTER)):
+        torch.manual_seed(0)
+        x = torch.randn(16384, K, device="cuda").bfloat16()
+        W = (torch.randn(R, K, device="cuda") * 0.02).bfloat16()
+        H0 = torch.zeros(K, K, device="cuda")
+        ops.hessian_accumulate_(H0, x)
+        del x
+        perm = torch.argsort(torch.diagonal(H0), descending=True, stable=True).to(torch.int32)
+        work = torch.empty_like(H0)
+
+        def chain():
+            work.copy_(H0)
+            return ops.gptq_hinv_(work, perm, divisor=8.0)
+
+        t_copy = timed(lambda: work.copy_(H0))
+        t_chain = timed(chain) - t_copy
+        U, dead, _ = ops.gptq_hinv_(H0.clone(), perm, divisor=8.0)
+        mn, mx = ops.minmax_groups(W, 128)
+        scale, _, _ = ops.calculate_qparams(mn, mx, ops.FMT_INT, 4, True)
+        g_idx = (torch.arange(K, dtype=torch.int32, device="cuda") // 128)[perm.long()]
+        t_loop = timed(lambda: ops.gptq_quantize(W, U, scale, None, ops.FMT_INT, 4, 1, K // 128, g_idx=g_idx,
+                                                 perm=perm, dead=dead))
+        print(f"| {R} x {K} | {t_chain:.2f} | {t_loop:.2f} |")
+        del H0, work, U
+
+    print()
+    print("| fp32 product C -= A B (llmc_sgemm) | M | N | K | us | TFLOP/s of the non-zero part |")
+    print("|---|---|---|---|---|---|")
+    cases = [
+        ("square", 8192, 8192, 8192, False, 0, 1.0),
+        ("inversion, 8192-wide level: L21 X11 (X11 lower triangular)", 6144, 8192, 8192, False, ops.SGEMM_B_LOWER_TRI, 0.5),
+        ("inversion, 8192-wide level: X22 T (X22 lower triangular)", 6144, 8192, 6144, False, ops.SGEMM_A_LOWER_TRI, 0.5),
+        ("inversion, 4096-wide level: L21 X11", 4096, 4096, 4096, False, ops.SGEMM_B_LOWER_TRI, 0.5),
+        ("trailing SYRK of the first 512-wide panel (lower triangle)", 13824, 13824, 512, True, ops.SGEMM_C_LOWER, 0.5),
+        ("trailing SYRK, half way", 7168, 7168, 512, True, ops.SGEMM_C_LOWER, 0.5),
+        ("column loop: far product of the first group", 4096, 13824, 512, False, 0, 1.0),
+        ("column loop: far product, half way", 4096, 7168, 512, False, 0, 1.0),
+        ("column loop: product inside a group", 4096, 384, 128, False, 0, 1.0),
+    ]
+    for name, M, N, Kc, trans_b, flags, frac in cases:
+        A = torch.randn(M, Kc, device="cuda")
+        B = torch.randn(N, Kc, device="cuda") if trans_b else torch.randn(Kc, N, device="cuda")
+        C = torch.zeros(M, N, device="cuda")
+        ms = timed(lambda: ops.sgemm_(C, A, B, -1.0, 1.0, trans_b, flags))
+        print(f"| {name} | {M} | {N} | {Kc} | {ms * 1e3:.1f} | {2.0 * M * N * Kc * frac / ms / 1e9:.0f} |")
+        del A, B, C
+
+
 def probe_moe(mode="both"):
     """One MoE expert layer (128 experts, hidden 2048, intermediate 768, top-8 routing of 4096 tokens: 384 expert
     Linears) through GPTQModifier W4A16: time of the calibration forward (grouped Hessian launches from the hooks)
@@ -439,6 +508,8 @@ def main():
                     "(--batches x --tokens calibration tokens) instead of the bench line")
     ap.add_argument("--layers", type=int, default=2, help="--probe-oneshot: decoder layers of the model (config: 32)")
     ap.add_argument("--vocab", type=int, default=32000, help="--probe-oneshot: vocabulary size (config: 128256)")
+    ap.add_argument("--probe-chain", action="store_true",
+                    help="time the Cholesky chain, the column loop and their fp32 products alone, print tables")
     ap.add_argument("--probe-moe", action="store_true",
                     help="print the timings of one 128-expert MoE layer through GPTQModifier instead of the bench line")
     a = ap.parse_args()
@@ -460,6 +531,9 @@ def main():
         return
     if a.probe_sparsegpt:
         probe_sparsegpt()
+        return
+    if a.probe_chain:
+        probe_chain()
         return
     if a.probe_moe:
         probe_moe(a.moe_mode)
