@@ -137,15 +137,20 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) __attribute__((amdgpu_waves
 
   // Workgroup ids are dealt round-robin to the 8 XCDs.  XCD x takes the tile rows x, 15 - x, 16 + x, 31 - x, ...
   // (a row's tiles share the A panel in that XCD's L2; the back-and-forth order balances the XCDs when the
-  // work of a row grows with its index, as it does for triangular operands), longest rows first.
-  // With fewer than 8 tile rows left in a group of 8, some XCDs get no row of this problem; the slot is rotated
+  // work of a row grows with its index, as it does for triangular operands), longest rows first.  With a lower
+  // triangular B the work of a tile falls with its column instead, so there the roles of rows and columns are
+  // swapped: tile columns are dealt to the XCDs (sharing the B panel), first columns first.
+  // With fewer than 8 rows left in a group of 8, some XCDs get no row of this problem; the slot is rotated
   // by the problem index times that remainder, so that the rows of successive problems fill the XCDs in turn.
+  const bool by_columns = g.b_lower_tri && !g.a_lower_tri && !g.c_lower;
+  const int major = by_columns ? tiles_x : tiles_y, minor = by_columns ? tiles_y : tiles_x;
   const int id = blockIdx.x;
-  const int x = (id + (int)blockIdx.z * (tiles_y & 7)) & 7, j = id >> 3;
-  const int i = j / tiles_x, tx = j - i * tiles_x;
+  const int x = (id + (int)blockIdx.z * (major & 7)) & 7, j = id >> 3;
+  const int i = j / minor, t = j - i * minor;
   const int rrow = 8 * i + ((i & 1) ? 7 - x : x);
-  if (rrow >= tiles_y) return;
-  const int ty = (g.a_lower_tri || g.c_lower) ? tiles_y - 1 - rrow : rrow;
+  if (rrow >= major) return;
+  const int ty = by_columns ? t : ((g.a_lower_tri || g.c_lower) ? tiles_y - 1 - rrow : rrow);
+  const int tx = by_columns ? rrow : t;
   const int m0 = ty * BM, n0 = tx * BN;
   if (g.c_lower && n0 > m0 + BM - 1) return;
   const int b1 = (int)blockIdx.z % g.batch, b2 = (int)blockIdx.z / g.batch;
@@ -319,7 +324,9 @@ int launch_x3(const GemmF32& g, hipStream_t st) {
     if (e != hipSuccess) return 1000 + (int)e;
     configured = true;
   }
-  const unsigned grid_x = 8u * (unsigned)((tiles_y + 7) / 8) * (unsigned)tiles_x;
+  const bool by_columns = g.b_lower_tri && !g.a_lower_tri && !g.c_lower;  // as in the kernel's tile order
+  const int major = by_columns ? tiles_x : tiles_y, minor = by_columns ? tiles_y : tiles_x;
+  const unsigned grid_x = 8u * (unsigned)((major + 7) / 8) * (unsigned)minor;
   hipLaunchKernelGGL(kern, dim3(grid_x, 1, (unsigned)(g.batch * nb2)), dim3(C::NTHREADS), smem, st, g, tiles_x, tiles_y);
   hipError_t e = hipGetLastError();
   return e == hipSuccess ? 0 : 1000 + (int)e;
