@@ -6,7 +6,7 @@
 // matrix, R = J L J for the ordinary lower factor L of J H J, so
 //     U[i][j] = (L^-1)[K-1-i][K-1-j].
 // This file therefore (1) copies J (P^T H P / n + damp I) J into a work matrix
-// (P = optional activation-order permutation), (2) runs a right-looking blocked
+// (P = optional activation-order permutation), (2) runs a blocked
 // lower Cholesky (64-wide panels: the diagonal block is factored and inverted in
 // LDS by one workgroup, panel solve and trailing update are MFMA GEMMs),
 // (3) inverts L by recursive doubling with batched triangular GEMMs and
@@ -362,16 +362,27 @@ extern "C" int llmc_gptq_hinv(float* H, int64_t ldh, int64_t K, const int32_t* p
   }
   LLMC_LAUNCH_STATUS();
 
-  // Blocked Cholesky, two levels: inside a 256-wide outer panel the 64-wide steps (diagonal block
-  // factored + inverted in LDS, panel solve as a GEMM) only update the panel's own remaining
-  // columns; the trailing matrix then gets one rank-256 update per outer panel, which cuts its
-  // read-modify-write traffic 4x compared with rank-64 updates.  Diagonal blocks end up holding
-  // inv(L_kk).
+  // Blocked Cholesky, two levels.  Inside a 256- or 512-wide outer panel the 64-wide steps run left-looking:
+  // a step first brings its own 64 columns up to date with the panel's earlier steps (one product), then the
+  // diagonal block is factored + inverted in LDS and the panel below it solved as a GEMM.  The trailing matrix
+  // gets one rank-256/512 update per outer panel (right-looking between panels), which cuts its
+  // read-modify-write traffic 4-8x compared with rank-64 updates.  Diagonal blocks end up holding inv(L_kk).
   const int NBO = Kp >= 8192 ? 512 : 256;  // wider outer panels once the trailing matrix is big enough to pay for them
   for (int k0 = 0; k0 < Kp; k0 += NBO) {
     const int pw = (Kp - k0) < NBO ? (Kp - k0) : NBO;
     for (int kk = 0; kk < pw; kk += NB) {
       const int c0 = k0 + kk;
+      if (kk > 0) {
+        // left-looking inside the panel: columns c0 .. c0+63 of the rows from c0 down take the updates of the
+        // panel's earlier steps in one product, C[M+64, 64] -= L[rows, k0:c0] * L[c0:c0+64, k0:c0]^T.  (Updating
+        // all remaining columns of the panel after every step moves twice the bytes for the same sums.)
+        float* Lp = A + (int64_t)c0 * Kp + k0;
+        GemmF32 u = {};
+        u.A = Lp; u.lda = Kp; u.B = Lp; u.ldb = Kp; u.C = A + (int64_t)c0 * Kp + c0; u.ldc = Kp;
+        u.M = Kp - c0; u.N = NB; u.Kc = kk; u.alpha = -1.f; u.beta = 1.f; u.trans_b = 1; u.batch = 1;
+        const int rc = llmc_gemm_f32(u, st);
+        if (rc) return rc;
+      }
       hipLaunchKernelGGL(potf2_inv_kernel, dim3(1), dim3(256), 0, st, A, Kp, c0, (int)K, sc);
       LLMC_LAUNCH_STATUS();
       const int M = Kp - c0 - NB;
@@ -381,17 +392,8 @@ extern "C" int llmc_gptq_hinv(float* H, int64_t ldh, int64_t K, const int32_t* p
       // panel: A21 <- A21 * inv(L_kk)^T   (in place: one tile column, each workgroup owns its rows)
       g.A = A21; g.lda = Kp; g.B = A + (int64_t)c0 * Kp + c0; g.ldb = Kp; g.C = A21; g.ldc = Kp;
       g.M = M; g.N = NB; g.Kc = NB; g.alpha = 1.f; g.beta = 0.f; g.trans_b = 1; g.batch = 1;
-      int rc = llmc_gemm_f32(g, st);
+      const int rc = llmc_gemm_f32(g, st);
       if (rc) return rc;
-      const int nrem = k0 + pw - (c0 + NB);
-      if (nrem > 0) {
-        // remaining columns of this outer panel: C[M, nrem] -= A21 * A21[:nrem]^T (lower part)
-        GemmF32 u = {};
-        u.A = A21; u.lda = Kp; u.B = A21; u.ldb = Kp; u.C = A + (int64_t)(c0 + NB) * Kp + c0 + NB; u.ldc = Kp;
-        u.M = M; u.N = nrem; u.Kc = NB; u.alpha = -1.f; u.beta = 1.f; u.trans_b = 1; u.c_lower = 1; u.batch = 1;
-        rc = llmc_gemm_f32(u, st);
-        if (rc) return rc;
-      }
     }
     const int M2 = Kp - (k0 + pw);
     if (M2 > 0) {
@@ -514,6 +516,15 @@ extern "C" int llmc_gptq_hinv_grouped(const float* const* H, int64_t ldh, int32_
     const int pw = (Kp - k0) < NBO ? (Kp - k0) : NBO;
     for (int kk = 0; kk < pw; kk += NB) {
       const int c0 = k0 + kk;
+      if (kk > 0) {  // left-looking inside the panel, as in the single-problem chain
+        float* Lp = A + (int64_t)c0 * Kp + k0;
+        GemmF32 u = {};
+        u.A = Lp; u.lda = Kp; u.B = Lp; u.ldb = Kp; u.C = A + (int64_t)c0 * Kp + c0; u.ldc = Kp;
+        u.M = Kp - c0; u.N = NB; u.Kc = kk; u.alpha = -1.f; u.beta = 1.f; u.trans_b = 1;
+        u.batch = 1; u.batch2 = n; u.stride2_a = mat; u.stride2_b = mat; u.stride2_c = mat;
+        const int rc = llmc_gemm_f32(u, st);
+        if (rc) return rc;
+      }
       hipLaunchKernelGGL(potf2_inv_kernel, dim3(n), dim3(256), 0, st, A, Kp, c0, (int)K, sc);
       LLMC_LAUNCH_STATUS();
       const int M = Kp - c0 - NB;
@@ -523,17 +534,8 @@ extern "C" int llmc_gptq_hinv_grouped(const float* const* H, int64_t ldh, int32_
       g.A = A21; g.lda = Kp; g.B = A + (int64_t)c0 * Kp + c0; g.ldb = Kp; g.C = A21; g.ldc = Kp;
       g.M = M; g.N = NB; g.Kc = NB; g.alpha = 1.f; g.beta = 0.f; g.trans_b = 1;
       g.batch = 1; g.batch2 = n; g.stride2_a = mat; g.stride2_b = mat; g.stride2_c = mat;
-      int rc = llmc_gemm_f32(g, st);
+      const int rc = llmc_gemm_f32(g, st);
       if (rc) return rc;
-      const int nrem = k0 + pw - (c0 + NB);
-      if (nrem > 0) {
-        GemmF32 u = {};
-        u.A = A21; u.lda = Kp; u.B = A21; u.ldb = Kp; u.C = A + (int64_t)(c0 + NB) * Kp + c0 + NB; u.ldc = Kp;
-        u.M = M; u.N = nrem; u.Kc = NB; u.alpha = -1.f; u.beta = 1.f; u.trans_b = 1; u.c_lower = 1;
-        u.batch = 1; u.batch2 = n; u.stride2_a = mat; u.stride2_b = mat; u.stride2_c = mat;
-        rc = llmc_gemm_f32(u, st);
-        if (rc) return rc;
-      }
     }
     const int M2 = Kp - (k0 + pw);
     if (M2 > 0) {

@@ -1558,17 +1558,21 @@ def test_linearize_moe_keeps_the_logits_of_transformers_moe_families(family):
 def test_scheduling_options_do_not_change_gptq_results_on_a_transformers_llama():
     """The scheduling fields of GPTQModifier (lock-step sets, stream concurrency, staging by reference or by
     copy, shared Hessians for identical inputs) leave every quantised parameter bit-identical; one Hessian launch
-    per hook call instead of staged launches changes the summation order only (>= 99.9 % identical weights)."""
+    per hook call instead of staged launches, or early flushes, change the summation order only (>= 99.9 %
+    identical weights without activation ordering)."""
     transformers = pytest.importorskip("transformers")
 
     from llmcompressor_amd import oneshot
     from llmcompressor_amd.modifiers.gptq import GPTQModifier
 
     cfg = transformers.LlamaConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=2,
-                                   num_attention_heads=4, num_key_value_heads=2, vocab_size=256,
+                                   num_attention_heads=4, num_key_value_heads=2, vocab_size=4096,
                                    max_position_embeddings=128)
     torch.manual_seed(3)
-    data = [{"input_ids": torch.randint(0, 256, (1, 128))} for _ in range(6)]
+    # four times as many tokens as the widest Linear has columns, drawn from a vocabulary far larger than the hidden
+    # size: with fewer distinct inputs the Hessians are close to singular and a last-bit change of one (another
+    # summation order) moves far more than 0.1 % of the codes
+    data = [{"input_ids": torch.randint(0, 4096, (1, 128))} for _ in range(16)]
 
     def run(**kw):
         torch.manual_seed(0)
@@ -1579,18 +1583,20 @@ def test_scheduling_options_do_not_change_gptq_results_on_a_transformers_llama()
 
     base = run()
     for kw in (dict(group_min_modules=0), dict(compress_concurrency=1), dict(group_min_modules=0, compress_concurrency=1),
-               dict(stage_by_reference=False), dict(share_identical_inputs=True), dict(stage_max_bytes=1 << 16)):
+               dict(stage_by_reference=False), dict(share_identical_inputs=True)):
         other = run(**kw)
         assert other.keys() == base.keys()
-        same_everywhere = all(torch.equal(base[n], other[n]) for n in base)
-        if "stage_max_bytes" in kw:  # early flushes regroup the token sums
-            agree = min((base[n] == other[n]).float().mean().item() for n in base if n.endswith("proj.weight"))
-            assert agree >= 0.999, (kw, agree)
-        else:
-            assert same_everywhere, kw
-    unstaged = run(hessian_batch_tokens=0)
-    agree = min((base[n] == unstaged[n]).float().mean().item() for n in base if n.endswith("proj.weight"))
-    assert agree >= 0.999, agree
+        assert all(torch.equal(base[n], other[n]) for n in base), kw
+    # Early flushes and unstaged launches regroup the token sums, so the Hessians differ in their last bits.
+    # Activation ordering sorts the Hessian diagonal, whose entries are nearly tied on this random model: a
+    # last-bit change reorders them and the column loop then visits the columns in another order (91 % identical
+    # codes here).  The regrouping itself is therefore compared without activation ordering.
+    plain = run(actorder=None)
+    for kw in (dict(stage_max_bytes=1 << 16), dict(hessian_batch_tokens=0)):
+        other = run(actorder=None, **kw)
+        agree = min((plain[n] == other[n]).float().mean().item() for n in plain if n.endswith("proj.weight"))
+        print(kw, "least agreement", agree)
+        assert agree >= 0.999, (kw, agree)
 
 
 def test_checkpoint_omits_zero_points_of_symmetric_activations(tmp_path):
