@@ -2,10 +2,10 @@
 
 fp32 inputs reproduce the reference's eight known-answer losses (tests/llmcompressor/observers/
 test_mse.py:9-42) to the reference's own abs=1e-10.  For bf16 weights every intermediate is
-rounded to bf16, so near-ties between neighbouring shrink steps are common; the device powf
-and the CPU's differ in the last fp32 bit, which can flip such a tie.  The stated bar is
-therefore: identical (min,max) for >= 99.5 % of the groups, and a quantisation error that
-is never worse than the oracle's choice by more than 2 %.
+rounded to bf16, so near-ties between neighbouring shrink steps are common; the kernels form
+|e|^2.4 as exp2(2.4 log2 e) in extended precision and fall back to powf only where the 16-bit
+rounding of the two could differ, so the search picks the oracle's (min, max) for every group:
+the fixed cases below assert equality (as the 60-case sweep in test_gpu_sweeps.py does).
 """
 import pytest
 import torch
@@ -15,7 +15,6 @@ from oracle import qformat as F
 
 pytestmark = pytest.mark.gpu
 
-GROUP_AGREEMENT = 0.995
 
 
 def _gpu_minmax(w, args, **kw):
@@ -79,7 +78,7 @@ def test_mse_matches_oracle_bf16(name):
     mn, mx = mn.cpu().reshape(emn.shape), mx.cpu().reshape(emx.shape)
     same = ((mn == emn) & (mx == emx)).float().mean().item()
     print(f"{name}: groups identical {same:.4f}")
-    assert same >= GROUP_AGREEMENT
+    assert torch.equal(mn, emn) and torch.equal(mx, emx), same
 
     # the chosen ranges are as good as the oracle's
     def qerr(a, b):
