@@ -340,8 +340,9 @@ def probe_chain():
 
 def probe_moe(mode="both"):
     """One MoE expert layer (128 experts, hidden 2048, intermediate 768, top-8 routing of 4096 tokens: 384 expert
-    Linears) through GPTQModifier W4A16: time of the calibration forward (grouped Hessian launches from the hooks)
-    and of the quantisation of the 384 Linears, with lock-step groups and with the per-module path.  Prints a table."""
+    Linears) through GPTQModifier W4A16 and NVFP4A16: time of the calibration forward (grouped Hessian launches from
+    the hooks) and of the quantisation of the 384 Linears, with lock-step groups and with the per-module path.
+    Prints a table."""
     import torch
 
     from llmcompressor_amd.core import LifecycleCallbacks, active_session
@@ -371,8 +372,10 @@ def probe_moe(mode="both"):
     w, idx = torch.topk(torch.softmax(logits, -1), TOPK, -1)
     print("| quantisation of the 384 expert Linears | forward + Hessians ms per batch | quantise ms | ms per Linear |")
     print("|---|---|---|---|")
-    variants = (("lock-step groups (default)", 8, "lockstep"), ("one module at a time, 4 streams", 0, "permodule"))
-    for label, gmin, key in variants:
+    variants = (("W4A16, lock-step groups (default)", 8, "lockstep", "W4A16"),
+                ("W4A16, one module at a time, 4 streams", 0, "permodule", "W4A16"),
+                ("NVFP4A16, lock-step groups (default)", 8, "lockstep", "NVFP4A16"))
+    for label, gmin, key, scheme in variants:
         if mode not in ("both", key):
             continue
         best = None
@@ -380,7 +383,7 @@ def probe_moe(mode="both"):
             for p in model.parameters():
                 if p.dtype == torch.bfloat16:
                     p.data.normal_(0, 0.02)
-            mod = GPTQModifier(targets="Linear", scheme="W4A16", group_min_modules=gmin)
+            mod = GPTQModifier(targets="Linear", scheme=scheme, group_min_modules=gmin)
             s = active_session()
             s.reset()
             s.initialize(model=model, recipe=mod)
