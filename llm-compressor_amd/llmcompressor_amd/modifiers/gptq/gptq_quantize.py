@@ -190,23 +190,42 @@ def quantize_weight_group(modules, hessians, hessian_divisors, blocksize: int = 
     divs = [hessian_divisors[i] for i in order]
     keys = [keys[i] for i in order]
     prep = []
-    for m, H in zip(mods, Hs):
+    # the column orders of all members in one sort (row-wise stable, so each row is what the per-module call sorts)
+    all_perms = None
+    if all(m.quantization_scheme.weights.actorder for m in mods):
+        all_perms = torch.argsort(torch.stack([torch.diagonal(H) for H in Hs]), dim=1, descending=True, stable=True)
+    base_g_idx = {}
+    for j, (m, H) in enumerate(zip(mods, Hs)):
         quant_args = m.quantization_scheme.weights
         strategy, actorder = quant_args.strategy, quant_args.actorder
         W = m.weight.data if m.weight.data.is_contiguous() else m.weight.data.contiguous()
         num_rows, num_columns = W.shape
-        perm = torch.argsort(torch.diagonal(H), descending=True, stable=True) if actorder else None
+        if all_perms is not None:
+            perm = all_perms[j]
+        else:
+            perm = torch.argsort(torch.diagonal(H), descending=True, stable=True) if actorder else None
         row_div, srow, divisor = _scale_layout(strategy, quant_args, num_rows, num_columns)
         g_idx = None
         if divisor is not None:
-            g_idx = torch.arange(num_columns, device=W.device, dtype=torch.int) // divisor
+            if (num_columns, divisor) not in base_g_idx:
+                base_g_idx[(num_columns, divisor)] = torch.arange(num_columns, device=W.device,
+                                                                  dtype=torch.int) // divisor
+            g_idx = base_g_idx[(num_columns, divisor)]
             if actorder == ActivationOrdering.WEIGHT:
-                g_idx = g_idx[perm]
+                if all_perms is not None:  # one gather for every member with this group width
+                    if ("permuted", divisor) not in base_g_idx:
+                        base_g_idx[("permuted", divisor)] = g_idx[all_perms]
+                    g_idx = base_g_idx[("permuted", divisor)][j]
+                else:
+                    g_idx = g_idx[perm]
         qp = m.weight_observer.get_qparams()
         prep.append(dict(args=quant_args, W=W, perm=perm, g_idx=g_idx, qp=qp, row_div=row_div, srow=srow,
                          zp=None if quant_args.symmetric else qp["zero_point"].to(torch.int8),
                          kscale=effective_scale(qp["scale"], quant_args, W.dtype)))
-    perms = torch.stack([p["perm"] for p in prep]) if prep[0]["perm"] is not None else None
+    if all_perms is not None:
+        perms = all_perms
+    else:
+        perms = torch.stack([p["perm"] for p in prep]) if prep[0]["perm"] is not None else None
 
     U, dead, info = llmc.gptq_prepare_hinv_grouped(Hs, perms, [float(d) for d in divs], float(percdamp))
 
