@@ -34,7 +34,8 @@ from ..quantization.calibration import observe, update_qparams
 from ..quantization.quantization import QuantizationMixin
 from ..utils.concurrent import run_on_streams
 from ..utils.hessian_staging import HessianStagingMixin
-from .gptq_quantize import (accumulate_hessian, make_empty_hessian, quantize_weight, quantize_weight_group,
+from .gptq_quantize import (accumulate_hessian, begin_weight_group, finish_weight_group, make_empty_hessian,
+                            quantize_weight, quantize_weight_group,
                             width_key)
 
 logger = logging.getLogger("llmcompressor_amd")
@@ -163,10 +164,13 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
 
     def on_sequential_epoch_end(self, state: State, event: Event, modules: list[torch.nn.Module] = (), **kwargs):
         modules = [m for m in modules if is_module_quantized(m)]
+        # The Cholesky chains of wide lock-step sets (the experts of an MoE layer) need the Hessians only: they
+        # are enqueued first, and the weights are observed on the host while they run.
+        started = self._begin_compress(list(self._num_samples.keys()))
         observe(modules, base_name="weight")
         self.sync_obs_act_stats(modules)
         update_qparams(modules, ACTIVATION_OBS)
-        self.compress_modules()
+        self._finish_compress(started)
 
     def on_calibration_end(self, state: State, event: Event, **kwargs):
         QuantizationMixin.end_calibration(self, state.model)
@@ -238,6 +242,11 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
         self.compress_module_list(list(self._num_samples.keys()))
 
     def compress_module_list(self, module_list):
+        self._finish_compress(self._begin_compress(module_list))
+
+    def _begin_compress(self, module_list):
+        """Flush what is pending, plan the jobs and enqueue the chains of the wide sets.  Returns
+        (launched wide sets, remaining jobs) for ``_finish_compress``; no weight observer is read here."""
         for module in module_list:  # followers get their own copy of the shared Hessian
             leader = self._leader.pop(module, None)
             if leader is not None:
@@ -254,9 +263,13 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
         # a set of many problems (the experts of an MoE layer) fills the chip by itself: such sets are enqueued one
         # after the other on the calling stream, with one host wait for all of them
         wide = [job for job in jobs if isinstance(job, list) and len(job) >= _WIDE_SET]
-        if wide:
-            self._finish_sets([self._launch_set(part) for part in wide])
-            jobs = [job for job in jobs if not (isinstance(job, list) and len(job) >= _WIDE_SET)]
+        jobs = [job for job in jobs if not (isinstance(job, list) and len(job) >= _WIDE_SET)]
+        return [self._begin_set(part) for part in wide], jobs
+
+    def _finish_compress(self, started):
+        begun, jobs = started
+        if begun:
+            self._finish_sets([self._end_set(b) for b in begun])
         if not jobs:
             return
         members = [m for job in jobs for m in (job if isinstance(job, list) else [job])]
@@ -312,6 +325,9 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
         self._finish_sets([self._launch_set(part, produced_on)], consumed_on)
 
     def _launch_set(self, part, produced_on=None):
+        return self._end_set(self._begin_set(part, produced_on))
+
+    def _begin_set(self, part, produced_on=None):
         hs = [self._hessians.pop(m) for m in part]
         tallies = [self._num_samples.pop(m) for m in part]
         if all(isinstance(t, torch.Tensor) and t.is_cuda for t in tallies):  # one transfer, not one per module
@@ -323,7 +339,13 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
         names = [self._module_names.get(m, m.__class__.__name__) for m in part]
         logger.info(f"Quantizing {len(part)} modules in lock-step ({names[0]} .. {names[-1]})")
         with torch.no_grad():
-            results = quantize_weight_group(part, hs, tallies, self.block_size, self.dampening_frac)
+            ctx = begin_weight_group(part, hs, tallies, self.dampening_frac)
+        return part, names, ctx
+
+    def _end_set(self, begun):
+        part, names, ctx = begun
+        with torch.no_grad():
+            results = finish_weight_group(ctx, self.block_size)
         return part, names, results
 
     def _finish_sets(self, launched, consumed_on=None):

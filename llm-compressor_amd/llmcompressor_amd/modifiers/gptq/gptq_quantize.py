@@ -23,7 +23,7 @@ logger = logging.getLogger("llmcompressor_amd")
 GPTQ_PRECISION = torch.float32
 
 __all__ = ["make_empty_hessian", "accumulate_hessian", "quantize_weight", "quantize_weight_tensors",
-           "quantize_weight_group", "group_key", "width_key"]
+           "quantize_weight_group", "begin_weight_group", "finish_weight_group", "group_key", "width_key"]
 
 
 def make_empty_hessian(module: torch.nn.Module, device: torch.device | None = None) -> torch.Tensor:
@@ -181,6 +181,13 @@ def quantize_weight_group(modules, hessians, hessian_divisors, blocksize: int = 
     and one lock-step column loop per set of equal shape and scheme, instead of a chain of small kernels per
     module.  Same results as calling ``quantize_weight`` on each.  Returns a list of
     (loss tensor, q_param_dict, info tensor) in the order of ``modules``."""
+    return finish_weight_group(begin_weight_group(modules, hessians, hessian_divisors, percdamp), blocksize)
+
+
+def begin_weight_group(modules, hessians, hessian_divisors, percdamp: float = 0.01):
+    """First half of ``quantize_weight_group``: column orders and the lock-step Cholesky chain, which need the
+    Hessians only.  The weight observers' statistics are not read before ``finish_weight_group``, so a caller may
+    enqueue the chains of several sets, observe the weights while they run, and finish afterwards."""
     n = len(modules)
     keys = [group_key(m, m.quantization_scheme.weights, H) for m, H in zip(modules, hessians)]
     # members of one column-loop set next to each other, so that their factors are one slice of the batch
@@ -189,21 +196,32 @@ def quantize_weight_group(modules, hessians, hessian_divisors, blocksize: int = 
     Hs = [hessians[i] for i in order]
     divs = [hessian_divisors[i] for i in order]
     keys = [keys[i] for i in order]
-    prep = []
     # the column orders of all members in one sort (row-wise stable, so each row is what the per-module call sorts)
     all_perms = None
     if all(m.quantization_scheme.weights.actorder for m in mods):
         all_perms = torch.argsort(torch.stack([torch.diagonal(H) for H in Hs]), dim=1, descending=True, stable=True)
+        perms = all_perms
+    else:
+        single = [torch.argsort(torch.diagonal(H), descending=True, stable=True)
+                  if m.quantization_scheme.weights.actorder else None for m, H in zip(mods, Hs)]
+        perms = torch.stack(single) if single[0] is not None else None
+    U, dead, info = llmc.gptq_prepare_hinv_grouped(Hs, perms, [float(d) for d in divs], float(percdamp))
+    return dict(n=n, order=order, mods=mods, keys=keys, perms=perms, all_perms=all_perms, U=U, dead=dead, info=info)
+
+
+def finish_weight_group(ctx, blocksize: int = 128):
+    """Second half of ``quantize_weight_group``: quantisation parameters from the weight observers, the lock-step
+    column loops on the factors of ``begin_weight_group``, and the results in the caller's order."""
+    n, order, mods, keys = ctx["n"], ctx["order"], ctx["mods"], ctx["keys"]
+    perms, all_perms, U, dead, info = ctx["perms"], ctx["all_perms"], ctx["U"], ctx["dead"], ctx["info"]
+    prep = []
     base_g_idx = {}
-    for j, (m, H) in enumerate(zip(mods, Hs)):
+    for j, m in enumerate(mods):
         quant_args = m.quantization_scheme.weights
         strategy, actorder = quant_args.strategy, quant_args.actorder
         W = m.weight.data if m.weight.data.is_contiguous() else m.weight.data.contiguous()
         num_rows, num_columns = W.shape
-        if all_perms is not None:
-            perm = all_perms[j]
-        else:
-            perm = torch.argsort(torch.diagonal(H), descending=True, stable=True) if actorder else None
+        perm = perms[j] if (perms is not None and actorder) else None
         row_div, srow, divisor = _scale_layout(strategy, quant_args, num_rows, num_columns)
         g_idx = None
         if divisor is not None:
@@ -222,12 +240,6 @@ def quantize_weight_group(modules, hessians, hessian_divisors, blocksize: int = 
         prep.append(dict(args=quant_args, W=W, perm=perm, g_idx=g_idx, qp=qp, row_div=row_div, srow=srow,
                          zp=None if quant_args.symmetric else qp["zero_point"].to(torch.int8),
                          kscale=effective_scale(qp["scale"], quant_args, W.dtype)))
-    if all_perms is not None:
-        perms = all_perms
-    else:
-        perms = torch.stack([p["perm"] for p in prep]) if prep[0]["perm"] is not None else None
-
-    U, dead, info = llmc.gptq_prepare_hinv_grouped(Hs, perms, [float(d) for d in divs], float(percdamp))
 
     outs, losses = [None] * n, [None] * n
     at = 0
