@@ -295,7 +295,8 @@ __global__ __launch_bounds__(256) void potf2_inv_kernel(float* __restrict__ A, i
   }
 }
 
-// U[i][j] = X[K-1-i][K-1-j] for j >= i, 0 below; identity when the factorisation failed
+// U[i][j] = X[K-1-i][K-1-j] for j >= i, 0 below; identity when the factorisation failed.  Four columns per
+// thread: a row of U is a row of X read backwards, so four neighbours of U are four neighbours of X.
 __global__ __launch_bounds__(256) void hinv_copyout_kernel(const float* __restrict__ X, int Kp, int K,
                                                            const HinvScalars* __restrict__ sc,
                                                            float* __restrict__ U, int64_t ldu,
@@ -307,17 +308,38 @@ __global__ __launch_bounds__(256) void hinv_copyout_kernel(const float* __restri
     X += (int64_t)blockIdx.z * Kp * Kp;
     if (info_out) info_out += blockIdx.z;
   }
-  const int j = blockIdx.x * 256 + threadIdx.x;
+  const int j0 = (blockIdx.x * 256 + threadIdx.x) * 4;
   const int i = blockIdx.y;
-  if (i == 0 && j == 0 && info_out) *info_out = sc->info;
-  if (j >= K) return;
-  float v = 0.f;
-  if (sc->info != 0) {
-    v = (i == j) ? 1.f : 0.f;
-  } else if (j >= i) {
-    v = X[(int64_t)(K - 1 - i) * Kp + (K - 1 - j)];
+  if (i == 0 && j0 == 0 && info_out) *info_out = sc->info;
+  if (j0 >= K) return;
+  const bool failed = sc->info != 0;
+  const float* xrow = X + (int64_t)(K - 1 - i) * Kp;
+  float* urow = U + (int64_t)i * ldu;
+  const bool vec = j0 + 3 < K && (K & 3) == 0 && (ldu & 3) == 0 && (((uintptr_t)U | (uintptr_t)X) & 15) == 0;
+  if (vec && !failed && j0 >= i) {  // four values of X at K-4-j0 .. K-1-j0, reversed
+    const float4 x = *(const float4*)(xrow + (K - 4 - j0));
+    *(float4*)(urow + j0) = make_float4(x.w, x.z, x.y, x.x);
+    return;
   }
-  U[(int64_t)i * ldu + j] = v;
+  float v[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int j = j0 + e;
+    v[e] = 0.f;
+    if (j < K) {
+      if (failed)
+        v[e] = (i == j) ? 1.f : 0.f;
+      else if (j >= i)
+        v[e] = xrow[K - 1 - j];
+    }
+  }
+  if (vec) {
+    *(float4*)(urow + j0) = make_float4(v[0], v[1], v[2], v[3]);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (j0 + e < K) urow[j0 + e] = v[e];
+  }
 }
 
 inline int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * b; }
@@ -437,7 +459,7 @@ extern "C" int llmc_gptq_hinv(float* H, int64_t ldh, int64_t K, const int32_t* p
     }
   }
 
-  hipLaunchKernelGGL(hinv_copyout_kernel, dim3((unsigned)((K + 255) / 256), (unsigned)K), dim3(256), 0, st, A, Kp,
+  hipLaunchKernelGGL(hinv_copyout_kernel, dim3((unsigned)((K + 1023) / 1024), (unsigned)K), dim3(256), 0, st, A, Kp,
                      (int)K, sc, H, ldh, info_out, (const HinvItem*)nullptr);
   LLMC_LAUNCH_STATUS();
   return 0;
@@ -581,7 +603,7 @@ extern "C" int llmc_gptq_hinv_grouped(const float* const* H, int64_t ldh, int32_
     }
   }
 
-  hipLaunchKernelGGL(hinv_copyout_kernel, dim3((unsigned)((K + 255) / 256), (unsigned)K, (unsigned)n), dim3(256), 0, st,
+  hipLaunchKernelGGL(hinv_copyout_kernel, dim3((unsigned)((K + 1023) / 1024), (unsigned)K, (unsigned)n), dim3(256), 0, st,
                      A, Kp, (int)K, sc, (float*)nullptr, ldu, info_out, (const HinvItem*)items);
   LLMC_LAUNCH_STATUS();
   return 0;
