@@ -88,8 +88,9 @@ def test_blocksize_independence(bs):
     assert agree >= 0.99
 
 
-def test_matches_textbook_gptq_fp64():
-    w, H = _problem(R=16, K=24, seed=3, dtype=torch.float32)
+@pytest.mark.parametrize("R,K,seed", [(16, 24, 3), (256, 256, 2)])
+def test_matches_textbook_gptq_fp64(R, K, seed):
+    w, H = _problem(R=R, K=K, seed=seed, dtype=torch.float32)
     args = F.QArgs(num_bits=4, strategy="group", group_size=8)
     obs = _obs(w, args)
     scale, zp = F.calculate_qparams(obs.min_vals, obs.max_vals, args)
@@ -101,7 +102,9 @@ def test_matches_textbook_gptq_fp64():
     Q = G.textbook_gptq_fp64(w, H, qcol)
     loss, out, info = G.quantize_weight(w, obs, args, H.clone())
     assert info["ok"]
-    assert (out["weight"].double() == Q).float().mean().item() >= 0.98
+    # fp32 blocked restatement against the un-blocked fp64 elimination: only a code whose pre-rounding value sits
+    # within fp32 noise of a rounding boundary may differ (65 536 elements in the larger case; measured: none)
+    assert (out["weight"].double() == Q).float().mean().item() >= 0.995
     # loss recomputed independently: 1/2 sum (w-q)^2/d^2 is >= 0 and finite
     assert loss >= 0 and torch.isfinite(torch.tensor(loss))
 
