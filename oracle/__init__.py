@@ -27,17 +27,25 @@ closed form or invariant says so here):
   un-blocked GPTQ in fp64, block-size independence, grid membership),
   ``moe.experts_forward`` (the reference's routing counts for 4 experts / top-2,
   the dense fp64 closed form).
-* parity unpinned (no reference-held vector exists; follows the public format
-  specs): MXFP4 E8M0 scale generation, ``pack_to_int32`` / ``pack_fp4_to_uint8``
-  byte layouts, fp8 storage, per-token dynamic FP8 scales, zero-scale epsilon
-  substitution, the BLOCK strategy inside the GPTQ column loop, the checkpoint
-  format name of int weights with quantised activations.  Cross-checks that do
-  not lift the status (``tests/test_oracle_golden.py``): the MXFP4 exponent rule
-  against the OCP Microscaling definition over every bf16 maximum (equal, or one
-  more where the rounding bump carries, mantissas >= 1.75); the E8M0 byte against
-  ``torch.float8_e8m0fnu``; per-token FP8 against the per-row helper a consumer
-  of such checkpoints applies (same reduce dimension, scales equal after rounding
-  to bf16, >= 95 % equal bytes, the rest one e4m3 step away).
+* pinned by independent definitions importable here (``tests/test_oracle_formats.py``; no reference-held bytes
+  exist for these): ``pack_fp4_to_uint8`` nibble order, sign bit and the -0 nibble, and the E8M0 byte with its
+  bias (the MXFP4 consumer decode of ``transformers.integrations.mxfp4`` gives back ``fake_quantize`` bit for
+  bit; swapped nibbles, a dropped -0 or a bias off by one fail); ``cast_to_fp4`` rounding and the e2m1 codes
+  (triton's OCP reference encoder over every bf16 value); the NVFP4 triple nibble / e4m3 scale byte / global
+  scale (decode written from the format); fp8 storage (nearest-even over a table of the 256 e4m3fn bytes built
+  from the bit fields, every bf16 input); ``pack_to_int32`` (shift-and-mask decode written from the published
+  ``pack_factor = 32 // num_bits`` definition, every code in every slot, and the reference-held int4 group
+  matrix of ``test_lifecycle.py`` through the packed words); the BLOCK strategy inside the GPTQ column loop
+  (diagonal Hessian => the reference-held block [2, 3] matrix of ``test_lifecycle.py``).
+* parity unpinned (no reference-held vector exists and nothing importable decides them; each sits behind one
+  function): MXFP4 E8M0 scale *generation* for group maxima with mantissa >= 1.75 (``mxfp4_scale_exponent``: the
+  bit-pattern rule's rounding bump carries there and gives one more than the OCP floor rule -- brute force over
+  every bf16 maximum in ``tests/test_oracle_golden.py`` shows the two rules differ exactly there); the zero-scale
+  epsilon substitution (``calculate_qparams``); the per-token dynamic FP8 reduce / scale-dtype path
+  (``compute_dynamic_scales_and_zp``; cross-checked against the per-row helper a consumer applies: same reduce
+  dimension, scales equal after rounding to bf16, >= 95 % equal bytes, the rest one e4m3 step away); the dtype in
+  which ``q * scale`` is formed when x is fp32 and the scale bf16 (``_dequantize``); the checkpoint format name of
+  int weights with quantised activations.
 * parity unpinned by reference vectors, pinned by mathematics only:
   ``sparsegpt.accumulate_hessian`` / ``sparsegpt.sparsify_weight`` (the
   reference's SparseGPT tests need hub models; see ``tests/test_oracle_sparsegpt.py``:

@@ -56,11 +56,17 @@ def hessian_inverse_factor(H, percdamp):
         return torch.eye(H.shape[0], dtype=H.dtype), False
 
 
-def quantize_weight(weight, observer: Observer, quant_args: QArgs, hessian, blocksize=128, percdamp=0.01):
+def quantize_weight(weight, observer: Observer, quant_args: QArgs, hessian, blocksize=128, percdamp=0.01,
+                    fused_update=False):
     """gptq_quantize.py:67-264.  ``weight`` [R,K] in its own dtype; ``hessian`` is consumed.
 
     Returns ``(loss, q_param_dict, info)`` where ``info['ok']`` is False when the
     identity (round-to-nearest) fallback was taken.
+
+    ``fused_update=True`` is NOT the reference: it forms the in-block update ``w - err * U[i, j]`` with one
+    rounding (an fma, which is what the device's block kernel issues) instead of rounding the outer product
+    first (gptq_quantize.py:232-233).  It exists so that a test can bound the effect of that one-rounding
+    difference on the codes.
     """
     strategy = quant_args.strategy
     actorder = quant_args.actorder
@@ -128,7 +134,11 @@ def quantize_weight(weight, observer: Observer, quant_args: QArgs, hessian, bloc
             Q1[:, i] = q
             losses1[:, i] = (w - q) ** 2 / d**2
             err1 = (w - q) / d
-            W1[:, i:] -= err1.unsqueeze(1).matmul(Hinv1[i, i:].unsqueeze(0))
+            if fused_update:
+                # exact product of two fp32 values in fp64, one rounding of the difference back to fp32
+                W1[:, i:] = (W1[:, i:].double() - err1.double().unsqueeze(1) * Hinv1[i, i:].double().unsqueeze(0)).float()
+            else:
+                W1[:, i:] -= err1.unsqueeze(1).matmul(Hinv1[i, i:].unsqueeze(0))
             Err1[:, i] = err1
         W[:, i1:i2] = Q1
         losses += torch.sum(losses1, 1) / 2

@@ -1,4 +1,5 @@
-"""Oracle: compressed-tensors storage formats (parity unpinned: no reference-held bytes).
+"""Oracle: compressed-tensors storage formats (no reference-held bytes exist; the layouts are pinned by
+independent decoders in ``tests/test_oracle_formats.py``, see ``oracle/__init__.py``).
 
 TEST INFRASTRUCTURE ONLY (see ``oracle/__init__.py``).
 

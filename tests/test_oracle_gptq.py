@@ -141,3 +141,29 @@ def test_upper_factor_identity():
     J = torch.eye(24, dtype=torch.float64).flip(0)
     Rr = J @ torch.linalg.cholesky(J @ Hd @ J) @ J
     assert torch.allclose(torch.linalg.inv(Rr), U.double(), atol=1e-4, rtol=1e-3)
+
+
+@pytest.mark.parametrize("T", [2048, 160])
+@pytest.mark.parametrize("fmt", ["w4a16", "nvfp4"])
+def test_one_rounding_in_block_update_changes_next_to_nothing(fmt, T):
+    """The device's block kernel applies ``w <- fma(-err, U[i][j], w)`` (one rounding); the reference rounds the outer
+    product, then subtracts (gptq_quantize.py:232-233).  Bound of the effect on the result, on a well-conditioned
+    Hessian (T >= K tokens) and on a rank-deficient one kept regular by the damping alone: at least 99.95 % of the
+    weights identical (measured at 768 x 2048: 100 % / 99.983 % for nvfp4 with 965 tokens)."""
+    torch.manual_seed(T)
+    R, K = 192, 512
+    x = (torch.randn(T, K) * torch.pow(2.0, 2.0 * torch.rand(K))).bfloat16()
+    w = (torch.randn(R, K) * 0.02).bfloat16()
+    H, _ = G.accumulate_hessian(x.unsqueeze(0), G.make_empty_hessian(K), torch.zeros(()))
+    if fmt == "w4a16":
+        args = F.QArgs(num_bits=4, strategy="group", group_size=128, actorder="weight")
+    else:
+        args = F.QArgs(num_bits=4, type="float", strategy="tensor_group", group_size=16,
+                       scale_dtype=torch.float8_e4m3fn, actorder="weight")
+    outs = []
+    for fused in (False, True):
+        _, out, info = G.quantize_weight(w, _obs(w, args), args, H.clone(), fused_update=fused)
+        assert info["ok"]
+        outs.append(out["weight"])
+    agree = (outs[0] == outs[1]).float().mean().item()
+    assert agree >= 0.9995, agree
