@@ -50,7 +50,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 def dominant_traffic_bytes(tokens_per_launch: int):
     """HBM bytes per launch of the dominant kernel, from the FETCH_SIZE / WRITE_SIZE counter runs whose raw
     averages and calibration are kept next to their summary (profiles/hessian_syrk_k14336_t65536_hbm_traffic.json);
-    None when no counter run exists for this launch size."""
+    None when no counter run exists for this launch size or the kernel's source has changed since that run."""
     path = os.path.join(ROOT, "profiles", "hessian_syrk_k14336_t65536_hbm_traffic.json")
     try:
         with open(path) as f:
@@ -58,6 +58,15 @@ def dominant_traffic_bytes(tokens_per_launch: int):
     except OSError:
         return None
     if int(rec.get("tokens_per_launch", -1)) != int(tokens_per_launch) or int(rec.get("K", -1)) != INTER:
+        return None
+    # the counters were read on one build of the kernel: a figure taken on other source is not reported
+    import hashlib
+
+    try:
+        with open(os.path.join(ROOT, rec.get("kernel_source", "")), "rb") as f:
+            if hashlib.sha256(f.read()).hexdigest() != rec.get("kernel_source_sha256"):
+                return None
+    except OSError:
         return None
     return float(rec["FETCH_SIZE_avg_per_dispatch"]) * rec["FETCH_SIZE_unit_bytes"] + \
         float(rec["WRITE_SIZE_avg_per_dispatch"]) * rec["WRITE_SIZE_unit_bytes"]
@@ -616,7 +625,7 @@ def main():
 
     ops.hessian_accumulate_segments_ = timed_segments
 
-    def step(record: bool, share: bool = False):
+    def step(record: bool, share: bool = False):  # the headline step accumulates one Hessian per module, as the reference does
         for name, r, k in LINEARS:
             getattr(layer, name).weight.data.copy_(originals[name])
         recording[0] = record

@@ -63,7 +63,11 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
 
     :param share_identical_inputs: Linears that are fed the very same tensor on every call (q/k/v, gate/up)
         have the same Hessian; accumulate it once and hand each of them a copy when it is compressed.
-        Results are identical; off by default, as the reference accumulates one Hessian per module.
+        Results are bit-identical to one accumulation per module.  A module shares only while the tensor it
+        receives is the very object (address, shape, strides, version) its leader has just accumulated, starting
+        with its first call; a module that shared and later receives another tensor, or misses a call of its
+        leader, raises (its leader has then already taken in a call the module did not see, so the two Hessians
+        cannot be separated after the fact) -- pass ``share_identical_inputs=False`` for such a model
 
     :param stage_by_reference: while staging, keep references to the hook's input tensors instead of copying
         them into a staging buffer, and hand the kernel the list of buffers.  Taken only for contiguous
@@ -90,7 +94,7 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
     actorder: ActivationOrdering | Sentinel | None = Sentinel("static")
     offload_hessians: bool = False
     hessian_batch_tokens: int = 65536
-    share_identical_inputs: bool = False
+    share_identical_inputs: bool = True
     compress_concurrency: int = 4
     group_min_modules: int = 3
     group_max_bytes: int = 8 << 30
@@ -106,6 +110,7 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
     _group_pending: list | None = PrivateAttr(default=None)
     _leader: dict = PrivateAttr(default_factory=dict)  # follower module -> module whose Hessian it shares
     _recent_input: tuple | None = PrivateAttr(default=None)  # (tensor kept alive, its version, leader)
+    _hook_calls: dict = PrivateAttr(default_factory=dict)  # module -> hook calls so far (leaders and followers)
     _streams: dict = PrivateAttr(default_factory=dict)
 
     def resolve_quantization_config(self) -> QuantizationConfig:
@@ -179,8 +184,10 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
     def calibrate_module(self, module: torch.nn.Module, args: tuple[torch.Tensor, ...], _output: torch.Tensor):
         """Forward hook: accumulate the Hessian of the module's input."""
         inp = args[0]
-        if self.share_identical_inputs and self._follows_recent_input(module, inp):
-            return
+        if self.share_identical_inputs:
+            self._hook_calls[module] = self._hook_calls.get(module, 0) + 1
+            if self._follows_recent_input(module, inp):
+                return
         grouped = (self._group_pending is not None and isinstance(module, torch.nn.Linear) and inp.is_cuda
                    and not self.offload_hessians and inp.dtype in (torch.bfloat16, torch.float16))
         if module not in self._num_samples:
@@ -218,7 +225,7 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
             return True
         if leader is not None:
             raise RuntimeError("share_identical_inputs: a module that shared its input with another one received a "
-                               "different tensor on a later call; disable share_identical_inputs for this model")
+                               "different tensor on a later call; pass share_identical_inputs=False for this model")
         self._recent_input = (inp, inp._version, module)
         return False
 
@@ -250,11 +257,18 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
         for module in module_list:  # followers get their own copy of the shared Hessian
             leader = self._leader.pop(module, None)
             if leader is not None:
+                if self._hook_calls.get(module) != self._hook_calls.get(leader):
+                    raise RuntimeError("share_identical_inputs: a module that shared its input with another one was "
+                                       f"called {self._hook_calls.get(module)} times, the module it shared with "
+                                       f"{self._hook_calls.get(leader)} times; pass share_identical_inputs=False for "
+                                       "this model")
                 self._flush(leader)
                 self._hessians[module] = self._hessians[leader].clone()
                 self._num_samples[module] = torch.tensor(float(self._num_samples[module]),
                                                          device=self._hessians[module].device)
         self._recent_input = None
+        for module in module_list:
+            self._hook_calls.pop(module, None)
         for module in module_list:  # pending activations go in on the calibration stream
             self._flush(module)
             self._staged.pop(module, None)
@@ -398,6 +412,7 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
         self._held = dict()
         self._held_bytes = 0
         self._leader = dict()
+        self._hook_calls = dict()
         self._recent_input = None
         return True
 
