@@ -374,7 +374,8 @@ def test_oneshot_datafree_rtn_and_checkpoint_round_trip(tmp_path, scheme, fmt):
     assert torch.isfinite(y.float()).all()
 
 
-def test_moe_gptq_zero_token_expert_is_zeroed():
+@pytest.mark.parametrize("share", [True, False])
+def test_moe_gptq_zero_token_expert_is_zeroed(share):
     """An expert that never receives a token keeps H = 0: every column is dead and its weight is zeroed."""
     from llmcompressor_amd.core import State, active_session
     from llmcompressor_amd.modeling import LinearExperts2D
@@ -391,8 +392,8 @@ def test_moe_gptq_zero_token_expert_is_zeroed():
             self.layers = torch.nn.ModuleList([experts])
 
     model = Wrap()
-    mod = GPTQModifier(targets="Linear", config_groups={"g": dict(targets=["Linear"], weights=dict(
-        num_bits=4, strategy="group", group_size=32))})
+    mod = GPTQModifier(targets="Linear", share_identical_inputs=share, config_groups={"g": dict(
+        targets=["Linear"], weights=dict(num_bits=4, strategy="group", group_size=32))})
     session = active_session()
     session.reset()
     session.initialize(model=model, recipe=mod)
@@ -413,8 +414,9 @@ def test_moe_gptq_zero_token_expert_is_zeroed():
     finally:
         ops.hessian_accumulate_grouped_ = raw_grouped
     # the experts' hook calls were flushed as grouped launches: per forward one for the gate/up width
-    # (2 x 4 problems) and one for the down width (4 problems)
-    assert sorted(calls) == [4, 4, 4, 8, 8, 8]
+    # (2 x 4 problems; 4 when an expert's up_proj shares the Hessian of its gate_proj, which is fed the same
+    # rows) and one for the down width (4 problems)
+    assert sorted(calls) == ([4, 4, 4, 4, 4, 4] if share else [4, 4, 4, 8, 8, 8])
     routed0 = x[(idx == 0).any(dim=1)].double()
     H0 = mod._hessians[experts[0].gate_proj]
     ref = 3 * 2 * (routed0.t() @ routed0)
