@@ -15,6 +15,7 @@
 // fallback) without a host round trip.
 #include <vector>
 
+#include "chol_block.h"
 #include "common.h"
 #include "gemm_f32.h"
 
@@ -153,145 +154,30 @@ __global__ __launch_bounds__(256) void hinv_copyin_rows_kernel(const float* __re
   }
 }
 
-// Factor the 64x64 diagonal block at (k0,k0) and replace it by the inverse of its factor.
-// The block and the growing inverse X = L^-1 live in registers: thread (ty, tx) of a 16 x 16 grid
-// owns the 4x4 sub-blocks L[4ty.., 4tx..] and X[4ty.., 4tx..].  Right-looking in steps of four
-// columns with one barrier per step: the owners publish the 64x4 column panel of the partly
-// factored block and the four matching rows of X through LDS; every thread then factors the 4x4
-// diagonal block itself (redundantly), solves its own rows of the panel against it and applies
-// the rank-4 updates  L[i][c] -= sum_j l_ij l_cj,  X[i][c] -= sum_j l_ij x_jc  to its sub-blocks,
-// so factor and inverse advance together.
+// Factor the 64x64 diagonal block at (k0,k0) and replace it by the inverse of its factor (chol_block.h).
 __global__ __launch_bounds__(256) void potf2_inv_kernel(float* __restrict__ A, int Kp, int k0, int K,
                                                         HinvScalars* sc) {
   A += (int64_t)blockIdx.x * Kp * Kp;  // grouped call: one workgroup per problem (a single problem has one workgroup)
   sc += blockIdx.x;
-  __shared__ __attribute__((aligned(16))) float colbuf[2][NB][4];  // panel: row i, columns j0..j0+3
-  __shared__ __attribute__((aligned(16))) float xrow[2][4][NB];    // rows j0..j0+3 of X
-  const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
-  float Lb[4][4], Xb[4][4];
+  __shared__ __attribute__((aligned(16))) float Xl[NB * cholblk::LDD];
+  __shared__ __attribute__((aligned(16))) cholblk::FactorScratch fs;
+  const int tid = threadIdx.x, w = tid >> 6, r = tid & 63;
+  float a[16];
+  {
+    const float* src = A + (int64_t)(k0 + r) * Kp + k0 + 16 * w;
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const float4 v = *(const float4*)(A + (int64_t)(k0 + 4 * ty + r) * Kp + k0 + 4 * tx);
-    const float e[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      Lb[r][c] = (4 * tx + c <= 4 * ty + r) ? e[c] : 0.f;
-      Xb[r][c] = (4 * tx + c == 4 * ty + r) ? 1.f : 0.f;
+    for (int q = 0; q < 4; ++q) {
+      const float4 v = *(const float4*)(src + 4 * q);
+      a[4 * q] = v.x; a[4 * q + 1] = v.y; a[4 * q + 2] = v.z; a[4 * q + 3] = v.w;
     }
   }
-  // x = p * G^-T for one 4-vector p (a row of the panel): forward substitution against the
-  // lower-triangular G with reciprocal diagonal gi
-  auto solve_row = [](const float4 p, const float (&G)[4][4], const float (&gi)[4], float (&l)[4]) {
-    l[0] = p.x * gi[0];
-    l[1] = (p.y - l[0] * G[1][0]) * gi[1];
-    l[2] = (p.z - l[0] * G[2][0] - l[1] * G[2][1]) * gi[2];
-    l[3] = (p.w - l[0] * G[3][0] - l[1] * G[3][1] - l[2] * G[3][2]) * gi[3];
-  };
-  for (int jb = 0; jb < NB / 4; ++jb) {
-    const int buf = jb & 1, j0 = 4 * jb;
-    if (tx == jb) {
+  const int bad = cholblk::factor_invert_64(a, Xl, fs);
+  // first failing pivot, 1-based index in the ORIGINAL (un-reversed) ordering
+  if (tid == 0 && bad < NB && k0 + bad < K) atomicCAS(&sc->info, 0, K - (k0 + bad));
 #pragma unroll
-      for (int r = 0; r < 4; ++r)
-        *(float4*)colbuf[buf][4 * ty + r] = make_float4(Lb[r][0], Lb[r][1], Lb[r][2], Lb[r][3]);
-    }
-    if (ty == jb) {
-#pragma unroll
-      for (int jj = 0; jj < 4; ++jj)
-        *(float4*)&xrow[buf][jj][4 * tx] = make_float4(Xb[jj][0], Xb[jj][1], Xb[jj][2], Xb[jj][3]);
-    }
-    __syncthreads();
-    if (ty < jb) continue;  // this thread's rows are final; it still reaches the barrier of every later step
-    // 4x4 Cholesky of the diagonal block
-    float D[4][4], G[4][4], gi[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const float4 v = *(const float4*)colbuf[buf][j0 + r];
-      D[r][0] = v.x; D[r][1] = v.y; D[r][2] = v.z; D[r][3] = v.w;
-    }
-#pragma unroll
-    for (int jj = 0; jj < 4; ++jj) {
-      float d = D[jj][jj];
-#pragma unroll
-      for (int k = 0; k < jj; ++k) d -= G[jj][k] * G[jj][k];
-      if (!(d > 0.f) || d > 3.0e38f) {
-        // first failing pivot, 1-based index in the ORIGINAL (un-reversed) ordering
-        if (tid == 255 && k0 + j0 + jj < K) atomicCAS(&sc->info, 0, K - (k0 + j0 + jj));
-        d = 1.f;
-      }
-      // 1/sqrt(d): hardware estimate plus one Newton step (the four pivots of a step form a
-      // dependent chain, so the full-precision sqrt and divide sequences would dominate it)
-      float rs = __builtin_amdgcn_rsqf(d);
-      rs = rs * (1.5f - 0.5f * d * rs * rs);
-      G[jj][jj] = d * rs;
-      gi[jj] = rs;
-#pragma unroll
-      for (int r = jj + 1; r < 4; ++r) {
-        float v = D[r][jj];
-#pragma unroll
-        for (int k = 0; k < jj; ++k) v -= G[r][k] * G[jj][k];
-        G[r][jj] = v * gi[jj];
-      }
-    }
-    // rows j0..j0+3 of the inverse: Xf = G^-1 * (published rows), for this thread's four columns
-    float Xf[4][4];
-    {
-      float4 xr[4];
-#pragma unroll
-      for (int jj = 0; jj < 4; ++jj) xr[jj] = *(const float4*)&xrow[buf][jj][4 * tx];
-      const float in[4][4] = {{xr[0].x, xr[0].y, xr[0].z, xr[0].w}, {xr[1].x, xr[1].y, xr[1].z, xr[1].w},
-                              {xr[2].x, xr[2].y, xr[2].z, xr[2].w}, {xr[3].x, xr[3].y, xr[3].z, xr[3].w}};
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        Xf[0][c] = in[0][c] * gi[0];
-        Xf[1][c] = (in[1][c] - G[1][0] * Xf[0][c]) * gi[1];
-        Xf[2][c] = (in[2][c] - G[2][0] * Xf[0][c] - G[2][1] * Xf[1][c]) * gi[2];
-        Xf[3][c] = (in[3][c] - G[3][0] * Xf[0][c] - G[3][1] * Xf[1][c] - G[3][2] * Xf[2][c]) * gi[3];
-      }
-    }
-    if (ty == jb) {
-#pragma unroll
-      for (int jj = 0; jj < 4; ++jj)
-#pragma unroll
-        for (int c = 0; c < 4; ++c) Xb[jj][c] = Xf[jj][c];
-      if (tx == jb) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-#pragma unroll
-          for (int c = 0; c < 4; ++c) Lb[r][c] = c <= r ? G[r][c] : 0.f;
-      }
-      continue;
-    }
-    // rows below the block: this thread's rows of the solved panel, then the rank-4 updates
-    float Lr[4][4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) solve_row(*(const float4*)colbuf[buf][4 * ty + r], G, gi, Lr[r]);
-#pragma unroll
-    for (int r = 0; r < 4; ++r)
-#pragma unroll
-      for (int c = 0; c < 4; ++c)
-        Xb[r][c] -= Lr[r][0] * Xf[0][c] + Lr[r][1] * Xf[1][c] + Lr[r][2] * Xf[2][c] + Lr[r][3] * Xf[3][c];
-    if (tx == jb) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-#pragma unroll
-        for (int c = 0; c < 4; ++c) Lb[r][c] = Lr[r][c];  // these four columns are final
-    } else if (tx > jb) {
-      float Lc[4][4];
-#pragma unroll
-      for (int c = 0; c < 4; ++c) solve_row(*(const float4*)colbuf[buf][4 * tx + c], G, gi, Lc[c]);
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-#pragma unroll
-        for (int c = 0; c < 4; ++c)
-          Lb[r][c] -= Lr[r][0] * Lc[c][0] + Lr[r][1] * Lc[c][1] + Lr[r][2] * Lc[c][2] + Lr[r][3] * Lc[c][3];
-    }
-  }
-#pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    float e[4];
-#pragma unroll
-    for (int c = 0; c < 4; ++c) e[c] = (4 * tx + c <= 4 * ty + r) ? Xb[r][c] : 0.f;
-    *(float4*)(A + (int64_t)(k0 + 4 * ty + r) * Kp + k0 + 4 * tx) = make_float4(e[0], e[1], e[2], e[3]);
+  for (int n = 0; n < 4; ++n) {
+    const int idx = tid + 256 * n, row = idx >> 4, c4 = (idx & 15) * 4;
+    *(float4*)(A + (int64_t)(k0 + row) * Kp + k0 + c4) = *(const float4*)(Xl + row * cholblk::LDD + c4);
   }
 }
 
