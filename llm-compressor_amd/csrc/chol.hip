@@ -155,30 +155,38 @@ __global__ __launch_bounds__(256) void hinv_copyin_rows_kernel(const float* __re
 }
 
 // Factor the 64x64 diagonal block at (k0,k0) and replace it by the inverse of its factor (chol_block.h).
-__global__ __launch_bounds__(256) void potf2_inv_kernel(float* __restrict__ A, int Kp, int k0, int K,
-                                                        HinvScalars* sc) {
+__global__ __launch_bounds__(cholblk::NT) void potf2_inv_kernel(float* __restrict__ A, int Kp, int k0, int K,
+                                                                HinvScalars* sc) {
   A += (int64_t)blockIdx.x * Kp * Kp;  // grouped call: one workgroup per problem (a single problem has one workgroup)
   sc += blockIdx.x;
-  __shared__ __attribute__((aligned(16))) float Xl[NB * cholblk::LDD];
-  __shared__ __attribute__((aligned(16))) cholblk::FactorScratch fs;
+  extern __shared__ __attribute__((aligned(16))) unsigned char potf2_smem[];
+  cholblk::FactorScratch& fs = *(cholblk::FactorScratch*)potf2_smem;
   const int tid = threadIdx.x, w = tid >> 6, r = tid & 63;
-  float a[16];
-  {
-    const float* src = A + (int64_t)(k0 + r) * Kp + k0 + 16 * w;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const float4 v = *(const float4*)(src + 4 * q);
-      a[4 * q] = v.x; a[4 * q + 1] = v.y; a[4 * q + 2] = v.z; a[4 * q + 3] = v.w;
-    }
+  {  // row r, columns 8w .. 8w+7 of the block into the column-major LDS copy
+    const float* src = A + (int64_t)(k0 + r) * Kp + k0 + 8 * w;
+    const float4 v0 = *(const float4*)src, v1 = *(const float4*)(src + 4);
+    fs.AT[8 * w + 0][r] = v0.x; fs.AT[8 * w + 1][r] = v0.y; fs.AT[8 * w + 2][r] = v0.z; fs.AT[8 * w + 3][r] = v0.w;
+    fs.AT[8 * w + 4][r] = v1.x; fs.AT[8 * w + 5][r] = v1.y; fs.AT[8 * w + 6][r] = v1.z; fs.AT[8 * w + 7][r] = v1.w;
   }
-  const int bad = cholblk::factor_invert_64(a, Xl, fs);
+  __syncthreads();
+  const int bad = cholblk::factor_invert_64(fs);
   // first failing pivot, 1-based index in the ORIGINAL (un-reversed) ordering
   if (tid == 0 && bad < NB && k0 + bad < K) atomicCAS(&sc->info, 0, K - (k0 + bad));
 #pragma unroll
-  for (int n = 0; n < 4; ++n) {
-    const int idx = tid + 256 * n, row = idx >> 4, c4 = (idx & 15) * 4;
-    *(float4*)(A + (int64_t)(k0 + row) * Kp + k0 + c4) = *(const float4*)(Xl + row * cholblk::LDD + c4);
+  for (int n = 0; n < 2; ++n) {
+    const int idx = tid + cholblk::NT * n, row = idx >> 4, c4 = (idx & 15) * 4;
+    *(float4*)(A + (int64_t)(k0 + row) * Kp + k0 + c4) = *(const float4*)&fs.X[row][c4];
   }
+}
+
+// the diagonal-block kernel keeps its working set in dynamic LDS (more than the 64 KiB a static array may take)
+inline int launch_potf2(float* A, int Kp, int k0, int K, HinvScalars* sc, int n, hipStream_t st) {
+  static const hipError_t configured = hipFuncSetAttribute(  // once per process (thread-safe static initialisation)
+      (const void*)potf2_inv_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(cholblk::FactorScratch));
+  if (configured != hipSuccess) return 1000 + (int)configured;
+  hipLaunchKernelGGL(potf2_inv_kernel, dim3(n), dim3(cholblk::NT), sizeof(cholblk::FactorScratch), st, A, Kp, k0, K, sc);
+  LLMC_LAUNCH_STATUS();
+  return 0;
 }
 
 // U[i][j] = X[K-1-i][K-1-j] for j >= i, 0 below; identity when the factorisation failed.  Four columns per
@@ -291,8 +299,10 @@ extern "C" int llmc_gptq_hinv(float* H, int64_t ldh, int64_t K, const int32_t* p
         const int rc = llmc_gemm_f32(u, st);
         if (rc) return rc;
       }
-      hipLaunchKernelGGL(potf2_inv_kernel, dim3(1), dim3(256), 0, st, A, Kp, c0, (int)K, sc);
-      LLMC_LAUNCH_STATUS();
+      {
+        const int prc = launch_potf2(A, Kp, c0, (int)K, sc, 1, st);
+        if (prc) return prc;
+      }
       const int M = Kp - c0 - NB;
       if (M <= 0) break;
       float* A21 = A + (int64_t)(c0 + NB) * Kp + c0;
@@ -433,8 +443,10 @@ extern "C" int llmc_gptq_hinv_grouped(const float* const* H, int64_t ldh, int32_
         const int rc = llmc_gemm_f32(u, st);
         if (rc) return rc;
       }
-      hipLaunchKernelGGL(potf2_inv_kernel, dim3(n), dim3(256), 0, st, A, Kp, c0, (int)K, sc);
-      LLMC_LAUNCH_STATUS();
+      {
+        const int prc = launch_potf2(A, Kp, c0, (int)K, sc, n, st);
+        if (prc) return prc;
+      }
       const int M = Kp - c0 - NB;
       if (M <= 0) break;
       float* A21 = A + (int64_t)(c0 + NB) * Kp + c0;
