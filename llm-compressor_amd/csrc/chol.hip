@@ -7,8 +7,9 @@
 //     U[i][j] = (L^-1)[K-1-i][K-1-j].
 // This file therefore (1) copies J (P^T H P / n + damp I) J into a work matrix
 // (P = optional activation-order permutation), (2) runs a blocked
-// lower Cholesky (64-wide panels: the diagonal block is factored and inverted in
-// LDS by one workgroup, panel solve and trailing update are MFMA GEMMs),
+// lower Cholesky (regions of 256 columns: 64-wide steps that factor and invert the
+// diagonal block and solve the region's rows in one launch, one more launch for the
+// rows below the region; the trailing update is a GEMM on the matrix cores),
 // (3) inverts L by recursive doubling with batched triangular GEMMs and
 // (4) writes the index-reversed result over H.  A non-positive pivot sets
 // *info and the output becomes the identity (the reference's round-to-nearest
@@ -154,39 +155,164 @@ __global__ __launch_bounds__(256) void hinv_copyin_rows_kernel(const float* __re
   }
 }
 
-// Factor the 64x64 diagonal block at (k0,k0) and replace it by the inverse of its factor (chol_block.h).
-__global__ __launch_bounds__(cholblk::NT) void potf2_inv_kernel(float* __restrict__ A, int Kp, int k0, int K,
-                                                                HinvScalars* sc) {
-  A += (int64_t)blockIdx.x * Kp * Kp;  // grouped call: one workgroup per problem (a single problem has one workgroup)
-  sc += blockIdx.x;
-  extern __shared__ __attribute__((aligned(16))) unsigned char potf2_smem[];
-  cholblk::FactorScratch& fs = *(cholblk::FactorScratch*)potf2_smem;
+// ---- a 256-wide region of the factorisation in two kinds of launches -------------------------------------------
+// The serial spine of the blocked factorisation is one 64 x 64 diagonal block after the other.  Inside a region
+// of up to four such blocks, step m is ONE launch (chol_region_step_kernel): every workgroup factors and inverts
+// the diagonal block m itself (the same arithmetic in each, so nothing has to cross workgroups), and workgroup
+// b > 0 then solves its own 64 rows of block column m against it, after bringing them up to date with the
+// region's earlier steps, and takes the new columns' contribution off its own diagonal block -- so that block
+// is complete when its turn comes.  The rows below the region are not on the spine: they are solved against
+// the whole region afterwards, one launch (chol_region_rows_kernel), 64 rows per workgroup, the block row kept
+// in LDS from one block column to the next.
+//
+// The inverses of the diagonal blocks' factors go to a side array Xs (block c0 / 64 at Xs + (c0 / 64) * 4096, dense
+// 64 x 64) and not over the diagonal block itself: within one launch every workgroup reads that block, whenever it
+// happens to start, so nothing may overwrite it before the launch has ended.  chol_scatter_diag_kernel moves them
+// into the diagonal blocks once the factorisation is complete (where the inversion expects them).
+struct RegionStepLds {
+  cholblk::FactorScratch fs;
+  float Abuf[NB][cholblk::LDD];
+  float Bbuf[NB][cholblk::LDD];
+};
+
+__global__ __launch_bounds__(cholblk::NT) void chol_region_step_kernel(float* __restrict__ A, int Kp, int r0, int m,
+                                                                       int K, HinvScalars* sc, float* __restrict__ Xs,
+                                                                       int64_t xs_stride) {
+  using namespace cholblk;
+  A += (int64_t)blockIdx.y * Kp * Kp;  // grouped call: blockIdx.y = problem
+  Xs += (int64_t)blockIdx.y * xs_stride;
+  sc += blockIdx.y;
+  extern __shared__ __attribute__((aligned(16))) unsigned char region_smem[];
+  RegionStepLds& L = *(RegionStepLds*)region_smem;
   const int tid = threadIdx.x, w = tid >> 6, r = tid & 63;
-  {  // row r, columns 8w .. 8w+7 of the block into the column-major LDS copy
-    const float* src = A + (int64_t)(k0 + r) * Kp + k0 + 8 * w;
-    const float4 v0 = *(const float4*)src, v1 = *(const float4*)(src + 4);
-    fs.AT[8 * w + 0][r] = v0.x; fs.AT[8 * w + 1][r] = v0.y; fs.AT[8 * w + 2][r] = v0.z; fs.AT[8 * w + 3][r] = v0.w;
-    fs.AT[8 * w + 4][r] = v1.x; fs.AT[8 * w + 5][r] = v1.y; fs.AT[8 * w + 6][r] = v1.z; fs.AT[8 * w + 7][r] = v1.w;
+  const int b = blockIdx.x;                // 0: owner of the diagonal block; b > 0: row block m + b of the region
+  const int c0 = r0 + NB * m;              // the step's block column
+  const int64_t rows = c0 + (int64_t)NB * b;
+  // the diagonal block's loads are issued first: their latency hides behind the products below
+  const float* dsrc = A + (int64_t)(c0 + r) * Kp + c0 + 8 * w;
+  const float4 d0 = *(const float4*)dsrc, d1 = *(const float4*)(dsrc + 4);
+  Acc64 acc, dg;
+  if (b > 0) {
+    // own rows of block column m, brought up to date with the region's earlier steps:
+    // acc = A[rows, c0..] - sum_{i<m} A[rows, cols_i] A[c0 rows, cols_i]^T
+    acc_load(acc, A + rows * Kp + c0, Kp, w, r);
+    acc_load(dg, A + rows * Kp + rows, Kp, w, r);  // this row block's own diagonal block, needed at the very end
+    for (int i = 0; i < m; ++i) {
+      BlockFetch fa, fb;
+      fa.fetch(A + rows * Kp + r0 + NB * i, Kp, tid);
+      fb.fetch(A + (int64_t)c0 * Kp + r0 + NB * i, Kp, tid);
+      if (i > 0) __syncthreads();  // the previous product has read the buffers
+      fa.put(L.Abuf, tid);
+      fb.put(L.Bbuf, tid);
+      __syncthreads();
+      mm64_nt<true>(acc, L.Abuf, L.Bbuf, w, r);
+    }
   }
+  L.fs.AT[8 * w + 0][r] = d0.x; L.fs.AT[8 * w + 1][r] = d0.y; L.fs.AT[8 * w + 2][r] = d0.z; L.fs.AT[8 * w + 3][r] = d0.w;
+  L.fs.AT[8 * w + 4][r] = d1.x; L.fs.AT[8 * w + 5][r] = d1.y; L.fs.AT[8 * w + 6][r] = d1.z; L.fs.AT[8 * w + 7][r] = d1.w;
   __syncthreads();
-  const int bad = cholblk::factor_invert_64(fs);
-  // first failing pivot, 1-based index in the ORIGINAL (un-reversed) ordering
-  if (tid == 0 && bad < NB && k0 + bad < K) atomicCAS(&sc->info, 0, K - (k0 + bad));
+  const int bad = factor_invert_64(L.fs);
+  if (b == 0) {
+    // first failing pivot, 1-based index in the ORIGINAL (un-reversed) ordering
+    if (tid == 0 && bad < NB && c0 + bad < K) atomicCAS(&sc->info, 0, K - (c0 + bad));
 #pragma unroll
-  for (int n = 0; n < 2; ++n) {
-    const int idx = tid + cholblk::NT * n, row = idx >> 4, c4 = (idx & 15) * 4;
-    *(float4*)(A + (int64_t)(k0 + row) * Kp + k0 + c4) = *(const float4*)&fs.X[row][c4];
+    for (int n = 0; n < 2; ++n) {
+      const int idx = tid + NT * n, row = idx >> 4, c4 = (idx & 15) * 4;
+      *(float4*)(Xs + (int64_t)(c0 / NB) * NB * NB + row * NB + c4) = *(const float4*)&L.fs.X[row][c4];
+    }
+    return;
+  }
+  // solve: R = acc * inv(L_mm)^T  (the barriers inside the factorisation separate this from the last product)
+  acc_store(acc, &L.Abuf[0][0], LDD, w, r);
+  __syncthreads();
+  Acc64 sol = {};
+  mm64_nt<false>(sol, L.Abuf, L.fs.X, w, r);
+  acc_store(sol, A + rows * Kp + c0, Kp, w, r);
+  __syncthreads();  // every wave has read Abuf
+  acc_store(sol, &L.Abuf[0][0], LDD, w, r);
+  // the new columns' contribution to this row block's own diagonal block: D_b -= R R^T
+  __syncthreads();
+  mm64_nt<true>(dg, L.Abuf, L.Abuf, w, r);
+  acc_store(dg, A + rows * Kp + rows, Kp, w, r);
+}
+
+struct RegionRowsLds {
+  float R[4][NB][cholblk::LDD];  // the workgroup's solved blocks of the region's block columns
+  float Abuf[NB][cholblk::LDD];
+  float Bbuf[NB][cholblk::LDD];
+};
+
+// rows row_start + 64 * blockIdx.x .. of the nb block columns of the region at r0, whose diagonal region is done
+__global__ __launch_bounds__(cholblk::NT) void chol_region_rows_kernel(float* __restrict__ A, int Kp, int r0, int nb,
+                                                                       int row_start, const float* __restrict__ Xs,
+                                                                       int64_t xs_stride) {
+  using namespace cholblk;
+  A += (int64_t)blockIdx.y * Kp * Kp;
+  Xs += (int64_t)blockIdx.y * xs_stride;
+  extern __shared__ __attribute__((aligned(16))) unsigned char rows_smem[];
+  RegionRowsLds& L = *(RegionRowsLds*)rows_smem;
+  const int tid = threadIdx.x, w = tid >> 6, r = tid & 63;
+  const int64_t rows = row_start + (int64_t)NB * blockIdx.x;
+  // schedule: for block column j the factor blocks (j, 0) .. (j, j-1) at A[r0 + 64 j rows, r0 + 64 i columns], then
+  // the inverse of the diagonal block's factor from the side array.  One block ahead is in flight while the current
+  // product runs.
+  const float* xs0 = Xs + (int64_t)(r0 / NB) * NB * NB;
+  BlockFetch next;
+  next.fetch(xs0, NB, tid);
+  Acc64 own[4];  // the workgroup's rows of the region's block columns: all loads in flight from the start
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    if (j < nb) acc_load(own[j], A + rows * Kp + r0 + NB * j, Kp, w, r);
+  bool first = true;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    if (j >= nb) break;
+    Acc64 acc = own[j];
+    for (int i = 0; i <= j; ++i) {
+      if (!first) __syncthreads();  // the previous product has read Bbuf (and Abuf)
+      first = false;
+      next.put(L.Bbuf, tid);
+      {  // the block after this one
+        int nj = j, ni = i + 1;
+        if (ni > nj) { nj = j + 1; ni = 0; }
+        if (nj < nb) {
+          if (ni == nj)
+            next.fetch(xs0 + (int64_t)nj * NB * NB, NB, tid);
+          else
+            next.fetch(A + (int64_t)(r0 + NB * nj) * Kp + r0 + NB * ni, Kp, tid);
+        }
+      }
+      if (i == j) acc_store(acc, &L.Abuf[0][0], LDD, w, r);
+      __syncthreads();
+      if (i < j) {
+        mm64_nt<true>(acc, L.R[i], L.Bbuf, w, r);
+      } else {
+        Acc64 sol = {};
+        mm64_nt<false>(sol, L.Abuf, L.Bbuf, w, r);
+        acc_store(sol, A + rows * Kp + r0 + NB * j, Kp, w, r);
+        acc_store(sol, &L.R[j][0][0], LDD, w, r);  // read by later products, after the barriers in between
+      }
+    }
   }
 }
 
-// the diagonal-block kernel keeps its working set in dynamic LDS (more than the 64 KiB a static array may take)
-inline int launch_potf2(float* A, int Kp, int k0, int K, HinvScalars* sc, int n, hipStream_t st) {
-  static const hipError_t configured = hipFuncSetAttribute(  // once per process (thread-safe static initialisation)
-      (const void*)potf2_inv_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(cholblk::FactorScratch));
-  if (configured != hipSuccess) return 1000 + (int)configured;
-  hipLaunchKernelGGL(potf2_inv_kernel, dim3(n), dim3(cholblk::NT), sizeof(cholblk::FactorScratch), st, A, Kp, k0, K, sc);
-  LLMC_LAUNCH_STATUS();
-  return 0;
+// diagonal block c of the work matrix <- Xs block c (after the factorisation, before the inversion)
+__global__ __launch_bounds__(256) void chol_scatter_diag_kernel(float* __restrict__ A, int Kp, const float* __restrict__ Xs,
+                                                                int64_t xs_stride) {
+  A += (int64_t)blockIdx.y * Kp * Kp;
+  Xs += (int64_t)blockIdx.y * xs_stride + (int64_t)blockIdx.x * NB * NB;
+  const int c0 = blockIdx.x * NB;
+#pragma unroll
+  for (int n = 0; n < 4; ++n) {
+    const int idx = threadIdx.x + 256 * n, row = idx >> 4, c4 = (idx & 15) * 4;
+    *(float4*)(A + (int64_t)(c0 + row) * Kp + c0 + c4) = *(const float4*)(Xs + row * NB + c4);
+  }
+}
+
+template <typename KernelT>
+inline int set_dynamic_lds(KernelT kernel, size_t bytes) {
+  const hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  return e == hipSuccess ? 0 : 1000 + (int)e;
 }
 
 // U[i][j] = X[K-1-i][K-1-j] for j >= i, 0 below; identity when the factorisation failed.  Four columns per
@@ -238,12 +364,76 @@ __global__ __launch_bounds__(256) void hinv_copyout_kernel(const float* __restri
 
 inline int64_t round_up(int64_t a, int64_t b) { return (a + b - 1) / b * b; }
 
+// floats of the temporary behind a work matrix: the inversion's first products (Kp^2 / 4) and, before that, the
+// side array of the diagonal blocks' inverses (64 Kp)
+inline int64_t hinv_temp_floats(int64_t Kp) { return Kp * Kp / 4 > NB * Kp ? Kp * Kp / 4 : NB * Kp; }
+
+// Blocked lower Cholesky of n work matrices (one every Kp^2 floats) in lock-step; Xs (one every xs_stride floats) takes
+// the inverses of the diagonal blocks' factors and is moved into the diagonal blocks at the end.
+//
+// Two levels.  An outer panel (512 wide once the trailing matrix is big enough to pay for it, else 256) ends with one
+// rank-256/512 update of the trailing matrix, which cuts that matrix's read-modify-write traffic 4-8x compared with
+// rank-64 updates.  Inside it, regions of 256 columns: four single-launch steps on the diagonal region, one launch for
+// the rows below it (see chol_region_step_kernel); the second region of a 512-wide panel first takes the first
+// region's update as one product.
+inline int chol_factor(float* A, int Kp, int K, HinvScalars* sc, float* Xs, int64_t xs_stride, int n, hipStream_t st) {
+  static const int cfg_step = set_dynamic_lds(chol_region_step_kernel, sizeof(RegionStepLds));
+  static const int cfg_rows = set_dynamic_lds(chol_region_rows_kernel, sizeof(RegionRowsLds));
+  if (cfg_step) return cfg_step;
+  if (cfg_rows) return cfg_rows;
+  const int64_t mat = (int64_t)Kp * Kp;
+  const int NBO = Kp >= 8192 ? 512 : 256;
+  constexpr int RW = 256;
+  for (int k0 = 0; k0 < Kp; k0 += NBO) {
+    const int pw = (Kp - k0) < NBO ? (Kp - k0) : NBO;
+    for (int r0 = k0; r0 < k0 + pw; r0 += RW) {
+      const int rw = (k0 + pw - r0) < RW ? (k0 + pw - r0) : RW;
+      const int nb = rw / NB;
+      if (r0 > k0) {
+        // columns r0 .. r0+rw of the rows from r0 down take the panel's first region in one product,
+        // C[M, rw] -= L[rows, k0:r0] L[r0:r0+rw, k0:r0]^T, lower part only (C starts on the matrix diagonal)
+        float* Lp = A + (int64_t)r0 * Kp + k0;
+        GemmF32 u = {};
+        u.A = Lp; u.lda = Kp; u.B = Lp; u.ldb = Kp; u.C = A + (int64_t)r0 * Kp + r0; u.ldc = Kp;
+        u.M = Kp - r0; u.N = rw; u.Kc = r0 - k0; u.alpha = -1.f; u.beta = 1.f; u.trans_b = 1; u.c_lower = 1;
+        u.batch = 1; u.batch2 = n; u.stride2_a = mat; u.stride2_b = mat; u.stride2_c = mat;
+        const int rc = llmc_gemm_f32(u, st);
+        if (rc) return rc;
+      }
+      for (int m = 0; m < nb; ++m) {
+        hipLaunchKernelGGL(chol_region_step_kernel, dim3(nb - m, n), dim3(cholblk::NT), sizeof(RegionStepLds), st, A, Kp,
+                           r0, m, K, sc, Xs, xs_stride);
+        LLMC_LAUNCH_STATUS();
+      }
+      const int below = (Kp - (r0 + rw)) / NB;
+      if (below > 0) {
+        hipLaunchKernelGGL(chol_region_rows_kernel, dim3(below, n), dim3(cholblk::NT), sizeof(RegionRowsLds), st, A, Kp,
+                           r0, nb, r0 + rw, (const float*)Xs, xs_stride);
+        LLMC_LAUNCH_STATUS();
+      }
+    }
+    const int M2 = Kp - (k0 + pw);
+    if (M2 > 0) {
+      float* P = A + (int64_t)(k0 + pw) * Kp + k0;
+      GemmF32 t = {};
+      t.A = P; t.lda = Kp; t.B = P; t.ldb = Kp; t.C = A + (int64_t)(k0 + pw) * ((int64_t)Kp + 1); t.ldc = Kp;
+      t.M = M2; t.N = M2; t.Kc = pw; t.alpha = -1.f; t.beta = 1.f; t.trans_b = 1; t.c_lower = 1;
+      t.batch = 1; t.batch2 = n; t.stride2_a = mat; t.stride2_b = mat; t.stride2_c = mat;
+      const int rc = llmc_gemm_f32(t, st);
+      if (rc) return rc;
+    }
+  }
+  hipLaunchKernelGGL(chol_scatter_diag_kernel, dim3(Kp / NB, n), dim3(256), 0, st, A, Kp, (const float*)Xs, xs_stride);
+  LLMC_LAUNCH_STATUS();
+  return 0;
+}
+
 }  // namespace
 
 extern "C" int64_t llmc_gptq_hinv_workspace_bytes(int64_t K) {
   const int64_t Kp = round_up(K, NB);
-  // work matrix + recursive-doubling temporary (at most Kp^2/4) + scalars
-  return (Kp * Kp + Kp * Kp / 4 + 64) * 4 + 256;
+  // work matrix + temporary (recursive doubling, side array of the diagonal inverses) + scalars
+  return (Kp * Kp + hinv_temp_floats(Kp) + 64) * 4 + 256;
 }
 
 extern "C" int llmc_gptq_hinv(float* H, int64_t ldh, int64_t K, const int32_t* perm, float divisor,
@@ -278,50 +468,9 @@ extern "C" int llmc_gptq_hinv(float* H, int64_t ldh, int64_t K, const int32_t* p
   }
   LLMC_LAUNCH_STATUS();
 
-  // Blocked Cholesky, two levels.  Inside a 256- or 512-wide outer panel the 64-wide steps run left-looking:
-  // a step first brings its own 64 columns up to date with the panel's earlier steps (one product), then the
-  // diagonal block is factored + inverted in LDS and the panel below it solved as a GEMM.  The trailing matrix
-  // gets one rank-256/512 update per outer panel (right-looking between panels), which cuts its
-  // read-modify-write traffic 4-8x compared with rank-64 updates.  Diagonal blocks end up holding inv(L_kk).
-  const int NBO = Kp >= 8192 ? 512 : 256;  // wider outer panels once the trailing matrix is big enough to pay for them
-  for (int k0 = 0; k0 < Kp; k0 += NBO) {
-    const int pw = (Kp - k0) < NBO ? (Kp - k0) : NBO;
-    for (int kk = 0; kk < pw; kk += NB) {
-      const int c0 = k0 + kk;
-      if (kk > 0) {
-        // left-looking inside the panel: columns c0 .. c0+63 of the rows from c0 down take the updates of the
-        // panel's earlier steps in one product, C[M+64, 64] -= L[rows, k0:c0] * L[c0:c0+64, k0:c0]^T.  (Updating
-        // all remaining columns of the panel after every step moves twice the bytes for the same sums.)
-        float* Lp = A + (int64_t)c0 * Kp + k0;
-        GemmF32 u = {};
-        u.A = Lp; u.lda = Kp; u.B = Lp; u.ldb = Kp; u.C = A + (int64_t)c0 * Kp + c0; u.ldc = Kp;
-        u.M = Kp - c0; u.N = NB; u.Kc = kk; u.alpha = -1.f; u.beta = 1.f; u.trans_b = 1; u.batch = 1;
-        const int rc = llmc_gemm_f32(u, st);
-        if (rc) return rc;
-      }
-      {
-        const int prc = launch_potf2(A, Kp, c0, (int)K, sc, 1, st);
-        if (prc) return prc;
-      }
-      const int M = Kp - c0 - NB;
-      if (M <= 0) break;
-      float* A21 = A + (int64_t)(c0 + NB) * Kp + c0;
-      GemmF32 g = {};
-      // panel: A21 <- A21 * inv(L_kk)^T   (in place: one tile column, each workgroup owns its rows)
-      g.A = A21; g.lda = Kp; g.B = A + (int64_t)c0 * Kp + c0; g.ldb = Kp; g.C = A21; g.ldc = Kp;
-      g.M = M; g.N = NB; g.Kc = NB; g.alpha = 1.f; g.beta = 0.f; g.trans_b = 1; g.batch = 1;
-      const int rc = llmc_gemm_f32(g, st);
-      if (rc) return rc;
-    }
-    const int M2 = Kp - (k0 + pw);
-    if (M2 > 0) {
-      float* P = A + (int64_t)(k0 + pw) * Kp + k0;
-      GemmF32 t = {};
-      t.A = P; t.lda = Kp; t.B = P; t.ldb = Kp; t.C = A + (int64_t)(k0 + pw) * ((int64_t)Kp + 1); t.ldc = Kp;
-      t.M = M2; t.N = M2; t.Kc = pw; t.alpha = -1.f; t.beta = 1.f; t.trans_b = 1; t.c_lower = 1; t.batch = 1;
-      const int rc = llmc_gemm_f32(t, st);
-      if (rc) return rc;
-    }
+  {
+    const int frc = chol_factor(A, Kp, (int)K, sc, T, 0, 1, st);
+    if (frc) return frc;
   }
 
   // inverse by recursive doubling: [[X11,0],[X21,X22]] with X21 = -X22 * L21 * X11
@@ -370,7 +519,7 @@ extern "C" int llmc_gptq_hinv(float* H, int64_t ldh, int64_t K, const int32_t* p
 extern "C" int64_t llmc_gptq_hinv_grouped_workspace_bytes(int64_t n, int64_t K) {
   const int64_t Kp = round_up(K, NB);
   return round_up(n * (int64_t)sizeof(HinvItem), 256) + round_up(n * (int64_t)sizeof(HinvScalars), 256) +
-         n * (Kp * Kp + Kp * Kp / 4) * 4 + 256;
+         n * (Kp * Kp + hinv_temp_floats(Kp)) * 4 + 256;
 }
 
 extern "C" int llmc_gptq_hinv_grouped(const float* const* H, int64_t ldh, int32_t n, int64_t K,
@@ -395,6 +544,7 @@ extern "C" int llmc_gptq_hinv_grouped(const float* const* H, int64_t ldh, int32_
   HinvScalars* sc = (HinvScalars*)wp; wp += round_up(n * (int64_t)sizeof(HinvScalars), 256);
   float* A = (float*)wp;
   float* T = A + (int64_t)n * mat;
+  const int64_t tstride = hinv_temp_floats(Kp);
   std::vector<HinvItem> host(n);
   for (int b = 0; b < n; ++b) {
     LLMC_CHECK_ARG(H[b] != nullptr && divisors[b] != 0.f, 1);
@@ -429,44 +579,9 @@ extern "C" int llmc_gptq_hinv_grouped(const float* const* H, int64_t ldh, int32_
   }
   LLMC_LAUNCH_STATUS();
 
-  const int NBO = Kp >= 8192 ? 512 : 256;
-  for (int k0 = 0; k0 < Kp; k0 += NBO) {
-    const int pw = (Kp - k0) < NBO ? (Kp - k0) : NBO;
-    for (int kk = 0; kk < pw; kk += NB) {
-      const int c0 = k0 + kk;
-      if (kk > 0) {  // left-looking inside the panel, as in the single-problem chain
-        float* Lp = A + (int64_t)c0 * Kp + k0;
-        GemmF32 u = {};
-        u.A = Lp; u.lda = Kp; u.B = Lp; u.ldb = Kp; u.C = A + (int64_t)c0 * Kp + c0; u.ldc = Kp;
-        u.M = Kp - c0; u.N = NB; u.Kc = kk; u.alpha = -1.f; u.beta = 1.f; u.trans_b = 1;
-        u.batch = 1; u.batch2 = n; u.stride2_a = mat; u.stride2_b = mat; u.stride2_c = mat;
-        const int rc = llmc_gemm_f32(u, st);
-        if (rc) return rc;
-      }
-      {
-        const int prc = launch_potf2(A, Kp, c0, (int)K, sc, n, st);
-        if (prc) return prc;
-      }
-      const int M = Kp - c0 - NB;
-      if (M <= 0) break;
-      float* A21 = A + (int64_t)(c0 + NB) * Kp + c0;
-      GemmF32 g = {};
-      g.A = A21; g.lda = Kp; g.B = A + (int64_t)c0 * Kp + c0; g.ldb = Kp; g.C = A21; g.ldc = Kp;
-      g.M = M; g.N = NB; g.Kc = NB; g.alpha = 1.f; g.beta = 0.f; g.trans_b = 1;
-      g.batch = 1; g.batch2 = n; g.stride2_a = mat; g.stride2_b = mat; g.stride2_c = mat;
-      const int rc = llmc_gemm_f32(g, st);
-      if (rc) return rc;
-    }
-    const int M2 = Kp - (k0 + pw);
-    if (M2 > 0) {
-      float* P = A + (int64_t)(k0 + pw) * Kp + k0;
-      GemmF32 t = {};
-      t.A = P; t.lda = Kp; t.B = P; t.ldb = Kp; t.C = A + (int64_t)(k0 + pw) * ((int64_t)Kp + 1); t.ldc = Kp;
-      t.M = M2; t.N = M2; t.Kc = pw; t.alpha = -1.f; t.beta = 1.f; t.trans_b = 1; t.c_lower = 1;
-      t.batch = 1; t.batch2 = n; t.stride2_a = mat; t.stride2_b = mat; t.stride2_c = mat;
-      const int rc = llmc_gemm_f32(t, st);
-      if (rc) return rc;
-    }
+  {
+    const int frc = chol_factor(A, Kp, (int)K, sc, T, tstride, n, st);
+    if (frc) return frc;
   }
 
   for (int64_t s = NB; s < Kp; s *= 2) {
@@ -488,14 +603,14 @@ extern "C" int llmc_gptq_hinv_grouped(const float* const* H, int64_t ldh, int32_
       g.A = L21; g.lda = Kp; g.B = X11; g.ldb = Kp; g.C = T; g.ldc = s;
       g.M = (int)s2; g.N = (int)s; g.Kc = (int)s; g.alpha = 1.f; g.beta = 0.f; g.b_lower_tri = 1;
       g.batch = (int)batch; g.stride_a = step; g.stride_b = step; g.stride_c = s * s;
-      g.batch2 = n; g.stride2_a = mat; g.stride2_b = mat; g.stride2_c = mat / 4;
+      g.batch2 = n; g.stride2_a = mat; g.stride2_b = mat; g.stride2_c = tstride;
       int rc = llmc_gemm_f32(g, st);
       if (rc) return rc;
       GemmF32 h = {};
       h.A = X22; h.lda = Kp; h.B = T; h.ldb = s; h.C = L21; h.ldc = Kp;
       h.M = (int)s2; h.N = (int)s; h.Kc = (int)s2; h.alpha = -1.f; h.beta = 0.f; h.a_lower_tri = 1;
       h.batch = (int)batch; h.stride_a = step; h.stride_b = s * s; h.stride_c = step;
-      h.batch2 = n; h.stride2_a = mat; h.stride2_b = mat / 4; h.stride2_c = mat;
+      h.batch2 = n; h.stride2_a = mat; h.stride2_b = tstride; h.stride2_c = mat;
       rc = llmc_gemm_f32(h, st);
       if (rc) return rc;
     }

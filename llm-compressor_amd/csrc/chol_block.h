@@ -248,3 +248,76 @@ __device__ __forceinline__ int factor_invert_64(FactorScratch& s) {
 }
 
 }  // namespace cholblk
+
+// ---- 64 x 64 products on the matrix cores, for the kernels that keep a block row of the factorisation in one
+// workgroup.  A 64 x 64 result is 16 tiles of 16 x 16; wave w of the eight owns the tiles (w / 2, 2 * (w % 2) + e),
+// e = 0, 1.  Tile layout of v_mfma_f32_16x16x4_f32: lane l holds column l % 16, rows 4 * (l / 16) + v.
+namespace cholblk {
+
+struct Acc64 {
+  v4f t[2];
+};
+
+// acc (+/-)= A * B^T with A and B row-major 64 x 64 blocks in LDS (row stride LDD).  The k index a lane group
+// feeds into a matrix instruction is free as long as both operands agree, so lane group g takes k = 16 g .. 16 g + 15
+// and reads its 16 values as four 16-byte loads.
+template <bool NEG>
+__device__ __forceinline__ void mm64_nt(Acc64& acc, const float (*A)[LDD], const float (*B)[LDD], int w, int lane) {
+  const int i = lane & 15, g = lane >> 4, ti = w >> 1;
+  float a[16];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const float4 x = *(const float4*)&A[16 * ti + i][16 * g + 4 * q];
+    a[4 * q] = NEG ? -x.x : x.x; a[4 * q + 1] = NEG ? -x.y : x.y; a[4 * q + 2] = NEG ? -x.z : x.z; a[4 * q + 3] = NEG ? -x.w : x.w;
+  }
+#pragma unroll
+  for (int e = 0; e < 2; ++e) {
+    const int tj = 2 * (w & 1) + e;
+    float b[16];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float4 x = *(const float4*)&B[16 * tj + i][16 * g + 4 * q];
+      b[4 * q] = x.x; b[4 * q + 1] = x.y; b[4 * q + 2] = x.z; b[4 * q + 3] = x.w;
+    }
+#pragma unroll
+    for (int kk = 0; kk < 16; ++kk) acc.t[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[kk], b[kk], acc.t[e], 0, 0, 0);
+  }
+}
+
+// the wave's two tiles of a 64 x 64 block at `p` (row stride ld, global or LDS)
+__device__ __forceinline__ void acc_load(Acc64& acc, const float* p, int64_t ld, int w, int lane) {
+  const int i = lane & 15, g = lane >> 4, ti = w >> 1;
+#pragma unroll
+  for (int e = 0; e < 2; ++e)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) acc.t[e][v] = p[(int64_t)(16 * ti + 4 * g + v) * ld + 16 * (2 * (w & 1) + e) + i];
+}
+__device__ __forceinline__ void acc_store(const Acc64& acc, float* p, int64_t ld, int w, int lane) {
+  const int i = lane & 15, g = lane >> 4, ti = w >> 1;
+#pragma unroll
+  for (int e = 0; e < 2; ++e)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) p[(int64_t)(16 * ti + 4 * g + v) * ld + 16 * (2 * (w & 1) + e) + i] = acc.t[e][v];
+}
+
+// a 64 x 64 block of a row-major global matrix through registers into a row-major LDS block: fetch() issues the
+// loads (two 16-byte loads per thread), put() stores them, so that a product can run in between
+struct BlockFetch {
+  float4 v[2];
+  __device__ __forceinline__ void fetch(const float* src, int64_t ld, int tid) {
+#pragma unroll
+    for (int n = 0; n < 2; ++n) {
+      const int idx = tid + NT * n;
+      v[n] = *(const float4*)(src + (int64_t)(idx >> 4) * ld + (idx & 15) * 4);
+    }
+  }
+  __device__ __forceinline__ void put(float (*dst)[LDD], int tid) const {
+#pragma unroll
+    for (int n = 0; n < 2; ++n) {
+      const int idx = tid + NT * n;
+      *(float4*)&dst[idx >> 4][(idx & 15) * 4] = v[n];
+    }
+  }
+};
+
+}  // namespace cholblk
