@@ -313,7 +313,11 @@ int llmc_gptq_quantize_grouped(const void* const* weight, int32_t w_dtype, int32
  * all row-major fp32.  Products whose shape is a whole number of 128- or 256-wide tiles run on the 16-bit
  * matrix cores with every operand split into three bf16 terms (six partial products, the dropped ones below
  * the rounding of an fp32 product); other shapes, and every shape with LLMC_SGEMM_FP32_MFMA, use the fp32
- * matrix instruction.  Structure flags are tile-granular promises about exact zeros in the operands. */
+ * matrix instruction.  Structure flags are tile-granular promises about exact zeros in the operands.
+ * Non-finite operands: the split form turns an infinite operand, or a finite one whose magnitude rounds to infinity
+ * in bf16 (above 3.39e38), into NaN (the remainder of the split is inf - inf), where the fp32 instruction gives an
+ * infinity; results for finite operands below that bound are as accurate as stated above.  Pass
+ * LLMC_SGEMM_FP32_MFMA when infinities must propagate as such. */
 enum {
   LLMC_SGEMM_C_LOWER = 1,      /* only tiles touching the lower triangle of C are computed and written     */
   LLMC_SGEMM_A_LOWER_TRI = 2,  /* A[m,k] == 0 for k > m                                                    */

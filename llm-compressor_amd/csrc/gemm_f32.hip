@@ -219,7 +219,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32 g, int vec) {
   if (ALL_FAST) {
     gemm_tile<BM, BN, TRANS_B, true, TRANS_A>(g, A, B, C, m0, n0, k_begin, k_end, As, Bs);
   } else {
-    const bool fast = vec && m0 + BM <= g.M && n0 + BN <= g.N && ((k_end - k_begin) % BK) == 0;
+    const bool fast = vec && m0 + BM <= g.M && n0 + BN <= g.N && ((k_end - k_begin) % BK) == 0 && g.ldc < (1 << 22);
     if (fast)
       gemm_tile<BM, BN, TRANS_B, true, TRANS_A>(g, A, B, C, m0, n0, k_begin, k_end, As, Bs);
     else
@@ -274,7 +274,9 @@ static int gemm_f32_mfma(const GemmF32& g, hipStream_t st) {
   const int bt = big ? 128 : 64;
   // every tile unconditional?  (a_lower_tri / b_lower_tri cut the contraction at tile edges, which
   // are multiples of BK for both tile sizes)
-  const bool all_fast = vec && g.M % bt == 0 && g.N % bt == 0 && g.Kc % BK == 0;
+  // (and the unconditional epilogue addresses a wave's strip of C with 32-bit byte offsets, up to 132 rows of ldc
+  // floats from the strip's origin: rows of 4M floats and more take the per-element path with 64-bit addresses)
+  const bool all_fast = vec && g.M % bt == 0 && g.N % bt == 0 && g.Kc % BK == 0 && g.ldc < (1 << 22);
   dim3 grid((g.N + bt - 1) / bt, (g.M + bt - 1) / bt, g.batch * nb2);
 #define LLMC_GEMM(BT, TB, AF) hipLaunchKernelGGL((gemm_f32_kernel<BT, BT, TB, AF>), grid, dim3(256), 0, st, g, vec)
   if (g.trans_a) {

@@ -346,7 +346,9 @@ int llmc_gemm_x3(const GemmF32& g, hipStream_t st) {
                        (g.stride_a & 3) == 0 && (g.stride_b & 3) == 0 &&
                        (nb2 == 1 || ((g.stride2_a & 3) == 0 && (g.stride2_b & 3) == 0));
   if (!aligned || g.Kc % XK || g.Kc < 64) return -1;
-  if (g.ldc > (1 << 28)) return -1;
+  // the epilogue addresses a wave's strip of C with 32-bit byte offsets (up to 68 rows of ldc floats from the
+  // strip's origin): wider rows than this go to the fp32 kernel's 64-bit path
+  if (g.ldc >= (1 << 22)) return -1;
   // Whether a product is split depends on its own shape only, never on how many independent problems
   // (batch2) share the launch, so that a grouped call gives the bits of its single calls.  Both tile shapes
   // add the partial products of an element in the same order, so the choice between them is free.

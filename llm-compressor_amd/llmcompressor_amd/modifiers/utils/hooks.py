@@ -2,6 +2,7 @@
 from __future__ import annotations
 
 import contextlib
+import weakref
 from functools import wraps
 from typing import Any, Callable, ClassVar
 
@@ -15,7 +16,9 @@ __all__ = ["HooksMixin"]
 class HooksMixin(BaseModel):
     _HOOKS_DISABLED: ClassVar[bool] = False
     _HOOKS_KEEP_ENABLED: ClassVar[set] = set()
-    _ALL_HANDLES: ClassVar[set] = set()  # every live handle of every modifier (for `keep` by module)
+    # every handle a modifier still refers to (for `keep` by module); weak, so that a handle removed directly with
+    # handle.remove() and dropped by its modifier does not stay alive here
+    _ALL_HANDLES: ClassVar[weakref.WeakSet] = weakref.WeakSet()
 
     _hooks: set = PrivateAttr(default_factory=set)
 
@@ -53,5 +56,6 @@ class HooksMixin(BaseModel):
             handles = self._hooks
         for h in list(handles):
             h.remove()
-        HooksMixin._ALL_HANDLES.difference_update(handles)
+        for h in list(handles):
+            HooksMixin._ALL_HANDLES.discard(h)
         self._hooks -= set(handles)

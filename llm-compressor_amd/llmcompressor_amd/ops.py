@@ -2,6 +2,9 @@
 from torch tensors and call the C ABI.  torch is only memory and streams here."""
 from __future__ import annotations
 
+import threading
+import weakref
+
 import torch
 
 from . import _lib
@@ -150,7 +153,14 @@ SCALE_PLAIN, SCALE_NVFP4, SCALE_MXFP4 = 0, 1, 2
 OUT_FAKEQUANT, OUT_CODES, OUT_PACKED = 0, 1, 2
 _TD = {BF16: torch.bfloat16, F16: torch.float16, F32: torch.float32}
 
-_ws_cache = {}
+class _WorkspaceStore(dict):
+    """The scratch buffers of one host thread, keyed by (device, stream)."""
+
+    __slots__ = ("__weakref__",)
+
+
+_ws_local = threading.local()  # a thread's store goes away with the thread, and its buffers with it
+_ws_stores = weakref.WeakSet()  # the stores of the threads still alive, for release_workspaces()
 
 
 def _workspace(device, nbytes: int) -> torch.Tensor:
@@ -158,15 +168,26 @@ def _workspace(device, nbytes: int) -> torch.Tensor:
 
     Several entry points issue more than one launch over their workspace, and ctypes releases the GIL during
     a call, so two host threads on one stream could interleave their launches: each thread therefore owns its
-    buffer (work of one thread on one stream is ordered by the stream)."""
-    import threading
-
-    key = (device, torch.cuda.current_stream(device).cuda_stream, threading.get_ident())
-    ws = _ws_cache.get(key)
+    buffer (work of one thread on one stream is ordered by the stream).  The buffers of a thread live in
+    thread-local storage: a worker thread that ends (a pool that is torn down) gives its buffers back."""
+    store = getattr(_ws_local, "store", None)
+    if store is None:
+        store = _ws_local.store = _WorkspaceStore()
+        _ws_stores.add(store)
+    key = (device, torch.cuda.current_stream(device).cuda_stream)
+    ws = store.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(max(nbytes, 1 << 16), dtype=torch.uint8, device=device)
-        _ws_cache[key] = ws
+        store[key] = ws
     return ws
+
+
+def release_workspaces() -> None:
+    """Drop the cached scratch buffers of every thread (the largest GPTQ workspace is R * K * 4 bytes and more).
+    Call it between phases when the memory is wanted back; work already enqueued keeps its buffer alive through
+    the caching allocator's stream ordering, and the next call allocates afresh."""
+    for store in list(_ws_stores):
+        store.clear()
 
 
 def _ptr(t):

@@ -206,13 +206,15 @@ def _calibrate_tail(model, layers, tail, dataloader, cache, device, returns_tupl
     def cached_output(*args, **kwargs):
         return (current["hidden"],) if returns_tuple else current["hidden"]
 
-    patched = []
+    missing = object()
+    patched = []  # (layer, the instance-level forward it carried before, or `missing`)
+    seen = 0
     try:
         for layer in layers[:-1]:
+            patched.append((layer, vars(layer).get("forward", missing)))
             layer.forward = hand_through
-            patched.append(layer)
+        patched.append((layers[-1], vars(layers[-1]).get("forward", missing)))
         layers[-1].forward = cached_output
-        patched.append(layers[-1])
         with HooksMixin.disable_hooks(keep=keep):
             for i, batch in enumerate(dataloader):
                 if i >= len(cache):
@@ -220,9 +222,19 @@ def _calibrate_tail(model, layers, tail, dataloader, cache, device, returns_tupl
                 current["hidden"] = cache.fetch(i)["args"][0]
                 batch = _to_device(batch, device)
                 model(**batch) if isinstance(batch, dict) else model(batch)
+                seen += 1
     finally:
-        for layer in patched:
-            del layer.forward  # back to the class's method
+        for layer, previous in patched:
+            if previous is missing:
+                del layer.forward  # back to the class's method
+            else:
+                layer.forward = previous  # a wrapper assigned on the instance (e.g. an offloading hook) stays in place
+    if seen < len(cache):
+        # a one-shot iterable is exhausted after the first pass: the modules after the last layer would be left
+        # with fewer samples than the layers (none at all, a zero Hessian), which must not pass silently
+        raise RuntimeError(
+            f"the calibration data yielded {seen} batches on the pass for the modules after the last layer, "
+            f"{len(cache)} on the first pass; pass a re-iterable dataloader (a list or a DataLoader)")
 
 
 def _handles_of(module: torch.nn.Module):

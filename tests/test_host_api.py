@@ -632,3 +632,61 @@ def test_owl_outlier_percentage_and_sparsity_mapping():
     stretched = (d - d.min()) * (2 * lmbda / (d.max() - d.min()))
     keep = stretched - stretched.mean() + (1 - target)
     assert abs(keep.mean().item() - (1 - target)) < 1e-12 and abs((keep.max() - keep.min()).item() - 2 * lmbda) < 1e-12
+
+
+def test_tail_pass_restores_instance_level_forwards_and_refuses_a_short_second_pass():
+    """The pass that calibrates what follows the last sequential layer short-circuits the layers by assigning
+    `forward` on the instances.  A layer that already carried an instance-level forward (a wrapper such as an
+    offloading hook) must get it back, a layer without one must fall back to its class, and a dataloader that is
+    exhausted after the first pass must raise instead of leaving the tail modules without samples."""
+    import torch
+
+    from llmcompressor_amd.pipelines import _calibrate_tail
+
+    class Layer(torch.nn.Module):
+        def forward(self, hidden_states):
+            return hidden_states + 1
+
+    class Model(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.layers = torch.nn.ModuleList([Layer(), Layer()])
+            self.head = torch.nn.Linear(4, 4, bias=False)
+
+        def forward(self, x):
+            for layer in self.layers:
+                x = layer(x)
+            return self.head(x)
+
+    class Cache:
+        def __init__(self, items):
+            self.items = items
+
+        def __len__(self):
+            return len(self.items)
+
+        def fetch(self, i):
+            return {"args": (self.items[i],)}
+
+    model = Model()
+    calls = []
+    original = model.layers[0].forward
+
+    def wrapper(hidden_states):  # what accelerate's add_hook_to_module leaves on an instance
+        calls.append(1)
+        return original(hidden_states)
+
+    model.layers[0].forward = wrapper
+    seen = []
+    model.head.register_forward_pre_hook(lambda m, a: seen.append(a[0].clone()))
+    batches = [torch.zeros(1, 4), torch.ones(1, 4)]
+    cache = Cache([torch.full((1, 4), 7.0), torch.full((1, 4), 9.0)])
+    _calibrate_tail(model, list(model.layers), [model.head], batches, cache, torch.device("cpu"), returns_tuple=False)
+    assert [t[0, 0].item() for t in seen] == [7.0, 9.0]  # the head saw the cached outputs of the last layer
+    assert vars(model.layers[0])["forward"] is wrapper and not calls  # wrapper back in place, not called meanwhile
+    assert "forward" not in vars(model.layers[1])  # back to the class's method
+    assert model(torch.zeros(1, 4)).shape == (1, 4) and calls == [1]
+    with pytest.raises(RuntimeError, match="re-iterable"):
+        _calibrate_tail(model, list(model.layers), [model.head], iter(batches[:1]), cache, torch.device("cpu"),
+                        returns_tuple=False)
+    assert vars(model.layers[0])["forward"] is wrapper and "forward" not in vars(model.layers[1])
