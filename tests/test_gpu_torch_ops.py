@@ -65,3 +65,37 @@ def test_torch_ops_refuse_host_tensors():
 
     with pytest.raises((NotImplementedError, RuntimeError)):
         torch.ops.llmc.minmax_observe(torch.zeros(4, 8, dtype=torch.bfloat16), 8)
+
+
+def test_workspaces_are_per_thread_and_go_away_with_the_thread():
+    """A call's scratch buffer is cached per (device, stream, host thread) in thread-local storage: a worker thread
+    that has ended no longer pins its buffer, and release_workspaces() drops the buffers of the live threads."""
+    import gc
+    import threading
+
+    import torch
+
+    from llmcompressor_amd import ops
+
+    ops.release_workspaces()
+    w = torch.randn(64, 256, device="cuda").bfloat16()
+    ops.minmax_groups(w, 64)
+    mine = [s for s in ops._ws_stores if s]
+    assert len(mine) == 1 and len(mine[0]) == 1
+    seen = []
+
+    def worker():
+        ops.minmax_groups(w, 64)
+        seen.append(len([s for s in ops._ws_stores if s]))
+
+    t = threading.Thread(target=worker)
+    t.start()
+    t.join()
+    assert seen == [2]  # the worker had a buffer of its own
+    del t
+    gc.collect()
+    assert len([s for s in ops._ws_stores if s]) == 1  # ... which went away with the thread
+    ops.release_workspaces()
+    assert not [s for s in ops._ws_stores if s]
+    mn, mx = ops.minmax_groups(w, 64)  # and the next call simply allocates again
+    assert torch.equal(mn, w.unflatten(-1, (-1, 64)).amin(-1))
