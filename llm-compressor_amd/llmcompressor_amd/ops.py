@@ -157,6 +157,10 @@ class _WorkspaceStore(dict):
     """The scratch buffers of one host thread, keyed by (device, stream)."""
 
     __slots__ = ("__weakref__",)
+    __hash__ = object.__hash__  # kept in a WeakSet: identity, not contents
+
+    def __eq__(self, other):
+        return self is other
 
 
 _ws_local = threading.local()  # a thread's store goes away with the thread, and its buffers with it
