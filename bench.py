@@ -502,6 +502,10 @@ def main():
     ap.add_argument("--stage-tokens", type=int, default=65536,
                     help="tokens staged per Hessian launch (GPTQModifier.hessian_batch_tokens; 0 = one launch per batch)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--group-min-modules", type=int, default=None,
+                    help="GPTQModifier.group_min_modules of the step (default: the modifier's own)")
+    ap.add_argument("--compress-concurrency", type=int, default=None,
+                    help="GPTQModifier.compress_concurrency of the step (default: the modifier's own)")
     ap.add_argument("--probe-dominant", type=int, default=0, metavar="N",
                     help="counter runs: launch only the dominant kernel N times (14336-wide Hessian, --stage-tokens "
                     "tokens) and N plain copies of a 1 GiB buffer (the known-size kernel the HBM counters are scaled by)")
@@ -629,9 +633,14 @@ def main():
         for name, r, k in LINEARS:
             getattr(layer, name).weight.data.copy_(originals[name])
         recording[0] = record
+        tuning = {}
+        if a.group_min_modules is not None:
+            tuning["group_min_modules"] = a.group_min_modules
+        if a.compress_concurrency is not None:
+            tuning["compress_concurrency"] = a.compress_concurrency
         modifier = GPTQModifier(targets="Linear", scheme="W4A16", actorder="static", block_size=128,
                                 dampening_frac=0.01, hessian_batch_tokens=a.stage_tokens,
-                                share_identical_inputs=share)
+                                share_identical_inputs=share, **tuning)
         session = active_session()
         session.reset()
         session.initialize(model=layer, recipe=modifier)
