@@ -690,3 +690,19 @@ def test_tail_pass_restores_instance_level_forwards_and_refuses_a_short_second_p
         _calibrate_tail(model, list(model.layers), [model.head], iter(batches[:1]), cache, torch.device("cpu"),
                         returns_tuple=False)
     assert vars(model.layers[0])["forward"] is wrapper and "forward" not in vars(model.layers[1])
+
+
+@pytest.mark.parametrize("shape", [(2, 3, 8, 8), (3, 8, 8)])
+def test_conv2d_hessian_branch_fails_the_way_the_reference_does(shape):
+    """/root/reference/src/llmcompressor/modifiers/gptq/gptq_quantize.py:36-56: every input is brought to three
+    dimensions before the Conv2d branch, where ``Unfold`` then takes it for one unbatched image and returns a
+    matrix, so the following three-axis ``permute`` raises.  The branch cannot succeed for any input in the
+    reference; the mirror applies the same operations in the same order and fails at the same one, before any
+    device call."""
+    from llmcompressor_amd.modifiers.gptq.gptq_quantize import accumulate_hessian, make_empty_hessian
+
+    conv = torch.nn.Conv2d(3, 8, 3, padding=1)
+    H = make_empty_hessian(conv)
+    assert H.shape == (3, 3)  # weight.shape[1], as in the reference (not in_channels * kernel area)
+    with pytest.raises(RuntimeError, match="permute"):
+        accumulate_hessian(torch.randn(*shape), conv, H, torch.zeros(1))
