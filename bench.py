@@ -379,6 +379,27 @@ def probe_moe(mode="both"):
     # a skewed router, as trained ones are: expert e is about e^-1.1 as likely as expert 1
     logits = torch.randn(T, E, device="cuda") + torch.log(1.0 / torch.arange(1, E + 1, device="cuda").float() ** 1.1)
     w, idx = torch.topk(torch.softmax(logits, -1), TOPK, -1)
+    from llmcompressor_amd.modeling import moe as moe_module
+
+    with torch.no_grad():  # the propagation pass: nothing observes the experts
+        for grouped in (False, True):
+            moe_module.GROUPED_FORWARD = grouped
+            for _ in range(2):
+                model.layers[0](x, idx, w.to(x.dtype))
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(5):
+                model.layers[0](x, idx, w.to(x.dtype))
+            torch.cuda.synchronize()
+            print(f"propagation forward, {'grouped launches' if grouped else 'per-expert calls'}: "
+                  f"{(time.perf_counter() - t0) / 5 * 1e3:.2f} ms per batch")
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        model.layers[0](x, idx, w.to(x.dtype))
+        e0.record()
+        model.layers[0](x, idx, w.to(x.dtype))
+        e1.record()
+        torch.cuda.synchronize()
+        print(f"propagation forward, grouped launches, device time between events: {e0.elapsed_time(e1):.2f} ms")
     print("| quantisation of the 384 expert Linears | forward + Hessians ms per batch | quantise ms | ms per Linear |")
     print("|---|---|---|---|")
     variants = (("W4A16, lock-step groups (default)", 8, "lockstep", "W4A16"),

@@ -348,6 +348,21 @@ int llmc_sparsegpt_sparsify(const void* weight, int32_t w_dtype, int64_t R, int6
                             int32_t preserve_sparsity_mask, void* out_weight, int64_t ldo,
                             float* loss_out, void* workspace, int64_t workspace_bytes, void* stream);
 
+/* Grouped Linear of the experts of an MoE block (the reference's loop: modeling/moe/linear_experts.py:235-268
+ * calls each expert's gate_proj / up_proj / down_proj on its own routed rows, one F.linear each):
+ *   y[r, s*N + n] = sum_k x[r, k] * W_{s,e(r)}[n, k]   for every routed row r, bf16 in, fp32 accumulation,
+ * one rounding to bf16.  x [rows, K] (row stride ldx) holds the routed rows expert after expert; `tiles`
+ * (device, int32 [ntiles][4], 16-byte aligned) lists runs of at most 128 rows of one expert as
+ * {expert, first row, rows, 0}; w (device array of splits * experts pointers, 16-byte aligned each) holds the
+ * [N, K] weights (row stride ldw) of split s and expert e at w[s * experts + e]; splits that share their input
+ * (gate and up) write side by side into y (row stride ldy >= splits * N).  N % 128 == 0, K % 64 == 0,
+ * dtype LLMC_BF16.  Rows no tile names are not written.  The sum over k runs in a different order than a
+ * library GEMM's, so results agree with F.linear to the last bf16 digit, not bit for bit: use it where hooks do
+ * not need the exact inputs of the reference's forward (the propagation pass of a sequential pipeline). */
+int llmc_grouped_linear(const void* x, int32_t dtype, int64_t ldx, const void* const* w, int64_t ldw,
+                        int32_t experts, int32_t splits, void* y, int64_t ldy, const int32_t* tiles,
+                        int32_t ntiles, int64_t N, int64_t K, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -6,6 +6,10 @@ Every expert is called on every forward, also with zero routed tokens (an expert
 token keeps a zero Hessian, so GPTQ zeroes its weight exactly as the reference does).  Inside
 ``moe_calibration_context()`` every expert sees all tokens; outputs are still combined with the routing
 weights of the tokens actually routed to it.
+
+When nothing observes the experts' Linears -- every hook on them was registered through ``HooksMixin`` and is
+switched off (the propagation pass of a sequential pipeline), no quantised forward is active -- the
+per-expert calls are replaced by two grouped launches over the routed-token buffer (``grouped_forward``).
 """
 from __future__ import annotations
 
@@ -20,6 +24,8 @@ __all__ = ["ExpertMLP", "LinearExperts2D", "Llama4LinearExperts", "moe_calibrati
            "get_non_linearized_moes", "linearize_moe"]
 
 _CALIBRATE_ALL_EXPERTS = False
+# replace the per-expert loop by grouped launches when no hook or quantised forward needs the single calls
+GROUPED_FORWARD = True
 
 
 @contextlib.contextmanager
@@ -52,6 +58,15 @@ class ExpertMLP(nn.Module):
         if self._gate_fn is None:
             return self.down_proj(self.act_fn(self.gate_proj(x)) * self.up_proj(x))
         return self.down_proj(self._gate_fn(torch.cat([self.gate_proj(x), self.up_proj(x)], dim=-1)))
+
+
+def _hooks_inert(module: nn.Module, hook_is_inert) -> bool:
+    """No hook of ``module`` would do anything if it were called now."""
+    for hooks in (module._forward_hooks, module._forward_pre_hooks, module._backward_hooks,
+                  module._backward_pre_hooks):
+        if hooks and not all(hook_is_inert(h) for h in hooks.values()):
+            return False
+    return True
 
 
 class LinearExperts2D(nn.ModuleList):
@@ -105,6 +120,89 @@ class LinearExperts2D(nn.ModuleList):
                               None if gub is None else gub.data, None if db is None else db.data,
                               apply_gate=apply_gate, gate_attributes=attributes)
 
+    # per instance switch for the grouped launches (see ``_grouped_plan``)
+    grouped_forward = True
+
+    def _grouped_plan(self, hidden_states: torch.Tensor):
+        """The experts' weights as two pointer tables, or None when the per-expert calls must stay: some hook on
+        an expert or one of its Linears would fire (only hooks registered through ``HooksMixin`` can be told to be
+        off), a Linear has a bias, a quantised forward is active, the experts are not plain ``ExpertMLP``s of
+        bf16 Linears of one shape, gradients are recorded, or the shapes do not fit the kernel's tiles.  The
+        grouped products add along k in another order than the library GEMM behind ``F.linear``: same values to
+        the last bf16 digit, not the same bits, which is why observed passes keep the loop."""
+        from ..modifiers.utils.hooks import hook_is_inert
+        from .. import ops
+
+        if (not hidden_states.is_cuda or hidden_states.dtype != torch.bfloat16 or torch.is_grad_enabled()
+                or len(self) == 0 or nn.modules.module._global_forward_hooks
+                or nn.modules.module._global_forward_pre_hooks):
+            return None
+        weights = ([], [], [])
+        first = self[0]
+        act_type, gate_fn = type(first._modules["act_fn"]), first._gate_fn
+        names = ("gate_proj", "up_proj", "down_proj")
+        for expert in self._modules.values():
+            d = expert.__dict__
+            if type(expert) is not ExpertMLP or "forward" in d or d["_gate_fn"] is not gate_fn:
+                return None
+            if (d["_forward_hooks"] or d["_forward_pre_hooks"] or d["_backward_hooks"]
+                    or d["_backward_pre_hooks"]) and not _hooks_inert(expert, hook_is_inert):
+                return None
+            mods = d["_modules"]
+            if type(mods["act_fn"]) is not act_type:
+                return None
+            for slot in range(3):
+                lin = mods[names[slot]]
+                d = lin.__dict__
+                if type(lin) is not nn.Linear or d["_parameters"]["bias"] is not None:
+                    return None
+                if (d["_forward_hooks"] or d["_forward_pre_hooks"] or d["_backward_hooks"]
+                        or d["_backward_pre_hooks"]) and not _hooks_inert(lin, hook_is_inert):
+                    return None
+                if "forward" in d and not (
+                        d.get("_llmc_forward_wrapped", False)
+                        and (d.get("quantization_scheme") is None or not d.get("quantization_enabled", True))):
+                    return None
+                weights[slot].append(d["_parameters"]["weight"])
+        if any(True for _ in first.act_fn.parameters()):
+            return None
+        key = tuple(w.data_ptr() for group in weights for w in group)
+        cached = self.__dict__.get("_grouped_cache")
+        if cached is not None and cached[0] == key and cached[1] == hidden_states.device:
+            return cached[2]
+        gate, up, down = weights
+        inter, hidden = gate[0].shape
+        for group, shape in ((gate, (inter, hidden)), (up, (inter, hidden)), (down, (hidden, inter))):
+            for w in group:
+                if (w.shape != shape or w.dtype != torch.bfloat16 or w.stride() != group[0].stride()
+                        or w.stride(1) != 1 or w.stride(0) % 8 or w.device != hidden_states.device):
+                    return None
+        if not (ops.grouped_linear_supported(inter, hidden, torch.bfloat16)
+                and ops.grouped_linear_supported(hidden, inter, torch.bfloat16)) or gate[0].stride() != up[0].stride():
+            return None
+        try:
+            plan = dict(gate_up=ops.weight_pointer_table(gate + up, hidden_states.device), ld_gate_up=gate[0].stride(0),
+                        down=ops.weight_pointer_table(down, hidden_states.device), ld_down=down[0].stride(0),
+                        inter=inter, hidden=hidden)
+        except ValueError:  # a weight that is not 16-byte aligned
+            return None
+        object.__setattr__(self, "_grouped_cache", (key, hidden_states.device, plan))
+        return plan
+
+    def _forward_grouped(self, plan, routed: torch.Tensor, counts) -> torch.Tensor:
+        """``expert(rows)`` for every expert's rows of ``routed`` (sorted by expert) in two launches."""
+        from .. import ops
+
+        E, inter = self.num_experts, plan["inter"]
+        tiles, ntiles = ops.grouped_linear_tiles(counts, routed.device)
+        gate_up = ops.grouped_linear(routed, plan["gate_up"], E, 2, inter, plan["ld_gate_up"], tiles, ntiles)
+        first = self[0]
+        if first._gate_fn is not None:
+            mid = first._gate_fn(gate_up)
+        else:
+            mid = first.act_fn(gate_up[:, :inter]) * gate_up[:, inter:]
+        return ops.grouped_linear(mid.contiguous(), plan["down"], E, 1, plan["hidden"], plan["ld_down"], tiles, ntiles)
+
     def forward(self, hidden_states: torch.Tensor, top_k_index: torch.Tensor, top_k_weights: torch.Tensor):
         """hidden_states [T,H]; top_k_index / top_k_weights [T,k].
 
@@ -128,16 +226,21 @@ class LinearExperts2D(nn.ModuleList):
             place = torch.empty_like(order)
             place[order] = torch.arange(order.numel(), device=order.device)
             place = place.view(k, T).sort(dim=0).values
-        routed = None if _CALIBRATE_ALL_EXPERTS else hidden_states[tok_sorted]
-        outs, at = [], 0
-        for e, expert in enumerate(self):
-            n = counts[e]
-            if _CALIBRATE_ALL_EXPERTS:
-                outs.append(expert(hidden_states)[tok_sorted[at:at + n]])
-            else:
-                outs.append(expert(routed[at:at + n]))
-            at += n
-        weighted = (torch.cat(outs) * top_k_weights[tok_sorted, slot_sorted, None]).to(hidden_states.dtype)
+        plan = self._grouped_plan(hidden_states) if GROUPED_FORWARD and self.grouped_forward else None
+        if plan is not None:
+            expert_out = self._forward_grouped(plan, hidden_states[tok_sorted], counts)
+        else:
+            routed = None if _CALIBRATE_ALL_EXPERTS else hidden_states[tok_sorted]
+            outs, at = [], 0
+            for e, expert in enumerate(self):
+                n = counts[e]
+                if _CALIBRATE_ALL_EXPERTS:
+                    outs.append(expert(hidden_states)[tok_sorted[at:at + n]])
+                else:
+                    outs.append(expert(routed[at:at + n]))
+                at += n
+            expert_out = torch.cat(outs)
+        weighted = (expert_out * top_k_weights[tok_sorted, slot_sorted, None]).to(hidden_states.dtype)
         final = torch.zeros_like(hidden_states)
         for j in range(k):
             final = final + weighted[place[j]]

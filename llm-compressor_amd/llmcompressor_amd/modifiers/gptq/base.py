@@ -264,8 +264,12 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
                                        "this model")
                 self._flush(leader)
                 self._hessians[module] = self._hessians[leader].clone()
-                self._num_samples[module] = torch.tensor(float(self._num_samples[module]),
-                                                         device=self._hessians[module].device)
+                # the tally in the form the leader keeps it (host number for experts, device scalar otherwise),
+                # filled on the device: no host transfer or wait per follower
+                tally = self._num_samples[leader]
+                count = float(self._num_samples[module])
+                self._num_samples[module] = (torch.full_like(tally, count) if isinstance(tally, torch.Tensor)
+                                             else count)
         self._recent_input = None
         for module in module_list:
             self._hook_calls.pop(module, None)

@@ -10,7 +10,17 @@ import torch
 from pydantic import BaseModel, PrivateAttr
 from torch.utils.hooks import RemovableHandle
 
-__all__ = ["HooksMixin"]
+__all__ = ["HooksMixin", "hook_is_inert"]
+
+
+def hook_is_inert(fn) -> bool:
+    """True for a hook function registered through ``HooksMixin.register_hook`` that is switched off right now
+    (``disable_hooks`` is active and its handle is not among the kept ones): calling it would return at once."""
+    handle = getattr(fn, "_llmc_handle", None)
+    if handle is None:
+        return False
+    handle = handle()
+    return handle is not None and HooksMixin._HOOKS_DISABLED and handle not in HooksMixin._HOOKS_KEEP_ENABLED
 
 
 class HooksMixin(BaseModel):
@@ -47,6 +57,7 @@ class HooksMixin(BaseModel):
         name = f"register_{hook_type}_hook" if hook_type else "register_hook"
         register = getattr(target, name)
         handle = register(wrapped_hook, **kwargs)
+        wrapped_hook._llmc_handle = weakref.ref(handle)
         self._hooks.add(handle)
         HooksMixin._ALL_HANDLES.add(handle)
         return handle

@@ -682,3 +682,60 @@ def sgemm_(C: torch.Tensor, A: torch.Tensor, B: torch.Tensor, alpha: float = 1.0
                                    M, N, Kc, float(alpha), float(beta), 1 if trans_b else 0, int(flags), _stream(C))
     _lib.check(rc, "llmc_sgemm")
     return C
+
+
+GROUPED_LINEAR_ROWS = 128  # rows of one expert per entry of the tile table
+
+
+def grouped_linear_tiles(counts, device) -> tuple[torch.Tensor, int]:
+    """Tile table of ``grouped_linear`` for experts whose routed rows lie one after the other: per run of at most
+    128 rows of one expert ``[expert, first row, rows, 0]`` (int32, on ``device``).  ``counts`` are the experts'
+    row counts (host integers); an expert without rows gets no entry."""
+    import numpy as np
+
+    counts = np.asarray(counts, dtype=np.int64)
+    per = (counts + GROUPED_LINEAR_ROWS - 1) // GROUPED_LINEAR_ROWS
+    n = int(per.sum())
+    table = np.zeros((max(n, 1), 4), dtype=np.int32)
+    if n:
+        expert = np.repeat(np.arange(counts.size), per)
+        first_tile = np.cumsum(per) - per                       # index of each expert's first entry
+        within = np.arange(n) - np.repeat(first_tile, per)      # entry number inside its expert
+        start = np.repeat(np.cumsum(counts) - counts, per) + within * GROUPED_LINEAR_ROWS
+        rows = np.minimum(np.repeat(counts, per) - within * GROUPED_LINEAR_ROWS, GROUPED_LINEAR_ROWS)
+        table[:, 0], table[:, 1], table[:, 2] = expert, start, rows
+    return torch.from_numpy(table).to(device), n
+
+
+def grouped_linear_supported(N: int, K: int, dtype) -> bool:
+    return dtype == torch.bfloat16 and N % 128 == 0 and K % 64 == 0
+
+
+def weight_pointer_table(weights, device) -> torch.Tensor:
+    """Device array of the data pointers of ``weights`` (each [N, K] bf16, unit column stride, one common row stride,
+    16-byte aligned), in the order ``grouped_linear`` expects: split-major, expert-minor."""
+    ptrs = [w.data_ptr() for w in weights]
+    if any(p & 15 for p in ptrs):
+        raise ValueError("weight_pointer_table: every weight must be 16-byte aligned")
+    return torch.tensor(ptrs, dtype=torch.int64, device=device)
+
+
+def grouped_linear(x: torch.Tensor, pointers: torch.Tensor, experts: int, splits: int, N: int, ldw: int,
+                   tiles: torch.Tensor, ntiles: int) -> torch.Tensor:
+    """y [rows, splits * N] (bf16): the rows the tile table assigns to expert e times the transposed weights
+    ``pointers[s * experts + e]`` ([N, K] bf16, row stride ldw) for every split s.  Every row of x must belong to
+    a tile (the output is not cleared)."""
+    _require_gpu(x, pointers, tiles)
+    assert x.ndim == 2 and x.dtype == torch.bfloat16 and x.stride(1) == 1
+    assert pointers.dtype == torch.int64 and pointers.numel() == experts * splits
+    assert tiles.dtype == torch.int32 and tiles.ndim == 2 and tiles.shape[1] == 4 and tiles.shape[0] >= ntiles
+    K = x.shape[1]
+    y = torch.empty((x.shape[0], splits * N), dtype=x.dtype, device=x.device)
+    if x.shape[0] == 0:
+        return y
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().llmc_grouped_linear(x.data_ptr(), _dt(x), x.stride(0), pointers.data_ptr(), ldw, experts,
+                                            splits, y.data_ptr(), y.stride(0), tiles.data_ptr(), ntiles, N, K,
+                                            _stream(x))
+    _lib.check(rc, "llmc_grouped_linear")
+    return y

@@ -1,0 +1,219 @@
+"""GPU: the grouped expert Linear (``llmc_grouped_linear``) and the grouped forward of ``LinearExperts2D``.
+
+The grouped products add along k in another order than the library GEMM behind ``F.linear``, so they are compared
+with the per-expert loop (the reference's forward, ``oracle/moe.py``) to a stated tolerance instead of bit for bit:
+at least 99.9 % of the outputs within one bf16 unit in the last place of the loop's value, all of them within a
+small multiple of the rounding of the fp32 sums, and neither further from the fp64 product than the other by more
+than that.  Where hooks observe the experts the loop itself must run, and that stays bit for bit.
+"""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _ulp_bf16(v: torch.Tensor) -> torch.Tensor:
+    """One unit in the last place of a bf16 value of this magnitude (8 significand bits)."""
+    return torch.pow(2.0, torch.floor(torch.log2(v.abs().float().clamp_min(1e-30))) - 7)
+
+
+def _assert_same_to_one_ulp(got, want, exact, what=""):
+    got, want = got.float(), want.float()
+    diff = (got - want).abs()
+    within = diff <= _ulp_bf16(want)
+    frac = within.float().mean().item()
+    assert frac >= 0.999, f"{what}: {frac:.5f} of the outputs within one bf16 ulp"
+    # the rest: results that cancellation made small against their terms; small against a typical output then
+    scale = exact.abs().float().mean().item()
+    assert bool((within | (diff <= 2.0 ** -9 * scale)).all()), what
+    eg, ew = (got.double() - exact).abs().mean().item(), (want.double() - exact).abs().mean().item()
+    assert eg <= 1.05 * ew + 1e-12, f"{what}: grouped error {eg:.3e} against the loop's {ew:.3e}"
+
+
+@pytest.mark.parametrize("N,K,splits", [(128, 64, 1), (768, 2048, 2), (2048, 768, 1), (256, 192, 3)])
+def test_grouped_linear_against_per_expert_linear(N, K, splits):
+    from llmcompressor_amd import ops
+
+    torch.manual_seed(N + K + splits)
+    counts = [0, 1, 127, 128, 129, 0, 300, 5, 1000, 64, 0]
+    E, rows = len(counts), sum(counts)
+    x = torch.randn(rows, K, device=DEV).bfloat16()
+    weights = [[(torch.randn(N, K, device=DEV) * K ** -0.5).bfloat16() for _ in range(E)] for _ in range(splits)]
+    table = ops.weight_pointer_table([w for group in weights for w in group], DEV)
+    tiles, ntiles = ops.grouped_linear_tiles(counts, DEV)
+    assert ntiles == sum(-(-c // 128) for c in counts)
+    y = ops.grouped_linear(x, table, E, splits, N, K, tiles, ntiles)
+    assert y.shape == (rows, splits * N) and y.dtype == torch.bfloat16
+    at = 0
+    for e, c in enumerate(counts):
+        for s in range(splits):
+            want = torch.nn.functional.linear(x[at:at + c], weights[s][e])
+            exact = x[at:at + c].double() @ weights[s][e].double().t()
+            if c:
+                _assert_same_to_one_ulp(y[at:at + c, s * N:(s + 1) * N], want, exact, f"expert {e} split {s}")
+        at += c
+
+
+def test_grouped_linear_reads_strided_rows_and_rejects_what_it_cannot_tile():
+    from llmcompressor_amd import _lib, ops
+
+    torch.manual_seed(0)
+    E, N, K = 3, 128, 128
+    big = torch.randn(200, 2 * K, device=DEV).bfloat16()
+    x = big[:, :K]  # row stride 2 K
+    wbig = [(torch.randn(N, K + 64, device=DEV) * 0.1).bfloat16() for _ in range(E)]
+    weights = [w[:, :K] for w in wbig]  # row stride K + 64
+    counts = [70, 0, 130]
+    tiles, ntiles = ops.grouped_linear_tiles(counts, DEV)
+    y = ops.grouped_linear(x, ops.weight_pointer_table(weights, DEV), E, 1, N, K + 64, tiles, ntiles)
+    want = torch.cat([torch.nn.functional.linear(x[:70], weights[0]), torch.nn.functional.linear(x[70:], weights[2])])
+    exact = torch.cat([x[:70].double() @ weights[0].double().t(), x[70:].double() @ weights[2].double().t()])
+    _assert_same_to_one_ulp(y, want, exact)
+    with pytest.raises(ValueError, match="argument 4"):  # N not a multiple of 128
+        ops.grouped_linear(x, ops.weight_pointer_table(weights, DEV), E, 1, 96, K + 64, tiles, ntiles)
+    with pytest.raises(ValueError):  # a weight that is not 16-byte aligned
+        ops.weight_pointer_table([wbig[0].view(-1)[1:1 + N * K].view(N, K)], DEV)
+    assert _lib.lib().llmc_grouped_linear(x.data_ptr(), 2, 2 * K, 0, K, E, 1, y.data_ptr(), N, tiles.data_ptr(), ntiles,
+                                          N, K, 0) < 0  # null pointer table
+
+
+def _moe(E, H, I, seed, apply_gate=None):
+    from llmcompressor_amd.modeling import LinearExperts2D
+
+    torch.manual_seed(seed)
+    experts = LinearExperts2D(E, H, I, torch.bfloat16, DEV, apply_gate=apply_gate)
+    for p in experts.parameters():
+        p.data.normal_(0, H ** -0.5)
+    return experts
+
+
+def _routing(T, E, k, idle=None):
+    logits = torch.randn(T, E, device=DEV) + torch.log(1.0 / torch.arange(1, E + 1, device=DEV).float() ** 1.1)
+    if idle is not None:
+        logits[:, idle] = -1e9
+    wts, idx = torch.topk(torch.softmax(logits, -1), k, -1)
+    return idx, wts.bfloat16()
+
+
+def _exact_forward(experts, x, idx, wts):
+    """sum_j w[t, j] * expert_{idx[t, j]}(x[t]) with every product in fp64."""
+    out = torch.zeros(x.shape, dtype=torch.float64, device=x.device)
+    xd = x.double()
+    for e, ex in enumerate(experts):
+        slot_hit = idx == e
+        tok = slot_hit.any(-1).nonzero().flatten()
+        if tok.numel() == 0:
+            continue
+        g, u, d = (m.weight.double() for m in (ex.gate_proj, ex.up_proj, ex.down_proj))
+        h = torch.nn.functional.silu(xd[tok] @ g.t()) * (xd[tok] @ u.t())
+        w = (wts.double() * slot_hit)[tok].sum(-1, keepdim=True)
+        out[tok] += (h @ d.t()) * w
+    return out
+
+
+@pytest.mark.parametrize("all_experts", [False, True])
+def test_forward_without_observers_uses_the_grouped_launches_and_agrees_with_the_loop(all_experts, monkeypatch):
+    from llmcompressor_amd import ops
+    from llmcompressor_amd.modeling import moe, moe_calibration_context
+    from oracle.moe import experts_forward
+
+    E, H, I, T, k = 32, 256, 128, 2048, 4
+    experts = _moe(E, H, I, 5)
+    x = torch.randn(T, H, device=DEV).bfloat16()
+    idx, wts = _routing(T, E, k, idle=9)
+    launches = []
+    real = ops.grouped_linear
+    monkeypatch.setattr(ops, "grouped_linear", lambda *a, **kw: launches.append(a[3]) or real(*a, **kw))
+    with torch.no_grad():
+        if all_experts:
+            with moe_calibration_context():
+                got = experts(x, idx, wts)
+        else:
+            got = experts(x, idx, wts)
+        assert launches == [2, 1]  # gate and up side by side, then down
+        want = experts_forward(list(experts), x, idx, wts)
+        monkeypatch.setattr(moe, "GROUPED_FORWARD", False)
+        assert torch.equal(experts(x, idx, wts), want) and launches == [2, 1]  # the switch restores the loop's bits
+    exact = _exact_forward(experts, x, idx, wts)
+    # the output adds k expert outputs, each rounded to bf16 once more: one ulp of the sum holds for fewer elements
+    diff = (got.float() - want.float()).abs()
+    within = diff <= 2 * _ulp_bf16(want.float())
+    assert within.float().mean().item() >= 0.995
+    assert bool((within | (diff <= 2.0 ** -7 * exact.abs().mean().item())).all())
+    eg, ew = (got.double() - exact).abs().mean().item(), (want.double() - exact).abs().mean().item()
+    assert eg <= 1.05 * ew
+
+
+def test_forward_with_observers_keeps_the_per_expert_calls(monkeypatch):
+    """A hook from outside, an active HooksMixin hook, a bias or recorded gradients keep the loop (bit for bit the
+    oracle's); HooksMixin hooks that are switched off do not."""
+    from llmcompressor_amd import ops
+    from llmcompressor_amd.modifiers.utils.hooks import HooksMixin
+    from oracle.moe import experts_forward
+
+    E, H, I, T, k = 8, 128, 128, 512, 2
+    experts = _moe(E, H, I, 6)
+    x = torch.randn(T, H, device=DEV).bfloat16()
+    idx, wts = _routing(T, E, k)
+    launches = []
+    real = ops.grouped_linear
+    monkeypatch.setattr(ops, "grouped_linear", lambda *a, **kw: launches.append(1) or real(*a, **kw))
+
+    class Owner(HooksMixin):
+        pass
+
+    owner, seen = Owner(), []
+    handles = [owner.register_hook(ex.down_proj, lambda m, a: seen.append(a[0].shape[0]), "forward_pre")
+               for ex in experts]
+    with torch.no_grad():
+        want = experts_forward(list(experts), x, idx, wts)
+        seen.clear()
+        assert torch.equal(experts(x, idx, wts), want) and not launches and len(seen) == E
+        with HooksMixin.disable_hooks(keep={handles[3]}):  # one hook kept on: still the loop
+            seen.clear()
+            assert torch.equal(experts(x, idx, wts), want) and not launches and len(seen) == 1
+        with HooksMixin.disable_hooks():
+            seen.clear()
+            experts(x, idx, wts)
+            assert launches == [1, 1] and not seen
+        owner.remove_hooks()
+        launches.clear()
+        outside = experts[2].gate_proj.register_forward_hook(lambda m, a, o: None)
+        assert torch.equal(experts(x, idx, wts), want) and not launches
+        outside.remove()
+        experts(x, idx, wts)
+        assert launches == [1, 1]
+    launches.clear()
+    experts(x, idx, wts)  # gradients recorded
+    assert not launches
+    with torch.no_grad():
+        experts[1].up_proj.bias = torch.nn.Parameter(torch.zeros(I, device=DEV, dtype=torch.bfloat16))
+        assert torch.equal(experts(x, idx, wts), experts_forward(list(experts), x, idx, wts)) and not launches
+
+
+def test_grouped_forward_follows_replaced_weights_and_a_custom_gate():
+    from oracle.moe import experts_forward
+
+    def apply_gate(self, gate_up):  # the fused module's own gating: clamp, then act(first half) * second half
+        g, u = gate_up.chunk(2, dim=-1)
+        return torch.nn.functional.gelu(g.clamp(max=1.0)) * u
+
+    E, H, I, T, k = 6, 128, 256, 700, 3
+    experts = _moe(E, H, I, 7, apply_gate=apply_gate)
+    x = torch.randn(T, H, device=DEV).bfloat16()
+    idx, wts = _routing(T, E, k)
+    with torch.no_grad():
+        for _ in range(2):
+            got = experts(x, idx, wts)
+            experts.grouped_forward = False
+            want = experts(x, idx, wts)
+            experts.grouped_forward = True
+            assert torch.equal(want, experts_forward(list(experts), x, idx, wts))
+            diff = (got.float() - want.float()).abs()
+            within = diff <= 2 * _ulp_bf16(want.float())
+            assert within.float().mean().item() >= 0.995
+            assert bool((within | (diff <= 2.0 ** -7 * want.float().abs().mean().item())).all())
+            # new storage for one weight (what a quantiser does when it assigns a fresh tensor): the second
+            # round must read it
+            experts[4].down_proj.weight.data = (experts[4].down_proj.weight.data * -1.0).clone()
