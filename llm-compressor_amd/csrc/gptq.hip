@@ -136,6 +136,7 @@ inline int allow_row_stage(KernT kern, int K) {
   return e == hipSuccess ? 0 : 1000 + (int)e;
 }
 
+
 // The block's [GB][GB] slice of U into LDS, zero outside the upper triangle and past `count`.  Addresses are
 // clamped into the block instead of predicated, so the loads of a batch are all in flight together.
 __device__ __forceinline__ void load_u_block(float* __restrict__ Hs, const float* __restrict__ U, int64_t ldu,
@@ -533,26 +534,30 @@ __device__ __forceinline__ float sgpt_saliency(float w, float d, bool masked) {
   return __fdiv_rn(num, __fmul_rn(d, d));
 }
 
-// First bin whose running total exceeds k; k becomes the rank inside that bin.  All 256 threads of the
-// workgroup take part; `scratch` holds 258 words.
+// First bin whose running total exceeds k (the last bin when none does); k becomes the rank inside that bin.
+// All 256 threads of the workgroup take part; `scratch` holds 258 words.  Thread t sums its nbins / 256
+// consecutive bins, a scan over the 256 sums (shuffles inside a wave, the four wave totals through LDS) finds
+// the one thread whose bins contain rank k, and that thread walks its few bins.
 __device__ __forceinline__ unsigned sgpt_find_bin(const unsigned* __restrict__ hist, int nbins, unsigned& k,
                                                   unsigned* scratch) {
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int per = nbins / 256;
   unsigned local = 0;
   for (int b = 0; b < per; ++b) local += hist[tid * per + b];
-  scratch[tid] = local;
+  unsigned incl = local;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const unsigned v = __shfl_up(incl, d);
+    if (lane >= d) incl += v;
+  }
+  if (lane == 63) scratch[wave] = incl;
   __syncthreads();
-  if (tid == 0) {
-    unsigned run = 0;
-    int t = 0;
-    for (; t < 255; ++t) {
-      if (run + scratch[t] > k) break;
-      run += scratch[t];
-    }
-    unsigned bin = (unsigned)(t * per);
+  for (int w = 0; w < wave; ++w) incl += scratch[w];
+  const unsigned excl = incl - local;
+  if (excl <= k && (k < incl || tid == 255)) {
+    unsigned run = excl, bin = (unsigned)(tid * per);
     for (int b = 0; b < per - 1; ++b) {
-      const unsigned h = hist[t * per + b];
+      const unsigned h = hist[tid * per + b];
       if (run + h > k) break;
       run += h;
       ++bin;
@@ -581,7 +586,9 @@ __global__ __launch_bounds__(256) void sgpt_hist_kernel(SgptParams p) {
   __syncthreads();
   const int64_t n = (int64_t)p.R * p.count;
   for (int64_t e = (int64_t)blockIdx.x * 256 + tid; e < n; e += (int64_t)gridDim.x * 256) {
-    const int r = (int)(e / p.count), c = (int)(e % p.count);
+    // a full block is 128 wide: shift and mask instead of a 64-bit division per element
+    const int r = p.count == GB ? (int)(e >> 7) : (int)(e / p.count);
+    const int c = p.count == GB ? (int)(e & (GB - 1)) : (int)(e % p.count);
     const int col = p.i1 + c;
     const bool masked = p.mask && p.mask[(int64_t)r * p.K + col];
     const float t = sgpt_saliency(p.Wf[(int64_t)r * p.K + col], p.U[(int64_t)col * p.ldu + col], masked);
@@ -869,6 +876,47 @@ extern "C" int llmc_sparsegpt_sparsify(const void* weight, int32_t w_dtype, int6
   return 0;
 }
 
+// The quantiser's blocked column loop for n problems of one shape (n = 1: the single call), lazy updates on
+// two levels.  After a block is quantised its scaled errors E_b update only the columns left in its group of
+// GROUP blocks (what the next block needs); the columns beyond the group get the whole group's errors in one
+// rank-(GROUP*bs) product.  Same sums as updating everything after every block, regrouped -- but the big part
+// of W is read and written a quarter as often, which is what bounds a rank-128 update.
+static int gptq_column_loop(void (*kern)(GptqBlockParams), GptqBlockParams p, int smem, unsigned wgs, int n, int64_t R,
+                            int64_t K, int bs, float* E, const float* U, int64_t ldu, int64_t u_stride, float* Wf,
+                            hipStream_t st) {
+  const int ldE = GROUP * GB;
+  p.ldE = ldE;
+  const int64_t gw = (int64_t)GROUP * bs;
+  auto product = [&](const float* A, int64_t k0, int64_t kc, int64_t c0, int64_t c1) {
+    GemmF32 g = {};
+    g.A = A; g.lda = ldE; g.B = U + k0 * ldu + c0; g.ldb = ldu; g.C = Wf + c0; g.ldc = K;
+    g.M = (int)R; g.N = (int)(c1 - c0); g.Kc = (int)kc; g.alpha = -1.f; g.beta = 1.f;
+    g.batch = 1; g.batch2 = n; g.stride2_a = R * (int64_t)ldE; g.stride2_b = u_stride; g.stride2_c = R * K;
+    return llmc_gemm_f32(g, st);
+  };
+  for (int64_t g0 = 0; g0 < K; g0 += gw) {
+    const int64_t gend = (g0 + gw) < K ? g0 + gw : K;
+    for (int64_t i1 = g0; i1 < gend; i1 += bs) {
+      const int count = (int)((gend - i1) < bs ? (gend - i1) : bs);
+      p.i1 = (int)i1;
+      p.count = count;
+      p.E = E + (i1 - g0);
+      hipLaunchKernelGGL(kern, dim3(wgs, (unsigned)n), dim3(256), smem, st, p);
+      LLMC_LAUNCH_STATUS();
+      const int64_t i2 = i1 + count;
+      if (i2 < gend) {
+        const int rc = product(p.E, i1, count, i2, gend);
+        if (rc) return rc;
+      }
+    }
+    if (gend < K) {
+      const int rc = product(E, g0, gend - g0, gend, K);
+      if (rc) return rc;
+    }
+  }
+  return 0;
+}
+
 extern "C" int64_t llmc_gptq_quantize_workspace_bytes(int64_t R, int64_t K) {
   return align256(R * K * 4) + align256(R * GROUP * GB * 4) + align256(R * 4);
 }
@@ -952,38 +1000,9 @@ extern "C" int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
   if (e != hipSuccess) return 1000 + (int)e;
   const unsigned wgs = (unsigned)((R + Q_ROWS_PER_WG - 1) / Q_ROWS_PER_WG);
-  // Lazy updates on two levels.  After a block is quantised its scaled errors E_b update only the
-  // columns left in its group of GROUP blocks (what the next block needs); the columns beyond the
-  // group get the whole group's errors in one rank-(GROUP*bs) product.  Same sums as updating
-  // everything after every block, regrouped -- but the big part of W is read and written a
-  // quarter as often, which is what bounds a rank-128 update.
-  const int ldE = GROUP * GB;
-  p.ldE = ldE;
-  for (int64_t g0 = 0; g0 < K; g0 += (int64_t)GROUP * bs) {
-    const int64_t gend = (g0 + (int64_t)GROUP * bs) < K ? g0 + (int64_t)GROUP * bs : K;
-    for (int64_t i1 = g0; i1 < gend; i1 += bs) {
-      const int count = (int)((gend - i1) < bs ? (gend - i1) : bs);
-      p.i1 = (int)i1;
-      p.count = count;
-      p.E = E + (i1 - g0);
-      hipLaunchKernelGGL(kern, dim3(wgs), dim3(256), smem, st, p);
-      LLMC_LAUNCH_STATUS();
-      const int64_t i2 = i1 + count;
-      if (i2 < gend) {
-        GemmF32 g = {};
-        g.A = p.E; g.lda = ldE; g.B = U + i1 * ldu + i2; g.ldb = ldu; g.C = Wf + i2; g.ldc = K;
-        g.M = (int)R; g.N = (int)(gend - i2); g.Kc = count; g.alpha = -1.f; g.beta = 1.f; g.batch = 1;
-        const int rc = llmc_gemm_f32(g, st);
-        if (rc) return rc;
-      }
-    }
-    if (gend < K) {
-      GemmF32 g = {};
-      g.A = E; g.lda = ldE; g.B = U + g0 * ldu + gend; g.ldb = ldu; g.C = Wf + gend; g.ldc = K;
-      g.M = (int)R; g.N = (int)(K - gend); g.Kc = (int)(gend - g0); g.alpha = -1.f; g.beta = 1.f; g.batch = 1;
-      const int rc = llmc_gemm_f32(g, st);
-      if (rc) return rc;
-    }
+  {
+    const int rc = gptq_column_loop(kern, p, smem, wgs, 1, R, K, bs, E, U, ldu, 0, Wf, st);
+    if (rc) return rc;
   }
 
 #define LLMC_FIN(DT)                                                                                                \
@@ -1112,35 +1131,9 @@ extern "C" int llmc_gptq_quantize_grouped(const void* const* weight, int32_t w_d
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
   if (e != hipSuccess) return 1000 + (int)e;
   const unsigned wgs = (unsigned)((R + Q_ROWS_PER_WG - 1) / Q_ROWS_PER_WG);
-  const int ldE = GROUP * GB;
-  p.ldE = ldE;
-  for (int64_t g0 = 0; g0 < K; g0 += (int64_t)GROUP * bs) {
-    const int64_t gend = (g0 + (int64_t)GROUP * bs) < K ? g0 + (int64_t)GROUP * bs : K;
-    for (int64_t i1 = g0; i1 < gend; i1 += bs) {
-      const int count = (int)((gend - i1) < bs ? (gend - i1) : bs);
-      p.i1 = (int)i1;
-      p.count = count;
-      p.E = E + (i1 - g0);
-      hipLaunchKernelGGL(kern, dim3(wgs, (unsigned)n), dim3(256), smem, st, p);
-      LLMC_LAUNCH_STATUS();
-      const int64_t i2 = i1 + count;
-      if (i2 < gend) {
-        GemmF32 g = {};
-        g.A = p.E; g.lda = ldE; g.B = U + i1 * ldu + i2; g.ldb = ldu; g.C = Wf + i2; g.ldc = K;
-        g.M = (int)R; g.N = (int)(gend - i2); g.Kc = count; g.alpha = -1.f; g.beta = 1.f;
-        g.batch = 1; g.batch2 = n; g.stride2_a = R * (int64_t)ldE; g.stride2_b = u_stride; g.stride2_c = R * K;
-        const int rc = llmc_gemm_f32(g, st);
-        if (rc) return rc;
-      }
-    }
-    if (gend < K) {
-      GemmF32 g = {};
-      g.A = E; g.lda = ldE; g.B = U + g0 * ldu + gend; g.ldb = ldu; g.C = Wf + gend; g.ldc = K;
-      g.M = (int)R; g.N = (int)(K - gend); g.Kc = (int)(gend - g0); g.alpha = -1.f; g.beta = 1.f;
-      g.batch = 1; g.batch2 = n; g.stride2_a = R * (int64_t)ldE; g.stride2_b = u_stride; g.stride2_c = R * K;
-      const int rc = llmc_gemm_f32(g, st);
-      if (rc) return rc;
-    }
+  {
+    const int rc = gptq_column_loop(kern, p, smem, wgs, n, R, K, bs, E, U, ldu, u_stride, Wf, st);
+    if (rc) return rc;
   }
 
 #define LLMC_FIN(DT)                                                                                            \
