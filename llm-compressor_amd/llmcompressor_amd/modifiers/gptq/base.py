@@ -254,7 +254,8 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
     def _begin_compress(self, module_list):
         """Flush what is pending, plan the jobs and enqueue the chains of the wide sets.  Returns
         (launched wide sets, remaining jobs) for ``_finish_compress``; no weight observer is read here."""
-        for module in module_list:  # followers get their own copy of the shared Hessian
+        followers = {}
+        for module in module_list:
             leader = self._leader.pop(module, None)
             if leader is not None:
                 if self._hook_calls.get(module) != self._hook_calls.get(leader):
@@ -262,22 +263,31 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
                                        f"called {self._hook_calls.get(module)} times, the module it shared with "
                                        f"{self._hook_calls.get(leader)} times; pass share_identical_inputs=False for "
                                        "this model")
-                self._flush(leader)
-                self._hessians[module] = self._hessians[leader].clone()
-                # the tally in the form the leader keeps it (host number for experts, device scalar otherwise),
-                # filled on the device: no host transfer or wait per follower
-                tally = self._num_samples[leader]
-                count = float(self._num_samples[module])
-                self._num_samples[module] = (torch.full_like(tally, count) if isinstance(tally, torch.Tensor)
-                                             else count)
+                followers[module] = leader
         self._recent_input = None
         for module in module_list:
             self._hook_calls.pop(module, None)
+        for leader in followers.values():
+            self._flush(leader)
         for module in module_list:  # pending activations go in on the calibration stream
             self._flush(module)
             self._staged.pop(module, None)
             self._held.pop(module, None)
+        for module, leader in followers.items():
+            # the leader's tensor itself for now, and the tally in the form the leader keeps it (host number for
+            # experts, device scalar otherwise), filled on the device: no host transfer or wait per follower
+            self._hessians[module] = self._hessians[leader]
+            tally = self._num_samples[leader]
+            count = float(self._num_samples[module])
+            self._num_samples[module] = torch.full_like(tally, count) if isinstance(tally, torch.Tensor) else count
         jobs = self._plan_jobs(list(module_list))
+        # A lock-step set leaves its Hessians untouched and factors a tensor it meets twice only once, so members of
+        # such sets keep sharing the leader's tensor.  The per-module path factors in place: a follower gets its own
+        # copy (made here, before any job starts) unless it and its leader both sit in lock-step sets.
+        in_sets = {m for job in jobs if isinstance(job, list) for m in job}
+        for module, leader in followers.items():
+            if not (module in in_sets and leader in in_sets):
+                self._hessians[module] = self._hessians[module].clone()
         # a set of many problems (the experts of an MoE layer) fills the chip by itself: such sets are enqueued one
         # after the other on the calling stream, with one host wait for all of them
         wide = [job for job in jobs if isinstance(job, list) and len(job) >= _WIDE_SET]

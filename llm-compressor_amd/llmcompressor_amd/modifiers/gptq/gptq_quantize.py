@@ -196,16 +196,34 @@ def begin_weight_group(modules, hessians, hessian_divisors, percdamp: float = 0.
     Hs = [hessians[i] for i in order]
     divs = [hessian_divisors[i] for i in order]
     keys = [keys[i] for i in order]
+    # Members that were given the very same Hessian tensor (Linears fed one input: q/k/v, gate/up) with the same
+    # divisor and the same ordering rule have the same column order and the same factor: the chain runs once per
+    # distinct Hessian and the members take copies of its results.
+    ordered = [bool(m.quantization_scheme.weights.actorder) for m in mods]
+    first_of, source = {}, []
+    for i, (H, d, o) in enumerate(zip(Hs, divs, ordered)):
+        source.append(first_of.setdefault((id(H), float(d), o), i))
+    distinct = sorted(set(source))
+    shared = len(distinct) < n
+    uH, udiv, uord = [Hs[i] for i in distinct], [divs[i] for i in distinct], [ordered[i] for i in distinct]
     # the column orders of all members in one sort (row-wise stable, so each row is what the per-module call sorts)
     all_perms = None
-    if all(m.quantization_scheme.weights.actorder for m in mods):
-        all_perms = torch.argsort(torch.stack([torch.diagonal(H) for H in Hs]), dim=1, descending=True, stable=True)
+    if all(uord):
+        all_perms = torch.argsort(torch.stack([torch.diagonal(H) for H in uH]), dim=1, descending=True, stable=True)
         perms = all_perms
     else:
-        single = [torch.argsort(torch.diagonal(H), descending=True, stable=True)
-                  if m.quantization_scheme.weights.actorder else None for m, H in zip(mods, Hs)]
+        single = [torch.argsort(torch.diagonal(H), descending=True, stable=True) if o else None
+                  for o, H in zip(uord, uH)]
         perms = torch.stack(single) if single[0] is not None else None
-    U, dead, info = llmc.gptq_prepare_hinv_grouped(Hs, perms, [float(d) for d in divs], float(percdamp))
+    U, dead, info = llmc.gptq_prepare_hinv_grouped(uH, perms, [float(d) for d in udiv], float(percdamp))
+    if shared:
+        slot = {i: j for j, i in enumerate(distinct)}
+        # through pinned memory, so that the host does not wait for the chain it has just enqueued
+        take = torch.tensor([slot[i] for i in source]).pin_memory().to(U.device, non_blocking=True)
+        U, dead, info = U[take], dead[take], info[take]
+        if perms is not None:
+            perms = perms[take]
+            all_perms = perms if all_perms is not None else None
     return dict(n=n, order=order, mods=mods, keys=keys, perms=perms, all_perms=all_perms, U=U, dead=dead, info=info)
 
 

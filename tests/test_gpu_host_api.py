@@ -1075,8 +1075,8 @@ def test_dynamic_group_and_tensor_activations_match_oracle(spec):
 @pytest.mark.parametrize("actorder", [None, "weight"])
 def test_gptq_same_width_linears_in_lock_step_match_per_module_path(actorder):
     """q/k/v/o/gate/up-like Linears (one width, different heights) plus one of another width: the same-width
-    ones share a lock-step Cholesky chain, equal shapes share a column loop; parameters are bit-identical to the
-    per-module path, with and without concurrency."""
+    ones share a lock-step Cholesky chain (one factorisation per distinct Hessian), equal shapes share a column
+    loop; parameters are bit-identical to the per-module path, with and without concurrency."""
     from llmcompressor_amd import ops
     from llmcompressor_amd.core import LifecycleCallbacks, active_session
     from llmcompressor_amd.modifiers.gptq import GPTQModifier
@@ -1125,7 +1125,9 @@ def test_gptq_same_width_linears_in_lock_step_match_per_module_path(actorder):
             ops.gptq_hinv_grouped = raw
         torch.cuda.synchronize()
         results.append((sizes, {n: p.detach().clone() for n, p in model.named_parameters()}))
-    assert results[0][0] == [] and results[1][0] == [6] and results[2][0] == [6]
+    # six Linears in the lock-step set, three distinct Hessians (q/k/v and gate/up are fed one tensor each and share
+    # theirs): the chain factors each distinct Hessian once
+    assert results[0][0] == [] and results[1][0] == [3] and results[2][0] == [3]
     for sizes, params in results[1:]:
         assert params.keys() == results[0][1].keys()
         for n in params:
