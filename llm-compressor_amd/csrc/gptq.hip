@@ -462,6 +462,75 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(GptqBlockParams p) {
   }
 }
 
+// The product inside a group of column blocks, W[:, c0:c1] -= E_b * U[i1:i1+128, c0:c1] with at most 384 columns:
+// 15 MB of traffic for a 4096-row weight, a few microseconds of matrix-core time -- a general tiled product
+// spends most of its 19 us ramping its pipeline up and down.  Here a workgroup owns 16 rows and all columns: each
+// wave takes every fourth 16-column tile, holds the 16 x 128 slice of E (negated) in registers for all its tiles,
+// fetches a tile's 128 x 16 slice of U straight from global memory (every workgroup reads the same 128 x 384
+// block, which stays in the L2) one tile ahead, and runs 32 v_mfma_f32_16x16x4_f32 per tile with the tile of W
+// as the accumulator's start value.  Lane group q = lane / 16 contributes the inner indices 32 q .. 32 q + 31, one
+// per instruction, so a lane's E values are eight consecutive float4.  Sums are fp32 fused multiply-adds of
+// exact products, as in the fp32 matrix kernel.
+struct GroupUpdate {
+  const float* E;   // [R, ldE]: the block's scaled errors (128 columns)
+  int64_t ldE;
+  const float* U;   // first row of the block's 128 rows of the factor, at column c0
+  int64_t ldu;
+  float* W;         // [R, K] work copy, at column c0
+  int64_t ldw;
+  int R, ntiles;    // ntiles = (c1 - c0) / 16
+  int64_t stride_e, stride_u, stride_w;  // per problem (blockIdx.y)
+};
+
+__global__ __launch_bounds__(256) void gptq_group_update_kernel(GroupUpdate g) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int c = lane & 15, q = lane >> 4;
+  const float* E = g.E + (int64_t)blockIdx.y * g.stride_e;
+  const float* U = g.U + (int64_t)blockIdx.y * g.stride_u;
+  float* W = g.W + (int64_t)blockIdx.y * g.stride_w;
+  const int row0 = blockIdx.x * 16;
+  const int ra = row0 + c < g.R ? row0 + c : g.R - 1;  // A operand: row c of the 16, inner indices 32 q + j
+  float a[32];
+  {
+    const float4* src = (const float4*)(E + (int64_t)ra * g.ldE + 32 * q);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float4 v = src[j];
+      a[4 * j] = -v.x; a[4 * j + 1] = -v.y; a[4 * j + 2] = -v.z; a[4 * j + 3] = -v.w;
+    }
+  }
+  auto fetch_b = [&](float* b, int tile) {  // B operand: column c of the tile, inner indices 32 q + j
+    const float* src = U + (int64_t)(32 * q) * g.ldu + tile * 16 + c;
+#pragma unroll
+    for (int j = 0; j < 32; ++j) b[j] = src[(int64_t)j * g.ldu];
+  };
+  float b0[32], b1[32];
+  int tile = wave;
+  if (tile < g.ntiles) fetch_b(b0, tile);
+  // accumulator element i of a lane: row 4 q + i, column c
+  auto run = [&](const float* b, int t) {
+    float* dst = W + (int64_t)(row0 + 4 * q) * g.ldw + t * 16 + c;
+    f32x4_t acc;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] = row0 + 4 * q + i < g.R ? dst[(int64_t)i * g.ldw] : 0.f;
+#pragma unroll
+    for (int j = 0; j < 32; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[j], b[j], acc, 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (row0 + 4 * q + i < g.R) dst[(int64_t)i * g.ldw] = acc[i];
+  };
+  while (tile < g.ntiles) {
+    if (tile + 4 < g.ntiles) fetch_b(b1, tile + 4);
+    run(b0, tile);
+    tile += 4;
+    if (tile >= g.ntiles) break;
+    if (tile + 4 < g.ntiles) fetch_b(b0, tile + 4);
+    run(b1, tile);
+    tile += 4;
+  }
+}
+
+
 template <int WDT>
 __global__ __launch_bounds__(256) void gptq_finalize_kernel(const float* __restrict__ Wf, int R, int K,
                                                             const int32_t* __restrict__ perm,
@@ -905,8 +974,18 @@ static int gptq_column_loop(void (*kern)(GptqBlockParams), GptqBlockParams p, in
       LLMC_LAUNCH_STATUS();
       const int64_t i2 = i1 + count;
       if (i2 < gend) {
-        const int rc = product(p.E, i1, count, i2, gend);
-        if (rc) return rc;
+        if (count == GB && (gend - i2) % 16 == 0 && (ldE & 3) == 0 && K < (1 << 30)) {
+          GroupUpdate gu;
+          gu.E = p.E; gu.ldE = ldE; gu.U = U + i1 * ldu + i2; gu.ldu = ldu; gu.W = Wf + i2; gu.ldw = K;
+          gu.R = (int)R; gu.ntiles = (int)((gend - i2) / 16);
+          gu.stride_e = R * (int64_t)ldE; gu.stride_u = u_stride; gu.stride_w = R * K;
+          hipLaunchKernelGGL(gptq_group_update_kernel, dim3((unsigned)((R + 15) / 16), (unsigned)n), dim3(256), 0, st,
+                             gu);
+          LLMC_LAUNCH_STATUS();
+        } else {
+          const int rc = product(p.E, i1, count, i2, gend);
+          if (rc) return rc;
+        }
       }
     }
     if (gend < K) {
