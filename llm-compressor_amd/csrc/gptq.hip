@@ -815,6 +815,21 @@ __global__ __launch_bounds__(256) void zero_u32_words_kernel(unsigned* p, int64_
 
 }  // namespace
 
+// enqueue gptq_group_update_kernel when the shapes fit it (a full 128-column block, a multiple of 16 columns to
+// update); returns -1 when the product is left to the general kernels
+static int launch_group_update(const float* Eb, int64_t ldE, const float* U, int64_t ldu, int64_t u_stride, float* Wf,
+                               int64_t R, int64_t K, int n, int64_t i1, int count, int64_t c0, int64_t c1,
+                               hipStream_t st) {
+  if (count != GB || (c1 - c0) % 16 != 0 || (ldE & 3) != 0 || K >= (1 << 30)) return -1;
+  GroupUpdate gu;
+  gu.E = Eb; gu.ldE = ldE; gu.U = U + i1 * ldu + c0; gu.ldu = ldu; gu.W = Wf + c0; gu.ldw = K;
+  gu.R = (int)R; gu.ntiles = (int)((c1 - c0) / 16);
+  gu.stride_e = R * ldE; gu.stride_u = u_stride; gu.stride_w = R * K;
+  hipLaunchKernelGGL(gptq_group_update_kernel, dim3((unsigned)((R + 15) / 16), (unsigned)n), dim3(256), 0, st, gu);
+  LLMC_LAUNCH_STATUS();
+  return 0;
+}
+
 extern "C" int64_t llmc_sparsegpt_workspace_bytes(int64_t R, int64_t K) {
   const int64_t slices = (K + SG_MIN_BLOCK - 1) / SG_MIN_BLOCK;
   return align256(R * K * 4) + align256(R * GROUP * GB * 4) + align256(R * 4) +
@@ -910,10 +925,13 @@ extern "C" int llmc_sparsegpt_sparsify(const void* weight, int32_t w_dtype, int6
       LLMC_LAUNCH_STATUS();
       const int64_t i2 = i1 + count;
       if (i2 < gend) {
-        GemmF32 g = {};
-        g.A = p.E; g.lda = ldE; g.B = U + i1 * ldu + i2; g.ldb = ldu; g.C = Wf + i2; g.ldc = K;
-        g.M = (int)R; g.N = (int)(gend - i2); g.Kc = count; g.alpha = -1.f; g.beta = 1.f; g.batch = 1;
-        const int rc = llmc_gemm_f32(g, st);
+        int rc = launch_group_update(p.E, ldE, U, ldu, 0, Wf, R, K, 1, i1, count, i2, gend, st);
+        if (rc < 0) {
+          GemmF32 g = {};
+          g.A = p.E; g.lda = ldE; g.B = U + i1 * ldu + i2; g.ldb = ldu; g.C = Wf + i2; g.ldc = K;
+          g.M = (int)R; g.N = (int)(gend - i2); g.Kc = count; g.alpha = -1.f; g.beta = 1.f; g.batch = 1;
+          rc = llmc_gemm_f32(g, st);
+        }
         if (rc) return rc;
         rezero(i2, gend);
         LLMC_LAUNCH_STATUS();
@@ -974,18 +992,9 @@ static int gptq_column_loop(void (*kern)(GptqBlockParams), GptqBlockParams p, in
       LLMC_LAUNCH_STATUS();
       const int64_t i2 = i1 + count;
       if (i2 < gend) {
-        if (count == GB && (gend - i2) % 16 == 0 && (ldE & 3) == 0 && K < (1 << 30)) {
-          GroupUpdate gu;
-          gu.E = p.E; gu.ldE = ldE; gu.U = U + i1 * ldu + i2; gu.ldu = ldu; gu.W = Wf + i2; gu.ldw = K;
-          gu.R = (int)R; gu.ntiles = (int)((gend - i2) / 16);
-          gu.stride_e = R * (int64_t)ldE; gu.stride_u = u_stride; gu.stride_w = R * K;
-          hipLaunchKernelGGL(gptq_group_update_kernel, dim3((unsigned)((R + 15) / 16), (unsigned)n), dim3(256), 0, st,
-                             gu);
-          LLMC_LAUNCH_STATUS();
-        } else {
-          const int rc = product(p.E, i1, count, i2, gend);
-          if (rc) return rc;
-        }
+        int rc = launch_group_update(p.E, ldE, U, ldu, u_stride, Wf, R, K, n, i1, count, i2, gend, st);
+        if (rc < 0) rc = product(p.E, i1, count, i2, gend);
+        if (rc) return rc;
       }
     }
     if (gend < K) {
