@@ -70,10 +70,13 @@ def _scale_layout(strategy, quant_args: QuantizationArgs, num_rows: int, num_col
 
 
 def quantize_weight_tensors(weight: torch.Tensor, observer, quant_args: QuantizationArgs, hessian: torch.Tensor,
-                            blocksize: int = 128, percdamp: float = 0.01, hessian_divisor: float = 1.0):
+                            blocksize: int = 128, percdamp: float = 0.01, hessian_divisor: float = 1.0,
+                            before_loop=None):
     """quantize_weight on bare tensors: ``weight`` [R,K], ``observer`` holding its statistics.
 
-    ``hessian_divisor`` folds the caller's ``H / num_samples`` into the factorisation's first pass."""
+    ``hessian_divisor`` folds the caller's ``H / num_samples`` into the factorisation's first pass.
+    ``before_loop`` (a callable or None) is called once the factorisation has been enqueued and before the
+    observer is read: a caller that starts this function while the observers still run passes its wait here."""
     strategy = quant_args.strategy
     actorder = quant_args.actorder
     final_shape, final_dtype = weight.shape, weight.dtype
@@ -89,6 +92,9 @@ def quantize_weight_tensors(weight: torch.Tensor, observer, quant_args: Quantiza
                        "falling back to actorder=None for this module.")
         actorder = None
 
+    if actorder == ActivationOrdering.GROUP and before_loop is not None:
+        before_loop()  # this ordering re-observes the weight below: not while the caller's observers still run
+        before_loop = None
     perm = None
     if actorder:
         # stable: equal diagonal entries keep their column order, so that the column order (and with it the
@@ -108,12 +114,14 @@ def quantize_weight_tensors(weight: torch.Tensor, observer, quant_args: Quantiza
         if actorder == ActivationOrdering.WEIGHT:
             g_idx = g_idx[perm]
 
-    qparams = observer.get_qparams()
-    scale, zero_point, global_scale = qparams["scale"], qparams["zero_point"], qparams["global_scale"]
-
     # dead columns, damping, Cholesky -> inverse -> upper factor; identity on failure
     dead, info = llmc.gptq_prepare_hinv_(H, perm, float(hessian_divisor), float(percdamp))
     U = H  # overwritten in place by the upper factor
+
+    if before_loop is not None:
+        before_loop()
+    qparams = observer.get_qparams()
+    scale, zero_point, global_scale = qparams["scale"], qparams["zero_point"], qparams["global_scale"]
 
     fmt, bits = kernel_format(quant_args)
     zp = None if quant_args.symmetric else zero_point.to(torch.int8)
@@ -141,7 +149,8 @@ def quantize_weight_tensors(weight: torch.Tensor, observer, quant_args: Quantiza
 
 
 def quantize_weight(module: torch.nn.Module, quant_args: QuantizationArgs, hessian: torch.Tensor,
-                    blocksize: int = 128, percdamp: float = 0.01, hessian_divisor: float = 1.0) -> tuple[float, dict]:
+                    blocksize: int = 128, percdamp: float = 0.01, hessian_divisor: float = 1.0,
+                    before_loop=None) -> tuple[float, dict]:
     """Quantize a module weight according to the GPTQ algorithm.
 
     :param module: module with weight being quantized (must carry ``weight_observer`` with statistics)
@@ -152,7 +161,7 @@ def quantize_weight(module: torch.nn.Module, quant_args: QuantizationArgs, hessi
     :return: loss, dict of weight / weight_scale / weight_zero_point [/ weight_global_scale / weight_g_idx]
     """
     return quantize_weight_tensors(module.weight.data, module.weight_observer, quant_args, hessian, blocksize,
-                                   percdamp, hessian_divisor)
+                                   percdamp, hessian_divisor, before_loop)
 
 
 def group_key(module: torch.nn.Module, quant_args: QuantizationArgs, hessian: torch.Tensor):

@@ -15,7 +15,7 @@ from pydantic import PrivateAttr
 from ....core import State
 from ....quantization import update_offload_parameter
 from ....utils.metric_logging import CompressionLogger
-from ...utils.concurrent import run_on_streams
+from ...utils.concurrent import SIDE_STREAMS, run_on_streams
 from ...utils.hessian_staging import HessianStagingMixin
 from .sgpt_base import SparsityModifierBase
 from .sgpt_sparsify import accumulate_hessian, make_empty_hessian, sparsify_weight
@@ -52,7 +52,7 @@ class SparseGPTModifier(SparsityModifierBase, HessianStagingMixin):
     _staged: dict = PrivateAttr(default_factory=dict)
     _held: dict = PrivateAttr(default_factory=dict)
     _held_bytes: int = PrivateAttr(default=0)
-    _streams: dict = PrivateAttr(default_factory=dict)
+    _streams: dict = PrivateAttr(default_factory=lambda: SIDE_STREAMS)
 
     def calibrate_module(self, module: torch.nn.Module, args: tuple[torch.Tensor, ...], _output: torch.Tensor):
         """Forward hook: accumulate the Hessian of the module's input."""
