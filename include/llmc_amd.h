@@ -257,6 +257,13 @@ int llmc_gptq_hinv(float* H, int64_t ldh, int64_t K, const int32_t* perm, float 
                    float percdamp, uint8_t* dead_out, void* workspace, int64_t workspace_bytes,
                    int32_t* info_out, void* stream);
 
+/* Column order of GPTQ's activation ordering (gptq_quantize.py:131-140: argsort of diag(H), descending): for each of
+ * the n Hessians (HOST array of n device pointers, fp32 [K, K], row stride ldh) the column numbers ordered by
+ * descending diagonal entry, equal entries in ascending column order (the result of a stable sort; the reference's
+ * unstable torch.argsort leaves the order of exact ties unspecified), NaN before every number.  out: device int64
+ * [n, K].  K <= 16384. */
+int llmc_diag_argsort_desc(const float* const* H, int64_t ldh, int32_t n, int64_t K, int64_t* out, void* stream);
+
 /* Grouped form for many small problems of one width (the experts of an MoE layer): the chain of
  * llmc_gptq_hinv run once for all n problems in lock-step, every kernel carrying one more batch
  * dimension.  H (and perm, or NULL) are HOST arrays of n device pointers, divisors a HOST array of n

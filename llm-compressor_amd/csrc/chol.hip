@@ -430,6 +430,82 @@ inline int chol_factor(float* A, int Kp, int K, HinvScalars* sc, float* Xs, int6
 
 }  // namespace
 
+namespace {
+// ---- activation order: argsort of the Hessian's diagonal, descending, equal entries in index order -------------
+// (gptq_quantize.py:131-140 sorts diag(H) with torch.argsort; a stable sort is what keeps equal entries in column
+// order.)  One workgroup per Hessian: the diagonal and the column numbers sit in LDS, padded to a power of two
+// with entries that sort last, and a bitonic network orders them by (value descending, index ascending) -- a total
+// order, so the network's result is the stable sort's.  NaN sorts before every number, as in torch.
+constexpr int ORDER_MAX_K = 16384;
+constexpr int ORDER_MAX_PROBLEMS = 256;
+struct OrderArgs {
+  const float* H[ORDER_MAX_PROBLEMS];
+};
+
+__device__ __forceinline__ bool order_before(float ka, int ia, float kb, int ib) {
+  const bool na = ka != ka, nb = kb != kb;
+  if (na != nb) return na;
+  if (!na && ka != kb) return ka > kb;
+  return ia < ib;
+}
+
+__global__ __launch_bounds__(1024) void diag_order_kernel(OrderArgs args, int64_t ldh, int K, int N,
+                                                          int64_t* __restrict__ out) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char order_smem[];
+  float* key = (float*)order_smem;
+  int* idx = (int*)(order_smem + (size_t)N * 4);
+  const float* H = args.H[blockIdx.x];
+  const int tid = threadIdx.x;
+  for (int i = tid; i < N; i += 1024) {
+    key[i] = i < K ? H[(int64_t)i * ldh + i] : -__builtin_inff();
+    idx[i] = i < K ? i : 0x7fffffff;
+  }
+  __syncthreads();
+  for (int k = 2; k <= N; k <<= 1) {
+    for (int j = k >> 1; j > 0; j >>= 1) {
+      for (int t = tid; t < N / 2; t += 1024) {
+        const int i = ((t & ~(j - 1)) << 1) | (t & (j - 1));  // the element of the pair with bit j clear
+        const int p = i | j;
+        const bool up = (i & k) == 0;  // this run ends up in order (first element first)
+        const float ka = key[i], kb = key[p];
+        const int ia = idx[i], ib = idx[p];
+        const bool in_order = order_before(ka, ia, kb, ib);
+        if (in_order != up) {
+          key[i] = kb; key[p] = ka;
+          idx[i] = ib; idx[p] = ia;
+        }
+      }
+      __syncthreads();
+    }
+  }
+  for (int i = tid; i < K; i += 1024) out[(int64_t)blockIdx.x * K + i] = idx[i];
+}
+}  // namespace
+
+extern "C" int llmc_diag_argsort_desc(const float* const* H, int64_t ldh, int32_t n, int64_t K, int64_t* out,
+                                      void* stream) {
+  LLMC_CHECK_ARG(H != nullptr && out != nullptr, 1);
+  LLMC_CHECK_ARG(n >= 0 && K > 0 && K <= ORDER_MAX_K && ldh >= K, 3);
+  int N = 2;
+  while (N < K) N <<= 1;
+  const size_t smem = (size_t)N * 8;
+  static const hipError_t configured = hipFuncSetAttribute(
+      (const void*)diag_order_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, ORDER_MAX_K * 8);
+  if (configured != hipSuccess) return 1000 + (int)configured;
+  for (int first = 0; first < n; first += ORDER_MAX_PROBLEMS) {
+    const int m = n - first < ORDER_MAX_PROBLEMS ? n - first : ORDER_MAX_PROBLEMS;
+    OrderArgs args;
+    for (int b = 0; b < m; ++b) {
+      LLMC_CHECK_ARG(H[first + b] != nullptr, 1);
+      args.H[b] = H[first + b];
+    }
+    hipLaunchKernelGGL(diag_order_kernel, dim3((unsigned)m), dim3(1024), smem, (hipStream_t)stream, args, ldh, (int)K,
+                       N, out + (int64_t)first * K);
+    LLMC_LAUNCH_STATUS();
+  }
+  return 0;
+}
+
 extern "C" int64_t llmc_gptq_hinv_workspace_bytes(int64_t K) {
   const int64_t Kp = round_up(K, NB);
   // work matrix + temporary (recursive doubling, side array of the diagonal inverses) + scalars

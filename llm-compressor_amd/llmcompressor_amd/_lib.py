@@ -99,6 +99,7 @@ SIGNATURES.update({
     "llmc_mse_observe_blocks": [_P, _I32, _I64, _I64, _I64, _I32, _I32, _I32, _I32, _I32, _I32, _I32, _F64, _I32,
                                 _F32, _F32, _P, _P, _P, _I64, _P],
 })
+SIGNATURES["llmc_diag_argsort_desc"] = [_P, _I64, _I32, _I64, _P, _P]
 SIGNATURES["llmc_grouped_linear"] = [_P, _I32, _I64, _P, _I64, _I32, _I32, _P, _I64, _P, _I32, _I64, _I64, _P]
 # functions whose return type is not int
 RESTYPES = {

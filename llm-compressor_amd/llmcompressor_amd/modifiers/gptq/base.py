@@ -9,7 +9,6 @@ from __future__ import annotations
 
 import contextlib
 import logging
-import threading
 
 import torch
 from pydantic import PrivateAttr
@@ -33,7 +32,7 @@ from ...utils.metric_logging import CompressionLogger
 from ..modifier import Modifier
 from ..quantization.calibration import observe, update_qparams
 from ..quantization.quantization import QuantizationMixin
-from ..utils.concurrent import SIDE_STREAMS, start_on_streams
+from ..utils.concurrent import SIDE_STREAMS, run_on_streams
 from ..utils.hessian_staging import HessianStagingMixin
 from .gptq_quantize import (accumulate_hessian, begin_weight_group, finish_weight_group, make_empty_hessian,
                             quantize_weight, quantize_weight_group,
@@ -47,12 +46,6 @@ _GPTQ_Q_PARAMS = ["weight", "weight_scale", "weight_zero_point", "weight_g_idx"]
 
 
 _WIDE_SET = 16  # problems per lock-step set from which the set runs alone on the calling stream
-
-
-def _set_flag() -> threading.Event:
-    flag = threading.Event()
-    flag.set()
-    return flag
 
 
 class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
@@ -119,9 +112,6 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
     _recent_input: tuple | None = PrivateAttr(default=None)  # (tensor kept alive, its version, leader)
     _hook_calls: dict = PrivateAttr(default_factory=dict)  # module -> hook calls so far (leaders and followers)
     _streams: dict = PrivateAttr(default_factory=lambda: SIDE_STREAMS)
-    # jobs started before the weight observers ran wait here before they read the observers' statistics;
-    # (flag, event recorded on the observers' stream after their kernels, or None)
-    _observed: list = PrivateAttr(default_factory=lambda: [_set_flag(), None])
 
     def resolve_quantization_config(self) -> QuantizationConfig:
         config = super().resolve_quantization_config()
@@ -181,20 +171,10 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
         modules = [m for m in modules if is_module_quantized(m)]
         # The Cholesky chains of wide lock-step sets (the experts of an MoE layer) need the Hessians only: they
         # are enqueued first, and the weights are observed on the host while they run.
-        # The other jobs start now as well, on their side streams: a job's chain needs its Hessians only, and it
-        # waits (``_wait_observed``) before it reads a weight observer.
-        flag = self._observed[0]
-        flag.clear()
-        self._observed[1] = None
-        try:
-            started = self._start_jobs(self._begin_compress(list(self._num_samples.keys())))
-            observe(modules, base_name="weight")
-            self.sync_obs_act_stats(modules)
-            update_qparams(modules, ACTIVATION_OBS)
-            if torch.cuda.is_available() and any(m.weight.is_cuda for m in modules if hasattr(m, "weight")):
-                self._observed[1] = torch.cuda.current_stream().record_event()
-        finally:
-            flag.set()  # also when observing failed: no worker stays blocked
+        started = self._begin_compress(list(self._num_samples.keys()))
+        observe(modules, base_name="weight")
+        self.sync_obs_act_stats(modules)
+        update_qparams(modules, ACTIVATION_OBS)
         self._finish_compress(started)
 
     def on_calibration_end(self, state: State, event: Event, **kwargs):
@@ -314,49 +294,29 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
         jobs = [job for job in jobs if not (isinstance(job, list) and len(job) >= _WIDE_SET)]
         return [self._begin_set(part) for part in wide], jobs
 
-    def _wait_observed(self):
-        """Called by a job between its chain and its column loop: until the weight observers hold their statistics,
-        and its stream behind the kernels that produced them."""
-        flag, event = self._observed
-        flag.wait()
-        event = self._observed[1]
-        if event is not None:
-            torch.cuda.current_stream().wait_event(event)
-
-    def _start_jobs(self, started):
-        """Start the jobs that can run side by side (one host thread and one HIP stream each, most expensive first
-        so that the widest module does not start last; see modifiers/utils/concurrent.py).  Returns
-        (launched wide sets, jobs left for the calling thread, running jobs or None)."""
+    def _finish_compress(self, started):
         begun, jobs = started
+        if begun:
+            self._finish_sets([self._end_set(b) for b in begun])
         if not jobs:
-            return begun, jobs, None
+            return
         members = [m for job in jobs for m in (job if isinstance(job, list) else [job])]
         workers = min(int(self.compress_concurrency), len(jobs))
         on_gpu = (all(m.weight.is_cuda and self._hessians[m].is_cuda for m in members)
                   and len({m.weight.device for m in members}) == 1)  # one device per call
         if workers <= 1 or not on_gpu or self.offload_hessians:
-            return begun, jobs, None
+            for job in jobs:
+                self._compress_job(job)
+            return
+        # several jobs at once, one host thread and one HIP stream each, most expensive first so that the
+        # widest module does not start last (see modifiers/utils/concurrent.py); results are unchanged
 
         def cost(job):
             return sum(float(m.weight.shape[1]) ** 3 + float(m.weight.shape[0]) * m.weight.shape[1] ** 2
                        for m in (job if isinstance(job, list) else [job]))
 
-        jobs = sorted(jobs, key=lambda job: -cost(job))
-        running = start_on_streams(jobs, self._compress_job, workers, members[0].weight.device, self._streams)
-        return begun, [], running
-
-    def _finish_compress(self, started):
-        if len(started) == 2:  # from ``_begin_compress`` directly: nothing runs yet
-            started = self._start_jobs(started)
-        begun, jobs, running = started
-        try:
-            if begun:
-                self._finish_sets([self._end_set(b) for b in begun])
-        finally:
-            if running is not None:
-                running.join()  # results are unchanged by the side streams
-        for job in jobs:
-            self._compress_job(job)
+        jobs.sort(key=lambda job: -cost(job))
+        run_on_streams(jobs, self._compress_job, workers, members[0].weight.device, self._streams)
 
     def _plan_jobs(self, modules):
         """Split the modules of one call into jobs: a list = Linears of one width that share a lock-step
@@ -390,9 +350,7 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
 
     def _compress_set(self, part, produced_on=None, consumed_on=None):
         """Linears of one width in lock-step (``quantize_weight_group``); parameters as on the per-module path."""
-        begun = self._begin_set(part, produced_on)
-        self._wait_observed()
-        self._finish_sets([self._end_set(begun)], consumed_on)
+        self._finish_sets([self._end_set(self._begin_set(part, produced_on))], consumed_on)
 
     def _begin_set(self, part, produced_on=None):
         hs = [self._hessians.pop(m) for m in part]
@@ -447,7 +405,6 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
                 blocksize=self.block_size,
                 percdamp=self.dampening_frac,
                 hessian_divisor=float(num_samples),
-                before_loop=self._wait_observed,
             )
             comp_logger.set_results(name="GPTQ", loss=loss)
         for attr, val in q_param_dict.items():

@@ -54,6 +54,17 @@ def accumulate_hessian(inp: torch.Tensor, module: torch.nn.Module, H: torch.Tens
     return H, num_samples
 
 
+def _diag_order(Hs) -> torch.Tensor:
+    """[n, K] column orders of the activation ordering: ``argsort(diag H, descending, stable)`` per Hessian (stable:
+    equal diagonal entries keep their column order, so the order and with it the result is reproducible; torch
+    leaves the order of ties unspecified otherwise).  One launch for Hessians the kernel takes, torch otherwise."""
+    H0 = Hs[0]
+    if (H0.is_cuda and H0.shape[0] <= ops.DIAG_ORDER_MAX_K
+            and all(H.dtype == torch.float32 and H.stride(1) == 1 and H.stride(0) == H0.stride(0) for H in Hs)):
+        return ops.diag_argsort_desc(Hs)
+    return torch.argsort(torch.stack([torch.diagonal(H) for H in Hs]), dim=1, descending=True, stable=True)
+
+
 def _scale_layout(strategy, quant_args: QuantizationArgs, num_rows: int, num_columns: int):
     """(row_div, scale_row_stride, base g_idx or None) of llmc_gptq_quantize."""
     S = QuantizationStrategy
@@ -70,13 +81,10 @@ def _scale_layout(strategy, quant_args: QuantizationArgs, num_rows: int, num_col
 
 
 def quantize_weight_tensors(weight: torch.Tensor, observer, quant_args: QuantizationArgs, hessian: torch.Tensor,
-                            blocksize: int = 128, percdamp: float = 0.01, hessian_divisor: float = 1.0,
-                            before_loop=None):
+                            blocksize: int = 128, percdamp: float = 0.01, hessian_divisor: float = 1.0):
     """quantize_weight on bare tensors: ``weight`` [R,K], ``observer`` holding its statistics.
 
-    ``hessian_divisor`` folds the caller's ``H / num_samples`` into the factorisation's first pass.
-    ``before_loop`` (a callable or None) is called once the factorisation has been enqueued and before the
-    observer is read: a caller that starts this function while the observers still run passes its wait here."""
+    ``hessian_divisor`` folds the caller's ``H / num_samples`` into the factorisation's first pass."""
     strategy = quant_args.strategy
     actorder = quant_args.actorder
     final_shape, final_dtype = weight.shape, weight.dtype
@@ -92,14 +100,11 @@ def quantize_weight_tensors(weight: torch.Tensor, observer, quant_args: Quantiza
                        "falling back to actorder=None for this module.")
         actorder = None
 
-    if actorder == ActivationOrdering.GROUP and before_loop is not None:
-        before_loop()  # this ordering re-observes the weight below: not while the caller's observers still run
-        before_loop = None
     perm = None
     if actorder:
         # stable: equal diagonal entries keep their column order, so that the column order (and with it the
         # result) is reproducible; torch leaves the order of ties unspecified otherwise
-        perm = torch.argsort(torch.diagonal(H), descending=True, stable=True)
+        perm = _diag_order([H])[0]
     if actorder == ActivationOrdering.GROUP:
         # re-observe the permuted weight so that groups are runs of the permuted columns.  The reference observes
         # its fp32 work copy here (gptq_quantize.py:88,111-114), so these statistics and the scales the column
@@ -114,14 +119,12 @@ def quantize_weight_tensors(weight: torch.Tensor, observer, quant_args: Quantiza
         if actorder == ActivationOrdering.WEIGHT:
             g_idx = g_idx[perm]
 
+    qparams = observer.get_qparams()
+    scale, zero_point, global_scale = qparams["scale"], qparams["zero_point"], qparams["global_scale"]
+
     # dead columns, damping, Cholesky -> inverse -> upper factor; identity on failure
     dead, info = llmc.gptq_prepare_hinv_(H, perm, float(hessian_divisor), float(percdamp))
     U = H  # overwritten in place by the upper factor
-
-    if before_loop is not None:
-        before_loop()
-    qparams = observer.get_qparams()
-    scale, zero_point, global_scale = qparams["scale"], qparams["zero_point"], qparams["global_scale"]
 
     fmt, bits = kernel_format(quant_args)
     zp = None if quant_args.symmetric else zero_point.to(torch.int8)
@@ -149,8 +152,7 @@ def quantize_weight_tensors(weight: torch.Tensor, observer, quant_args: Quantiza
 
 
 def quantize_weight(module: torch.nn.Module, quant_args: QuantizationArgs, hessian: torch.Tensor,
-                    blocksize: int = 128, percdamp: float = 0.01, hessian_divisor: float = 1.0,
-                    before_loop=None) -> tuple[float, dict]:
+                    blocksize: int = 128, percdamp: float = 0.01, hessian_divisor: float = 1.0) -> tuple[float, dict]:
     """Quantize a module weight according to the GPTQ algorithm.
 
     :param module: module with weight being quantized (must carry ``weight_observer`` with statistics)
@@ -161,7 +163,7 @@ def quantize_weight(module: torch.nn.Module, quant_args: QuantizationArgs, hessi
     :return: loss, dict of weight / weight_scale / weight_zero_point [/ weight_global_scale / weight_g_idx]
     """
     return quantize_weight_tensors(module.weight.data, module.weight_observer, quant_args, hessian, blocksize,
-                                   percdamp, hessian_divisor, before_loop)
+                                   percdamp, hessian_divisor)
 
 
 def group_key(module: torch.nn.Module, quant_args: QuantizationArgs, hessian: torch.Tensor):
@@ -218,11 +220,10 @@ def begin_weight_group(modules, hessians, hessian_divisors, percdamp: float = 0.
     # the column orders of all members in one sort (row-wise stable, so each row is what the per-module call sorts)
     all_perms = None
     if all(uord):
-        all_perms = torch.argsort(torch.stack([torch.diagonal(H) for H in uH]), dim=1, descending=True, stable=True)
+        all_perms = _diag_order(uH)
         perms = all_perms
     else:
-        single = [torch.argsort(torch.diagonal(H), descending=True, stable=True) if o else None
-                  for o, H in zip(uord, uH)]
+        single = [_diag_order([H])[0] if o else None for o, H in zip(uord, uH)]
         perms = torch.stack(single) if single[0] is not None else None
     U, dead, info = llmc.gptq_prepare_hinv_grouped(uH, perms, [float(d) for d in udiv], float(percdamp))
     if shared:

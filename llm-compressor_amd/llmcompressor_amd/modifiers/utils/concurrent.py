@@ -13,34 +13,17 @@ from typing import Callable, Dict, List
 
 import torch
 
-__all__ = ["run_on_streams", "start_on_streams", "SIDE_STREAMS"]
+__all__ = ["run_on_streams", "SIDE_STREAMS"]
 
 # the side streams of every device, shared by all modifiers of the process: creating a stream and giving it its
 # first submission costs about 0.4 ms, and one modifier after the other uses them, never two at a time
 SIDE_STREAMS: Dict[torch.device, list] = {}
 
 
-class _Running:
-    """Jobs started by ``start_on_streams``; ``join`` waits for them, makes the caller's stream wait for the side
-    streams and re-raises the first exception of a worker."""
-
-    def __init__(self, threads, streams, main, errors):
-        self._threads, self._streams, self._main, self._errors = threads, streams, main, errors
-
-    def join(self) -> None:
-        for t in self._threads:
-            t.join()
-        for s in self._streams:
-            self._main.wait_stream(s)
-        if self._errors:
-            raise self._errors[0]
-
-
-def start_on_streams(jobs: List, work: Callable, workers: int, device: torch.device,
-                     stream_cache: Dict[torch.device, list]) -> _Running:
-    """Start ``work(job, produced_on=side_stream, consumed_on=caller_stream)`` for every job, in list order, at
-    most ``workers`` at a time, and return at once; ``join()`` on the result ends the run.  The first exception
-    stops the remaining jobs and is re-raised by ``join``."""
+def run_on_streams(jobs: List, work: Callable, workers: int, device: torch.device,
+                   stream_cache: Dict[torch.device, list]) -> None:
+    """``work(job, produced_on=side_stream, consumed_on=caller_stream)`` for every job, in list order, at most
+    ``workers`` at a time.  The first exception stops the remaining jobs and is re-raised on the caller."""
     jobs = list(jobs)
     streams = stream_cache.setdefault(device, [])
     while len(streams) < max(workers, 4):
@@ -71,11 +54,9 @@ def start_on_streams(jobs: List, work: Callable, workers: int, device: torch.dev
     threads = [threading.Thread(target=worker, args=(s,), daemon=True) for s in streams[:workers]]
     for t in threads:
         t.start()
-    return _Running(threads, streams[:workers], main, errors)
-
-
-def run_on_streams(jobs: List, work: Callable, workers: int, device: torch.device,
-                   stream_cache: Dict[torch.device, list]) -> None:
-    """``work(job, produced_on=side_stream, consumed_on=caller_stream)`` for every job, in list order, at most
-    ``workers`` at a time.  The first exception stops the remaining jobs and is re-raised on the caller."""
-    start_on_streams(jobs, work, workers, device, stream_cache).join()
+    for t in threads:
+        t.join()
+    for s in streams[:workers]:
+        main.wait_stream(s)
+    if errors:
+        raise errors[0]

@@ -739,3 +739,26 @@ def grouped_linear(x: torch.Tensor, pointers: torch.Tensor, experts: int, splits
                                             _stream(x))
     _lib.check(rc, "llmc_grouped_linear")
     return y
+
+
+DIAG_ORDER_MAX_K = 16384
+
+
+def diag_argsort_desc(Hs) -> torch.Tensor:
+    """int64 [n, K]: for each fp32 Hessian of ``Hs`` (one width, one row stride) its column numbers by descending
+    diagonal entry, equal entries in column order -- ``torch.argsort(diag, descending=True, stable=True)`` in one
+    launch for all of them."""
+    import ctypes
+
+    H0 = Hs[0]
+    _require_gpu(H0)
+    K = H0.shape[0]
+    for H in Hs:
+        assert H.dtype == torch.float32 and H.shape == (K, K) and H.stride(1) == 1 and H.stride(0) == H0.stride(0)
+        assert H.device == H0.device
+    out = torch.empty((len(Hs), K), dtype=torch.int64, device=H0.device)
+    hp = (ctypes.c_void_p * len(Hs))(*[H.data_ptr() for H in Hs])
+    with torch.cuda.device(H0.device):
+        rc = _lib.lib().llmc_diag_argsort_desc(hp, H0.stride(0), len(Hs), K, out.data_ptr(), _stream(H0))
+    _lib.check(rc, "llmc_diag_argsort_desc")
+    return out

@@ -436,3 +436,30 @@ def test_gptq_grouped_at_moe_layer_size(R, K):
     assert torch.isfinite(loss).all() and float(loss[17]) == 0.0
     routed = [b for b in range(n) if counts[b] >= K]
     assert all(float(loss[b]) > 0 for b in routed)
+
+
+@pytest.mark.parametrize("K,n", [(64, 1), (1000, 3), (4096, 6), (14336, 1), (16384, 2), (2048, 300)])
+def test_diag_argsort_is_torchs_stable_descending_argsort(K, n):
+    """The column order of the activation ordering from one launch: equal to
+    ``torch.argsort(diag, descending=True, stable=True)`` (the reference sorts with torch's unstable argsort,
+    gptq_quantize.py:131-140, which agrees wherever no two entries are equal), including runs of exact ties,
+    zeros of either sign, infinities and NaN."""
+    from llmcompressor_amd import ops
+
+    g = torch.Generator().manual_seed(K + n)
+    Hs = []
+    for b in range(n):
+        d = torch.rand(K, generator=g) * 10
+        d[torch.randperm(K, generator=g)[: K // 5]] = 3.25      # a run of exact ties
+        d[torch.randperm(K, generator=g)[: K // 9]] = 0.0
+        d[torch.randperm(K, generator=g)[: K // 11]] = -0.0
+        if b % 2 and K > 100:
+            d[7], d[K - 3], d[K // 2] = float("inf"), float("-inf"), float("nan")
+            d[11] = float("nan")
+        H = torch.randn(K, K, generator=g) if K <= 4096 else torch.zeros(K, K)
+        H.diagonal().copy_(d)
+        Hs.append(H.to("cuda"))
+    got = ops.diag_argsort_desc(Hs)
+    want = torch.argsort(torch.stack([torch.diagonal(H) for H in Hs]), dim=1, descending=True, stable=True)
+    assert got.dtype == torch.int64 and got.shape == (n, K)
+    assert torch.equal(got, want)
