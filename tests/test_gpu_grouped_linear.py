@@ -217,3 +217,53 @@ def test_grouped_forward_follows_replaced_weights_and_a_custom_gate():
             # new storage for one weight (what a quantiser does when it assigns a fresh tensor): the second
             # round must read it
             experts[4].down_proj.weight.data = (experts[4].down_proj.weight.data * -1.0).clone()
+
+
+def test_oneshot_uses_grouped_launches_only_where_nothing_observes_the_experts(monkeypatch):
+    """oneshot GPTQ on a random-init transformers Qwen3-MoE (two layers): the calibration pass of a layer runs the
+    per-expert calls (its hooks feed the Hessians), the propagation pass the grouped launches.  With the grouped
+    forward switched off the first layer comes out bit for bit the same (its calibration inputs do not depend on the
+    switch); the second layer, calibrated on activations that differ in the last bf16 digit of a few elements, agrees
+    on nearly all weights."""
+    transformers = pytest.importorskip("transformers")
+    import copy
+
+    from llmcompressor_amd import oneshot, ops
+    from llmcompressor_amd.modeling import moe
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+    from llmcompressor_amd.modifiers.utils.hooks import HooksMixin
+
+    torch.manual_seed(0)
+    cfg = transformers.Qwen3MoeConfig(hidden_size=128, intermediate_size=256, moe_intermediate_size=128,
+                                      num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2,
+                                      head_dim=32, vocab_size=256, max_position_embeddings=128, num_experts=8,
+                                      num_experts_per_tok=2)
+    base = transformers.Qwen3MoeForCausalLM(cfg).to(torch.bfloat16).to(DEV)
+    data = [{"input_ids": torch.randint(0, 256, (1, 64))} for _ in range(8)]
+    launches = []
+    real = ops.grouped_linear
+    monkeypatch.setattr(ops, "grouped_linear",
+                        lambda *a, **kw: launches.append(HooksMixin._HOOKS_DISABLED) or real(*a, **kw))
+    results = []
+    for grouped in (True, False):
+        monkeypatch.setattr(moe, "GROUPED_FORWARD", grouped)
+        launches.clear()
+        model = copy.deepcopy(base)
+        oneshot(model=model, recipe=GPTQModifier(targets="Linear", scheme="W4A16",
+                                                 ignore=["lm_head", "re:.*mlp.gate$"]),
+                dataset=data, moe_calibrate_all_experts=False)
+        if grouped:
+            # two launches per batch and layer, every one of them with the hooks switched off
+            assert len(launches) == 2 * len(data) * cfg.num_hidden_layers and all(launches)
+        else:
+            assert not launches
+        results.append({n: p.detach().clone() for n, p in model.named_parameters()})
+    on, off = results
+    assert on.keys() == off.keys()
+    for name in on:
+        if ".layers.0." in name or "embed" in name:
+            assert torch.equal(on[name], off[name]), name
+    later = [n for n in on if ".layers.1." in n and n.endswith("experts.3.down_proj.weight")]
+    assert later
+    for name in later:
+        assert (on[name] == off[name]).float().mean().item() >= 0.98, name
