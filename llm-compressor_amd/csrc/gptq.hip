@@ -208,12 +208,23 @@ struct GptqBlockParams {
 // covers columns j*QCW + t*QG .. +QG-1.  The lane that owns a run quantises its QG columns by itself (the
 // serial chain of a row never crosses lanes inside a run), then the QG scaled errors are broadcast to the team
 // once and every lane applies them, in column order, to the runs that are still open.
-constexpr int QTEAM = 4;
-constexpr int QCPL = GB / QTEAM;   // 32 columns per lane
+// Two team sizes are built.  Four lanes per row (one DPP quad, 32 columns per lane, 64 rows per workgroup) is the
+// layout for many rows: few waves, each doing as little redundant work as possible.  Sixteen lanes per row (8
+// columns per lane, 16 rows per workgroup) spreads a problem of a few thousand rows over every CU, one wave per
+// SIMD, and each wave applies a run's errors to two runs per lane instead of eight: the per-block time is bound
+// by one wave's instruction issue, so it falls with the instruction count.  Both apply the same operations to
+// every element in the same order, so they give the same bits.
 constexpr int QG = 4;              // neighbouring columns per run
-constexpr int QNCH = QCPL / QG;    // 8 runs per lane
-constexpr int QCW = QTEAM * QG;    // 16 columns per round of the team
-constexpr int Q_ROWS_PER_WG = 256 / QTEAM;
+template <int TEAM>
+struct QLayout {
+  static constexpr int QTEAM = TEAM;
+  static constexpr int QCPL = GB / TEAM;   // columns per lane
+  static constexpr int QNCH = QCPL / QG;   // runs per lane
+  static constexpr int QCW = TEAM * QG;    // columns per round of the team
+  static constexpr int ROWS_PER_WG = 256 / TEAM;
+};
+// rows (of all problems of a launch) up to which the sixteen-lane layout is used
+constexpr int64_t Q_WIDE_TEAM_MAX_ROWS = 8192;
 
 // ---- divisions of the column loop.  x / s goes through the hoisted reciprocal y of s (see make_fastdiv():
 // the steps of the correctly rounded division with the divisor's part taken out).  The short form gives the
@@ -294,19 +305,21 @@ __device__ __noinline__ QRun gptq_run_exact(float4 w, float4 s, float4 z, float4
 }
 
 // the registers of one lane: QCPL columns of one row, their scales, the scales' reciprocals, zero points
-template <bool HAS_ZP>
+template <bool HAS_ZP, int TEAM>
 struct QLane {
+  static constexpr int QNCH = QLayout<TEAM>::QNCH;
   float4 w[QNCH], sv[QNCH], yv[QNCH], zv[HAS_ZP ? QNCH : 1];
 };
 
 // Round J of the team: for each lane in turn, its run J is quantised and the errors applied to everything
 // that is still open.  Columns at or past `count` hold w = 0, scale 1, d = 1 and zero rows of U: they
 // quantise to zero with zero error, so only the stores look at `count`.
-template <int J, int FMT, int SD, bool HAS_ZP>
-__device__ __forceinline__ void gptq_round(QLane<HAS_ZP>& r, const float* __restrict__ Hs,
+template <int J, int FMT, int SD, bool HAS_ZP, int TEAM>
+__device__ __forceinline__ void gptq_round(QLane<HAS_ZP, TEAM>& r, const float* __restrict__ Hs,
                                            const float* __restrict__ Dd, const float* __restrict__ Dy, int tl,
                                            int count, bool live, float* __restrict__ wrow,
                                            float* __restrict__ erow, const QFormat& f, int bits, float& loss) {
+  constexpr int QTEAM = TEAM, QNCH = QLayout<TEAM>::QNCH, QCW = QLayout<TEAM>::QCW;
 #pragma unroll 1
   for (int li = 0; li < QTEAM; ++li) {
     const int i0 = J * QCW + li * QG;  // first column of this run
@@ -356,9 +369,10 @@ __device__ __forceinline__ void gptq_round(QLane<HAS_ZP>& r, const float* __rest
 }
 
 // the block's weights, scales and zero points of one lane; SDT = dtype of the stored scales
-template <int SDT, bool HAS_ZP>
-__device__ __forceinline__ void gptq_load_lane(QLane<HAS_ZP>& r, const GptqBlockParams& p, int row, int tl,
+template <int SDT, bool HAS_ZP, int TEAM>
+__device__ __forceinline__ void gptq_load_lane(QLane<HAS_ZP, TEAM>& r, const GptqBlockParams& p, int row, int tl,
                                                bool live) {
+  constexpr int QCPL = QLayout<TEAM>::QCPL, QNCH = QLayout<TEAM>::QNCH, QCW = QLayout<TEAM>::QCW;
   const int rowc = live ? row : p.R - 1;  // every load stays inside the arrays; dead lanes are blanked below
   const float* wsrc = p.Wf + (int64_t)rowc * p.K + p.i1;
   const int64_t sbase = ((int64_t)rowc / p.row_div) * p.srow;
@@ -403,8 +417,10 @@ __device__ __forceinline__ void gptq_load_lane(QLane<HAS_ZP>& r, const GptqBlock
   if (!HAS_ZP) r.zv[0] = make_float4(0.f, 0.f, 0.f, 0.f);
 }
 
-template <int FMT, int SD, bool HAS_ZP>
+template <int FMT, int SD, bool HAS_ZP, int TEAM>
 __global__ __launch_bounds__(256) void gptq_block_kernel(GptqBlockParams p) {
+  constexpr int QTEAM = TEAM, QNCH = QLayout<TEAM>::QNCH, QCW = QLayout<TEAM>::QCW;
+  constexpr int Q_ROWS_PER_WG = QLayout<TEAM>::ROWS_PER_WG;
   // [GB][GB] slice of U, zero outside the upper triangle; then its diagonal and the diagonal's reciprocals
   extern __shared__ __attribute__((aligned(16))) float Hs[];
   float* Dd = Hs + GB * GB;
@@ -432,22 +448,25 @@ __global__ __launch_bounds__(256) void gptq_block_kernel(GptqBlockParams p) {
   float* wrow = p.Wf + (int64_t)row * p.K + p.i1;
   float* erow = p.E + (int64_t)row * p.ldE;
 
-  QLane<HAS_ZP> r;
+  QLane<HAS_ZP, TEAM> r;
   if (p.scale_dt == LLMC_BF16)
-    gptq_load_lane<LLMC_BF16, HAS_ZP>(r, p, row, tl, live);
+    gptq_load_lane<LLMC_BF16, HAS_ZP, TEAM>(r, p, row, tl, live);
   else if (p.scale_dt == LLMC_F16)
-    gptq_load_lane<LLMC_F16, HAS_ZP>(r, p, row, tl, live);
+    gptq_load_lane<LLMC_F16, HAS_ZP, TEAM>(r, p, row, tl, live);
   else
-    gptq_load_lane<LLMC_F32, HAS_ZP>(r, p, row, tl, live);
+    gptq_load_lane<LLMC_F32, HAS_ZP, TEAM>(r, p, row, tl, live);
   __syncthreads();
 
   float loss = 0.f;
-#define LLMC_ROUND(J) \
-  if (J * QCW < count) gptq_round<J, FMT, SD, HAS_ZP>(r, Hs, Dd, Dy, tl, count, live, wrow, erow, f, p.bits, loss);
+#define LLMC_ROUND(J)                                                                                          \
+  if constexpr (J < QNCH) {                                                                                    \
+    if (J * QCW < count)                                                                                       \
+      gptq_round<J, FMT, SD, HAS_ZP, TEAM>(r, Hs, Dd, Dy, tl, count, live, wrow, erow, f, p.bits, loss);       \
+  }
   LLMC_ROUND(0) LLMC_ROUND(1) LLMC_ROUND(2) LLMC_ROUND(3)
   LLMC_ROUND(4) LLMC_ROUND(5) LLMC_ROUND(6) LLMC_ROUND(7)
 #undef LLMC_ROUND
-  static_assert(QNCH == 8, "one LLMC_ROUND per run of a lane");
+  static_assert(QNCH <= 8, "one LLMC_ROUND per run of a lane");
 
   if (live) {
     // the runs that were never reached carry no error into the trailing products
@@ -1072,8 +1091,11 @@ extern "C" int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R
   const int smem = (GB * GB + 2 * GB) * 4;
   void (*kern)(GptqBlockParams) = nullptr;
   const bool hz = zero_point != nullptr;
-#define LLMC_PICK(F, S)                                                         \
-  if (p.fmt == F && p.sd == S) kern = hz ? gptq_block_kernel<F, S, true> : gptq_block_kernel<F, S, false>;
+  const bool wide_team = R <= Q_WIDE_TEAM_MAX_ROWS;
+#define LLMC_PICK(F, S)                                                                                  \
+  if (p.fmt == F && p.sd == S)                                                                           \
+    kern = wide_team ? (hz ? gptq_block_kernel<F, S, true, 16> : gptq_block_kernel<F, S, false, 16>)     \
+                     : (hz ? gptq_block_kernel<F, S, true, 4> : gptq_block_kernel<F, S, false, 4>);
   LLMC_PICK(LLMC_FMT_INT, LLMC_BF16)
   LLMC_PICK(LLMC_FMT_INT, LLMC_F16)
   LLMC_PICK(LLMC_FMT_INT, LLMC_F32)
@@ -1087,7 +1109,8 @@ extern "C" int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R
   if (kern == nullptr) return -17;
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
   if (e != hipSuccess) return 1000 + (int)e;
-  const unsigned wgs = (unsigned)((R + Q_ROWS_PER_WG - 1) / Q_ROWS_PER_WG);
+  const int rows_per_wg = wide_team ? QLayout<16>::ROWS_PER_WG : QLayout<4>::ROWS_PER_WG;
+  const unsigned wgs = (unsigned)((R + rows_per_wg - 1) / rows_per_wg);
   {
     const int rc = gptq_column_loop(kern, p, smem, wgs, 1, R, K, bs, E, U, ldu, 0, Wf, st);
     if (rc) return rc;
@@ -1203,8 +1226,11 @@ extern "C" int llmc_gptq_quantize_grouped(const void* const* weight, int32_t w_d
   const int smem = (GB * GB + 2 * GB) * 4;
   void (*kern)(GptqBlockParams) = nullptr;
   const bool hz = zero_point != nullptr;
-#define LLMC_PICK(F, S)                                                         \
-  if (p.fmt == F && p.sd == S) kern = hz ? gptq_block_kernel<F, S, true> : gptq_block_kernel<F, S, false>;
+  const bool wide_team = (int64_t)n * R <= Q_WIDE_TEAM_MAX_ROWS;
+#define LLMC_PICK(F, S)                                                                                  \
+  if (p.fmt == F && p.sd == S)                                                                           \
+    kern = wide_team ? (hz ? gptq_block_kernel<F, S, true, 16> : gptq_block_kernel<F, S, false, 16>)     \
+                     : (hz ? gptq_block_kernel<F, S, true, 4> : gptq_block_kernel<F, S, false, 4>);
   LLMC_PICK(LLMC_FMT_INT, LLMC_BF16)
   LLMC_PICK(LLMC_FMT_INT, LLMC_F16)
   LLMC_PICK(LLMC_FMT_INT, LLMC_F32)
@@ -1218,7 +1244,8 @@ extern "C" int llmc_gptq_quantize_grouped(const void* const* weight, int32_t w_d
   if (kern == nullptr) return -19;
   hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
   if (e != hipSuccess) return 1000 + (int)e;
-  const unsigned wgs = (unsigned)((R + Q_ROWS_PER_WG - 1) / Q_ROWS_PER_WG);
+  const int rows_per_wg = wide_team ? QLayout<16>::ROWS_PER_WG : QLayout<4>::ROWS_PER_WG;
+  const unsigned wgs = (unsigned)((R + rows_per_wg - 1) / rows_per_wg);
   {
     const int rc = gptq_column_loop(kern, p, smem, wgs, n, R, K, bs, E, U, ldu, u_stride, Wf, st);
     if (rc) return rc;
