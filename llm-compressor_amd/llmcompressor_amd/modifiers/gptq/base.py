@@ -182,22 +182,30 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
         self.remove_hooks()
 
     def calibrate_module(self, module: torch.nn.Module, args: tuple[torch.Tensor, ...], _output: torch.Tensor):
-        """Forward hook: accumulate the Hessian of the module's input."""
+        """Forward hook: accumulate the Hessian of the module's input.
+
+        The hook runs once per Linear and batch (384 times per forward of an MoE layer), so it reads the modifier's
+        private state through the one dictionary pydantic keeps it in instead of one attribute lookup each (those
+        go through ``BaseModel.__getattr__``, about a microsecond apiece)."""
         inp = args[0]
+        priv = self.__pydantic_private__
         if self.share_identical_inputs:
-            self._hook_calls[module] = self._hook_calls.get(module, 0) + 1
-            if self._follows_recent_input(module, inp):
+            calls = priv["_hook_calls"]
+            calls[module] = calls.get(module, 0) + 1
+            if self._follows_recent_input(module, inp, priv):
                 return
-        grouped = (self._group_pending is not None and isinstance(module, torch.nn.Linear) and inp.is_cuda
+        num_samples = priv["_num_samples"]
+        pending = priv["_group_pending"]
+        grouped = (pending is not None and isinstance(module, torch.nn.Linear) and inp.is_cuda
                    and not self.offload_hessians and inp.dtype in (torch.bfloat16, torch.float16))
-        if module not in self._num_samples:
+        if module not in num_samples:
             device = inp.device if inp.is_cuda else module.weight.device
             init_device = "cpu" if self.offload_hessians else device
-            self._hessians[module] = make_empty_hessian(module, device=init_device)
+            priv["_hessians"][module] = make_empty_hessian(module, device=init_device)
             # an expert's tally stays on the host: hundreds of one-element device additions per forward otherwise
-            self._num_samples[module] = 0.0 if grouped else torch.zeros(tuple(), device=device)
+            num_samples[module] = 0.0 if grouped else torch.zeros(tuple(), device=device)
         if grouped:
-            self._group_pending.append((module, inp))
+            pending.append((module, inp))
             return
         if (self.hessian_batch_tokens > 0 and not self.offload_hessians and isinstance(module, torch.nn.Linear)
                 and inp.dtype in (torch.bfloat16, torch.float16)):  # fp32 inputs go straight to the fp32 product
@@ -208,25 +216,27 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
                 inp, module, self._hessians[module], self._num_samples[module])
 
     # -- shared Hessians (see ``share_identical_inputs``)
-    def _follows_recent_input(self, module, inp) -> bool:
+    def _follows_recent_input(self, module, inp, priv=None) -> bool:
         """True when `module` just received the tensor that the previous hook call accumulated for
         another module of the same width; then only its sample count advances.  The previous input is
         kept referenced, so no later tensor can take its address while it is being compared."""
-        recent = self._recent_input
+        priv = self.__pydantic_private__ if priv is None else priv
+        recent = priv["_recent_input"]
         same = (recent is not None and recent[2] is not module and inp.data_ptr() == recent[0].data_ptr()
                 and inp.shape == recent[0].shape and inp.dtype == recent[0].dtype and inp.stride() == recent[0].stride()
                 and inp._version == recent[1] and isinstance(module, torch.nn.Linear)
                 and module.in_features == recent[2].in_features)
-        leader = self._leader.get(module)
-        if same and (leader is recent[2] or (leader is None and module not in self._num_samples)):
-            self._leader[module] = recent[2]
+        leaders, num_samples = priv["_leader"], priv["_num_samples"]
+        leader = leaders.get(module)
+        if same and (leader is recent[2] or (leader is None and module not in num_samples)):
+            leaders[module] = recent[2]
             n = 1 if inp.ndim == 2 else inp.shape[0]
-            self._num_samples[module] = self._num_samples.get(module, 0) + n
+            num_samples[module] = num_samples.get(module, 0) + n
             return True
         if leader is not None:
             raise RuntimeError("share_identical_inputs: a module that shared its input with another one received a "
                                "different tensor on a later call; pass share_identical_inputs=False for this model")
-        self._recent_input = (inp, inp._version, module)
+        priv["_recent_input"] = (inp, inp._version, module)
         return False
 
     # -- expert groups (see the class docstring)

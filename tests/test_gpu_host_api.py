@@ -738,7 +738,9 @@ def test_gptq_concurrent_module_compression_is_identical():
         results.append((streams, {n: p.detach().clone() for n, p in model.named_parameters()}))
     (s1, w1), (s4, w4) = results
     assert len(s1) == 6 and len(set(s1)) == 1
-    assert len(s4) == 6 and len(set(s4)) > 1 and s1[0] not in s4
+    # every job ran on a side stream (how many of the four a run uses depends on how fast the first worker drains
+    # the queue of these tiny jobs)
+    assert len(s4) == 6 and 1 <= len(set(s4)) <= 4 and s1[0] not in s4
     assert w1.keys() == w4.keys()
     for n in w1:
         assert torch.equal(w1[n], w4[n]), n
