@@ -331,12 +331,16 @@ def test_hinv_grouped_is_bit_identical_to_single_calls(K, n, actorder):
 
 @pytest.mark.parametrize("R,K,n,fmt_case", [(96, 768, 5, "int4_sym"), (64, 512, 4, "int4_asym_actorder"),
                                             (48, 256, 3, "nvfp4"), (1024, 4096, 2, "int4_sym"),
-                                            (1024, 4608, 2, "int4_asym_actorder")])
+                                            (1024, 4608, 2, "int4_asym_actorder"),
+                                            (3072, 512, 3, "int4_asym_actorder"), (3080, 256, 3, "nvfp4")])
 def test_gptq_quantize_grouped_is_bit_identical_to_single_calls(R, K, n, fmt_case):
     """llmc_gptq_quantize_grouped on the factors of llmc_gptq_hinv_grouped: identical weights and losses to n
     single calls (int4 symmetric g128, int4 asymmetric g64 with activation ordering, NVFP4 with global scales).
-    The two larger cases reach the split-bf16 products of the trailing updates (the small ones stay on the fp32
-    matrix instructions), whose choice must not depend on how many problems a call carries."""
+    The two 1024-row cases reach the split-bf16 products of the trailing updates (the small ones stay on the fp32
+    matrix instructions), whose choice must not depend on how many problems a call carries.  In the last two the
+    grouped call carries more than 8192 rows and runs the block kernel with four lanes per row while the single
+    calls use sixteen: the two layouts must give the same bits (3080 rows: a last workgroup that is partly empty in
+    both)."""
     from llmcompressor_amd import ops
 
     torch.manual_seed(R + K)
