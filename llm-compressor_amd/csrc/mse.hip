@@ -32,6 +32,7 @@ struct MseParams {
   void* max0;        // [N]
   uint64_t* masks;   // [N][MASK_WORDS]
   uint64_t* flags;   // [MASK_WORDS] zero-initialised
+  const uint16_t* powtab;  // a^norm rounded to dt for every non-negative 16-bit a (see mse_powtab_kernel), or NULL
   // importance-weighted variant (observers/imatrix.py:255-328): the error |fq(x) - x|^norm is formed and
   // summed in fp32 (values are quantised in dt as before) and weighted per input channel
   int err32;
@@ -220,8 +221,9 @@ __device__ __forceinline__ void unpack8t(const uint4& v, float* x) {
 }
 
 // sum over 8 elements of |fq(x) - x|^norm, every intermediate rounded to DT
-template <int DT, int FMT, bool HAS_ZP>
-__device__ __forceinline__ float chunk_error(const float (&x)[8], float s, float zp, const QFormat& f, float norm) {
+template <int DT, int FMT, bool HAS_ZP, bool TAB>
+__device__ __forceinline__ float chunk_error(const float (&x)[8], float s, float zp, const QFormat& f, float norm,
+                                             const uint16_t* __restrict__ tab) {
   float v[8];
   const FastDiv d = make_fastdiv(s);
   bool big = false, small = false;
@@ -270,6 +272,25 @@ __device__ __forceinline__ float chunk_error(const float (&x)[8], float s, float
     }
   }
   float err = 0.f;
+  if (TAB) {
+    // a is a non-negative value of the 16-bit dtype: its power, already rounded, sits in the table at a's bits
+    uint32_t at[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      float dq = v[j];
+      if (HAS_ZP) dq = round16_finite<DT>(dq - zp);
+      dq = round16_finite<DT>(dq * s);
+      const float a = fabsf(round16_finite<DT>(dq - x[j]));
+      at[j] = DT == LLMC_BF16 ? (__float_as_uint(a) >> 16) : (uint32_t)f32_to_f16_bits(a);
+    }
+    uint32_t pw[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) pw[j] = tab[at[j] & 0x7fffu];
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      err += DT == LLMC_BF16 ? __uint_as_float(pw[j] << 16) : f16_bits_to_f32((uint16_t)pw[j]);
+    return err;
+  }
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     float dq = v[j];
@@ -289,11 +310,30 @@ __device__ __forceinline__ float chunk_error(const float (&x)[8], float s, float
 }
 
 // 16-bit inputs, groups of g = 8*L consecutive elements (L a power of two <= 64 lanes per group)
-template <int DT, int FMT, bool SYM>
-__global__ __launch_bounds__(256) void mse_team_fast_kernel(MseParams p, int64_t ngroups, int ng, int g, int lshift,
-                                                            int64_t ldw) {
+// TAB: the power comes from p.powtab, copied into LDS (64 KiB) when the workgroup starts: a lookup instead of the
+// two dozen issue slots of exp2(norm * log2 a) with its exactness guard.  Workgroups of 1024 threads then (the two
+// that fit a CU's LDS put eight waves on every SIMD), and a workgroup walks over the groups in strides of the
+// grid, so that the table is fetched a few hundred times per call and not once per 1024 threads of work.
+template <int DT, int FMT, bool SYM, bool TAB>
+__global__ __launch_bounds__(TAB ? 512 : 256) void mse_team_fast_kernel(MseParams p, int64_t ngroups, int ng, int g,
+                                                                         int lshift, int64_t ldw) {
+  constexpr int BLOCK = TAB ? 512 : 256;
+  extern __shared__ __attribute__((aligned(16))) uint16_t powlds[];
+  if (TAB) {
+    const uint4* src = (const uint4*)p.powtab;
+    uint4* dst = (uint4*)powlds;
+#pragma unroll
+    for (int k = 0; k < 65536 / 16 / BLOCK; ++k) dst[k * BLOCK + threadIdx.x] = src[k * BLOCK + threadIdx.x];
+    __syncthreads();
+  }
   const int L = 1 << lshift;
-  const int64_t gtid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  uint64_t any[MASK_WORDS];  // OR of this thread's masks over its groups
+#pragma unroll
+  for (int wd = 0; wd < MASK_WORDS; ++wd) any[wd] = 0ull;
+  const int64_t threads = ngroups << lshift;
+  // the bound is uniform over the workgroup, so every lane of a group's team takes part in every shuffle
+  for (int64_t base = (int64_t)blockIdx.x * BLOCK; base < threads; base += (int64_t)gridDim.x * BLOCK) {
+  const int64_t gtid = base + threadIdx.x;
   const int64_t grp = gtid >> lshift;
   const int sub = (int)(gtid & (L - 1));
   const bool live = grp < ngroups;
@@ -328,7 +368,7 @@ __global__ __launch_bounds__(256) void mse_team_fast_kernel(MseParams p, int64_t
     float s, zp;
     int e;
     qparams_from_minmax(smin, smax, DT, f, SYM, p.scale_mode, 1.f, &s, &zp, &e);
-    float err = chunk_error<DT, FMT, !SYM>(xv, s, zp, f, p.norm);
+    float err = chunk_error<DT, FMT, !SYM, TAB>(xv, s, zp, f, p.norm, powlds);
     for (int o = L >> 1; o > 0; o >>= 1) err += __shfl_xor(err, o, 64);
     err = round_to<DT>(err);
     if (err < best) {
@@ -348,24 +388,47 @@ __global__ __launch_bounds__(256) void mse_team_fast_kernel(MseParams p, int64_t
 #pragma unroll
     for (int wd = 0; wd < MASK_WORDS; ++wd) p.masks[grp * MASK_WORDS + wd] = mask[wd];
   }
-  or_flags(p.flags, mask);
+#pragma unroll
+  for (int wd = 0; wd < MASK_WORDS; ++wd) any[wd] |= mask[wd];
+  }
+  or_flags(p.flags, any);
+}
+
+// a^norm rounded to dt for each of the 32768 non-negative 16-bit values a, as 16-bit patterns: exactly what the
+// eager pow gives element by element, evaluated once per call instead of once per element and candidate
+__global__ __launch_bounds__(256) void mse_powtab_kernel(uint16_t* __restrict__ tab, float norm, int dt) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  const float a = dt == LLMC_BF16 ? bf16_bits_to_f32((uint16_t)i) : f16_bits_to_f32((uint16_t)i);
+  const float r = pow_eager(a, norm, dt);
+  tab[i] = dt == LLMC_BF16 ? f32_to_bf16_bits(r) : f32_to_f16_bits(r);
+}
+
+template <int DT, int FMT, bool SYM>
+int launch_team_fast_one(const MseParams& p, int64_t n, int ng, int g, int lshift, int64_t ldw, hipStream_t st) {
+  const int64_t threads = n << lshift;
+  if (p.powtab != nullptr) {
+    auto kern = mse_team_fast_kernel<DT, FMT, SYM, true>;
+    static const hipError_t configured =
+        hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
+    if (configured != hipSuccess) return 1000 + (int)configured;
+    const int64_t wgs = (threads + 511) / 512;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(wgs < 4096 ? wgs : 4096)), dim3(512), 65536, st, p, n, ng, g, lshift, ldw);
+  } else {
+    hipLaunchKernelGGL((mse_team_fast_kernel<DT, FMT, SYM, false>), dim3((unsigned)((threads + 255) / 256)),
+                       dim3(256), 0, st, p, n, ng, g, lshift, ldw);
+  }
+  return 0;
 }
 
 template <int DT>
-void launch_team_fast(const MseParams& p, int64_t n, int ng, int g, int lshift, int64_t ldw, hipStream_t st) {
-  const int64_t threads = n << lshift;
-  const dim3 grid((unsigned)((threads + 255) / 256)), block(256);
-#define LLMC_MSE(F, S) hipLaunchKernelGGL((mse_team_fast_kernel<DT, F, S>), grid, block, 0, st, p, n, ng, g, lshift, ldw)
-  if (p.fmt == LLMC_FMT_INT) {
-    if (p.symmetric) LLMC_MSE(LLMC_FMT_INT, true);
-    else LLMC_MSE(LLMC_FMT_INT, false);
-  } else if (p.fmt == LLMC_FMT_FP8) {
-    if (p.symmetric) LLMC_MSE(LLMC_FMT_FP8, true);
-    else LLMC_MSE(LLMC_FMT_FP8, false);
-  } else {
-    LLMC_MSE(LLMC_FMT_FP4, true);
-  }
-#undef LLMC_MSE
+int launch_team_fast(const MseParams& p, int64_t n, int ng, int g, int lshift, int64_t ldw, hipStream_t st) {
+  if (p.fmt == LLMC_FMT_INT)
+    return p.symmetric ? launch_team_fast_one<DT, LLMC_FMT_INT, true>(p, n, ng, g, lshift, ldw, st)
+                       : launch_team_fast_one<DT, LLMC_FMT_INT, false>(p, n, ng, g, lshift, ldw, st);
+  if (p.fmt == LLMC_FMT_FP8)
+    return p.symmetric ? launch_team_fast_one<DT, LLMC_FMT_FP8, true>(p, n, ng, g, lshift, ldw, st)
+                       : launch_team_fast_one<DT, LLMC_FMT_FP8, false>(p, n, ng, g, lshift, ldw, st);
+  return launch_team_fast_one<DT, LLMC_FMT_FP4, true>(p, n, ng, g, lshift, ldw, st);
 }
 
 struct GenericLayout {
@@ -517,6 +580,7 @@ float round_host(float v, int dt) {
 struct Workspace {
   uint64_t* flags;
   int* last;
+  uint16_t* powtab;
   void* min0;
   void* max0;
   uint64_t* masks;
@@ -527,6 +591,7 @@ Workspace carve(void* ws, int64_t n) {
   Workspace w;
   w.flags = (uint64_t*)c; c += 256;
   w.last = (int*)c; c += 256;
+  w.powtab = (uint16_t*)c; c += 65536;
   w.min0 = c; c += align256(n * 4);
   w.max0 = c; c += align256(n * 4);
   w.masks = (uint64_t*)c;
@@ -557,7 +622,7 @@ int setup(MseParams& p, Workspace& w, void* workspace, int64_t n, hipStream_t st
 }  // namespace
 
 extern "C" int64_t llmc_mse_workspace_bytes(int64_t n_groups) {
-  return 512 + 2 * align256(n_groups * 4) + align256(n_groups * MASK_WORDS * 8);
+  return 512 + 65536 + 2 * align256(n_groups * 4) + align256(n_groups * MASK_WORDS * 8);
 }
 
 static int check_common(int32_t dtype, int32_t fmt, int32_t num_bits, int32_t scale_mode, int32_t steps,
@@ -598,10 +663,15 @@ extern "C" int llmc_mse_observe_groups(const void* x, int32_t dtype, int64_t R, 
   if (team && (fmt != LLMC_FMT_FP4 || symmetric)) {
     int lshift = 0;
     while ((1 << lshift) < L) ++lshift;
-    if (dtype == LLMC_BF16)
-      launch_team_fast<LLMC_BF16>(p, n, (int)(K / group), (int)group, lshift, ldw, st);
-    else
-      launch_team_fast<LLMC_F16>(p, n, (int)(K / group), (int)group, lshift, ldw, st);
+    if (p.norm != 2.0f && p.norm != 3.0f && p.norm != 0.5f) {  // the other exponents have closed forms
+      hipLaunchKernelGGL(mse_powtab_kernel, dim3(128), dim3(256), 0, st, w.powtab, p.norm, dtype);
+      LLMC_LAUNCH_STATUS();
+      p.powtab = w.powtab;
+    }
+    const int lrc = dtype == LLMC_BF16
+                        ? launch_team_fast<LLMC_BF16>(p, n, (int)(K / group), (int)group, lshift, ldw, st)
+                        : launch_team_fast<LLMC_F16>(p, n, (int)(K / group), (int)group, lshift, ldw, st);
+    if (lrc) return lrc;
   } else if (team) {
     const int64_t threads = n * L;
     hipLaunchKernelGGL(mse_team_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, p, n,
