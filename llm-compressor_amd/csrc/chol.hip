@@ -107,7 +107,9 @@ __global__ __launch_bounds__(256) void hinv_copyin_kernel(const float* __restric
 // coalesced into LDS and the permuted columns are picked there (element-wise the gather costs one cache line
 // per value).  Rows of up to COPYIN_STAGE_MAX values.
 constexpr int COPYIN_STAGE_MAX = 16384;
-__global__ __launch_bounds__(256) void hinv_copyin_rows_kernel(const float* __restrict__ H, int64_t ldh, int K,
+// Launched with 256 threads per row, or with 1024 for rows of more than 8192 values: a row of 14336 floats takes
+// 56 KB of LDS, two workgroups fit a CU, and with 256 threads each the CU would hold 8 waves' worth of loads.
+__global__ __launch_bounds__(1024) void hinv_copyin_rows_kernel(const float* __restrict__ H, int64_t ldh, int K,
                                                                int Kp, const int32_t* __restrict__ perm, float div,
                                                                const HinvScalars* __restrict__ sc,
                                                                float* __restrict__ A,
@@ -119,30 +121,30 @@ __global__ __launch_bounds__(256) void hinv_copyin_rows_kernel(const float* __re
     sc += blockIdx.y;
     A += (int64_t)blockIdx.y * Kp * Kp;
   }
-  const int i = blockIdx.x, tid = threadIdx.x;
+  const int i = blockIdx.x, tid = threadIdx.x, nt = blockDim.x;
   float* out = A + (int64_t)i * Kp;
   if (i >= K) {  // identity padding
-    for (int j = tid; j < Kp; j += 256) out[j] = (i == j) ? 1.f : 0.f;
+    for (int j = tid; j < Kp; j += nt) out[j] = (i == j) ? 1.f : 0.f;
     return;
   }
   const float* src = H + (int64_t)perm[K - 1 - i] * ldh;
   constexpr int BATCH = 8;
-  for (int c0 = 0; c0 < K; c0 += 256 * BATCH) {
+  for (int c0 = 0; c0 < K; c0 += nt * BATCH) {
     float v[BATCH];
 #pragma unroll
     for (int b = 0; b < BATCH; ++b) {
-      const int c = c0 + b * 256 + tid;
+      const int c = c0 + b * nt + tid;
       v[b] = src[c < K ? c : K - 1];
     }
 #pragma unroll
     for (int b = 0; b < BATCH; ++b) {
-      const int c = c0 + b * 256 + tid;
+      const int c = c0 + b * nt + tid;
       if (c < K) rowbuf[c] = v[b];
     }
   }
   __syncthreads();
   const float damp = sc->damp;
-  for (int j = tid; j < Kp; j += 256) {
+  for (int j = tid; j < Kp; j += nt) {
     float v = 0.f;
     if (j <= i) {
       v = rowbuf[perm[K - 1 - j]] / div;
@@ -536,7 +538,7 @@ extern "C" int llmc_gptq_hinv(float* H, int64_t ldh, int64_t K, const int32_t* p
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)K * 4);
       if (e != hipSuccess) return 1000 + (int)e;
     }
-    hipLaunchKernelGGL(hinv_copyin_rows_kernel, dim3(Kp), dim3(256), (size_t)K * 4, st, H, ldh, (int)K, Kp, perm,
+    hipLaunchKernelGGL(hinv_copyin_rows_kernel, dim3(Kp), dim3(K > 8192 ? 1024 : 256), (size_t)K * 4, st, H, ldh, (int)K, Kp, perm,
                        divisor, sc, A, (const HinvItem*)nullptr);
   } else {
     hipLaunchKernelGGL(hinv_copyin_kernel, dim3((Kp + 255) / 256, Kp), dim3(256), 0, st, H, ldh, (int)K, Kp, perm,
@@ -647,7 +649,7 @@ extern "C" int llmc_gptq_hinv_grouped(const float* const* H, int64_t ldh, int32_
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)K * 4);
       if (e != hipSuccess) return 1000 + (int)e;
     }
-    hipLaunchKernelGGL(hinv_copyin_rows_kernel, dim3(Kp, n), dim3(256), (size_t)K * 4, st, (const float*)nullptr, ldh,
+    hipLaunchKernelGGL(hinv_copyin_rows_kernel, dim3(Kp, n), dim3(K > 8192 ? 1024 : 256), (size_t)K * 4, st, (const float*)nullptr, ldh,
                        (int)K, Kp, (const int32_t*)nullptr, 1.f, sc, A, (const HinvItem*)items);
   } else {
     hipLaunchKernelGGL(hinv_copyin_kernel, dim3((Kp + 255) / 256, Kp, n), dim3(256), 0, st, (const float*)nullptr, ldh,

@@ -60,7 +60,7 @@ __global__ __launch_bounds__(256) void gptq_prepare_w_kernel(const void* __restr
 constexpr int ROW_STAGE_MAX = 16384;
 
 template <int WDT>
-__global__ __launch_bounds__(256) void gptq_prepare_w_rows_kernel(const void* __restrict__ w, int64_t ldw, int R,
+__global__ __launch_bounds__(1024) void gptq_prepare_w_rows_kernel(const void* __restrict__ w, int64_t ldw, int R,
                                                                   int K, const int32_t* __restrict__ perm,
                                                                   const uint8_t* __restrict__ dead,
                                                                   float* __restrict__ Wf,
@@ -72,23 +72,23 @@ __global__ __launch_bounds__(256) void gptq_prepare_w_rows_kernel(const void* __
     if (dead) dead += (int64_t)blockIdx.y * K;
     Wf += (int64_t)blockIdx.y * R * K;
   }
-  const int r = blockIdx.x, tid = threadIdx.x;
+  const int r = blockIdx.x, tid = threadIdx.x, nt = blockDim.x;  // 256 threads, 1024 for rows above 8192 values
   constexpr int BATCH = 8;
-  for (int c0 = 0; c0 < K; c0 += 256 * BATCH) {
+  for (int c0 = 0; c0 < K; c0 += nt * BATCH) {
     float v[BATCH];
 #pragma unroll
     for (int b = 0; b < BATCH; ++b) {
-      const int c = c0 + b * 256 + tid;
+      const int c = c0 + b * nt + tid;
       v[b] = load_as_f32<WDT>(w, (int64_t)r * ldw + (c < K ? c : K - 1));
     }
 #pragma unroll
     for (int b = 0; b < BATCH; ++b) {
-      const int c = c0 + b * 256 + tid;
+      const int c = c0 + b * nt + tid;
       if (c < K) rowbuf[c] = v[b];
     }
   }
   __syncthreads();
-  for (int c = tid; c < K; c += 256) {
+  for (int c = tid; c < K; c += nt) {
     float v = rowbuf[perm[c]];
     if (dead && dead[c]) v = 0.f;
     Wf[(int64_t)r * K + c] = v;
@@ -96,7 +96,7 @@ __global__ __launch_bounds__(256) void gptq_prepare_w_rows_kernel(const void* __
 }
 
 template <int WDT>
-__global__ __launch_bounds__(256) void gptq_finalize_rows_kernel(const float* __restrict__ Wf, int R, int K,
+__global__ __launch_bounds__(1024) void gptq_finalize_rows_kernel(const float* __restrict__ Wf, int R, int K,
                                                                  const int32_t* __restrict__ perm,
                                                                  void* __restrict__ out, int64_t ldo,
                                                                  const GptqItem* __restrict__ items) {
@@ -106,26 +106,26 @@ __global__ __launch_bounds__(256) void gptq_finalize_rows_kernel(const float* __
     perm += (int64_t)blockIdx.y * K;
     Wf += (int64_t)blockIdx.y * R * K;
   }
-  const int r = blockIdx.x, tid = threadIdx.x;
+  const int r = blockIdx.x, tid = threadIdx.x, nt = blockDim.x;  // 256 threads, 1024 for rows above 8192 values
   constexpr int BATCH = 8;
-  for (int c0 = 0; c0 < K; c0 += 256 * BATCH) {
+  for (int c0 = 0; c0 < K; c0 += nt * BATCH) {
     float v[BATCH];
     int dst[BATCH];
 #pragma unroll
     for (int b = 0; b < BATCH; ++b) {
-      const int c = c0 + b * 256 + tid;
+      const int c = c0 + b * nt + tid;
       const int cc = c < K ? c : K - 1;
       v[b] = Wf[(int64_t)r * K + cc];
       dst[b] = perm[cc];
     }
 #pragma unroll
     for (int b = 0; b < BATCH; ++b) {
-      const int c = c0 + b * 256 + tid;
+      const int c = c0 + b * nt + tid;
       if (c < K) rowbuf[dst[b]] = v[b];
     }
   }
   __syncthreads();
-  for (int c = tid; c < K; c += 256) store_from_f32<WDT>(out, (int64_t)r * ldo + c, rowbuf[c]);
+  for (int c = tid; c < K; c += nt) store_from_f32<WDT>(out, (int64_t)r * ldo + c, rowbuf[c]);
 }
 
 // dynamic LDS above 48 KB has to be asked for once per kernel
@@ -1065,7 +1065,7 @@ extern "C" int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R
   if (by_rows) {                                                                                                    \
     const int arc = allow_row_stage(gptq_prepare_w_rows_kernel<DT>, (int)K);                                        \
     if (arc) return arc;                                                                                            \
-    hipLaunchKernelGGL((gptq_prepare_w_rows_kernel<DT>), dim3((unsigned)R), dim3(256), (size_t)K * 4, st, weight, ldw, \
+    hipLaunchKernelGGL((gptq_prepare_w_rows_kernel<DT>), dim3((unsigned)R), dim3(K > 8192 ? 1024 : 256), (size_t)K * 4, st, weight, ldw, \
                        (int)R, (int)K, perm, dead, Wf, (const GptqItem*)nullptr);                                   \
   } else {                                                                                                          \
     hipLaunchKernelGGL((gptq_prepare_w_kernel<DT>), grid2, dim3(256), 0, st, weight, ldw, (int)R, (int)K, perm, dead, \
@@ -1120,7 +1120,7 @@ extern "C" int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R
   if (by_rows) {                                                                                                    \
     const int arc = allow_row_stage(gptq_finalize_rows_kernel<DT>, (int)K);                                         \
     if (arc) return arc;                                                                                            \
-    hipLaunchKernelGGL((gptq_finalize_rows_kernel<DT>), dim3((unsigned)R), dim3(256), (size_t)K * 4, st, Wf, (int)R,   \
+    hipLaunchKernelGGL((gptq_finalize_rows_kernel<DT>), dim3((unsigned)R), dim3(K > 8192 ? 1024 : 256), (size_t)K * 4, st, Wf, (int)R,   \
                        (int)K, perm, out_weight, ldo, (const GptqItem*)nullptr);                                    \
   } else {                                                                                                          \
     hipLaunchKernelGGL((gptq_finalize_kernel<DT>), grid2, dim3(256), 0, st, Wf, (int)R, (int)K, perm, out_weight, ldo); \
@@ -1200,7 +1200,7 @@ extern "C" int llmc_gptq_quantize_grouped(const void* const* weight, int32_t w_d
   if (by_rows) {                                                                                                \
     const int arc = allow_row_stage(gptq_prepare_w_rows_kernel<DT>, (int)K);                                    \
     if (arc) return arc;                                                                                        \
-    hipLaunchKernelGGL((gptq_prepare_w_rows_kernel<DT>), dim3((unsigned)R, (unsigned)n), dim3(256), (size_t)K * 4, \
+    hipLaunchKernelGGL((gptq_prepare_w_rows_kernel<DT>), dim3((unsigned)R, (unsigned)n), dim3(K > 8192 ? 1024 : 256), (size_t)K * 4, \
                        st, (const void*)nullptr, ldw, (int)R, (int)K, perm, dead, Wf, (const GptqItem*)items);  \
   } else {                                                                                                      \
     hipLaunchKernelGGL((gptq_prepare_w_kernel<DT>), grid3, dim3(256), 0, st, (const void*)nullptr, ldw, (int)R, \
@@ -1255,7 +1255,7 @@ extern "C" int llmc_gptq_quantize_grouped(const void* const* weight, int32_t w_d
   if (by_rows) {                                                                                                \
     const int arc = allow_row_stage(gptq_finalize_rows_kernel<DT>, (int)K);                                     \
     if (arc) return arc;                                                                                        \
-    hipLaunchKernelGGL((gptq_finalize_rows_kernel<DT>), dim3((unsigned)R, (unsigned)n), dim3(256), (size_t)K * 4,  \
+    hipLaunchKernelGGL((gptq_finalize_rows_kernel<DT>), dim3((unsigned)R, (unsigned)n), dim3(K > 8192 ? 1024 : 256), (size_t)K * 4,  \
                        st, Wf, (int)R, (int)K, perm, (void*)nullptr, ldo, (const GptqItem*)items);              \
   } else {                                                                                                      \
     hipLaunchKernelGGL((gptq_finalize_kernel<DT>), grid3, dim3(256), 0, st, Wf, (int)R, (int)K, perm,           \
