@@ -437,31 +437,32 @@ namespace {
 // (gptq_quantize.py:131-140 sorts diag(H) with torch.argsort; a stable sort is what keeps equal entries in column
 // order.)  One workgroup per Hessian: the diagonal and the column numbers sit in LDS, padded to a power of two
 // with entries that sort last, and a bitonic network orders them by (value descending, index ascending) -- a total
-// order, so the network's result is the stable sort's.  NaN sorts before every number, as in torch.
+// order, so the network's result is the stable sort's.  NaN sorts before every number, as in torch; the two zeros
+// compare equal.
 constexpr int ORDER_MAX_K = 16384;
 constexpr int ORDER_MAX_PROBLEMS = 256;
 struct OrderArgs {
   const float* H[ORDER_MAX_PROBLEMS];
 };
 
-__device__ __forceinline__ bool order_before(float ka, int ia, float kb, int ib) {
-  const bool na = ka != ka, nb = kb != kb;
-  if (na != nb) return na;
-  if (!na && ka != kb) return ka > kb;
-  return ia < ib;
+// (value, index) as one 64-bit key whose ascending order is "value descending, index ascending": the float's bits
+// are mapped to an unsigned that grows with the value (both zeros to one key, every NaN to one key above +inf),
+// complemented, and the index goes into the low half.
+__device__ __forceinline__ unsigned long long order_key(float v, int i) {
+  uint32_t u = __float_as_uint(v);
+  if (v != v) u = 0x7fc00000u;          // one NaN
+  if ((u << 1) == 0u) u = 0u;           // -0 -> +0
+  u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+  return ((unsigned long long)(~u) << 32) | (unsigned)i;
 }
 
 __global__ __launch_bounds__(1024) void diag_order_kernel(OrderArgs args, int64_t ldh, int K, int N,
                                                           int64_t* __restrict__ out) {
   extern __shared__ __attribute__((aligned(16))) unsigned char order_smem[];
-  float* key = (float*)order_smem;
-  int* idx = (int*)(order_smem + (size_t)N * 4);
+  unsigned long long* key = (unsigned long long*)order_smem;
   const float* H = args.H[blockIdx.x];
   const int tid = threadIdx.x;
-  for (int i = tid; i < N; i += 1024) {
-    key[i] = i < K ? H[(int64_t)i * ldh + i] : -__builtin_inff();
-    idx[i] = i < K ? i : 0x7fffffff;
-  }
+  for (int i = tid; i < N; i += 1024) key[i] = i < K ? order_key(H[(int64_t)i * ldh + i], i) : ~0ull;
   __syncthreads();
   for (int k = 2; k <= N; k <<= 1) {
     for (int j = k >> 1; j > 0; j >>= 1) {
@@ -469,18 +470,16 @@ __global__ __launch_bounds__(1024) void diag_order_kernel(OrderArgs args, int64_
         const int i = ((t & ~(j - 1)) << 1) | (t & (j - 1));  // the element of the pair with bit j clear
         const int p = i | j;
         const bool up = (i & k) == 0;  // this run ends up in order (first element first)
-        const float ka = key[i], kb = key[p];
-        const int ia = idx[i], ib = idx[p];
-        const bool in_order = order_before(ka, ia, kb, ib);
-        if (in_order != up) {
-          key[i] = kb; key[p] = ka;
-          idx[i] = ib; idx[p] = ia;
+        const unsigned long long a = key[i], b = key[p];
+        if ((a < b) != up) {
+          key[i] = b;
+          key[p] = a;
         }
       }
       __syncthreads();
     }
   }
-  for (int i = tid; i < K; i += 1024) out[(int64_t)blockIdx.x * K + i] = idx[i];
+  for (int i = tid; i < K; i += 1024) out[(int64_t)blockIdx.x * K + i] = (int64_t)(key[i] & 0xffffffffull);
 }
 }  // namespace
 
