@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the calibration-time quantization hot path on one MI355X.
 
-Workload (BASELINE.json configs[3], one decoder layer per step): GPTQ W4A16 g128,
+Workload (the fourth of the benchmark configurations, one decoder layer per step): GPTQ W4A16 g128,
 activation ordering "static", of the seven Linears of a random-init
 Llama-3-8B-shaped decoder layer.  A step is
 
