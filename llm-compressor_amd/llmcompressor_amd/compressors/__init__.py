@@ -31,7 +31,7 @@ from ..quantization import (
 )
 from ..quantization.lifecycle import effective_scale, kernel_format, scale_indexing
 
-__all__ = ["infer_format", "compress_module", "decompress_weight", "compress_model_state_dict",
+__all__ = ["infer_format", "resolve_format", "compress_module", "decompress_weight", "compress_model_state_dict",
            "save_pretrained_compressed", "quantization_config_dict", "CompressionFormat"]
 
 
@@ -65,6 +65,36 @@ def infer_format(scheme: QuantizationScheme) -> str:
     if w.type == QuantizationType.INT:
         return CompressionFormat.int_quantized
     return CompressionFormat.naive_quantized
+
+
+def resolve_format(scheme: QuantizationScheme, override=None) -> str:
+    """The format a scheme's weights are written in: the inferred one, or the caller's ``quantization_format``
+    (a string with hyphens or underscores, or an enum member with such a ``value``) when the codes of the scheme
+    can be stored that way.  The reference's W4AFP8 example saves with ``quantization_format="pack-quantized"``
+    (examples/quantization_w4a8_fp8/llama3_example.py:76-80, docs/guides/saving_a_model.md:54-79): int4 codes
+    next to quantised activations are inferred as one code per byte and packed eight per word on request."""
+    inferred = infer_format(scheme)
+    if override is None:
+        return inferred
+    fmt = str(getattr(override, "value", override)).replace("_", "-")
+    w = scheme.weights
+    if w is None or fmt in (inferred, CompressionFormat.dense):
+        return CompressionFormat.dense if w is None else fmt
+    is_int = w.type == QuantizationType.INT
+    fits = {
+        CompressionFormat.pack_quantized: is_int and w.num_bits in (4, 8),
+        CompressionFormat.int_quantized: is_int,
+        CompressionFormat.naive_quantized: is_int or w.num_bits == 8,
+        CompressionFormat.float_quantized: not is_int and w.num_bits == 8,
+        CompressionFormat.nvfp4_pack_quantized: not is_int and w.num_bits == 4 and not w.is_mx,
+        CompressionFormat.mxfp4_pack_quantized: not is_int and w.num_bits == 4 and w.is_mx,
+    }
+    if fmt not in fits:
+        raise ValueError(f"unknown quantization_format {fmt!r}; known: {sorted(fits) + [CompressionFormat.dense]}")
+    if not fits[fmt]:
+        raise ValueError(f"quantization_format {fmt!r} cannot hold {w.num_bits}-bit {w.type.value} weights "
+                         f"(inferred format: {inferred!r})")
+    return fmt
 
 
 def _run(weight, scale, zp, args: QuantizationArgs, mode, g_idx=None, global_scale=None):
@@ -198,7 +228,7 @@ def decompress_weight(tensors: Dict[str, torch.Tensor], args: QuantizationArgs, 
     return (vals.unflatten(-1, (-1, args.group_size)) * s.unsqueeze(-1)).flatten(-2).to(dtype)
 
 
-def compress_model_state_dict(model: torch.nn.Module) -> Dict[str, torch.Tensor]:
+def compress_model_state_dict(model: torch.nn.Module, quantization_format=None) -> Dict[str, torch.Tensor]:
     """Full state dict with every quantised module's weight replaced by its packed tensors."""
     quantised = {name: m for name, m in model.named_modules()
                  if is_module_quantized(m) and getattr(m.quantization_scheme, "weights", None) is not None
@@ -207,7 +237,7 @@ def compress_model_state_dict(model: torch.nn.Module) -> Dict[str, torch.Tensor]
     skip = set()
     for name, m in quantised.items():
         prefix = f"{name}." if name else ""
-        for k, v in compress_module(m).items():
+        for k, v in compress_module(m, fmt=resolve_format(m.quantization_scheme, quantization_format)).items():
             out[prefix + k] = v
         for k, _ in list(m.named_parameters(recurse=False)) + list(m.named_buffers(recurse=False)):
             skip.add(prefix + k)
@@ -218,14 +248,15 @@ def compress_model_state_dict(model: torch.nn.Module) -> Dict[str, torch.Tensor]
     return out
 
 
-def quantization_config_dict(model: torch.nn.Module, save_compressed: bool = True) -> Optional[dict]:
+def quantization_config_dict(model: torch.nn.Module, save_compressed: bool = True,
+                             quantization_format=None) -> Optional[dict]:
     config: Optional[QuantizationConfig] = getattr(model, "quantization_config", None)
     if config is None or not isinstance(config, QuantizationConfig):
         return None
     formats = set()
     groups = {}
     for name, scheme in config.config_groups.items():
-        fmt = infer_format(scheme) if save_compressed else CompressionFormat.dense
+        fmt = resolve_format(scheme, quantization_format) if save_compressed else CompressionFormat.dense
         formats.add(fmt)
         d = scheme.model_dump(mode="json")
         d["format"] = fmt

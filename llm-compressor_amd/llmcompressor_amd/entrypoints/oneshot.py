@@ -43,7 +43,11 @@ class Oneshot:
 
     def __call__(self):
         from ..modeling.moe import get_non_linearized_moes, linearize_moe
+        from ..transformers.compression.compressed_tensors_utils import modify_save_pretrained
 
+        # reference: entrypoints/utils.py:96 -- from here on ``model.save_pretrained(dir, save_compressed=True,
+        # quantization_format=None)`` writes the compressed checkpoint
+        modify_save_pretrained(self.model)
         if get_non_linearized_moes(self.model):  # reference: entrypoints/oneshot.py:237-243
             logger.warning("Detected an MoE model whose experts are stored as fused 3-D tensors; replacing them "
                            "by per-expert Linears so that they can be calibrated and quantized.")
@@ -55,10 +59,14 @@ class Oneshot:
                            f"recognised ({left[0]}, ...); they stay as they are and their weights are not quantized.")
         self.apply_recipe_modifiers(self.dataset)
         if self.output_dir is not None:
-            from ..compressors import save_pretrained_compressed
+            if getattr(getattr(self.model, "save_pretrained", None), "_overridden", False):
+                # reference: entrypoints/utils.py:122-124
+                self.model.save_pretrained(self.output_dir, save_compressed=self.save_compressed)
+            else:  # a plain torch module has no writer of its own
+                from ..compressors import save_pretrained_compressed
 
-            save_pretrained_compressed(self.model, self.output_dir, save_compressed=self.save_compressed,
-                                       recipe=active_session().lifecycle.recipe)
+                save_pretrained_compressed(self.model, self.output_dir, save_compressed=self.save_compressed,
+                                           recipe=active_session().lifecycle.recipe)
         return self.model
 
     def apply_recipe_modifiers(self, calibration_dataloader):

@@ -312,6 +312,12 @@ _PRESETS = {
         input_activations=dict(num_bits=8, type="int", symmetric=True, strategy="token", dynamic=True,
                                observer=None),
     ),
+    # int4 group weights, fp8 per-token activations (reference: examples/quantization_w4a8_fp8/llama3_example.py:53)
+    "W4AFP8": dict(
+        weights=dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128, dynamic=False),
+        input_activations=dict(num_bits=8, type="float", symmetric=True, strategy="token", dynamic=True,
+                               observer=None),
+    ),
     "FP8": dict(
         weights=dict(num_bits=8, type="float", symmetric=True, strategy="tensor", dynamic=False),
         input_activations=dict(num_bits=8, type="float", symmetric=True, strategy="tensor", dynamic=False),

@@ -1486,6 +1486,68 @@ def test_kv_cache_scheme_calibrates_k_and_v_scales_on_a_transformers_llama(tmp_p
     assert "model.layers.0.self_attn.q_proj.weight_scale" in sd
 
 
+def test_save_pretrained_after_oneshot_writes_the_compressed_checkpoint(tmp_path):
+    """The call the reference's examples end with (examples/quantization_w4a8_fp8/llama3_example.py:53-80):
+    ``oneshot`` without ``output_dir``, then ``model.save_pretrained(dir, save_compressed=True,
+    quantization_format="pack-quantized")``.  W4AFP8 through GPTQModifier on a transformers Llama: packed words
+    decode to the weights the model holds, ``config.json`` names the format, ``recipe.yaml`` is written; the
+    inferred format stores the same codes one per byte; ``save_compressed=False`` keeps dense weights."""
+    transformers = pytest.importorskip("transformers")
+
+    from safetensors.torch import load_file
+
+    from llmcompressor_amd import oneshot
+    from llmcompressor_amd.compressors import decompress_weight
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+
+    torch.manual_seed(0)
+    cfg = transformers.LlamaConfig(hidden_size=128, intermediate_size=256, num_hidden_layers=2,
+                                   num_attention_heads=4, num_key_value_heads=2, vocab_size=256,
+                                   max_position_embeddings=128)
+    model = transformers.LlamaForCausalLM(cfg).to(torch.bfloat16).to(DEV)
+    data = [{"input_ids": torch.randint(0, 256, (1, 64))} for _ in range(4)]
+    oneshot(model=model, dataset=data, recipe=GPTQModifier(targets="Linear", scheme="W4AFP8", ignore=["lm_head"]))
+    lin = model.model.layers[1].mlp.down_proj
+    args = lin.quantization_scheme.weights
+    assert lin.quantization_scheme.input_activations.type.value == "float"
+
+    packed_dir, bytes_dir, dense_dir = (str(tmp_path / n) for n in ("packed", "bytes", "dense"))
+    model.save_pretrained(packed_dir, save_compressed=True, quantization_format="pack-quantized")
+    model.save_pretrained(bytes_dir)
+    model.save_pretrained(dense_dir, save_compressed=False)
+    with pytest.raises(ValueError, match="cannot hold"):
+        model.save_pretrained(str(tmp_path / "bad"), quantization_format="float-quantized")
+    assert not os.path.exists(str(tmp_path / "bad"))
+
+    name = "model.layers.1.mlp.down_proj."
+    sd = load_file(os.path.join(packed_dir, "model.safetensors"))
+    assert sd[name + "weight_packed"].dtype == torch.int32 and sd[name + "weight_packed"].shape == (128, 256 // 8)
+    assert name + "weight" not in sd and "lm_head.weight" in sd
+    assert not any("observer" in k for k in sd)
+    tensors = {k[len(name):]: v.to(DEV) for k, v in sd.items() if k.startswith(name)}
+    assert torch.equal(decompress_weight(tensors, args, "pack-quantized"), lin.weight.data)
+    q = json.load(open(os.path.join(packed_dir, "config.json")))
+    assert q["model_type"] == "llama"
+    q = q["quantization_config"]
+    assert q["format"] == "pack-quantized" and q["quantization_status"] == "compressed"
+    group = next(iter(q["config_groups"].values()))
+    assert group["format"] == "pack-quantized" and group["input_activations"]["type"] == "float"
+    assert "lm_head" in q["ignore"]
+    assert "GPTQModifier" in open(os.path.join(packed_dir, "recipe.yaml")).read()
+    assert os.path.exists(os.path.join(packed_dir, "generation_config.json"))
+
+    sd8 = load_file(os.path.join(bytes_dir, "model.safetensors"))
+    assert sd8[name + "weight"].dtype == torch.int8
+    tensors8 = {k[len(name):]: v.to(DEV) for k, v in sd8.items() if k.startswith(name)}
+    assert torch.equal(decompress_weight(tensors8, args, "int-quantized"), lin.weight.data)
+    assert json.load(open(os.path.join(bytes_dir, "config.json")))["quantization_config"]["format"] == "int-quantized"
+
+    sdd = load_file(os.path.join(dense_dir, "model.safetensors"))
+    assert torch.equal(sdd[name + "weight"].to(DEV), lin.weight.data) and name + "weight_scale" in sdd
+    qd = json.load(open(os.path.join(dense_dir, "config.json")))["quantization_config"]
+    assert qd["format"] == "dense" and qd["quantization_status"] == "frozen"
+
+
 def test_gptq_beats_round_to_nearest_end_to_end_on_a_transformers_llama():
     """The whole pipeline on a 4-layer transformers Llama with anisotropic activations: W4A16 through
     GPTQModifier (sequential, error feedback from calibration data) gives a clearly smaller logit error on

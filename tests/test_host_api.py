@@ -256,6 +256,67 @@ def test_format_inference(preset, fmt):
     assert infer_format(w8a16_float) == CompressionFormat.naive_quantized
 
 
+def test_quantization_format_override():
+    """``save_pretrained(..., quantization_format=...)``: the reference's W4AFP8 example stores its int4 codes
+    packed on request (examples/quantization_w4a8_fp8/llama3_example.py:76-80); a format that cannot hold a
+    scheme's codes is refused before anything is written."""
+    from llmcompressor_amd.compressors import resolve_format
+
+    w4afp8 = preset_name_to_scheme("W4AFP8", ["Linear"])
+    assert w4afp8.weights.num_bits == 4 and w4afp8.weights.group_size == 128
+    assert w4afp8.input_activations.type.value == "float" and w4afp8.input_activations.dynamic is True
+    assert resolve_format(w4afp8) == CompressionFormat.int_quantized
+    assert resolve_format(w4afp8, "pack-quantized") == CompressionFormat.pack_quantized
+    assert resolve_format(w4afp8, "pack_quantized") == CompressionFormat.pack_quantized
+
+    class _Enum:  # compressed_tensors.QuantizationFormat members carry the string in ``value``
+        value = "pack-quantized"
+
+    assert resolve_format(w4afp8, _Enum) == CompressionFormat.pack_quantized
+    assert resolve_format(w4afp8, "dense") == CompressionFormat.dense
+    with pytest.raises(ValueError, match="cannot hold"):
+        resolve_format(w4afp8, "float-quantized")
+    with pytest.raises(ValueError, match="cannot hold"):
+        resolve_format(preset_name_to_scheme("FP8", ["Linear"]), "pack-quantized")
+    with pytest.raises(ValueError, match="cannot hold"):
+        resolve_format(preset_name_to_scheme("NVFP4A16", ["Linear"]), "mxfp4-pack-quantized")
+    with pytest.raises(ValueError, match="unknown quantization_format"):
+        resolve_format(w4afp8, "marlin-24")
+    assert resolve_format(preset_name_to_scheme("W8A8", ["Linear"]), "naive-quantized") == "naive-quantized"
+
+
+def test_oneshot_wraps_save_pretrained(tmp_path):
+    """After ``oneshot`` the model's own ``save_pretrained`` takes ``save_compressed`` / ``quantization_format``
+    (reference: entrypoints/utils.py:96, compressed_tensors_utils.py:86-190); wrapping twice changes nothing and
+    an un-quantised model is written as transformers writes it, with no ``quantization_config``."""
+    import json
+
+    from safetensors import safe_open
+    from transformers import LlamaConfig, LlamaForCausalLM
+
+    import llmcompressor_amd
+    from llmcompressor.transformers.compression.compressed_tensors_utils import modify_save_pretrained
+
+    model = LlamaForCausalLM(LlamaConfig(vocab_size=64, hidden_size=32, intermediate_size=64, num_hidden_layers=1,
+                                         num_attention_heads=2, num_key_value_heads=2))
+    llmcompressor_amd.oneshot(model=model, recipe=None)
+    first = model.save_pretrained
+    assert getattr(first, "_overridden", False)
+    modify_save_pretrained(model)
+    assert model.save_pretrained is first
+    model.save_pretrained(str(tmp_path / "a"), save_compressed=True)
+    model.save_pretrained(str(tmp_path / "b"), save_compressed=False, quantization_format="dense")
+    for sub in ("a", "b"):
+        with open(tmp_path / sub / "config.json") as f:
+            assert "quantization_config" not in json.load(f)
+        with safe_open(str(tmp_path / sub / "model.safetensors"), "pt") as f:
+            keys = set(f.keys())
+        assert "model.layers.0.self_attn.q_proj.weight" in keys and not any("observer" in k for k in keys)
+    plain = torch.nn.Linear(4, 4)
+    modify_save_pretrained(plain)  # no ``save_pretrained``: left alone
+    assert not hasattr(plain, "save_pretrained")
+
+
 def test_moe_token_routing_counts():
     # reference: tests/llmcompressor/modeling/test_linear_experts.py:12-106 (hidden 16, inter 32, 4 experts, top-2)
     from llmcompressor_amd.modeling import LinearExperts2D, moe_calibration_context
