@@ -1,7 +1,8 @@
 """oneshot(): apply a recipe to a model with optional calibration data (reference: entrypoints/oneshot.py:316-481).
 
-Accepts an instantiated ``torch.nn.Module`` and a ready ``DataLoader`` / list of batches (the
-reference passes a DataLoader straight through, datasets/utils.py:143-144).  Loading models or
+Accepts an instantiated ``torch.nn.Module`` and, as ``dataset``, a ready ``DataLoader`` / list of batches (the
+reference passes a DataLoader straight through, datasets/utils.py:143-144) or an in-memory ``datasets.Dataset``
+(sampled, truncated and batched as the reference does, ``llmcompressor_amd.datasets``).  Loading models or
 datasets by hub name needs network access and is not part of this build.
 """
 from __future__ import annotations
@@ -38,6 +39,7 @@ class Oneshot:
         self.pipeline = pipeline
         self.stage = stage
         self.save_compressed = save_compressed
+        self.processor = kwargs.pop("processor", None) or kwargs.pop("tokenizer", None)
         self.dataset_args = _DatasetArgs(sequential_targets=sequential_targets, pipeline=pipeline,
                                          moe_calibrate_all_experts=moe_calibrate_all_experts, **kwargs)
 
@@ -57,7 +59,12 @@ class Oneshot:
         if left:
             logger.warning(f"{len(left)} fused expert modules have a layout or forward signature that is not "
                            f"recognised ({left[0]}, ...); they stay as they are and their weights are not quantized.")
-        self.apply_recipe_modifiers(self.dataset)
+        from ..datasets import get_calibration_dataloader
+
+        # an in-memory `datasets.Dataset` becomes a DataLoader (num_calibration_samples, max_seq_length,
+        # batch_size, shuffle_calibration_samples, data_collator, ...); loaders and lists of batches pass through
+        self.apply_recipe_modifiers(get_calibration_dataloader(self.dataset, self.processor,
+                                                               **vars(self.dataset_args)))
         if self.output_dir is not None:
             if getattr(getattr(self.model, "save_pretrained", None), "_overridden", False):
                 # reference: entrypoints/utils.py:122-124

@@ -1505,8 +1505,17 @@ def test_save_pretrained_after_oneshot_writes_the_compressed_checkpoint(tmp_path
                                    num_attention_heads=4, num_key_value_heads=2, vocab_size=256,
                                    max_position_embeddings=128)
     model = transformers.LlamaForCausalLM(cfg).to(torch.bfloat16).to(DEV)
-    data = [{"input_ids": torch.randint(0, 256, (1, 64))} for _ in range(4)]
-    oneshot(model=model, dataset=data, recipe=GPTQModifier(targets="Linear", scheme="W4AFP8", ignore=["lm_head"]))
+    # calibration data as the examples pass it: a tokenised in-memory dataset, sampled and truncated by oneshot
+    datasets = pytest.importorskip("datasets")
+    rows = [torch.randint(0, 256, (n,)).tolist() for n in (80, 64, 72, 96, 40, 66)]
+    ds = datasets.Dataset.from_dict({"input_ids": rows, "attention_mask": [[1] * len(r) for r in rows]})
+    seen = []
+    spy = model.model.embed_tokens.register_forward_pre_hook(lambda m, a: seen.append(tuple(a[0].shape)))
+    oneshot(model=model, dataset=ds, num_calibration_samples=4, max_seq_length=64,
+            shuffle_calibration_samples=False,
+            recipe=GPTQModifier(targets="Linear", scheme="W4AFP8", ignore=["lm_head"]))
+    spy.remove()
+    assert seen and set(seen) == {(1, 64)} and len(seen) % 4 == 0  # the four longest rows, cut to 64 tokens
     lin = model.model.layers[1].mlp.down_proj
     args = lin.quantization_scheme.weights
     assert lin.quantization_scheme.input_activations.type.value == "float"

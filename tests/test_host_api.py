@@ -767,3 +767,83 @@ def test_conv2d_hessian_branch_fails_the_way_the_reference_does(shape):
     assert H.shape == (3, 3)  # weight.shape[1], as in the reference (not in_channels * kernel area)
     with pytest.raises(RuntimeError, match="permute"):
         accumulate_hessian(torch.randn(*shape), conv, H, torch.zeros(1))
+
+
+def test_calibration_dataloader_from_an_in_memory_dataset():
+    """``oneshot(dataset=<datasets.Dataset>, num_calibration_samples=..., max_seq_length=...)`` as the reference's
+    examples call it (datasets/utils.py:122-393): sampler, truncating collator, tokenisation of a text column,
+    pass-through of ready loaders, refusal of hub names."""
+    datasets = pytest.importorskip("datasets")
+    from torch.utils.data import DataLoader
+
+    from llmcompressor.datasets import LengthAwareSampler, get_calibration_dataloader
+
+    lengths = [5, 9, 3, 12, 7, 8]
+    ds = datasets.Dataset.from_dict({
+        "input_ids": [list(range(1, n + 1)) for n in lengths],
+        "attention_mask": [[1] * n for n in lengths],
+    })
+    # longest first without shuffling; the shortest samples are the ones left out
+    loader = get_calibration_dataloader(ds, num_calibration_samples=4, shuffle_calibration_samples=False,
+                                        max_seq_length=10)
+    assert isinstance(loader, DataLoader) and len(loader) == 4
+    batches = list(loader)
+    assert [b["input_ids"].shape for b in batches] == [(1, 10), (1, 9), (1, 8), (1, 7)]
+    assert batches[0]["input_ids"].dtype == torch.int64 and batches[0]["attention_mask"].shape == (1, 10)
+    assert torch.equal(batches[1]["input_ids"][0], torch.arange(1, 10))
+    assert list(LengthAwareSampler(ds, num_samples=3)) == [3, 1, 5]
+    # a batch is cut to its shortest member
+    loader = get_calibration_dataloader(ds, num_calibration_samples=6, shuffle_calibration_samples=False, batch_size=2)
+    assert [tuple(b["input_ids"].shape) for b in loader] == [(2, 9), (2, 7), (2, 3)]
+    # default: a random subset, each sample at most once
+    torch.manual_seed(0)
+    loader = get_calibration_dataloader(ds, num_calibration_samples=5)
+    seen = sorted(int(b["input_ids"].shape[1]) for b in loader)
+    assert len(seen) == 5 and len(set(seen)) == 5 and set(seen) <= set(lengths)
+    # more samples requested than there are
+    assert len(get_calibration_dataloader(ds, num_calibration_samples=512)) == 6
+    # a DatasetDict falls back to its train split; a named split is taken as asked
+    dd = datasets.DatasetDict({"train": ds, "test": ds.select(range(2))})
+    assert len(get_calibration_dataloader(dd)) == 6
+    assert len(get_calibration_dataloader(dd, splits="test")) == 2
+    assert len(get_calibration_dataloader(dd, splits={"calibration": "test"})) == 2
+    with pytest.raises(ValueError, match="train"):
+        get_calibration_dataloader(datasets.DatasetDict({"validation": ds}))
+
+    # a text column is tokenised with truncation and (by default) padding to max_seq_length
+    class Tok:
+        model_max_length = 16
+        calls = []
+
+        def __call__(self, text, padding=False, max_length=None, truncation=False):
+            Tok.calls.append((padding, max_length, truncation))
+            ids = [ord(c) % 50 + 1 for c in text][: max_length if truncation else None]
+            mask = [1] * len(ids)
+            if padding == "max_length":
+                ids, mask = ids + [0] * (max_length - len(ids)), mask + [0] * (max_length - len(mask))
+            return {"input_ids": ids, "attention_mask": mask}
+
+    text = datasets.Dataset.from_dict({"text": ["hello world", "a much longer line of text than that"], "n": [1, 2]})
+    loader = get_calibration_dataloader(text, Tok(), max_seq_length=8, shuffle_calibration_samples=False)
+    got = list(loader)
+    assert set(got[0].keys()) == {"input_ids", "attention_mask"} and got[0]["input_ids"].shape == (1, 8)
+    assert Tok.calls[0] == ("max_length", 8, True)
+    loader = get_calibration_dataloader(text, Tok(), max_seq_length=64, pad_to_max_length=False,
+                                        shuffle_calibration_samples=False)
+    assert [b["input_ids"].shape[1] for b in loader] == [16, 11]  # clipped to the tokenizer's model_max_length
+    with pytest.raises(ValueError, match="tokenize"):
+        get_calibration_dataloader(text)
+    with pytest.raises(ValueError, match="text_column"):
+        get_calibration_dataloader(text, Tok(), text_column="prompt")
+    # pass-through and refusals
+    ready = [{"input_ids": torch.ones(1, 4, dtype=torch.long)}]
+    assert get_calibration_dataloader(ready) is ready
+    dl = DataLoader(ready)
+    assert get_calibration_dataloader(dl) is dl and get_calibration_dataloader(None) is None
+    with pytest.raises(ValueError, match="network"):
+        get_calibration_dataloader("open_platypus")
+    with pytest.raises(ValueError, match="Unknown data collator"):
+        get_calibration_dataloader(ds, data_collator="nope")
+    custom = get_calibration_dataloader(ds, data_collator=lambda feats: {"n": len(feats)}, batch_size=3,
+                                        shuffle_calibration_samples=False)
+    assert [b["n"] for b in custom] == [3, 3]
