@@ -60,6 +60,11 @@ class Oneshot:
             logger.warning(f"{len(left)} fused expert modules have a layout or forward signature that is not "
                            f"recognised ({left[0]}, ...); they stay as they are and their weights are not quantized.")
         from ..datasets import get_calibration_dataloader
+        from ..pipelines.onload import place_model
+
+        # reference: set_onload_device(model, get_main_device()) at the head of every pipeline -- a model that
+        # arrives on the host is computed on the GPU: moved there whole if it fits, else layer by layer
+        self.dataset_args.onload_device = place_model(self.model)
 
         # an in-memory `datasets.Dataset` becomes a DataLoader (num_calibration_samples, max_seq_length,
         # batch_size, shuffle_calibration_samples, data_collator, ...); loaders and lists of batches pass through

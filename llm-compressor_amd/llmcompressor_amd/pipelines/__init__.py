@@ -124,7 +124,24 @@ class SequentialPipeline(CalibrationPipeline):
     def __call__(self, model, dataloader, dataset_args=None):
         targets = getattr(dataset_args, "sequential_targets", None) if dataset_args is not None else None
         layers = find_decoder_layers(model, targets)
-        device = next(model.parameters()).device
+        # a model too large to stay on the GPU: what surrounds the layers (embeddings, final norm, head) is
+        # brought over for the whole run, each layer for its two passes, and everything returns to the host
+        onload = getattr(dataset_args, "onload_device", None) if dataset_args is not None else None
+        home = next(model.parameters()).device
+        device = onload if onload is not None else home
+        inside = {id(x) for l in layers for x in l.modules()}
+        rest = [m for m in model.modules() if id(m) not in inside]
+        if onload is not None:
+            for m in rest:
+                m._apply(lambda t: t.to(onload), recurse=False)
+        try:
+            self._run(model, dataloader, dataset_args, layers, rest, device, onload, home)
+        finally:
+            if onload is not None:
+                for m in model.modules():
+                    m._apply(lambda t: t.to(home), recurse=False)
+
+    def _run(self, model, dataloader, dataset_args, layers, rest, device, onload, home):
         LifecycleCallbacks.calibration_start()
         with calibration_forward_context(model), DisableQuantization(model):
             # capture the first layer's inputs for every batch (activations stay on the device)
@@ -134,8 +151,6 @@ class SequentialPipeline(CalibrationPipeline):
                 captured.append((args, kwargs))
                 raise _StopForward()
 
-            inside = {id(x) for l in layers for x in l.modules()}
-            rest = [m for m in model.modules() if id(m) not in inside]
             before = set()  # modules that run ahead of the first layer (their hooks fire in this capture pass)
             trackers = [m.register_forward_pre_hook(lambda mod, args: before.add(id(mod))) for m in rest]
             handle = layers[0].register_forward_pre_hook(grab, with_kwargs=True)
@@ -161,6 +176,8 @@ class SequentialPipeline(CalibrationPipeline):
             del captured
             returns_tuple = False
             for idx, layer in enumerate(layers):
+                if onload is not None:
+                    layer.to(onload)
                 # pass 1: calibrate (hooks fire: Hessians / activation observers)
                 for inputs in cache.iter_prefetch():
                     layer(*inputs["args"], **inputs["kwargs"])
@@ -173,6 +190,8 @@ class SequentialPipeline(CalibrationPipeline):
                         returns_tuple = isinstance(out, (tuple, list))
                         hidden = out[0] if returns_tuple else out
                         cache.update(i, {"args": (hidden,) + tuple(inputs["args"][1:])})
+                if onload is not None:
+                    layer.to(home)
             # what follows the last layer (final norm, lm_head): the reference's last traced subgraph holds it
             # (pipelines/sequential/pipeline.py:136-181), so a module there that a modifier hooked is calibrated too
             tail = [m for m in rest if id(m) not in before and _has_calibration_hooks(m)]
@@ -248,6 +267,7 @@ def _handles_of(module: torch.nn.Module):
 @CalibrationPipeline.register("datafree")
 class DataFreePipeline(CalibrationPipeline):
     def __call__(self, model, dataloader=None, dataset_args=None):
+        _refuse_layerwise(dataset_args, "datafree")
         LifecycleCallbacks.calibration_start()
         LifecycleCallbacks.sequential_epoch_end(modules=list(model.modules()))
         LifecycleCallbacks.calibration_end()
@@ -256,6 +276,7 @@ class DataFreePipeline(CalibrationPipeline):
 @CalibrationPipeline.register("basic")
 class BasicPipeline(CalibrationPipeline):
     def __call__(self, model, dataloader, dataset_args=None):
+        _refuse_layerwise(dataset_args, "basic")
         device = next(model.parameters()).device
         LifecycleCallbacks.calibration_start()
         with calibration_forward_context(model):
@@ -279,6 +300,14 @@ class IndependentPipeline(CalibrationPipeline):
                 pipeline(model, dataloader, dataset_args)
         finally:
             recipe.modifiers = mods
+
+
+def _refuse_layerwise(dataset_args, name: str):
+    if dataset_args is not None and getattr(dataset_args, "onload_device", None) is not None:
+        raise RuntimeError(
+            f"the model does not fit in GPU memory and the {name!r} pipeline works on the whole model at once; "
+            "quantise the checkpoint shard by shard with `model_free_ptq`, or use a recipe that calibrates "
+            "through the sequential pipeline")
 
 
 def _to_device(batch, device):

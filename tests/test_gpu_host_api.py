@@ -1557,6 +1557,55 @@ def test_save_pretrained_after_oneshot_writes_the_compressed_checkpoint(tmp_path
     assert qd["format"] == "dense" and qd["quantization_status"] == "frozen"
 
 
+def test_a_model_on_the_host_is_calibrated_on_the_gpu(monkeypatch):
+    """The reference's examples hand ``oneshot`` a model that sits in host memory and its pipelines onload it
+    (pipelines/sequential/pipeline.py:85-87).  Here a model that fits is moved to the GPU and stays there; one that
+    does not is calibrated with one layer on the GPU at a time and ends where it came from.  Both give the bits
+    of the run on a model its caller placed on the GPU."""
+    transformers = pytest.importorskip("transformers")
+
+    from llmcompressor_amd import oneshot
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+    from llmcompressor_amd.modifiers.quantization import QuantizationModifier
+    from llmcompressor_amd.pipelines import onload
+
+    def make():
+        torch.manual_seed(0)
+        cfg = transformers.LlamaConfig(hidden_size=128, intermediate_size=256, num_hidden_layers=3,
+                                       num_attention_heads=4, num_key_value_heads=2, vocab_size=256,
+                                       max_position_embeddings=128)
+        return transformers.LlamaForCausalLM(cfg).to(torch.bfloat16)
+
+    torch.manual_seed(1)
+    data = [{"input_ids": torch.randint(0, 256, (1, 64))} for _ in range(4)]
+
+    def run(model):
+        oneshot(model=model, dataset=data,
+                recipe=GPTQModifier(targets=["Linear"], scheme="W4A16", ignore=[]))  # lm_head too: the tail pass
+        return {k: v.detach().cpu() for k, v in model.state_dict().items()}
+
+    placed = make().to(DEV)
+    want = run(placed)
+    resident = make()
+    got = run(resident)
+    assert all(p.device.type == "cuda" for p in resident.parameters())
+    assert want.keys() == got.keys() and all(torch.equal(want[k], got[k]) for k in want)
+
+    monkeypatch.setattr(onload, "RESIDENT_FRACTION", 0.0)
+    streamed = make()
+    where = []
+    probe = streamed.model.layers[1].mlp.down_proj.register_forward_pre_hook(
+        lambda m, a: where.append((m.weight.device.type, streamed.model.layers[2].mlp.down_proj.weight.device.type)))
+    got = run(streamed)
+    probe.remove()
+    assert where and set(where) == {("cuda", "cpu")}  # layer 1 computes on the GPU while layer 2 waits on the host
+    assert all(p.device.type == "cpu" for p in streamed.parameters())
+    assert all(b.device.type == "cpu" for b in streamed.buffers())
+    assert want.keys() == got.keys() and all(torch.equal(want[k], got[k]) for k in want)
+    with pytest.raises(RuntimeError, match="model_free_ptq"):
+        oneshot(model=make(), recipe=QuantizationModifier(targets="Linear", scheme="FP8_DYNAMIC", ignore=["lm_head"]))
+
+
 def test_gptq_beats_round_to_nearest_end_to_end_on_a_transformers_llama():
     """The whole pipeline on a 4-layer transformers Llama with anisotropic activations: W4A16 through
     GPTQModifier (sequential, error feedback from calibration data) gives a clearly smaller logit error on
