@@ -18,7 +18,7 @@ from torch.utils.data import DataLoader, RandomSampler, Sampler
 logger = logging.getLogger("llmcompressor_amd")
 
 __all__ = ["get_calibration_dataloader", "format_calibration_data", "DataCollatorWithTruncation",
-           "LengthAwareSampler", "DATASET_DEFAULTS"]
+           "LengthAwareSampler", "DATASET_DEFAULTS", "get_rank_partition"]
 
 # reference: args/dataset_arguments.py (the fields this path reads, with their defaults)
 DATASET_DEFAULTS = dict(num_calibration_samples=512, shuffle_calibration_samples=True, batch_size=1,
@@ -192,3 +192,18 @@ def get_calibration_dataloader(dataset, processor=None, **args):
     if "input_ids" not in dataset.column_names:
         dataset = _tokenize(dataset, processor, a)
     return format_calibration_data(dataset, processor, **a)
+
+
+def get_rank_partition(split: str, num_samples: int) -> str:
+    """``"train[start:end]"`` for this process's share of ``num_samples`` (reference: datasets/utils.py:398-431);
+    with one process that is all of them."""
+    import math
+
+    import torch.distributed as dist
+
+    assert "[" not in split, "Split string should not already contain partitioning brackets"
+    rank = dist.get_rank() if dist.is_available() and dist.is_initialized() else 0
+    world = dist.get_world_size() if dist.is_available() and dist.is_initialized() else 1
+    start = math.floor(num_samples * (rank / world))
+    end = math.floor(num_samples * ((rank + 1) / world))
+    return f"{split}[{start}:{end}]"

@@ -130,8 +130,8 @@ class LinearExperts2D(nn.ModuleList):
         bf16 Linears of one shape, gradients are recorded, or the shapes do not fit the kernel's tiles.  The
         grouped products add along k in another order than the library GEMM behind ``F.linear``: same values to
         the last bf16 digit, not the same bits, which is why observed passes keep the loop."""
-        from ..modifiers.utils.hooks import hook_is_inert
-        from .. import ops
+        from ...modifiers.utils.hooks import hook_is_inert
+        from ... import ops
 
         if (not hidden_states.is_cuda or hidden_states.dtype != torch.bfloat16 or torch.is_grad_enabled()
                 or len(self) == 0 or nn.modules.module._global_forward_hooks
@@ -191,7 +191,7 @@ class LinearExperts2D(nn.ModuleList):
 
     def _forward_grouped(self, plan, routed: torch.Tensor, counts) -> torch.Tensor:
         """``expert(rows)`` for every expert's rows of ``routed`` (sorted by expert) in two launches."""
-        from .. import ops
+        from ... import ops
 
         E, inter = self.num_experts, plan["inter"]
         tiles, ntiles = ops.grouped_linear_tiles(counts, routed.device)

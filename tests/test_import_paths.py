@@ -34,6 +34,67 @@ def test_llmcompressor_root_is_an_alias_of_this_package():
         importlib.import_module("llmcompressor.no_such_module")
 
 
+# import lines of the reference's examples, docs and tests that touch this path (examples/quantization_*,
+# examples/quantizing_moe, examples/model_free_ptq, examples/big_models_with_sequential_onloading, docs/guides)
+_REFERENCE_IMPORT_LINES = [
+    "from llmcompressor import oneshot, model_free_ptq",
+    "from llmcompressor.transformers import oneshot",
+    "from llmcompressor.modifiers import Modifier",
+    "from llmcompressor.modifiers.gptq import GPTQModifier",
+    "from llmcompressor.modifiers.quantization import GPTQModifier, QuantizationModifier",
+    "from llmcompressor.modifiers.pruning import SparseGPTModifier",
+    "from llmcompressor.modifiers.pruning.sparsegpt import SparseGPTModifier",
+    "from llmcompressor.modifiers.obcq import SparseGPTModifier",
+    "from llmcompressor.modifiers.gptq.gptq_quantize import quantize_weight, accumulate_hessian, make_empty_hessian",
+    "from llmcompressor.modifiers.pruning.sparsegpt.sgpt_sparsify import sparsify_weight",
+    "from llmcompressor.modifiers.quantization.calibration import initialize_observer, update_qparams, observe",
+    "from llmcompressor.modifiers.utils.hooks import HooksMixin",
+    "from llmcompressor.observers import Observer",
+    "from llmcompressor.observers.base import Observer, QParamsDict",
+    "from llmcompressor.observers.helpers import flatten_for_calibration",
+    "from llmcompressor.core import State, Event, EventType",
+    "from llmcompressor.core import active_session, create_session, reset_session",
+    "from llmcompressor.recipe import Recipe",
+    "from llmcompressor.args import DatasetArguments",
+    "from llmcompressor.utils import load_context, dispatch_for_generation",
+    "from llmcompressor.utils.dev import get_main_device",
+    "from llmcompressor.utils.helpers import calibration_forward_context, DisableQuantization",
+    "from llmcompressor.datasets.utils import get_rank_partition, get_calibration_dataloader",
+    "from llmcompressor.pipelines.cache import IntermediatesCache",
+    "from llmcompressor.pipelines.registry import CalibrationPipeline",
+    "from llmcompressor.modeling.moe.linear_experts import LinearExperts2D",
+    "from llmcompressor.modeling.moe.linearize import linearize_moe, load_quantizable_moe",
+    "from llmcompressor.modeling.moe.context import moe_calibration_context",
+    "from llmcompressor.entrypoints.model_free import model_free_ptq",
+    "from llmcompressor.transformers.compression.compressed_tensors_utils import modify_save_pretrained",
+]
+
+
+@pytest.mark.parametrize("line", _REFERENCE_IMPORT_LINES)
+def test_reference_import_lines_resolve(line):
+    import llmcompressor  # noqa: F401
+
+    scope = {}
+    exec(line, scope)
+    names = [n.strip() for n in line.split(" import ")[1].split(",")]
+    assert all(scope[n] is not None for n in names)
+
+
+def test_helpers_the_examples_wrap_their_loading_in():
+    import torch
+
+    from llmcompressor.datasets.utils import get_rank_partition
+    from llmcompressor.modeling.moe.linearize import load_quantizable_moe
+    from llmcompressor.utils import dispatch_for_generation, load_context
+
+    with load_context(), load_quantizable_moe():
+        model = torch.nn.Linear(4, 4)
+    assert dispatch_for_generation(model) is model  # no GPU here: stays on the host
+    assert get_rank_partition("train_sft", 256) == "train_sft[0:256]"
+    with pytest.raises(AssertionError):
+        get_rank_partition("train[:5]", 5)
+
+
 @pytest.mark.parametrize("root", ["llmcompressor", "llmcompressor_amd"])
 def test_deprecated_gptq_location_warns_and_reexports(root):
     import llmcompressor  # noqa: F401  (installs the alias finder)
