@@ -331,9 +331,9 @@ def model_free_ptq(model_stub, save_directory, scheme=None, config: Optional[Qua
         raise NotImplementedError("checkpoint converters are not part of this build")
     model_files = _checkpoint_files(model_stub)
     config = validate_config(config, scheme, ignore)
+    if isinstance(device, (list, tuple)):  # the reference spreads shards over several GPUs; one GPU here
+        device = device[0] if device else None
     device = torch.device(device if device is not None else "cuda:0")
-    if isinstance(device, (list, tuple)):
-        device = torch.device(device[0])
     os.makedirs(save_directory, exist_ok=True)
 
     for rel, path in model_files.items():

@@ -497,7 +497,7 @@ def test_model_free_ptq_round_trip(tmp_path, scheme):
         sch = QuantizationScheme(targets=["Linear"], weights=QuantizationArgs(num_bits=4, strategy="group", group_size=32))
         total, wmap = model_free_ptq(src, dst, scheme=sch, ignore=ignore, device="cuda:0")
     else:
-        total, wmap = model_free_ptq(src, dst, scheme=scheme, ignore=ignore, device="cuda:0")
+        total, wmap = model_free_ptq(src, dst, scheme=scheme, ignore=ignore, device=["cuda:0"])
     out = {}
     for fn in sorted(set(wmap.values())):
         with safe_open(f"{dst}/{fn}", framework="pt") as f:
