@@ -259,11 +259,12 @@ def probe_sparsegpt():
         W = (torch.randn(R, K, device="cuda") * 0.02).bfloat16()
         H0 = torch.zeros(K, K, device="cuda")
         ops.hessian_accumulate_(H0, x)
-        t_f = timed(lambda: ops.gptq_hinv_(H0.clone(), None, divisor=4.0))
-        U, dead, _ = ops.gptq_hinv_(H0.clone(), None, divisor=4.0)
-        t_u = timed(lambda: ops.sparsegpt_sparsify(W, U, 0.5, dead=dead))
-        t_s = timed(lambda: ops.sparsegpt_sparsify(W, U, 0.5, prune_n=2, prune_m=4, dead=dead))
-        Q, _ = ops.sparsegpt_sparsify(W, U, 0.5, dead=dead)
+        form = ops.gptq_factor_form(K, 128)  # what sparsify_weight picks at this width
+        t_f = timed(lambda: ops.gptq_hinv_(H0.clone(), None, divisor=4.0, form=form))
+        U, dead, _ = ops.gptq_hinv_(H0.clone(), None, divisor=4.0, form=form)
+        t_u = timed(lambda: ops.sparsegpt_sparsify(W, U, 0.5, dead=dead, form=form))
+        t_s = timed(lambda: ops.sparsegpt_sparsify(W, U, 0.5, prune_n=2, prune_m=4, dead=dead, form=form))
+        Q, _ = ops.sparsegpt_sparsify(W, U, 0.5, dead=dead, form=form)
         print(f"| {R} x {K} | {t_f:.2f} | {t_u:.2f} | {t_s:.2f} | {(Q == 0).float().mean().item():.4f} |")
         if keep is None:
             keep = (x.cpu(), W.cpu())
@@ -297,8 +298,8 @@ def probe_chain():
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / n
 
-    print("| Linear (rows x columns) | Cholesky chain ms | column loop ms |")
-    print("|---|---|---|")
+    print("| Linear (rows x columns) | Cholesky chain ms | column loop ms | chain, full inverse factor ms | loop on it ms |")
+    print("|---|---|---|---|---|")
     for R, K in ((HIDDEN, HIDDEN), (INTER, HIDDEN), (HIDDEN, INTER)):
         torch.manual_seed(0)
         x = torch.randn(16384, K, device="cuda").bfloat16()
@@ -309,20 +310,26 @@ def probe_chain():
         perm = torch.argsort(torch.diagonal(H0), descending=True, stable=True).to(torch.int32)
         work = torch.empty_like(H0)
 
-        def chain():
-            work.copy_(H0)
-            return ops.gptq_hinv_(work, perm, divisor=8.0)
-
-        t_copy = timed(lambda: work.copy_(H0))
-        t_chain = timed(chain) - t_copy
-        U, dead, _ = ops.gptq_hinv_(H0.clone(), perm, divisor=8.0)
         mn, mx = ops.minmax_groups(W, 128)
         scale, _, _ = ops.calculate_qparams(mn, mx, ops.FMT_INT, 4, True)
         g_idx = (torch.arange(K, dtype=torch.int32, device="cuda") // 128)[perm.long()]
-        t_loop = timed(lambda: ops.gptq_quantize(W, U, scale, None, ops.FMT_INT, 4, 1, K // 128, g_idx=g_idx,
-                                                 perm=perm, dead=dead))
-        print(f"| {R} x {K} | {t_chain:.2f} | {t_loop:.2f} |")
-        del H0, work, U
+        t_copy = timed(lambda: work.copy_(H0))
+        cells = []
+        # the form quantize_weight uses at this width (the factor of H outside 512-column diagonal blocks), then the
+        # reference's full inverse factor
+        for form in (ops.gptq_factor_form(K, 128), ops.FACTOR_INVERSE):
+            def chain():
+                work.copy_(H0)
+                return ops.gptq_hinv_(work, perm, divisor=8.0, form=form)
+
+            t_chain = timed(chain) - t_copy
+            U, dead, _ = ops.gptq_hinv_(H0.clone(), perm, divisor=8.0, form=form)
+            t_loop = timed(lambda: ops.gptq_quantize(W, U, scale, None, ops.FMT_INT, 4, 1, K // 128, g_idx=g_idx,
+                                                     perm=perm, dead=dead, form=form))
+            cells += [f"{t_chain:.2f}", f"{t_loop:.2f}"]
+            del U
+        print(f"| {R} x {K} | " + " | ".join(cells) + " |")
+        del H0, work
 
     print()
     print("| fp32 product C -= A B (llmc_sgemm) | M | N | K | us | TFLOP/s of the non-zero part |")

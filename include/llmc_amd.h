@@ -251,11 +251,26 @@ int llmc_dynamic_per_token_quantize(const void* x, int32_t x_dtype, int64_t N, i
  * non-positive pivot; in that case H becomes the identity, which is the
  * reference's round-to-nearest fallback on _LinAlgError (gptq_quantize.py:157-164).
  * perm may be NULL.  workspace must be 256-byte aligned.
+ *
+ * form selects what H holds afterwards.  LLMC_FACTOR_INVERSE: U as above.  LLMC_FACTOR_GROUPS (K a multiple of
+ * 512): inside every aligned 512-column diagonal block the same U (a diagonal block of the inverse of a
+ * triangular matrix is the inverse of its diagonal block); outside those blocks the upper Cholesky factor V of
+ * the damped H itself (V V^T = H, V = U^-1), i.e. the chain stops before the triangular inverse is carried
+ * across blocks, which is a third of its arithmetic.  llmc_gptq_quantize takes either form and gives the same
+ * result up to fp32 rounding, and so does llmc_sparsegpt_sparsify (its block size must then be 128).
+ * llmc_gptq_factor_form(K, blocksize) is the form the library prefers for a quantize_weight / sparsify_weight
+ * call.
  */
+enum {
+  LLMC_FACTOR_INVERSE = 0,
+  LLMC_FACTOR_GROUPS = 1,
+  LLMC_FACTOR_GROUP_WIDTH = 512
+};
+int32_t llmc_gptq_factor_form(int64_t K, int32_t blocksize);
 int64_t llmc_gptq_hinv_workspace_bytes(int64_t K);
 int llmc_gptq_hinv(float* H, int64_t ldh, int64_t K, const int32_t* perm, float divisor,
-                   float percdamp, uint8_t* dead_out, void* workspace, int64_t workspace_bytes,
-                   int32_t* info_out, void* stream);
+                   float percdamp, int32_t form, uint8_t* dead_out, void* workspace,
+                   int64_t workspace_bytes, int32_t* info_out, void* stream);
 
 /* Column order of GPTQ's activation ordering (gptq_quantize.py:131-140: argsort of diag(H), descending): for each of
  * the n Hessians (HOST array of n device pointers, fp32 [K, K], row stride ldh) the column numbers ordered by
@@ -273,7 +288,7 @@ int llmc_diag_argsort_desc(const float* const* H, int64_t ldh, int32_t n, int64_
 int64_t llmc_gptq_hinv_grouped_workspace_bytes(int64_t n, int64_t K);
 int llmc_gptq_hinv_grouped(const float* const* H, int64_t ldh, int32_t n, int64_t K,
                            const int32_t* const* perm, const float* divisors, float percdamp,
-                           uint8_t* dead_out, float* U_out, int64_t ldu, void* workspace,
+                           int32_t form, uint8_t* dead_out, float* U_out, int64_t ldu, void* workspace,
                            int64_t workspace_bytes, int32_t* info_out, void* stream);
 
 /* ---- a8/a9: GPTQ block column loop ---------------------------------------------
@@ -288,6 +303,11 @@ int llmc_gptq_hinv_grouped(const float* const* H, int64_t ldh, int32_t n, int64_
  * (per tensor: row_div >= R; per channel: row_div 1, stride 1; per group: stride K/g and
  * g_idx[c] = group of permuted column c; block strategy: row_div = block height).
  * blocksize above 128 runs as 128-wide blocks (same result up to fp32 summation order).
+ *
+ * form says what U holds (see llmc_gptq_hinv).  With LLMC_FACTOR_GROUPS (blocksize >= 128) the columns beyond a
+ * 512-column group are not updated after the group; instead each group first takes what all earlier groups owe it,
+ *     W[:, G] += ((W0 - Q)[:, :g0] @ V[:g0, G]) @ U[G, G]        (W0: the weights before the loop, Q: quantised),
+ * which equals -Err[:, :g0] @ U[:g0, G] without ever forming U outside the diagonal blocks.
  */
 int64_t llmc_gptq_quantize_workspace_bytes(int64_t R, int64_t K);
 int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R, int64_t K, int64_t ldw,
@@ -295,7 +315,7 @@ int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R, int64_t K
                        const void* scale, int32_t scale_dtype, const int8_t* zero_point,
                        const float* global_scale, const int32_t* g_idx, int64_t row_div,
                        int64_t scale_row_stride, int32_t fmt, int32_t num_bits, int32_t blocksize,
-                       void* out_weight, int64_t ldo, float* loss_out, void* workspace,
+                       int32_t form, void* out_weight, int64_t ldo, float* loss_out, void* workspace,
                        int64_t workspace_bytes, void* stream);
 
 /* Grouped form of llmc_gptq_quantize for n problems of one shape and scheme (the expert Linears of an MoE
@@ -310,8 +330,8 @@ int llmc_gptq_quantize_grouped(const void* const* weight, int32_t w_dtype, int32
                                int32_t scale_dtype, const int8_t* const* zero_point,
                                const float* const* global_scale, const int32_t* const* g_idx,
                                int64_t row_div, int64_t scale_row_stride, int32_t fmt, int32_t num_bits,
-                               int32_t blocksize, void* const* out_weight, int64_t ldo, float* loss_out,
-                               void* workspace, int64_t workspace_bytes, void* stream);
+                               int32_t blocksize, int32_t form, void* const* out_weight, int64_t ldo,
+                               float* loss_out, void* workspace, int64_t workspace_bytes, void* stream);
 
 /* ---- fp32 product of the lazy trailing updates ----------------------------------------------------
  * Replaces the matmul of W[:, i2:] -= Err1.matmul(Hinv[i1:i2, i2:]) (gptq_quantize.py:245) and the products
@@ -351,7 +371,7 @@ int llmc_sgemm(const float* A, int64_t lda, const float* B, int64_t ldb, float* 
 int64_t llmc_sparsegpt_workspace_bytes(int64_t R, int64_t K);
 int llmc_sparsegpt_sparsify(const void* weight, int32_t w_dtype, int64_t R, int64_t K, int64_t ldw,
                             const float* U, int64_t ldu, const uint8_t* dead, double sparsity,
-                            int32_t prune_n, int32_t prune_m, int32_t blocksize,
+                            int32_t prune_n, int32_t prune_m, int32_t blocksize, int32_t form,
                             int32_t preserve_sparsity_mask, void* out_weight, int64_t ldo,
                             float* loss_out, void* workspace, int64_t workspace_bytes, void* stream);
 

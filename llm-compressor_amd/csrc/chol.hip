@@ -513,10 +513,28 @@ extern "C" int64_t llmc_gptq_hinv_workspace_bytes(int64_t K) {
   return (Kp * Kp + hinv_temp_floats(Kp) + 64) * 4 + 256;
 }
 
+// Width up to which the inverse of the factor is formed: everything for LLMC_FACTOR_INVERSE, the aligned
+// 512-wide diagonal blocks for LLMC_FACTOR_GROUPS (the recursive doubling stops there, which leaves the Cholesky
+// factor itself outside those blocks; in the reversed index order of the work matrix the blocks start at
+// multiples of 512 exactly when K is one).
+inline int64_t inverse_width(int32_t form, int64_t Kp) { return form == LLMC_FACTOR_GROUPS ? LLMC_FACTOR_GROUP_WIDTH : Kp; }
+
+// The chain saves the part of the triangular inverse that crosses blocks (a third of its arithmetic, growing with
+// K^3: 0.6 ms at K = 4096, 7.3 ms at 14336), the column loop pays three more launches and one 512-wide product per
+// group (0.06 - 0.1 ms per group, growing with K): from 8192 columns on the first outweighs the second for every
+// number of rows; at 4096 columns the two cancel.
+constexpr int64_t FACTOR_GROUPS_MIN_K = 8192;
+
+extern "C" int32_t llmc_gptq_factor_form(int64_t K, int32_t blocksize) {
+  return (K % LLMC_FACTOR_GROUP_WIDTH == 0 && K >= FACTOR_GROUPS_MIN_K && blocksize >= 128) ? LLMC_FACTOR_GROUPS
+                                                                                             : LLMC_FACTOR_INVERSE;
+}
+
 extern "C" int llmc_gptq_hinv(float* H, int64_t ldh, int64_t K, const int32_t* perm, float divisor,
-                              float percdamp, uint8_t* dead_out, void* workspace, int64_t workspace_bytes,
-                              int32_t* info_out, void* stream) {
+                              float percdamp, int32_t form, uint8_t* dead_out, void* workspace,
+                              int64_t workspace_bytes, int32_t* info_out, void* stream) {
   LLMC_CHECK_ARG(H != nullptr, 1);
+  LLMC_CHECK_ARG(form == LLMC_FACTOR_INVERSE || (form == LLMC_FACTOR_GROUPS && K % LLMC_FACTOR_GROUP_WIDTH == 0), 7);
   LLMC_CHECK_ARG(ldh >= K, 2);
   LLMC_CHECK_ARG(K > 0 && K <= 65536, 3);
   LLMC_CHECK_ARG(divisor != 0.f, 5);
@@ -551,7 +569,7 @@ extern "C" int llmc_gptq_hinv(float* H, int64_t ldh, int64_t K, const int32_t* p
   }
 
   // inverse by recursive doubling: [[X11,0],[X21,X22]] with X21 = -X22 * L21 * X11
-  for (int64_t s = NB; s < Kp; s *= 2) {
+  for (int64_t s = NB; s < inverse_width(form, Kp); s *= 2) {
     const int64_t full = Kp / (2 * s);
     const int64_t rem = Kp % (2 * s);
     const int64_t step = 2 * s * ((int64_t)Kp + 1);
@@ -601,9 +619,10 @@ extern "C" int64_t llmc_gptq_hinv_grouped_workspace_bytes(int64_t n, int64_t K) 
 
 extern "C" int llmc_gptq_hinv_grouped(const float* const* H, int64_t ldh, int32_t n, int64_t K,
                                       const int32_t* const* perm, const float* divisors, float percdamp,
-                                      uint8_t* dead_out, float* U_out, int64_t ldu, void* workspace,
+                                      int32_t form, uint8_t* dead_out, float* U_out, int64_t ldu, void* workspace,
                                       int64_t workspace_bytes, int32_t* info_out, void* stream) {
   LLMC_CHECK_ARG(H != nullptr && ldh >= K, 1);
+  LLMC_CHECK_ARG(form == LLMC_FACTOR_INVERSE || (form == LLMC_FACTOR_GROUPS && K % LLMC_FACTOR_GROUP_WIDTH == 0), 8);
   LLMC_CHECK_ARG(n >= 0 && n <= 4096, 3);
   if (n == 0) return 0;
   LLMC_CHECK_ARG(K > 0 && K <= 65536, 4);
@@ -661,7 +680,7 @@ extern "C" int llmc_gptq_hinv_grouped(const float* const* H, int64_t ldh, int32_
     if (frc) return frc;
   }
 
-  for (int64_t s = NB; s < Kp; s *= 2) {
+  for (int64_t s = NB; s < inverse_width(form, Kp); s *= 2) {
     const int64_t full = Kp / (2 * s);
     const int64_t rem = Kp % (2 * s);
     const int64_t step = 2 * s * ((int64_t)Kp + 1);

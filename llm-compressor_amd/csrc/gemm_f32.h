@@ -26,6 +26,9 @@ struct GemmF32 {
   // batching over blockIdx.z
   int batch;
   int64_t stride_a, stride_b, stride_c;
+  // contraction length of the last block of the batch when it differs from Kc (a contraction cut into
+  // `batch` pieces whose last one is shorter); 0 = Kc like the others
+  int kc_last;
   // second batch level (independent problems, each with `batch` blocks): blockIdx.z = b + batch * b2;
   // 0 or 1 = none
   int batch2;

@@ -214,7 +214,7 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(GemmF32 g, int vec) {
   const float* B = g.B + (int64_t)b1 * g.stride_b + (int64_t)b2 * g.stride2_b;
   float* C = g.C + (int64_t)b1 * g.stride_c + (int64_t)b2 * g.stride2_c;
   const int k_begin = g.b_lower_tri ? (n0 / BK) * BK : 0;
-  int k_end = g.Kc;
+  int k_end = (g.kc_last > 0 && b1 == g.batch - 1) ? g.kc_last : g.Kc;
   if (g.a_lower_tri && m0 + BM < k_end) k_end = m0 + BM;
   if (ALL_FAST) {
     gemm_tile<BM, BN, TRANS_B, true, TRANS_A>(g, A, B, C, m0, n0, k_begin, k_end, As, Bs);
@@ -276,7 +276,8 @@ static int gemm_f32_mfma(const GemmF32& g, hipStream_t st) {
   // are multiples of BK for both tile sizes)
   // (and the unconditional epilogue addresses a wave's strip of C with 32-bit byte offsets, up to 132 rows of ldc
   // floats from the strip's origin: rows of 4M floats and more take the per-element path with 64-bit addresses)
-  const bool all_fast = vec && g.M % bt == 0 && g.N % bt == 0 && g.Kc % BK == 0 && g.ldc < (1 << 22);
+  const bool all_fast = vec && g.M % bt == 0 && g.N % bt == 0 && g.Kc % BK == 0 && g.kc_last % BK == 0 &&
+                        g.ldc < (1 << 22);
   dim3 grid((g.N + bt - 1) / bt, (g.M + bt - 1) / bt, g.batch * nb2);
 #define LLMC_GEMM(BT, TB, AF) hipLaunchKernelGGL((gemm_f32_kernel<BT, BT, TB, AF>), grid, dim3(256), 0, st, g, vec)
   if (g.trans_a) {

@@ -158,7 +158,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) __attribute__((amdgpu_waves
   const float* B = g.B + (int64_t)b1 * g.stride_b + (int64_t)b2 * g.stride2_b;
   float* Cm = g.C + (int64_t)b1 * g.stride_c + (int64_t)b2 * g.stride2_c;
   const int k_begin = g.b_lower_tri ? (n0 / XK) * XK : 0;
-  int k_end = g.Kc;
+  int k_end = (g.kc_last > 0 && b1 == g.batch - 1) ? g.kc_last : g.Kc;
   if (g.a_lower_tri && m0 + BM < k_end) k_end = m0 + BM;
   const int nsteps = (k_end - k_begin) / XK;
 
@@ -345,7 +345,7 @@ int llmc_gemm_x3(const GemmF32& g, hipStream_t st) {
   const bool aligned = (g.lda & 3) == 0 && (g.ldb & 3) == 0 && (((uintptr_t)g.A | (uintptr_t)g.B) & 15) == 0 &&
                        (g.stride_a & 3) == 0 && (g.stride_b & 3) == 0 &&
                        (nb2 == 1 || ((g.stride2_a & 3) == 0 && (g.stride2_b & 3) == 0));
-  if (!aligned || g.Kc % XK || g.Kc < 64) return -1;
+  if (!aligned || g.Kc % XK || g.Kc < 64 || g.kc_last % XK) return -1;
   // the epilogue addresses a wave's strip of C with 32-bit byte offsets (up to 68 rows of ldc floats from the
   // strip's origin): wider rows than this go to the fp32 kernel's 64-bit path
   if (g.ldc >= (1 << 22)) return -1;

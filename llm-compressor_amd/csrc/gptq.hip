@@ -819,12 +819,19 @@ __global__ __launch_bounds__(256) void sgpt_mask_kernel(const float* __restrict_
   if (i < n) mask[i] = Wf[i] == 0.f ? 1 : 0;
 }
 
-// the trailing updates leave preserved zeros alone: put them back after an unmasked product
+// the trailing updates leave preserved zeros alone: put them back after an unmasked product.  In the left-looking
+// form the update that is thrown away here has to stay visible to the later groups (their share of the earlier
+// errors is computed from W0 - Q, which equals Err U only while every update is kept): it is taken out of the
+// group's copy of W0 in Df, so that W0 - Q becomes what Err U is.
 __global__ __launch_bounds__(256) void sgpt_rezero_kernel(float* __restrict__ Wf, const uint8_t* __restrict__ mask,
-                                                          int K, int c0, int c1) {
+                                                          int K, int c0, int c1, float* __restrict__ Df) {
   const int c = c0 + blockIdx.x * 256 + threadIdx.x;
   const int r = blockIdx.y;
-  if (c < c1 && mask[(int64_t)r * K + c]) Wf[(int64_t)r * K + c] = 0.f;
+  const int64_t at = (int64_t)r * K + c;
+  if (c < c1 && mask[at]) {
+    if (Df) Df[at] -= Wf[at];
+    Wf[at] = 0.f;
+  }
 }
 
 __global__ __launch_bounds__(256) void zero_u32_words_kernel(unsigned* p, int64_t n) {
@@ -849,18 +856,123 @@ static int launch_group_update(const float* Eb, int64_t ldE, const float* U, int
   return 0;
 }
 
+// ---- left-looking form of the far updates (LLMC_FACTOR_GROUPS) ------------------------------------------------
+// With E = Err and D = W0 - Q (weights before the loop minus quantised weights) the loop's invariants are
+// D = E U and E = D V (V = U^-1 upper triangular, V V^T = H), so what the columns of a group G owe to all
+// earlier columns, -E[:, :g0] U[:g0, G], equals (D[:, :g0] V[:g0, G]) U[G, G]: the factor of H itself outside
+// the diagonal blocks and the inverse only inside them.  Per group: one product with a contraction over all
+// earlier columns, cut into `splits` pieces so that it fills the chip; a pass that adds the pieces in a fixed
+// order, keeps W0's columns and negates the sum; one 512-wide product with the group's diagonal block; the
+// group's blocks as in the other form; a pass that turns the kept W0 into D.
+constexpr int LEFT_MAX_SPLITS = 16;
+
+// pieces of the contraction for a weight of R rows: enough 256 x 256 (128 x 128 below 256 rows' multiple) tiles
+// for one per CU.  Depends on R only, never on how many problems share a launch.
+inline int left_split_cap(int64_t R) {
+  const int64_t tiles = (R % 256 == 0) ? (R / 256) * (LLMC_FACTOR_GROUP_WIDTH / 256)
+                                       : ((R + 127) / 128) * (LLMC_FACTOR_GROUP_WIDTH / 128);
+  int64_t s = (256 + tiles - 1) / tiles;
+  return (int)(s < 1 ? 1 : (s > LEFT_MAX_SPLITS ? LEFT_MAX_SPLITS : s));
+}
+
+inline int64_t left_extra_bytes(int64_t n, int64_t R, int64_t K) {
+  // D (W0, then W0 - Q), the pieces of the product, the negated sum
+  return align256(n * R * K * 4) + align256(n * left_split_cap(R) * R * LLMC_FACTOR_GROUP_WIDTH * 4) +
+         align256(n * R * LLMC_FACTOR_GROUP_WIDTH * 4);
+}
+
+// D[:, G] = W[:, G] (the untouched columns of the group) and, when there are pieces, C = -(P_0 + P_1 + ...)
+__global__ __launch_bounds__(256) void left_begin_group_kernel(const float* __restrict__ Wf, float* __restrict__ Df,
+                                                               int64_t K, int64_t g0, int64_t R,
+                                                               const float* __restrict__ P, int pieces,
+                                                               int64_t piece_stride, int64_t problem_stride_p,
+                                                               float* __restrict__ Cn) {
+  constexpr int GW = LLMC_FACTOR_GROUP_WIDTH;
+  const int64_t b = blockIdx.y;
+  const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;  // element of the [R, GW] group slice
+  if (idx >= R * GW) return;
+  const int64_t row = idx / GW, col = idx % GW;
+  const int64_t w = b * R * K + row * K + g0 + col;
+  *(float4*)(Df + w) = *(const float4*)(Wf + w);
+  if (pieces > 0) {
+    const float* p = P + b * problem_stride_p + idx;
+    float4 a = *(const float4*)p;
+    for (int s = 1; s < pieces; ++s) {
+      const float4 v = *(const float4*)(p + s * piece_stride);
+      a.x += v.x; a.y += v.y; a.z += v.z; a.w += v.w;
+    }
+    *(float4*)(Cn + b * R * GW + idx) = make_float4(-a.x, -a.y, -a.z, -a.w);
+  }
+}
+
+// D[:, G] -= W[:, G] (W holds the quantised values of the group now)
+__global__ __launch_bounds__(256) void left_end_group_kernel(const float* __restrict__ Wf, float* __restrict__ Df,
+                                                             int64_t K, int64_t g0, int64_t R) {
+  constexpr int GW = LLMC_FACTOR_GROUP_WIDTH;
+  const int64_t b = blockIdx.y;
+  const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (idx >= R * GW) return;
+  const int64_t w = b * R * K + (idx / GW) * K + g0 + idx % GW;
+  float4 d = *(const float4*)(Df + w);
+  const float4 q = *(const float4*)(Wf + w);
+  d.x -= q.x; d.y -= q.y; d.z -= q.z; d.w -= q.w;
+  *(float4*)(Df + w) = d;
+}
+
+// what the group [g0, g0 + 512) owes to the columns before it, added to Wf[:, G]; `extra` is the memory behind
+// the other work buffers (left_extra_bytes)
+static int left_begin_group(int n, int64_t R, int64_t K, int64_t g0, const float* U, int64_t ldu, int64_t u_stride,
+                            float* Wf, char* extra, hipStream_t st) {
+  constexpr int64_t GW = LLMC_FACTOR_GROUP_WIDTH;
+  float* Df = (float*)extra;
+  float* P = (float*)(extra + align256(n * R * K * 4));
+  const int cap = left_split_cap(R);
+  float* Cn = (float*)((char*)P + align256(n * cap * R * GW * 4));
+  const int64_t piece_stride = R * GW, problem_stride_p = (int64_t)cap * piece_stride;
+  int pieces = 0;
+  if (g0 > 0) {
+    const int64_t m = g0 / GW;                      // earlier groups
+    const int64_t per = (m + cap - 1) / cap;        // groups per piece
+    pieces = (int)((m + per - 1) / per);
+    const int64_t chunk = per * GW, last = g0 - (pieces - 1) * chunk;
+    GemmF32 g = {};
+    g.A = Df; g.lda = K; g.B = U + g0; g.ldb = ldu; g.C = P; g.ldc = GW;
+    g.M = (int)R; g.N = (int)GW; g.Kc = (int)chunk; g.alpha = 1.f; g.beta = 0.f;
+    g.batch = pieces; g.stride_a = chunk; g.stride_b = chunk * ldu; g.stride_c = piece_stride;
+    g.kc_last = last == chunk ? 0 : (int)last;
+    g.batch2 = n; g.stride2_a = R * K; g.stride2_b = u_stride; g.stride2_c = problem_stride_p;
+    const int rc = llmc_gemm_f32(g, st);
+    if (rc) return rc;
+  }
+  hipLaunchKernelGGL(left_begin_group_kernel, dim3((unsigned)((R * GW / 4 + 255) / 256), (unsigned)n), dim3(256), 0, st,
+                     (const float*)Wf, Df, K, g0, R, (const float*)P, pieces, piece_stride, problem_stride_p, Cn);
+  LLMC_LAUNCH_STATUS();
+  if (g0 > 0) {
+    GemmF32 h = {};  // Wf[:, G] -= Cn U[G, G]; U holds exact zeros below the diagonal
+    h.A = Cn; h.lda = GW; h.B = U + g0 * ldu + g0; h.ldb = ldu; h.C = Wf + g0; h.ldc = K;
+    h.M = (int)R; h.N = (int)GW; h.Kc = (int)GW; h.alpha = -1.f; h.beta = 1.f;
+    h.batch = 1; h.batch2 = n; h.stride2_a = R * GW; h.stride2_b = u_stride; h.stride2_c = R * K;
+    const int rc = llmc_gemm_f32(h, st);
+    if (rc) return rc;
+  }
+  return 0;
+}
+
 extern "C" int64_t llmc_sparsegpt_workspace_bytes(int64_t R, int64_t K) {
   const int64_t slices = (K + SG_MIN_BLOCK - 1) / SG_MIN_BLOCK;
   return align256(R * K * 4) + align256(R * GROUP * GB * 4) + align256(R * 4) +
-         align256(slices * SG_HIST_WORDS * 4) + align256(R * K);
+         align256(slices * SG_HIST_WORDS * 4) + align256(R * K) +
+         (K % LLMC_FACTOR_GROUP_WIDTH == 0 ? left_extra_bytes(1, R, K) : 0);
 }
 
 extern "C" int llmc_sparsegpt_sparsify(const void* weight, int32_t w_dtype, int64_t R, int64_t K, int64_t ldw,
                                        const float* U, int64_t ldu, const uint8_t* dead, double sparsity,
-                                       int32_t prune_n, int32_t prune_m, int32_t blocksize,
+                                       int32_t prune_n, int32_t prune_m, int32_t blocksize, int32_t form,
                                        int32_t preserve_sparsity_mask, void* out_weight, int64_t ldo,
                                        float* loss_out, void* workspace, int64_t workspace_bytes, void* stream) {
   LLMC_CHECK_ARG(weight != nullptr, 1);
+  LLMC_CHECK_ARG(form == LLMC_FACTOR_INVERSE ||
+                     (form == LLMC_FACTOR_GROUPS && K % LLMC_FACTOR_GROUP_WIDTH == 0 && blocksize == GB), 13);
   LLMC_CHECK_ARG(w_dtype >= 0 && w_dtype <= 2, 2);
   LLMC_CHECK_ARG(R > 0 && R < (1ll << 24), 3);
   LLMC_CHECK_ARG(K > 0 && K < (1ll << 31), 4);
@@ -885,6 +997,9 @@ extern "C" int llmc_sparsegpt_sparsify(const void* weight, int32_t w_dtype, int6
   float* loss_rows = (float*)wp; wp += align256(R * 4);
   unsigned* hist = (unsigned*)wp; wp += align256(((K + SG_MIN_BLOCK - 1) / SG_MIN_BLOCK) * SG_HIST_WORDS * 4);
   uint8_t* mask = preserve_sparsity_mask ? (uint8_t*)wp : nullptr;
+  wp += align256(R * K);
+  char* extra = wp;
+  const bool left = form == LLMC_FACTOR_GROUPS;
 
   dim3 grid2((unsigned)((K + 255) / 256), (unsigned)R);
 #define LLMC_PREP(DT) \
@@ -920,12 +1035,18 @@ extern "C" int llmc_sparsegpt_sparsify(const void* weight, int32_t w_dtype, int6
   auto rezero = [&](int64_t c0, int64_t c1) {  // preserved zeros in columns [c0, c1) back to zero
     if (!mask || c0 >= c1) return;
     hipLaunchKernelGGL(sgpt_rezero_kernel, dim3((unsigned)((c1 - c0 + 255) / 256), (unsigned)R), dim3(256), 0, st, Wf,
-                       mask, (int)K, (int)c0, (int)c1);
+                       mask, (int)K, (int)c0, (int)c1, left ? (float*)extra : (float*)nullptr);
   };
   // the same two-level lazy updates as the quantiser's loop
   int64_t blk = 0;
   for (int64_t g0 = 0; g0 < K; g0 += (int64_t)GROUP * bs) {
     const int64_t gend = (g0 + (int64_t)GROUP * bs) < K ? g0 + (int64_t)GROUP * bs : K;
+    if (left && (g0 > 0 || gend < K)) {  // what the group owes to the earlier columns, from the factor of H
+      const int rc = left_begin_group(1, R, K, g0, U, ldu, 0, Wf, extra, st);
+      if (rc) return rc;
+      if (g0 > 0) rezero(g0, gend);
+      LLMC_LAUNCH_STATUS();
+    }
     for (int64_t i1 = g0; i1 < gend; i1 += bs, ++blk) {
       const int count = (int)((gend - i1) < bs ? (gend - i1) : bs);
       p.i1 = (int)i1;
@@ -956,7 +1077,11 @@ extern "C" int llmc_sparsegpt_sparsify(const void* weight, int32_t w_dtype, int6
         LLMC_LAUNCH_STATUS();
       }
     }
-    if (gend < K) {
+    if (gend < K && left) {
+      hipLaunchKernelGGL(left_end_group_kernel, dim3((unsigned)((R * (gend - g0) / 4 + 255) / 256), 1), dim3(256), 0, st,
+                         (const float*)Wf, (float*)extra, K, g0, R);
+      LLMC_LAUNCH_STATUS();
+    } else if (gend < K) {
       GemmF32 g = {};
       g.A = E; g.lda = ldE; g.B = U + g0 * ldu + gend; g.ldb = ldu; g.C = Wf + gend; g.ldc = K;
       g.M = (int)R; g.N = (int)(K - gend); g.Kc = (int)(gend - g0); g.alpha = -1.f; g.beta = 1.f; g.batch = 1;
@@ -989,10 +1114,11 @@ extern "C" int llmc_sparsegpt_sparsify(const void* weight, int32_t w_dtype, int6
 // of W is read and written a quarter as often, which is what bounds a rank-128 update.
 static int gptq_column_loop(void (*kern)(GptqBlockParams), GptqBlockParams p, int smem, unsigned wgs, int n, int64_t R,
                             int64_t K, int bs, float* E, const float* U, int64_t ldu, int64_t u_stride, float* Wf,
-                            hipStream_t st) {
+                            int form, char* extra, hipStream_t st) {
   const int ldE = GROUP * GB;
   p.ldE = ldE;
   const int64_t gw = (int64_t)GROUP * bs;
+  const bool left = form == LLMC_FACTOR_GROUPS;  // the callers have checked gw == 512 and K % 512 == 0
   auto product = [&](const float* A, int64_t k0, int64_t kc, int64_t c0, int64_t c1) {
     GemmF32 g = {};
     g.A = A; g.lda = ldE; g.B = U + k0 * ldu + c0; g.ldb = ldu; g.C = Wf + c0; g.ldc = K;
@@ -1002,6 +1128,10 @@ static int gptq_column_loop(void (*kern)(GptqBlockParams), GptqBlockParams p, in
   };
   for (int64_t g0 = 0; g0 < K; g0 += gw) {
     const int64_t gend = (g0 + gw) < K ? g0 + gw : K;
+    if (left && (g0 > 0 || gend < K)) {  // the only group of a 512-wide weight needs neither D nor a sum
+      const int rc = left_begin_group(n, R, K, g0, U, ldu, u_stride, Wf, extra, st);
+      if (rc) return rc;
+    }
     for (int64_t i1 = g0; i1 < gend; i1 += bs) {
       const int count = (int)((gend - i1) < bs ? (gend - i1) : bs);
       p.i1 = (int)i1;
@@ -1017,15 +1147,22 @@ static int gptq_column_loop(void (*kern)(GptqBlockParams), GptqBlockParams p, in
       }
     }
     if (gend < K) {
-      const int rc = product(E, g0, gend - g0, gend, K);
-      if (rc) return rc;
+      if (left) {
+        hipLaunchKernelGGL(left_end_group_kernel, dim3((unsigned)((R * gw / 4 + 255) / 256), (unsigned)n), dim3(256), 0,
+                           st, (const float*)Wf, (float*)extra, K, g0, R);
+        LLMC_LAUNCH_STATUS();
+      } else {
+        const int rc = product(E, g0, gend - g0, gend, K);
+        if (rc) return rc;
+      }
     }
   }
   return 0;
 }
 
 extern "C" int64_t llmc_gptq_quantize_workspace_bytes(int64_t R, int64_t K) {
-  return align256(R * K * 4) + align256(R * GROUP * GB * 4) + align256(R * 4);
+  return align256(R * K * 4) + align256(R * GROUP * GB * 4) + align256(R * 4) +
+         (K % LLMC_FACTOR_GROUP_WIDTH == 0 ? left_extra_bytes(1, R, K) : 0);
 }
 
 extern "C" int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R, int64_t K, int64_t ldw,
@@ -1033,9 +1170,11 @@ extern "C" int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R
                                   const void* scale, int32_t scale_dtype, const int8_t* zero_point,
                                   const float* global_scale, const int32_t* g_idx, int64_t row_div,
                                   int64_t scale_row_stride, int32_t fmt, int32_t num_bits, int32_t blocksize,
-                                  void* out_weight, int64_t ldo, float* loss_out, void* workspace,
+                                  int32_t form, void* out_weight, int64_t ldo, float* loss_out, void* workspace,
                                   int64_t workspace_bytes, void* stream) {
   LLMC_CHECK_ARG(weight != nullptr, 1);
+  LLMC_CHECK_ARG(form == LLMC_FACTOR_INVERSE ||
+                     (form == LLMC_FACTOR_GROUPS && K % LLMC_FACTOR_GROUP_WIDTH == 0 && blocksize >= GB), 20);
   LLMC_CHECK_ARG(w_dtype >= 0 && w_dtype <= 2, 2);
   LLMC_CHECK_ARG(R > 0 && R < (1ll << 31), 3);
   LLMC_CHECK_ARG(K > 0 && K < (1ll << 31), 4);
@@ -1058,6 +1197,7 @@ extern "C" int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R
   float* Wf = (float*)workspace;
   float* E = (float*)((char*)workspace + align256(R * K * 4));
   float* loss_rows = (float*)((char*)E + align256(R * GROUP * GB * 4));
+  char* extra = (char*)loss_rows + align256(R * 4);
 
   dim3 grid2((unsigned)((K + 255) / 256), (unsigned)R);
   const bool by_rows = perm != nullptr && K <= ROW_STAGE_MAX;  // permuted columns: gather and scatter a row in LDS
@@ -1112,7 +1252,7 @@ extern "C" int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R
   const int rows_per_wg = wide_team ? QLayout<16>::ROWS_PER_WG : QLayout<4>::ROWS_PER_WG;
   const unsigned wgs = (unsigned)((R + rows_per_wg - 1) / rows_per_wg);
   {
-    const int rc = gptq_column_loop(kern, p, smem, wgs, 1, R, K, bs, E, U, ldu, 0, Wf, st);
+    const int rc = gptq_column_loop(kern, p, smem, wgs, 1, R, K, bs, E, U, ldu, 0, Wf, form, extra, st);
     if (rc) return rc;
   }
 
@@ -1143,7 +1283,7 @@ extern "C" int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R
 
 extern "C" int64_t llmc_gptq_quantize_grouped_workspace_bytes(int64_t n, int64_t R, int64_t K) {
   return align256(n * (int64_t)sizeof(GptqItem)) + align256(n * R * K * 4) + align256(n * R * GROUP * GB * 4) +
-         align256(n * R * 4);
+         align256(n * R * 4) + (K % LLMC_FACTOR_GROUP_WIDTH == 0 ? left_extra_bytes(n, R, K) : 0);
 }
 
 extern "C" int llmc_gptq_quantize_grouped(const void* const* weight, int32_t w_dtype, int32_t n, int64_t R, int64_t K,
@@ -1152,9 +1292,11 @@ extern "C" int llmc_gptq_quantize_grouped(const void* const* weight, int32_t w_d
                                           int32_t scale_dtype, const int8_t* const* zero_point,
                                           const float* const* global_scale, const int32_t* const* g_idx,
                                           int64_t row_div, int64_t scale_row_stride, int32_t fmt, int32_t num_bits,
-                                          int32_t blocksize, void* const* out_weight, int64_t ldo, float* loss_out,
-                                          void* workspace, int64_t workspace_bytes, void* stream) {
+                                          int32_t blocksize, int32_t form, void* const* out_weight, int64_t ldo,
+                                          float* loss_out, void* workspace, int64_t workspace_bytes, void* stream) {
   LLMC_CHECK_ARG(weight != nullptr, 1);
+  LLMC_CHECK_ARG(form == LLMC_FACTOR_INVERSE ||
+                     (form == LLMC_FACTOR_GROUPS && K % LLMC_FACTOR_GROUP_WIDTH == 0 && blocksize >= GB), 22);
   LLMC_CHECK_ARG(w_dtype >= 0 && w_dtype <= 2, 2);
   LLMC_CHECK_ARG(n >= 0 && n <= 4096, 3);
   if (n == 0) return 0;
@@ -1178,7 +1320,8 @@ extern "C" int llmc_gptq_quantize_grouped(const void* const* weight, int32_t w_d
   GptqItem* items = (GptqItem*)wp; wp += align256(n * (int64_t)sizeof(GptqItem));
   float* Wf = (float*)wp; wp += align256(n * R * K * 4);
   float* E = (float*)wp; wp += align256(n * R * GROUP * GB * 4);
-  float* loss_rows = (float*)wp;
+  float* loss_rows = (float*)wp; wp += align256(n * R * 4);
+  char* extra = wp;
   std::vector<GptqItem> host(n);
   for (int b = 0; b < n; ++b) {
     LLMC_CHECK_ARG(weight[b] != nullptr && scale[b] != nullptr && out_weight[b] != nullptr, 1);
@@ -1247,7 +1390,7 @@ extern "C" int llmc_gptq_quantize_grouped(const void* const* weight, int32_t w_d
   const int rows_per_wg = wide_team ? QLayout<16>::ROWS_PER_WG : QLayout<4>::ROWS_PER_WG;
   const unsigned wgs = (unsigned)((R + rows_per_wg - 1) / rows_per_wg);
   {
-    const int rc = gptq_column_loop(kern, p, smem, wgs, n, R, K, bs, E, U, ldu, u_stride, Wf, st);
+    const int rc = gptq_column_loop(kern, p, smem, wgs, n, R, K, bs, E, U, ldu, u_stride, Wf, form, extra, st);
     if (rc) return rc;
   }
 

@@ -374,7 +374,7 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
         names = [self._module_names.get(m, m.__class__.__name__) for m in part]
         logger.info(f"Quantizing {len(part)} modules in lock-step ({names[0]} .. {names[-1]})")
         with torch.no_grad():
-            ctx = begin_weight_group(part, hs, tallies, self.dampening_frac)
+            ctx = begin_weight_group(part, hs, tallies, self.dampening_frac, self.block_size)
         return part, names, ctx
 
     def _end_set(self, begun):

@@ -349,8 +349,18 @@ def dynamic_per_token_quantize(x, fmt: int = FMT_FP8, bits: int = 8, out_mode: i
     return out, scale
 
 
-def gptq_hinv_(H: torch.Tensor, perm=None, divisor: float = 1.0, percdamp: float = 0.01):
-    """In place: H -> upper factor U of (H/divisor [permuted] + damping)^-1.
+FACTOR_INVERSE, FACTOR_GROUPS, FACTOR_GROUP_WIDTH = 0, 1, 512
+
+
+def gptq_factor_form(K: int, blocksize: int = 128) -> int:
+    """The form of the factor the library prefers for a quantize_weight call on K columns: FACTOR_GROUPS where
+    the column loop can work from the Cholesky factor of H itself (K a multiple of 512), else FACTOR_INVERSE."""
+    return int(_lib.lib().llmc_gptq_factor_form(int(K), int(blocksize)))
+
+
+def gptq_hinv_(H: torch.Tensor, perm=None, divisor: float = 1.0, percdamp: float = 0.01, form: int = FACTOR_INVERSE):
+    """In place: H -> upper factor U of (H/divisor [permuted] + damping)^-1; with form = FACTOR_GROUPS only inside
+    the aligned 512-column diagonal blocks, the upper Cholesky factor of the damped H itself outside them.
 
     Returns (U (= H), dead uint8 [K], info int32 [1] on device)."""
     _require_gpu(H)
@@ -364,12 +374,13 @@ def gptq_hinv_(H: torch.Tensor, perm=None, divisor: float = 1.0, percdamp: float
     ws = _workspace(H.device, nbytes)
     with torch.cuda.device(H.device):
         rc = _lib.lib().llmc_gptq_hinv(H.data_ptr(), H.stride(0), K, _ptr(perm), float(divisor), float(percdamp),
-                                       dead.data_ptr(), ws.data_ptr(), ws.numel(), info.data_ptr(), _stream(H))
+                                       int(form), dead.data_ptr(), ws.data_ptr(), ws.numel(), info.data_ptr(),
+                                       _stream(H))
     _lib.check(rc, "llmc_gptq_hinv")
     return H, dead, info
 
 
-def gptq_hinv_grouped(Hs, perms=None, divisors=None, percdamp: float = 0.01):
+def gptq_hinv_grouped(Hs, perms=None, divisors=None, percdamp: float = 0.01, form: int = FACTOR_INVERSE):
     """gptq_hinv_ for n Hessians of one width in lock-step.  Hs: list of fp32 [K,K] (left untouched); perms:
     int32 [n,K] tensor or None; divisors: list of floats.  Returns (U [n,K,K] fp32, dead [n,K] uint8, info [n])."""
     import ctypes
@@ -394,16 +405,18 @@ def gptq_hinv_grouped(Hs, perms=None, divisors=None, percdamp: float = 0.01):
     nbytes = _lib.lib().llmc_gptq_hinv_grouped_workspace_bytes(n, K)
     ws = _workspace(H0.device, nbytes)
     with torch.cuda.device(H0.device):
-        rc = _lib.lib().llmc_gptq_hinv_grouped(hp, H0.stride(0), n, K, pp, dv, float(percdamp), dead.data_ptr(),
-                                              U.data_ptr(), K, ws.data_ptr(), ws.numel(), info.data_ptr(),
-                                              _stream(H0))
+        rc = _lib.lib().llmc_gptq_hinv_grouped(hp, H0.stride(0), n, K, pp, dv, float(percdamp), int(form),
+                                              dead.data_ptr(), U.data_ptr(), K, ws.data_ptr(), ws.numel(),
+                                              info.data_ptr(), _stream(H0))
     _lib.check(rc, "llmc_gptq_hinv_grouped")
     return U, dead, info
 
 
 def gptq_quantize(weight, U, scale, zero_point, fmt: int, bits: int, row_div: int, scale_row_stride: int,
-                  g_idx=None, perm=None, dead=None, global_scale=None, blocksize: int = 128):
-    """The GPTQ column loop.  Returns (quantised-dequantised weight in weight.dtype, loss fp32 [1])."""
+                  g_idx=None, perm=None, dead=None, global_scale=None, blocksize: int = 128,
+                  form: int = FACTOR_INVERSE):
+    """The GPTQ column loop on a factor of the given form (see gptq_hinv_).  Returns (quantised-dequantised weight
+    in weight.dtype, loss fp32 [1])."""
     global_scale = _gs32(global_scale)
     _require_gpu(weight, U, scale)
     assert weight.ndim == 2 and weight.stride(1) == 1 and U.stride(1) == 1
@@ -424,14 +437,15 @@ def gptq_quantize(weight, U, scale, zero_point, fmt: int, bits: int, row_div: in
         rc = _lib.lib().llmc_gptq_quantize(
             weight.data_ptr(), _dt(weight), R, K, weight.stride(0), U.data_ptr(), U.stride(0), _ptr(perm),
             _ptr(dead), scale.data_ptr(), _dt(scale), _ptr(zero_point), _ptr(global_scale), _ptr(g_idx), row_div,
-            scale_row_stride, fmt, bits, blocksize, out.data_ptr(), K, loss.data_ptr(), ws.data_ptr(), ws.numel(),
-            _stream(weight))
+            scale_row_stride, fmt, bits, blocksize, int(form), out.data_ptr(), K, loss.data_ptr(), ws.data_ptr(),
+            ws.numel(), _stream(weight))
     _lib.check(rc, "llmc_gptq_quantize")
     return out, loss
 
 
 def gptq_quantize_grouped(weights, U, scales, zero_points, fmt: int, bits: int, row_div: int, scale_row_stride: int,
-                          g_idxs=None, perms=None, dead=None, global_scales=None, blocksize: int = 128):
+                          g_idxs=None, perms=None, dead=None, global_scales=None, blocksize: int = 128,
+                          form: int = FACTOR_INVERSE):
     """gptq_quantize for n weights of one shape in lock-step.  weights / scales / zero_points / g_idxs /
     global_scales: lists of n tensors (the last three may be None); U [n,K,K] fp32; perms [n,K] int32 or None;
     dead [n,K] uint8 or None.  Returns (list of quantised-dequantised weights, loss fp32 [n])."""
@@ -471,16 +485,16 @@ def gptq_quantize_grouped(weights, U, scales, zero_points, fmt: int, bits: int, 
     with torch.cuda.device(w0.device):
         rc = _lib.lib().llmc_gptq_quantize_grouped(
             wp, _dt(w0), n, R, K, w0.stride(0), U.data_ptr(), K, K * K, _ptr(perms), _ptr(dead), sp, _dt(keep[0]),
-            zp, gp, ip, row_div, scale_row_stride, fmt, bits, blocksize, op, K, loss.data_ptr(), ws.data_ptr(),
-            ws.numel(), _stream(w0))
+            zp, gp, ip, row_div, scale_row_stride, fmt, bits, blocksize, int(form), op, K, loss.data_ptr(),
+            ws.data_ptr(), ws.numel(), _stream(w0))
     _lib.check(rc, "llmc_gptq_quantize_grouped")
     return outs, loss
 
 
 def sparsegpt_sparsify(weight, U, sparsity: float, prune_n: int = 0, prune_m: int = 0, dead=None,
-                       blocksize: int = 128, preserve_sparsity_mask: bool = False):
-    """The SparseGPT column loop on the factor U of gptq_hinv_.  Returns (pruned weight in weight.dtype,
-    loss fp32 [1])."""
+                       blocksize: int = 128, preserve_sparsity_mask: bool = False, form: int = FACTOR_INVERSE):
+    """The SparseGPT column loop on the factor U of gptq_hinv_ (of the given form).  Returns (pruned weight in
+    weight.dtype, loss fp32 [1])."""
     _require_gpu(weight, U)
     assert weight.ndim == 2 and weight.stride(1) == 1 and U.stride(1) == 1
     R, K = weight.shape
@@ -498,8 +512,9 @@ def sparsegpt_sparsify(weight, U, sparsity: float, prune_n: int = 0, prune_m: in
     with torch.cuda.device(weight.device):
         rc = _lib.lib().llmc_sparsegpt_sparsify(
             weight.data_ptr(), _dt(weight), R, K, weight.stride(0), U.data_ptr(), U.stride(0), _ptr(dead),
-            float(sparsity), int(prune_n), int(prune_m), int(blocksize), 1 if preserve_sparsity_mask else 0,
-            out.data_ptr(), K, loss.data_ptr(), ws.data_ptr(), ws.numel(), _stream(weight))
+            float(sparsity), int(prune_n), int(prune_m), int(blocksize), int(form),
+            1 if preserve_sparsity_mask else 0, out.data_ptr(), K, loss.data_ptr(), ws.data_ptr(), ws.numel(),
+            _stream(weight))
     _lib.check(rc, "llmc_sparsegpt_sparsify")
     return out, loss
 

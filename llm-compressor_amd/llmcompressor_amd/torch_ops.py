@@ -60,49 +60,52 @@ _register("hessian_accum_grouped_(Tensor(a!)[] Hs, Tensor[] Xs, float alpha=2.0,
 
 # ---- damped Cholesky chain and the column loop ------------------------------------------------------------------
 
-def _gptq_prepare_hinv_(H, perm=None, divisor=1.0, percdamp=0.01):
-    _, dead, info = _impl.gptq_hinv_(H, perm, divisor=divisor, percdamp=percdamp)
+def _gptq_prepare_hinv_(H, perm=None, divisor=1.0, percdamp=0.01, form=0):
+    _, dead, info = _impl.gptq_hinv_(H, perm, divisor=divisor, percdamp=percdamp, form=form)
     return dead, info
 
 
-def _gptq_prepare_hinv_grouped(Hs, perms=None, divisors=None, percdamp=0.01):
-    return _impl.gptq_hinv_grouped(list(Hs), perms, None if divisors is None else list(divisors), percdamp)
+def _gptq_prepare_hinv_grouped(Hs, perms=None, divisors=None, percdamp=0.01, form=0):
+    return _impl.gptq_hinv_grouped(list(Hs), perms, None if divisors is None else list(divisors), percdamp, form=form)
 
 
 def _gptq_quantize(W, Hinv, scale, zero_point, fmt, num_bits, row_div, scale_row_stride, g_idx=None, perm=None,
-                   dead=None, global_scale=None, blocksize=128):
+                   dead=None, global_scale=None, blocksize=128, form=0):
     return _impl.gptq_quantize(W, Hinv, scale, zero_point, fmt, num_bits, row_div, scale_row_stride, g_idx=g_idx,
-                               perm=perm, dead=dead, global_scale=global_scale, blocksize=blocksize)
+                               perm=perm, dead=dead, global_scale=global_scale, blocksize=blocksize, form=form)
 
 
 def _gptq_quantize_grouped(Ws, Hinv, scales, zero_points, fmt, num_bits, row_div, scale_row_stride, g_idxs=None,
-                           perms=None, dead=None, global_scales=None, blocksize=128):
+                           perms=None, dead=None, global_scales=None, blocksize=128, form=0):
     outs, loss = _impl.gptq_quantize_grouped(
         list(Ws), Hinv, list(scales), None if zero_points is None else list(zero_points), fmt, num_bits, row_div,
         scale_row_stride, g_idxs=None if g_idxs is None else list(g_idxs), perms=perms, dead=dead,
-        global_scales=None if global_scales is None else list(global_scales), blocksize=blocksize)
+        global_scales=None if global_scales is None else list(global_scales), blocksize=blocksize, form=form)
     return outs, loss
 
 
 def _sparsegpt_sparsify(W, Hinv, sparsity, prune_n=0, prune_m=0, dead=None, blocksize=128,
-                        preserve_sparsity_mask=False):
+                        preserve_sparsity_mask=False, form=0):
     return _impl.sparsegpt_sparsify(W, Hinv, sparsity, prune_n=prune_n, prune_m=prune_m, dead=dead,
-                                    blocksize=blocksize, preserve_sparsity_mask=preserve_sparsity_mask)
+                                    blocksize=blocksize, preserve_sparsity_mask=preserve_sparsity_mask, form=form)
 
 
-_register("gptq_prepare_hinv_(Tensor(a!) H, Tensor? perm=None, float divisor=1.0, float percdamp=0.01) "
+_register("gptq_prepare_hinv_(Tensor(a!) H, Tensor? perm=None, float divisor=1.0, float percdamp=0.01, int form=0) "
           "-> (Tensor dead, Tensor info)", _gptq_prepare_hinv_)
-_register("gptq_prepare_hinv_grouped(Tensor[] Hs, Tensor? perms=None, float[]? divisors=None, float percdamp=0.01) "
+_register("gptq_prepare_hinv_grouped(Tensor[] Hs, Tensor? perms=None, float[]? divisors=None, float percdamp=0.01, "
+          "int form=0) "
           "-> (Tensor U, Tensor dead, Tensor info)", _gptq_prepare_hinv_grouped)
 _register("gptq_quantize(Tensor W, Tensor Hinv, Tensor scale, Tensor? zero_point, int fmt, int num_bits, int row_div, "
           "int scale_row_stride, Tensor? g_idx=None, Tensor? perm=None, Tensor? dead=None, Tensor? global_scale=None, "
-          "int blocksize=128) -> (Tensor weight, Tensor loss)", _gptq_quantize)
+          "int blocksize=128, int form=0) -> (Tensor weight, Tensor loss)", _gptq_quantize)
 _register("gptq_quantize_grouped(Tensor[] Ws, Tensor Hinv, Tensor[] scales, Tensor[]? zero_points, int fmt, "
           "int num_bits, int row_div, int scale_row_stride, Tensor[]? g_idxs=None, Tensor? perms=None, "
-          "Tensor? dead=None, Tensor[]? global_scales=None, int blocksize=128) -> (Tensor[] weights, Tensor loss)",
+          "Tensor? dead=None, Tensor[]? global_scales=None, int blocksize=128, int form=0) "
+          "-> (Tensor[] weights, Tensor loss)",
           _gptq_quantize_grouped)
 _register("sparsegpt_sparsify(Tensor W, Tensor Hinv, float sparsity, int prune_n=0, int prune_m=0, Tensor? dead=None, "
-          "int blocksize=128, bool preserve_sparsity_mask=False) -> (Tensor weight, Tensor loss)", _sparsegpt_sparsify)
+          "int blocksize=128, bool preserve_sparsity_mask=False, int form=0) -> (Tensor weight, Tensor loss)",
+          _sparsegpt_sparsify)
 
 
 # ---- observers ---------------------------------------------------------------------------------------------------

@@ -26,9 +26,11 @@ def _gpu(x, W, n_samples, **kw):
     K = W.shape[1]
     H = torch.zeros(K, K, device=DEV)
     ops.hessian_accumulate_(H, x.to(DEV))
-    U, dead, info = ops.gptq_hinv_(H, None, divisor=float(n_samples), percdamp=kw.pop("dampening_frac", 0.01))
+    form = kw.pop("form", ops.FACTOR_INVERSE)
+    U, dead, info = ops.gptq_hinv_(H, None, divisor=float(n_samples), percdamp=kw.pop("dampening_frac", 0.01),
+                                   form=form)
     assert int(info.item()) == 0
-    Q, loss = ops.sparsegpt_sparsify(W.to(DEV), U, dead=dead, **kw)
+    Q, loss = ops.sparsegpt_sparsify(W.to(DEV), U, dead=dead, form=form, **kw)
     return Q.cpu(), float(loss.item())
 
 
@@ -84,6 +86,36 @@ def test_sparsify_matches_oracle(case):
             assert int((Qg[:, c0:c0 + cnt] == 0).sum()) == int(R * cnt * kw["sparsity"]) + 1
     if kw.get("preserve_sparsity_mask"):
         assert torch.all(Qg[W == 0] == 0)
+
+
+GROUPED_FACTOR_CASES = [
+    dict(R=64, K=1024, kw=dict(sparsity=0.5)),
+    dict(R=96, K=1536, kw=dict(sparsity=0.5, prune_n=2, prune_m=4)),
+    dict(R=64, K=1024, zero_frac=0.3, kw=dict(sparsity=0.6, preserve_sparsity_mask=True)),
+]
+
+
+@pytest.mark.parametrize("case", GROUPED_FACTOR_CASES, ids=[str(i) for i in range(len(GROUPED_FACTOR_CASES))])
+def test_sparsify_from_the_grouped_factor_matches_oracle(case):
+    """The loop in its left-looking form (the Cholesky factor of H outside the 512-column diagonal blocks, what
+    wide weights use) against the oracle's U-based loop, and against the other form on the device."""
+    from llmcompressor_amd import ops
+
+    R, K = case["R"], case["K"]
+    x, W = _problem(R, K, 2 * K, 300 + R + K, torch.bfloat16, case.get("zero_frac", 0.0))
+    Qg, lg = _gpu(x, W, 8, form=ops.FACTOR_GROUPS, **dict(case["kw"]))
+    Qi, li = _gpu(x, W, 8, **dict(case["kw"]))
+    lo, Qo = _oracle(x, W, 8, **dict(case["kw"]))
+    for other, lother in ((Qo, lo), (Qi, li)):
+        assert ((Qg == 0) == (other == 0)).float().mean().item() >= 0.999
+        both = (Qg != 0) & (other != 0)
+        rel = ((Qg.double() - other.double())[both].norm() / other.double()[both].norm()).item()
+        assert rel < 6e-3, rel
+        assert abs(lg - lother) <= 0.01 * abs(lother) + 1e-9
+    if case["kw"].get("preserve_sparsity_mask"):
+        assert torch.all(Qg[W == 0] == 0)
+    if case["kw"].get("prune_n"):
+        assert torch.all((Qg == 0).reshape(R, K // 4, 4).sum(-1) == 2)
 
 
 def test_sparsify_rejects_unsupported_structures():
