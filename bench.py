@@ -409,10 +409,14 @@ def probe_moe(mode="both"):
         print(f"propagation forward, grouped launches, device time between events: {e0.elapsed_time(e1):.2f} ms")
     print("| quantisation of the 384 expert Linears | forward + Hessians ms per batch | quantise ms | ms per Linear |")
     print("|---|---|---|---|")
-    variants = (("W4A16, lock-step groups (default)", 8, "lockstep", "W4A16"),
-                ("W4A16, one module at a time, 4 streams", 0, "permodule", "W4A16"),
-                ("NVFP4A16, lock-step groups (default)", 8, "lockstep", "NVFP4A16"))
-    for label, gmin, key, scheme in variants:
+    from llmcompressor_amd.modeling.moe import moe_calibration_context
+
+    variants = (("W4A16, lock-step groups (default)", 8, "lockstep", "W4A16", False),
+                ("W4A16, one module at a time, 4 streams", 0, "permodule", "W4A16", False),
+                ("NVFP4A16, lock-step groups (default)", 8, "lockstep", "NVFP4A16", False),
+                ("W4A16, lock-step groups, every expert calibrated on all tokens (`moe_calibrate_all_experts`, the "
+                 "`oneshot` default)", 8, "lockstep", "W4A16", True))
+    for label, gmin, key, scheme, all_experts in variants:
         if mode not in ("both", key):
             continue
         best = None
@@ -425,7 +429,7 @@ def probe_moe(mode="both"):
             s.reset()
             s.initialize(model=model, recipe=mod)
             LifecycleCallbacks.calibration_start()
-            with torch.no_grad():
+            with torch.no_grad(), moe_calibration_context(all_experts):
                 model.layers[0](x, idx, w.to(x.dtype))  # first batch: the Hessians are allocated here
                 torch.cuda.synchronize()
                 t0 = time.perf_counter()

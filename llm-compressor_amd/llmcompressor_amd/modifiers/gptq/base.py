@@ -109,7 +109,8 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
     _held_bytes: int = PrivateAttr(default=0)
     _group_pending: list | None = PrivateAttr(default=None)
     _leader: dict = PrivateAttr(default_factory=dict)  # follower module -> module whose Hessian it shares
-    _recent_input: tuple | None = PrivateAttr(default=None)  # (tensor kept alive, its version, leader)
+    # per input width: (tensor kept alive, its version, leader) of the last input that was accumulated
+    _recent_input: dict = PrivateAttr(default_factory=dict)
     _hook_calls: dict = PrivateAttr(default_factory=dict)  # module -> hook calls so far (leaders and followers)
     _streams: dict = PrivateAttr(default_factory=lambda: SIDE_STREAMS)
 
@@ -217,15 +218,17 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
 
     # -- shared Hessians (see ``share_identical_inputs``)
     def _follows_recent_input(self, module, inp, priv=None) -> bool:
-        """True when `module` just received the tensor that the previous hook call accumulated for
-        another module of the same width; then only its sample count advances.  The previous input is
-        kept referenced, so no later tensor can take its address while it is being compared."""
+        """True when `module` received the tensor that the last accumulating hook call of its input width took
+        in for another module; then only its sample count advances.  Kept per width, so that modules of another
+        width called in between (an expert's down_proj between its own and the next expert's gate_proj, which with
+        ``moe_calibrate_all_experts`` all receive the block's input) do not end the run.  The previous inputs are
+        kept referenced, so no later tensor can take their address while it is being compared."""
         priv = self.__pydantic_private__ if priv is None else priv
-        recent = priv["_recent_input"]
+        width = module.in_features if isinstance(module, torch.nn.Linear) else None
+        recent = priv["_recent_input"].get(width) if width is not None else None
         same = (recent is not None and recent[2] is not module and inp.data_ptr() == recent[0].data_ptr()
                 and inp.shape == recent[0].shape and inp.dtype == recent[0].dtype and inp.stride() == recent[0].stride()
-                and inp._version == recent[1] and isinstance(module, torch.nn.Linear)
-                and module.in_features == recent[2].in_features)
+                and inp._version == recent[1])
         leaders, num_samples = priv["_leader"], priv["_num_samples"]
         leader = leaders.get(module)
         if same and (leader is recent[2] or (leader is None and module not in num_samples)):
@@ -236,7 +239,8 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
         if leader is not None:
             raise RuntimeError("share_identical_inputs: a module that shared its input with another one received a "
                                "different tensor on a later call; pass share_identical_inputs=False for this model")
-        priv["_recent_input"] = (inp, inp._version, module)
+        if width is not None:
+            priv["_recent_input"][width] = (inp, inp._version, module)
         return False
 
     # -- expert groups (see the class docstring)
@@ -274,7 +278,7 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
                                        f"{self._hook_calls.get(leader)} times; pass share_identical_inputs=False for "
                                        "this model")
                 followers[module] = leader
-        self._recent_input = None
+        self._recent_input = dict()
         for module in module_list:
             self._hook_calls.pop(module, None)
         for leader in followers.values():
@@ -434,7 +438,7 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
         self._held_bytes = 0
         self._leader = dict()
         self._hook_calls = dict()
-        self._recent_input = None
+        self._recent_input = dict()
         return True
 
     @contextlib.contextmanager

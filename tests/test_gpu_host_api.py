@@ -431,6 +431,67 @@ def test_moe_gptq_zero_token_expert_is_zeroed(share):
     assert torch.count_nonzero(experts[0].gate_proj.weight) > 0
 
 
+def test_moe_all_experts_calibration_shares_one_hessian_across_experts():
+    """``moe_calibrate_all_experts`` (the ``oneshot`` default, reference entrypoints/oneshot.py:350): every expert's
+    gate_proj and up_proj receive the block's whole input, so one Hessian and one factorisation serve all of them
+    (an expert's down_proj, of another width, is called in between and does not end the run); the weights are the
+    bits of the run that keeps one Hessian per Linear."""
+    from llmcompressor_amd import ops
+    from llmcompressor_amd.core import LifecycleCallbacks, active_session
+    from llmcompressor_amd.modeling import LinearExperts2D, moe_calibration_context
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+    from llmcompressor_amd.modifiers.gptq import gptq_quantize as gq
+
+    torch.manual_seed(0)
+    E, H, I, T = 6, 128, 64, 160
+    fused = (torch.randn(E, 2 * I, H) * 0.05, torch.randn(E, H, I) * 0.05)
+    x = torch.randn(T, H, device=DEV).bfloat16()
+    idx = torch.stack([torch.arange(T) % E, (torch.arange(T) + 2) % E], dim=1).to(DEV)
+    wts = torch.full((T, 2), 0.5, device=DEV, dtype=torch.bfloat16)
+    out = {}
+    for share in (True, False):
+        experts = LinearExperts2D.from_fused(*fused).to(DEV).to(torch.bfloat16)
+
+        class Wrap(torch.nn.Module):
+            def __init__(self):
+                super().__init__()
+                self.layers = torch.nn.ModuleList([experts])
+
+        model = Wrap()
+        mod = GPTQModifier(targets="Linear", share_identical_inputs=share, config_groups={"g": dict(
+            targets=["Linear"], weights=dict(num_bits=4, strategy="group", group_size=32))})
+        session = active_session()
+        session.reset()
+        session.initialize(model=model, recipe=mod)
+        LifecycleCallbacks.calibration_start()
+        launches, chains = [], []
+        raw_grouped, raw_hinv = ops.hessian_accumulate_grouped_, ops.gptq_hinv_grouped
+        ops.hessian_accumulate_grouped_ = lambda Hs, xs, **kw: (launches.append((len(Hs), xs[0].shape[1])),
+                                                                 raw_grouped(Hs, xs, **kw))[1]
+        ops.gptq_hinv_grouped = lambda Hs, *a, **kw: (chains.append((len(Hs), Hs[0].shape[0])), raw_hinv(Hs, *a, **kw))[1]
+        try:
+            with torch.no_grad(), moe_calibration_context(True):
+                for _ in range(2):
+                    experts(x, idx, wts)
+            LifecycleCallbacks.sequential_epoch_end(modules=list(model.modules()))
+        finally:
+            ops.hessian_accumulate_grouped_, ops.gptq_hinv_grouped = raw_grouped, raw_hinv
+        LifecycleCallbacks.calibration_end()
+        session.finalize()
+        per_forward = sorted(launches[: len(launches) // 2])
+        if share:
+            assert per_forward == [(1, H), (E, I)]          # one problem for all twelve gate / up projections
+            assert sorted(chains) == [(1, H), (E, I)]       # and one factorisation
+        else:
+            assert per_forward == [(E, I), (2 * E, H)]
+            assert sorted(chains) == [(E, I), (2 * E, H)]
+        out[share] = {k: v.detach().clone() for k, v in experts.state_dict().items()}
+    assert out[True].keys() == out[False].keys()
+    for k in out[True]:
+        assert torch.equal(out[True][k], out[False][k]), k
+    assert torch.count_nonzero(out[True]["3.down_proj.weight"]) > 0
+
+
 def _write_checkpoint(root, seed=0):
     """A two-shard toy checkpoint: q/k/v of layer 0 split across the shards, one fused-experts tensor."""
     import json
