@@ -608,3 +608,93 @@ def test_grouped_calls_give_the_bits_of_single_calls_in_the_grouped_factor_form(
         ob, lb = ops.gptq_quantize(Ws[b], Ub, scales[b], None, ops.FMT_INT, 4, 1, K // g, g_idx=gidx[b], perm=perms[b],
                                    dead=db, form=form)
         assert torch.equal(ob, outs[b]) and torch.equal(lb.reshape(()), loss[b])
+
+
+def _grid_values(fmt_name, bits):
+    if fmt_name == "fp4":
+        pos = torch.tensor([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0])
+        return torch.cat([-pos.flip(0), pos])
+    return torch.arange(-(1 << (bits - 1)), 1 << (bits - 1)).float()
+
+
+@pytest.mark.parametrize(
+    "R,K,fmt_name,bits,group,sym,actorder,dead_cols,n",
+    [
+        (1, 1024, "int", 4, 128, True, False, 0, 1),        # a single row: every product on the fp32 instruction
+        (17, 1536, "int", 4, 32, False, True, 3, 1),        # zero points, permuted columns, dead columns
+        (100, 9216, "int", 4, 128, True, True, 0, 1),       # 17 earlier groups in 9 pieces, the last one shorter
+        (513, 1024, "int", 8, 1024, True, False, 0, 1),     # per-channel scales, rows one past a tile
+        (64, 2048, "fp4", 4, 16, True, False, 5, 2),        # NVFP4 grid with a global scale, two problems in lock-step
+        (130, 1536, "fp8", 8, 1536, True, True, 0, 3),      # fp8 codes per channel, three problems
+    ],
+)
+def test_factor_forms_agree_over_shapes_and_formats(R, K, fmt_name, bits, group, sym, actorder, dead_cols, n):
+    """Edge shapes of the left-looking loop against the right-looking one on the device (which the oracle tests
+    pin): >= 99.9 % identical weights, values on the format's grid, equal losses, dead columns zeroed -- for single
+    and grouped calls."""
+    from llmcompressor_amd import ops
+
+    torch.manual_seed(R * 7 + K)
+    dev = "cuda"
+    fmt = {"int": ops.FMT_INT, "fp4": ops.FMT_FP4, "fp8": ops.FMT_FP8}[fmt_name]
+    T = max(2 * K, 2048)
+    Hs, Ws, scales, zps, gss, perms, gidx = [], [], [], [], [], [], []
+    for b in range(n):
+        x = torch.randn(T, K, device=dev) * (0.25 + 2 * torch.rand(K, device=dev))
+        if dead_cols:
+            x[:, torch.randperm(K, device=dev)[:dead_cols]] = 0
+        x = x.bfloat16()
+        H = torch.zeros(K, K, device=dev)
+        ops.hessian_accumulate_(H, x)
+        Hs.append(H)
+        w = (torch.randn(R, K, device=dev) * 0.02).bfloat16()
+        Ws.append(w)
+        mn, mx = ops.minmax_groups(w, group)
+        gs = None
+        if fmt_name == "fp4":
+            gs = (448.0 * 6.0 / w.abs().max().float()).reshape(1)
+            s, z, _ = ops.calculate_qparams(mn, mx, fmt, bits, True, ops.SCALE_NVFP4, gs)
+        else:
+            s, z, _ = ops.calculate_qparams(mn, mx, fmt, bits, sym)
+        scales.append(s)
+        zps.append(None if sym else z.to(torch.int8))
+        gss.append(gs)
+        perm = torch.argsort(torch.diag(H), descending=True, stable=True).to(torch.int32) if actorder else None
+        perms.append(perm)
+        g = torch.arange(K, dtype=torch.int32, device=dev) // group
+        gidx.append(g[perm.long()] if actorder else g)
+    pstack = torch.stack(perms) if actorder else None
+    results = {}
+    for form in (ops.FACTOR_INVERSE, ops.FACTOR_GROUPS):
+        if n == 1:
+            U, dead, info = ops.gptq_hinv_(Hs[0].clone(), perms[0], divisor=3.0, form=form)
+            wq, loss = ops.gptq_quantize(Ws[0], U, scales[0], zps[0], fmt, bits, 1, K // group, g_idx=gidx[0],
+                                         perm=perms[0], dead=dead, global_scale=gss[0], form=form)
+            outs, losses, deads = [wq], loss.reshape(1), dead.reshape(1, K)
+        else:
+            U, deads, info = ops.gptq_hinv_grouped([H.clone() for H in Hs], pstack, [3.0] * n, 0.01, form=form)
+            outs, losses = ops.gptq_quantize_grouped(
+                Ws, U, scales, None if sym else zps, fmt, bits, 1, K // group, g_idxs=gidx, perms=pstack, dead=deads,
+                global_scales=gss if fmt_name == "fp4" else None, form=form)
+        assert int(info.abs().sum()) == 0
+        results[form] = ([o.clone() for o in outs], losses.clone(), deads.clone())
+    (oa, la, da), (ob, lb, db) = results[ops.FACTOR_INVERSE], results[ops.FACTOR_GROUPS]
+    assert torch.equal(da, db) and int(da.sum()) == dead_cols * n
+    grid = _grid_values(fmt_name, bits).to(dev) if fmt_name != "fp8" else None
+    for b in range(n):
+        agree = (oa[b] == ob[b]).float().mean().item()
+        assert agree >= CODE_AGREEMENT, (b, agree)
+        assert abs(float(la[b]) - float(lb[b])) <= 5e-3 * abs(float(la[b])) + 1e-12
+        if actorder:
+            inv = torch.empty(K, dtype=torch.long, device=dev)
+            inv[perms[b].long()] = torch.arange(K, device=dev)
+            dead_orig = db[b].bool()[inv]
+        else:
+            dead_orig = db[b].bool()
+        assert torch.count_nonzero(ob[b][:, dead_orig]) == 0
+        if grid is not None and sym and fmt_name == "int":
+            s_full = scales[b].float().repeat_interleave(group, dim=1)[:, :K]
+            q = ob[b].float() / s_full
+            # q * scale was rounded to bf16: the quotient is an integer to within 2^-8 of its magnitude
+            assert torch.all((q - q.round()).abs() <= 0.005 * q.abs() + 1e-6)
+            assert q.round().min() >= grid.min() and q.round().max() <= grid.max()
