@@ -307,9 +307,10 @@ int llmc_gptq_hinv_grouped(const float* const* H, int64_t ldh, int32_t n, int64_
  * form says what U holds (see llmc_gptq_hinv).  With LLMC_FACTOR_GROUPS (blocksize >= 128) the columns beyond a
  * 512-column group are not updated after the group; instead each group first takes what all earlier groups owe it,
  *     W[:, G] += ((W0 - Q)[:, :g0] @ V[:g0, G]) @ U[G, G]        (W0: the weights before the loop, Q: quantised),
- * which equals -Err[:, :g0] @ U[:g0, G] without ever forming U outside the diagonal blocks.
+ * which equals -Err[:, :g0] @ U[:g0, G] without ever forming U outside the diagonal blocks.  That form needs more
+ * workspace (a second [R, K] fp32 matrix and the pieces of the product), hence the form argument of the size query.
  */
-int64_t llmc_gptq_quantize_workspace_bytes(int64_t R, int64_t K);
+int64_t llmc_gptq_quantize_workspace_bytes(int64_t R, int64_t K, int32_t form);
 int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R, int64_t K, int64_t ldw,
                        const float* U, int64_t ldu, const int32_t* perm, const uint8_t* dead,
                        const void* scale, int32_t scale_dtype, const int8_t* zero_point,
@@ -323,7 +324,7 @@ int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R, int64_t K
  * device pointers (zero_point / global_scale / g_idx may be NULL as in the single call); U is device
  * [n][K][ldu] with problem stride u_stride (as written by llmc_gptq_hinv_grouped), perm device [n, K] int32
  * or NULL, dead device [n, K] bytes or NULL, loss_out device [n].  Results are bit-identical to n single calls. */
-int64_t llmc_gptq_quantize_grouped_workspace_bytes(int64_t n, int64_t R, int64_t K);
+int64_t llmc_gptq_quantize_grouped_workspace_bytes(int64_t n, int64_t R, int64_t K, int32_t form);
 int llmc_gptq_quantize_grouped(const void* const* weight, int32_t w_dtype, int32_t n, int64_t R, int64_t K,
                                int64_t ldw, const float* U, int64_t ldu, int64_t u_stride,
                                const int32_t* perm, const uint8_t* dead, const void* const* scale,
@@ -368,7 +369,7 @@ int llmc_sgemm(const float* A, int64_t lda, const float* B, int64_t ldb, float* 
  *     trailing updates (:193-198) and count towards the target (:143-151).  The caller checks
  *     that the existing sparsity does not exceed the target (:127-133 raises).
  * out_weight receives the pruned weight in w_dtype, *loss_out the sum of (w - q)^2 / d^2 / 2. */
-int64_t llmc_sparsegpt_workspace_bytes(int64_t R, int64_t K);
+int64_t llmc_sparsegpt_workspace_bytes(int64_t R, int64_t K, int32_t form);
 int llmc_sparsegpt_sparsify(const void* weight, int32_t w_dtype, int64_t R, int64_t K, int64_t ldw,
                             const float* U, int64_t ldu, const uint8_t* dead, double sparsity,
                             int32_t prune_n, int32_t prune_m, int32_t blocksize, int32_t form,

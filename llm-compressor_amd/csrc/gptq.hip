@@ -875,9 +875,16 @@ inline int left_split_cap(int64_t R) {
   return (int)(s < 1 ? 1 : (s > LEFT_MAX_SPLITS ? LEFT_MAX_SPLITS : s));
 }
 
-inline int64_t left_extra_bytes(int64_t n, int64_t R, int64_t K) {
-  // D (W0, then W0 - Q), the pieces of the product, the negated sum
-  return align256(n * R * K * 4) + align256(n * left_split_cap(R) * R * LLMC_FACTOR_GROUP_WIDTH * 4) +
+// workspace behind the other buffers, for the left-looking form only: D (W0, then W0 - Q), the pieces of the
+// product (never more of them than there are earlier groups), the negated sum
+inline int64_t left_pieces_max(int64_t R, int64_t K) {
+  const int64_t earlier = K / LLMC_FACTOR_GROUP_WIDTH - 1;
+  const int64_t cap = left_split_cap(R);
+  return earlier < 1 ? 1 : (earlier < cap ? earlier : cap);
+}
+inline int64_t left_extra_bytes(int64_t n, int64_t R, int64_t K, int form) {
+  if (form != LLMC_FACTOR_GROUPS) return 0;
+  return align256(n * R * K * 4) + align256(n * left_pieces_max(R, K) * R * LLMC_FACTOR_GROUP_WIDTH * 4) +
          align256(n * R * LLMC_FACTOR_GROUP_WIDTH * 4);
 }
 
@@ -927,8 +934,9 @@ static int left_begin_group(int n, int64_t R, int64_t K, int64_t g0, const float
   float* Df = (float*)extra;
   float* P = (float*)(extra + align256(n * R * K * 4));
   const int cap = left_split_cap(R);
-  float* Cn = (float*)((char*)P + align256(n * cap * R * GW * 4));
-  const int64_t piece_stride = R * GW, problem_stride_p = (int64_t)cap * piece_stride;
+  const int64_t slots = left_pieces_max(R, K);  // pieces the workspace holds per problem (pieces <= slots below)
+  float* Cn = (float*)((char*)P + align256(n * slots * R * GW * 4));
+  const int64_t piece_stride = R * GW, problem_stride_p = slots * piece_stride;
   int pieces = 0;
   if (g0 > 0) {
     const int64_t m = g0 / GW;                      // earlier groups
@@ -958,11 +966,10 @@ static int left_begin_group(int n, int64_t R, int64_t K, int64_t g0, const float
   return 0;
 }
 
-extern "C" int64_t llmc_sparsegpt_workspace_bytes(int64_t R, int64_t K) {
+extern "C" int64_t llmc_sparsegpt_workspace_bytes(int64_t R, int64_t K, int32_t form) {
   const int64_t slices = (K + SG_MIN_BLOCK - 1) / SG_MIN_BLOCK;
   return align256(R * K * 4) + align256(R * GROUP * GB * 4) + align256(R * 4) +
-         align256(slices * SG_HIST_WORDS * 4) + align256(R * K) +
-         (K % LLMC_FACTOR_GROUP_WIDTH == 0 ? left_extra_bytes(1, R, K) : 0);
+         align256(slices * SG_HIST_WORDS * 4) + align256(R * K) + left_extra_bytes(1, R, K, form);
 }
 
 extern "C" int llmc_sparsegpt_sparsify(const void* weight, int32_t w_dtype, int64_t R, int64_t K, int64_t ldw,
@@ -986,7 +993,7 @@ extern "C" int llmc_sparsegpt_sparsify(const void* weight, int32_t w_dtype, int6
   LLMC_CHECK_ARG(blocksize > 0 && blocksize <= GB && (nm ? blocksize % prune_m == 0 : blocksize >= SG_MIN_BLOCK), 12);
   LLMC_CHECK_ARG(out_weight != nullptr && ldo >= K, 14);
   LLMC_CHECK_ARG(workspace != nullptr && (((uintptr_t)workspace) & 255) == 0, 17);
-  LLMC_CHECK_ARG(workspace_bytes >= llmc_sparsegpt_workspace_bytes(R, K), 18);
+  LLMC_CHECK_ARG(workspace_bytes >= llmc_sparsegpt_workspace_bytes(R, K, form), 18);
   hipStream_t st = (hipStream_t)stream;
   const int bs = blocksize;
   const int64_t nblocks = (K + bs - 1) / bs;
@@ -1160,9 +1167,8 @@ static int gptq_column_loop(void (*kern)(GptqBlockParams), GptqBlockParams p, in
   return 0;
 }
 
-extern "C" int64_t llmc_gptq_quantize_workspace_bytes(int64_t R, int64_t K) {
-  return align256(R * K * 4) + align256(R * GROUP * GB * 4) + align256(R * 4) +
-         (K % LLMC_FACTOR_GROUP_WIDTH == 0 ? left_extra_bytes(1, R, K) : 0);
+extern "C" int64_t llmc_gptq_quantize_workspace_bytes(int64_t R, int64_t K, int32_t form) {
+  return align256(R * K * 4) + align256(R * GROUP * GB * 4) + align256(R * 4) + left_extra_bytes(1, R, K, form);
 }
 
 extern "C" int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R, int64_t K, int64_t ldw,
@@ -1188,7 +1194,7 @@ extern "C" int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R
   LLMC_CHECK_ARG(blocksize > 0, 19);
   LLMC_CHECK_ARG(out_weight != nullptr && ldo >= K, 20);
   LLMC_CHECK_ARG(workspace != nullptr && (((uintptr_t)workspace) & 255) == 0, 23);
-  LLMC_CHECK_ARG(workspace_bytes >= llmc_gptq_quantize_workspace_bytes(R, K), 24);
+  LLMC_CHECK_ARG(workspace_bytes >= llmc_gptq_quantize_workspace_bytes(R, K, form), 24);
   hipStream_t st = (hipStream_t)stream;
   // the result does not depend on the block width mathematically (lazy batching only
   // regroups fp32 sums); widths above what fits on chip run as 128-wide blocks
@@ -1281,9 +1287,9 @@ extern "C" int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R
 // Every kernel of llmc_gptq_quantize is launched once for all problems (one more grid dimension, GEMM batch):
 // the serial chain of column blocks is as long as one problem's while each launch carries n times the rows.
 
-extern "C" int64_t llmc_gptq_quantize_grouped_workspace_bytes(int64_t n, int64_t R, int64_t K) {
+extern "C" int64_t llmc_gptq_quantize_grouped_workspace_bytes(int64_t n, int64_t R, int64_t K, int32_t form) {
   return align256(n * (int64_t)sizeof(GptqItem)) + align256(n * R * K * 4) + align256(n * R * GROUP * GB * 4) +
-         align256(n * R * 4) + (K % LLMC_FACTOR_GROUP_WIDTH == 0 ? left_extra_bytes(n, R, K) : 0);
+         align256(n * R * 4) + left_extra_bytes(n, R, K, form);
 }
 
 extern "C" int llmc_gptq_quantize_grouped(const void* const* weight, int32_t w_dtype, int32_t n, int64_t R, int64_t K,
@@ -1311,7 +1317,7 @@ extern "C" int llmc_gptq_quantize_grouped(const void* const* weight, int32_t w_d
   LLMC_CHECK_ARG(blocksize > 0, 21);
   LLMC_CHECK_ARG(out_weight != nullptr && ldo >= K, 22);
   LLMC_CHECK_ARG(workspace != nullptr && (((uintptr_t)workspace) & 255) == 0, 25);
-  LLMC_CHECK_ARG(workspace_bytes >= llmc_gptq_quantize_grouped_workspace_bytes(n, R, K), 26);
+  LLMC_CHECK_ARG(workspace_bytes >= llmc_gptq_quantize_grouped_workspace_bytes(n, R, K, form), 26);
   LLMC_CHECK_ARG(n < 65535 && (K + 255) / 256 < 65535, 3);
   hipStream_t st = (hipStream_t)stream;
   const int bs = blocksize > GB ? GB : blocksize;

@@ -54,10 +54,10 @@ SIGNATURES = {
     "llmc_hessian_accumulate_grouped": [_P, _I64, _P, _I64, _P, _I32, _I64, _I32, _F32, _I32, _P],
     "llmc_gptq_hinv_grouped_workspace_bytes": [_I64, _I64],
     "llmc_gptq_hinv_grouped": [_P, _I64, _I32, _I64, _P, _P, _F32, _I32, _P, _P, _I64, _P, _I64, _P, _P],
-    "llmc_gptq_quantize_grouped_workspace_bytes": [_I64, _I64, _I64],
+    "llmc_gptq_quantize_grouped_workspace_bytes": [_I64, _I64, _I64, _I32],
     "llmc_gptq_quantize_grouped": [_P, _I32, _I32, _I64, _I64, _I64, _P, _I64, _I64, _P, _P, _P, _I32, _P, _P, _P, _I64,
                                    _I64, _I32, _I32, _I32, _I32, _P, _I64, _P, _P, _I64, _P],
-    "llmc_sparsegpt_workspace_bytes": [_I64, _I64],
+    "llmc_sparsegpt_workspace_bytes": [_I64, _I64, _I32],
     "llmc_sparsegpt_sparsify": [_P, _I32, _I64, _I64, _I64, _P, _I64, _P, ctypes.c_double, _I32, _I32, _I32, _I32, _I32,
                                 _P, _I64, _P, _P, _I64, _P],
     "llmc_hessian_accumulate_segments": [_P, _I64, _P, _I32, _I64, _I64, _I64, _I64, _I32, _F32, _I32, _P, _I64, _P],
@@ -76,7 +76,7 @@ SIGNATURES.update({
     "llmc_gptq_hinv_workspace_bytes": [_I64],
     "llmc_gptq_hinv": [_P, _I64, _I64, _P, _F32, _F32, _I32, _P, _P, _I64, _P, _P],
     "llmc_gptq_factor_form": [_I64, _I32],
-    "llmc_gptq_quantize_workspace_bytes": [_I64, _I64],
+    "llmc_gptq_quantize_workspace_bytes": [_I64, _I64, _I32],
     "llmc_gptq_quantize": [_P, _I32, _I64, _I64, _I64, _P, _I64, _P, _P, _P, _I32, _P, _P, _P, _I64, _I64,
                            _I32, _I32, _I32, _I32, _P, _I64, _P, _P, _I64, _P],
 })

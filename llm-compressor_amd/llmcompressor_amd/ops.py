@@ -431,7 +431,7 @@ def gptq_quantize(weight, U, scale, zero_point, fmt: int, bits: int, row_div: in
         perm = perm.to(torch.int32).contiguous()
     out = torch.empty((R, K), dtype=weight.dtype, device=weight.device)
     loss = torch.empty(1, dtype=torch.float32, device=weight.device)
-    nbytes = _lib.lib().llmc_gptq_quantize_workspace_bytes(R, K)
+    nbytes = _lib.lib().llmc_gptq_quantize_workspace_bytes(R, K, int(form))
     ws = _workspace(weight.device, nbytes)
     with torch.cuda.device(weight.device):
         rc = _lib.lib().llmc_gptq_quantize(
@@ -476,7 +476,7 @@ def gptq_quantize_grouped(weights, U, scales, zero_points, fmt: int, bits: int, 
         perms = perms.to(torch.int32).contiguous()
     outs = [torch.empty((R, K), dtype=w0.dtype, device=w0.device) for _ in range(n)]
     loss = torch.empty(n, dtype=torch.float32, device=w0.device)
-    nbytes = _lib.lib().llmc_gptq_quantize_grouped_workspace_bytes(n, R, K)
+    nbytes = _lib.lib().llmc_gptq_quantize_grouped_workspace_bytes(n, R, K, int(form))
     ws = _workspace(w0.device, nbytes)
     wp = (ctypes.c_void_p * n)(*[w.data_ptr() for w in weights])
     op = (ctypes.c_void_p * n)(*[o.data_ptr() for o in outs])
@@ -507,7 +507,7 @@ def sparsegpt_sparsify(weight, U, sparsity: float, prune_n: int = 0, prune_m: in
                          f"{blocksize} in [32, 128]")
     out = torch.empty((R, K), dtype=weight.dtype, device=weight.device)
     loss = torch.empty(1, dtype=torch.float32, device=weight.device)
-    nbytes = _lib.lib().llmc_sparsegpt_workspace_bytes(R, K)
+    nbytes = _lib.lib().llmc_sparsegpt_workspace_bytes(R, K, int(form))
     ws = _workspace(weight.device, nbytes)
     with torch.cuda.device(weight.device):
         rc = _lib.lib().llmc_sparsegpt_sparsify(
