@@ -253,10 +253,11 @@ int llmc_dynamic_per_token_quantize(const void* x, int32_t x_dtype, int64_t N, i
  * perm may be NULL.  workspace must be 256-byte aligned.
  *
  * form selects what H holds afterwards.  LLMC_FACTOR_INVERSE: U as above.  LLMC_FACTOR_GROUPS (K a multiple of
- * 512): inside every aligned 512-column diagonal block the same U (a diagonal block of the inverse of a
- * triangular matrix is the inverse of its diagonal block); outside those blocks the upper Cholesky factor V of
- * the damped H itself (V V^T = H, V = U^-1), i.e. the chain stops before the triangular inverse is carried
- * across blocks, which is a third of its arithmetic.  llmc_gptq_quantize takes either form and gives the same
+ * 128): inside every 512-column diagonal block the same U (a diagonal block of the inverse of a triangular matrix
+ * is the inverse of its diagonal block); outside those blocks the upper Cholesky factor V of the damped H itself
+ * (V V^T = H, V = U^-1), i.e. the chain stops before the triangular inverse is carried across blocks, which is a
+ * third of its arithmetic.  The blocks are aligned to the last column: [K-512, K), [K-1024, K-512), ..., and a
+ * first block of the K % 512 columns that are left.  llmc_gptq_quantize takes either form and gives the same
  * result up to fp32 rounding, and so does llmc_sparsegpt_sparsify (its block size must then be 128).
  * llmc_gptq_factor_form(K, blocksize) is the form the library prefers for a quantize_weight / sparsify_weight
  * call.

@@ -513,10 +513,12 @@ extern "C" int64_t llmc_gptq_hinv_workspace_bytes(int64_t K) {
   return (Kp * Kp + hinv_temp_floats(Kp) + 64) * 4 + 256;
 }
 
-// Width up to which the inverse of the factor is formed: everything for LLMC_FACTOR_INVERSE, the aligned
-// 512-wide diagonal blocks for LLMC_FACTOR_GROUPS (the recursive doubling stops there, which leaves the Cholesky
-// factor itself outside those blocks; in the reversed index order of the work matrix the blocks start at
-// multiples of 512 exactly when K is one).
+// Width up to which the inverse of the factor is formed: everything for LLMC_FACTOR_INVERSE, 512-wide diagonal
+// blocks for LLMC_FACTOR_GROUPS (the recursive doubling stops there, which leaves the Cholesky factor itself outside
+// those blocks).  The work matrix is in reversed index order, so the blocks start at multiples of 512 counted from
+// the LAST column: [K - 512, K), [K - 1024, K - 512), ... and a first block of the K % 512 columns that are left
+// (K must be a multiple of 128, so that the work matrix has no padding and the column loop's 128-column blocks do
+// not straddle two of them).
 inline int64_t inverse_width(int32_t form, int64_t Kp) { return form == LLMC_FACTOR_GROUPS ? LLMC_FACTOR_GROUP_WIDTH : Kp; }
 
 // The chain saves the part of the triangular inverse that crosses blocks (a third of its arithmetic, growing with
@@ -526,15 +528,14 @@ inline int64_t inverse_width(int32_t form, int64_t Kp) { return form == LLMC_FAC
 constexpr int64_t FACTOR_GROUPS_MIN_K = 8192;
 
 extern "C" int32_t llmc_gptq_factor_form(int64_t K, int32_t blocksize) {
-  return (K % LLMC_FACTOR_GROUP_WIDTH == 0 && K >= FACTOR_GROUPS_MIN_K && blocksize >= 128) ? LLMC_FACTOR_GROUPS
-                                                                                             : LLMC_FACTOR_INVERSE;
+  return (K % 128 == 0 && K >= FACTOR_GROUPS_MIN_K && blocksize >= 128) ? LLMC_FACTOR_GROUPS : LLMC_FACTOR_INVERSE;
 }
 
 extern "C" int llmc_gptq_hinv(float* H, int64_t ldh, int64_t K, const int32_t* perm, float divisor,
                               float percdamp, int32_t form, uint8_t* dead_out, void* workspace,
                               int64_t workspace_bytes, int32_t* info_out, void* stream) {
   LLMC_CHECK_ARG(H != nullptr, 1);
-  LLMC_CHECK_ARG(form == LLMC_FACTOR_INVERSE || (form == LLMC_FACTOR_GROUPS && K % LLMC_FACTOR_GROUP_WIDTH == 0), 7);
+  LLMC_CHECK_ARG(form == LLMC_FACTOR_INVERSE || (form == LLMC_FACTOR_GROUPS && K % 128 == 0), 7);
   LLMC_CHECK_ARG(ldh >= K, 2);
   LLMC_CHECK_ARG(K > 0 && K <= 65536, 3);
   LLMC_CHECK_ARG(divisor != 0.f, 5);
@@ -622,7 +623,7 @@ extern "C" int llmc_gptq_hinv_grouped(const float* const* H, int64_t ldh, int32_
                                       int32_t form, uint8_t* dead_out, float* U_out, int64_t ldu, void* workspace,
                                       int64_t workspace_bytes, int32_t* info_out, void* stream) {
   LLMC_CHECK_ARG(H != nullptr && ldh >= K, 1);
-  LLMC_CHECK_ARG(form == LLMC_FACTOR_INVERSE || (form == LLMC_FACTOR_GROUPS && K % LLMC_FACTOR_GROUP_WIDTH == 0), 8);
+  LLMC_CHECK_ARG(form == LLMC_FACTOR_INVERSE || (form == LLMC_FACTOR_GROUPS && K % 128 == 0), 8);
   LLMC_CHECK_ARG(n >= 0 && n <= 4096, 3);
   if (n == 0) return 0;
   LLMC_CHECK_ARG(K > 0 && K <= 65536, 4);

@@ -861,16 +861,26 @@ static int launch_group_update(const float* Eb, int64_t ldE, const float* U, int
 // D = E U and E = D V (V = U^-1 upper triangular, V V^T = H), so what the columns of a group G owe to all
 // earlier columns, -E[:, :g0] U[:g0, G], equals (D[:, :g0] V[:g0, G]) U[G, G]: the factor of H itself outside
 // the diagonal blocks and the inverse only inside them.  Per group: one product with a contraction over all
-// earlier columns, cut into `splits` pieces so that it fills the chip; a pass that adds the pieces in a fixed
-// order, keeps W0's columns and negates the sum; one 512-wide product with the group's diagonal block; the
-// group's blocks as in the other form; a pass that turns the kept W0 into D.
+// earlier columns, cut into pieces so that it fills the chip; a pass that adds the pieces in a fixed order,
+// keeps W0's columns and negates the sum; one 512-wide product with the group's diagonal block; the group's
+// blocks as in the other form; a pass that turns the kept W0 into D.
+// The groups are the chain's diagonal blocks, which are aligned to the END of the column range (the chain works
+// in reversed index order): 512 columns each, except that the first one holds the K % 512 columns that are left
+// over when K is not a multiple of 512.
 constexpr int LEFT_MAX_SPLITS = 16;
+constexpr int64_t LEFT_GW = LLMC_FACTOR_GROUP_WIDTH;
+
+// end of the group that starts at column g0
+inline int64_t left_group_end(int64_t g0, int64_t K) {
+  const int64_t first = K % LEFT_GW ? K % LEFT_GW : LEFT_GW;
+  const int64_t e = g0 == 0 ? first : g0 + LEFT_GW;
+  return e < K ? e : K;
+}
 
 // pieces of the contraction for a weight of R rows: enough 256 x 256 (128 x 128 below 256 rows' multiple) tiles
 // for one per CU.  Depends on R only, never on how many problems share a launch.
 inline int left_split_cap(int64_t R) {
-  const int64_t tiles = (R % 256 == 0) ? (R / 256) * (LLMC_FACTOR_GROUP_WIDTH / 256)
-                                       : ((R + 127) / 128) * (LLMC_FACTOR_GROUP_WIDTH / 128);
+  const int64_t tiles = (R % 256 == 0) ? (R / 256) * (LEFT_GW / 256) : ((R + 127) / 128) * (LEFT_GW / 128);
   int64_t s = (256 + tiles - 1) / tiles;
   return (int)(s < 1 ? 1 : (s > LEFT_MAX_SPLITS ? LEFT_MAX_SPLITS : s));
 }
@@ -878,27 +888,27 @@ inline int left_split_cap(int64_t R) {
 // workspace behind the other buffers, for the left-looking form only: D (W0, then W0 - Q), the pieces of the
 // product (never more of them than there are earlier groups), the negated sum
 inline int64_t left_pieces_max(int64_t R, int64_t K) {
-  const int64_t earlier = K / LLMC_FACTOR_GROUP_WIDTH - 1;
+  const int64_t earlier = (K + LEFT_GW - 1) / LEFT_GW - 1;
   const int64_t cap = left_split_cap(R);
   return earlier < 1 ? 1 : (earlier < cap ? earlier : cap);
 }
 inline int64_t left_extra_bytes(int64_t n, int64_t R, int64_t K, int form) {
   if (form != LLMC_FACTOR_GROUPS) return 0;
-  return align256(n * R * K * 4) + align256(n * left_pieces_max(R, K) * R * LLMC_FACTOR_GROUP_WIDTH * 4) +
-         align256(n * R * LLMC_FACTOR_GROUP_WIDTH * 4);
+  return align256(n * R * K * 4) + align256(n * left_pieces_max(R, K) * R * LEFT_GW * 4) + align256(n * R * LEFT_GW * 4);
 }
+inline bool left_form_fits(int64_t K, int blocksize) { return K % GB == 0 && blocksize >= GB; }
 
-// D[:, G] = W[:, G] (the untouched columns of the group) and, when there are pieces, C = -(P_0 + P_1 + ...)
+// D[:, G] = W[:, G] (the untouched columns of the group, gw of them) and, when there are pieces (gw = 512 then),
+// C = -(P_0 + P_1 + ...)
 __global__ __launch_bounds__(256) void left_begin_group_kernel(const float* __restrict__ Wf, float* __restrict__ Df,
-                                                               int64_t K, int64_t g0, int64_t R,
+                                                               int64_t K, int64_t g0, int gw, int64_t R,
                                                                const float* __restrict__ P, int pieces,
                                                                int64_t piece_stride, int64_t problem_stride_p,
                                                                float* __restrict__ Cn) {
-  constexpr int GW = LLMC_FACTOR_GROUP_WIDTH;
   const int64_t b = blockIdx.y;
-  const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;  // element of the [R, GW] group slice
-  if (idx >= R * GW) return;
-  const int64_t row = idx / GW, col = idx % GW;
+  const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;  // element of the [R, gw] group slice
+  if (idx >= R * gw) return;
+  const int64_t row = idx / gw, col = idx % gw;
   const int64_t w = b * R * K + row * K + g0 + col;
   *(float4*)(Df + w) = *(const float4*)(Wf + w);
   if (pieces > 0) {
@@ -908,29 +918,29 @@ __global__ __launch_bounds__(256) void left_begin_group_kernel(const float* __re
       const float4 v = *(const float4*)(p + s * piece_stride);
       a.x += v.x; a.y += v.y; a.z += v.z; a.w += v.w;
     }
-    *(float4*)(Cn + b * R * GW + idx) = make_float4(-a.x, -a.y, -a.z, -a.w);
+    *(float4*)(Cn + b * R * gw + idx) = make_float4(-a.x, -a.y, -a.z, -a.w);
   }
 }
 
 // D[:, G] -= W[:, G] (W holds the quantised values of the group now)
 __global__ __launch_bounds__(256) void left_end_group_kernel(const float* __restrict__ Wf, float* __restrict__ Df,
-                                                             int64_t K, int64_t g0, int64_t R) {
-  constexpr int GW = LLMC_FACTOR_GROUP_WIDTH;
+                                                             int64_t K, int64_t g0, int gw, int64_t R) {
   const int64_t b = blockIdx.y;
   const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
-  if (idx >= R * GW) return;
-  const int64_t w = b * R * K + (idx / GW) * K + g0 + idx % GW;
+  if (idx >= R * gw) return;
+  const int64_t w = b * R * K + (idx / gw) * K + g0 + idx % gw;
   float4 d = *(const float4*)(Df + w);
   const float4 q = *(const float4*)(Wf + w);
   d.x -= q.x; d.y -= q.y; d.z -= q.z; d.w -= q.w;
   *(float4*)(Df + w) = d;
 }
 
-// what the group [g0, g0 + 512) owes to the columns before it, added to Wf[:, G]; `extra` is the memory behind
+// what the group that starts at g0 owes to the columns before it, added to Wf[:, G]; `extra` is the memory behind
 // the other work buffers (left_extra_bytes)
 static int left_begin_group(int n, int64_t R, int64_t K, int64_t g0, const float* U, int64_t ldu, int64_t u_stride,
                             float* Wf, char* extra, hipStream_t st) {
-  constexpr int64_t GW = LLMC_FACTOR_GROUP_WIDTH;
+  constexpr int64_t GW = LEFT_GW;
+  const int gw = (int)(left_group_end(g0, K) - g0);  // 512 for every group but possibly the first
   float* Df = (float*)extra;
   float* P = (float*)(extra + align256(n * R * K * 4));
   const int cap = left_split_cap(R);
@@ -939,21 +949,22 @@ static int left_begin_group(int n, int64_t R, int64_t K, int64_t g0, const float
   const int64_t piece_stride = R * GW, problem_stride_p = slots * piece_stride;
   int pieces = 0;
   if (g0 > 0) {
-    const int64_t m = g0 / GW;                      // earlier groups
-    const int64_t per = (m + cap - 1) / cap;        // groups per piece
-    pieces = (int)((m + per - 1) / per);
-    const int64_t chunk = per * GW, last = g0 - (pieces - 1) * chunk;
+    const int64_t m = (g0 + GW - 1) / GW;           // earlier groups (the first one may be short)
+    const int64_t per = (m + cap - 1) / cap;        // groups' worth of columns per piece
+    const int64_t chunk = per * GW;
+    pieces = (int)((g0 + chunk - 1) / chunk);
+    const int64_t last = g0 - (pieces - 1) * chunk;
     GemmF32 g = {};
     g.A = Df; g.lda = K; g.B = U + g0; g.ldb = ldu; g.C = P; g.ldc = GW;
-    g.M = (int)R; g.N = (int)GW; g.Kc = (int)chunk; g.alpha = 1.f; g.beta = 0.f;
+    g.M = (int)R; g.N = (int)GW; g.Kc = (int)(pieces == 1 ? last : chunk); g.alpha = 1.f; g.beta = 0.f;
     g.batch = pieces; g.stride_a = chunk; g.stride_b = chunk * ldu; g.stride_c = piece_stride;
-    g.kc_last = last == chunk ? 0 : (int)last;
+    g.kc_last = (pieces == 1 || last == chunk) ? 0 : (int)last;
     g.batch2 = n; g.stride2_a = R * K; g.stride2_b = u_stride; g.stride2_c = problem_stride_p;
     const int rc = llmc_gemm_f32(g, st);
     if (rc) return rc;
   }
-  hipLaunchKernelGGL(left_begin_group_kernel, dim3((unsigned)((R * GW / 4 + 255) / 256), (unsigned)n), dim3(256), 0, st,
-                     (const float*)Wf, Df, K, g0, R, (const float*)P, pieces, piece_stride, problem_stride_p, Cn);
+  hipLaunchKernelGGL(left_begin_group_kernel, dim3((unsigned)((R * gw / 4 + 255) / 256), (unsigned)n), dim3(256), 0, st,
+                     (const float*)Wf, Df, K, g0, gw, R, (const float*)P, pieces, piece_stride, problem_stride_p, Cn);
   LLMC_LAUNCH_STATUS();
   if (g0 > 0) {
     GemmF32 h = {};  // Wf[:, G] -= Cn U[G, G]; U holds exact zeros below the diagonal
@@ -963,6 +974,14 @@ static int left_begin_group(int n, int64_t R, int64_t K, int64_t g0, const float
     const int rc = llmc_gemm_f32(h, st);
     if (rc) return rc;
   }
+  return 0;
+}
+
+static int left_end_group(int n, int64_t R, int64_t K, int64_t g0, const float* Wf, char* extra, hipStream_t st) {
+  const int gw = (int)(left_group_end(g0, K) - g0);
+  hipLaunchKernelGGL(left_end_group_kernel, dim3((unsigned)((R * gw / 4 + 255) / 256), (unsigned)n), dim3(256), 0, st, Wf,
+                     (float*)extra, K, g0, gw, R);
+  LLMC_LAUNCH_STATUS();
   return 0;
 }
 
@@ -979,7 +998,7 @@ extern "C" int llmc_sparsegpt_sparsify(const void* weight, int32_t w_dtype, int6
                                        float* loss_out, void* workspace, int64_t workspace_bytes, void* stream) {
   LLMC_CHECK_ARG(weight != nullptr, 1);
   LLMC_CHECK_ARG(form == LLMC_FACTOR_INVERSE ||
-                     (form == LLMC_FACTOR_GROUPS && K % LLMC_FACTOR_GROUP_WIDTH == 0 && blocksize == GB), 13);
+                     (form == LLMC_FACTOR_GROUPS && left_form_fits(K, blocksize) && blocksize == GB), 13);
   LLMC_CHECK_ARG(w_dtype >= 0 && w_dtype <= 2, 2);
   LLMC_CHECK_ARG(R > 0 && R < (1ll << 24), 3);
   LLMC_CHECK_ARG(K > 0 && K < (1ll << 31), 4);
@@ -1046,8 +1065,8 @@ extern "C" int llmc_sparsegpt_sparsify(const void* weight, int32_t w_dtype, int6
   };
   // the same two-level lazy updates as the quantiser's loop
   int64_t blk = 0;
-  for (int64_t g0 = 0; g0 < K; g0 += (int64_t)GROUP * bs) {
-    const int64_t gend = (g0 + (int64_t)GROUP * bs) < K ? g0 + (int64_t)GROUP * bs : K;
+  for (int64_t g0 = 0, gend = 0; g0 < K; g0 = gend) {
+    gend = left ? left_group_end(g0, K) : ((g0 + (int64_t)GROUP * bs) < K ? g0 + (int64_t)GROUP * bs : K);
     if (left && (g0 > 0 || gend < K)) {  // what the group owes to the earlier columns, from the factor of H
       const int rc = left_begin_group(1, R, K, g0, U, ldu, 0, Wf, extra, st);
       if (rc) return rc;
@@ -1085,9 +1104,8 @@ extern "C" int llmc_sparsegpt_sparsify(const void* weight, int32_t w_dtype, int6
       }
     }
     if (gend < K && left) {
-      hipLaunchKernelGGL(left_end_group_kernel, dim3((unsigned)((R * (gend - g0) / 4 + 255) / 256), 1), dim3(256), 0, st,
-                         (const float*)Wf, (float*)extra, K, g0, R);
-      LLMC_LAUNCH_STATUS();
+      const int rc = left_end_group(1, R, K, g0, Wf, extra, st);
+      if (rc) return rc;
     } else if (gend < K) {
       GemmF32 g = {};
       g.A = E; g.lda = ldE; g.B = U + g0 * ldu + gend; g.ldb = ldu; g.C = Wf + gend; g.ldc = K;
@@ -1125,7 +1143,7 @@ static int gptq_column_loop(void (*kern)(GptqBlockParams), GptqBlockParams p, in
   const int ldE = GROUP * GB;
   p.ldE = ldE;
   const int64_t gw = (int64_t)GROUP * bs;
-  const bool left = form == LLMC_FACTOR_GROUPS;  // the callers have checked gw == 512 and K % 512 == 0
+  const bool left = form == LLMC_FACTOR_GROUPS;  // the callers have checked gw == 512 and K % 128 == 0
   auto product = [&](const float* A, int64_t k0, int64_t kc, int64_t c0, int64_t c1) {
     GemmF32 g = {};
     g.A = A; g.lda = ldE; g.B = U + k0 * ldu + c0; g.ldb = ldu; g.C = Wf + c0; g.ldc = K;
@@ -1133,9 +1151,9 @@ static int gptq_column_loop(void (*kern)(GptqBlockParams), GptqBlockParams p, in
     g.batch = 1; g.batch2 = n; g.stride2_a = R * (int64_t)ldE; g.stride2_b = u_stride; g.stride2_c = R * K;
     return llmc_gemm_f32(g, st);
   };
-  for (int64_t g0 = 0; g0 < K; g0 += gw) {
-    const int64_t gend = (g0 + gw) < K ? g0 + gw : K;
-    if (left && (g0 > 0 || gend < K)) {  // the only group of a 512-wide weight needs neither D nor a sum
+  for (int64_t g0 = 0, gend = 0; g0 < K; g0 = gend) {
+    gend = left ? left_group_end(g0, K) : ((g0 + gw) < K ? g0 + gw : K);
+    if (left && (g0 > 0 || gend < K)) {  // the only group of a narrow weight needs neither D nor a sum
       const int rc = left_begin_group(n, R, K, g0, U, ldu, u_stride, Wf, extra, st);
       if (rc) return rc;
     }
@@ -1155,9 +1173,8 @@ static int gptq_column_loop(void (*kern)(GptqBlockParams), GptqBlockParams p, in
     }
     if (gend < K) {
       if (left) {
-        hipLaunchKernelGGL(left_end_group_kernel, dim3((unsigned)((R * gw / 4 + 255) / 256), (unsigned)n), dim3(256), 0,
-                           st, (const float*)Wf, (float*)extra, K, g0, R);
-        LLMC_LAUNCH_STATUS();
+        const int rc = left_end_group(n, R, K, g0, Wf, extra, st);
+        if (rc) return rc;
       } else {
         const int rc = product(E, g0, gend - g0, gend, K);
         if (rc) return rc;
@@ -1180,7 +1197,7 @@ extern "C" int llmc_gptq_quantize(const void* weight, int32_t w_dtype, int64_t R
                                   int64_t workspace_bytes, void* stream) {
   LLMC_CHECK_ARG(weight != nullptr, 1);
   LLMC_CHECK_ARG(form == LLMC_FACTOR_INVERSE ||
-                     (form == LLMC_FACTOR_GROUPS && K % LLMC_FACTOR_GROUP_WIDTH == 0 && blocksize >= GB), 20);
+                     (form == LLMC_FACTOR_GROUPS && left_form_fits(K, blocksize)), 20);
   LLMC_CHECK_ARG(w_dtype >= 0 && w_dtype <= 2, 2);
   LLMC_CHECK_ARG(R > 0 && R < (1ll << 31), 3);
   LLMC_CHECK_ARG(K > 0 && K < (1ll << 31), 4);
@@ -1302,7 +1319,7 @@ extern "C" int llmc_gptq_quantize_grouped(const void* const* weight, int32_t w_d
                                           float* loss_out, void* workspace, int64_t workspace_bytes, void* stream) {
   LLMC_CHECK_ARG(weight != nullptr, 1);
   LLMC_CHECK_ARG(form == LLMC_FACTOR_INVERSE ||
-                     (form == LLMC_FACTOR_GROUPS && K % LLMC_FACTOR_GROUP_WIDTH == 0 && blocksize >= GB), 22);
+                     (form == LLMC_FACTOR_GROUPS && left_form_fits(K, blocksize)), 22);
   LLMC_CHECK_ARG(w_dtype >= 0 && w_dtype <= 2, 2);
   LLMC_CHECK_ARG(n >= 0 && n <= 4096, 3);
   if (n == 0) return 0;

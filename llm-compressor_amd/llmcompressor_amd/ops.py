@@ -354,13 +354,15 @@ FACTOR_INVERSE, FACTOR_GROUPS, FACTOR_GROUP_WIDTH = 0, 1, 512
 
 def gptq_factor_form(K: int, blocksize: int = 128) -> int:
     """The form of the factor the library prefers for a quantize_weight call on K columns: FACTOR_GROUPS where
-    the column loop can work from the Cholesky factor of H itself (K a multiple of 512), else FACTOR_INVERSE."""
+    the column loop can work from the Cholesky factor of H itself and the shorter chain pays for the loop's extra
+    launches (K a multiple of 128, from 8192 columns on), else FACTOR_INVERSE."""
     return int(_lib.lib().llmc_gptq_factor_form(int(K), int(blocksize)))
 
 
 def gptq_hinv_(H: torch.Tensor, perm=None, divisor: float = 1.0, percdamp: float = 0.01, form: int = FACTOR_INVERSE):
     """In place: H -> upper factor U of (H/divisor [permuted] + damping)^-1; with form = FACTOR_GROUPS only inside
-    the aligned 512-column diagonal blocks, the upper Cholesky factor of the damped H itself outside them.
+    the 512-column diagonal blocks (aligned to the last column), the upper Cholesky factor of the damped H itself
+    outside them.
 
     Returns (U (= H), dead uint8 [K], info int32 [1] on device)."""
     _require_gpu(H)

@@ -478,14 +478,23 @@ def test_factor_form_choice():
     assert ops.gptq_factor_form(14336, 128) == ops.FACTOR_GROUPS
     assert ops.gptq_factor_form(8192, 512) == ops.FACTOR_GROUPS
     assert ops.gptq_factor_form(4096, 128) == ops.FACTOR_INVERSE   # the chain's saving does not pay for the loop's cost
-    assert ops.gptq_factor_form(14336 + 256, 128) == ops.FACTOR_INVERSE  # groups would not line up with the chain's blocks
+    assert ops.gptq_factor_form(11008 + 8192, 128) == ops.FACTOR_GROUPS  # not a multiple of 512: a short first group
+    assert ops.gptq_factor_form(14336 + 64, 128) == ops.FACTOR_INVERSE   # 128-column blocks would straddle two groups
     assert ops.gptq_factor_form(14336, 64) == ops.FACTOR_INVERSE   # narrower column blocks
 
 
-@pytest.mark.parametrize("K,use_perm", [(1024, False), (1536, True), (2048, True)])
+def _groups(K):
+    """Column ranges of the diagonal blocks: 512 wide, aligned to the last column, the first one what is left."""
+    first = K % 512 or 512
+    edges = [0] + list(range(first, K + 1, 512))
+    return list(zip(edges[:-1], edges[1:]))
+
+
+@pytest.mark.parametrize("K,use_perm", [(1024, False), (1536, True), (2048, True), (1152, True), (1920, False)])
 def test_grouped_factor_is_the_cholesky_factor_outside_the_diagonal_blocks(K, use_perm):
-    """form = FACTOR_GROUPS against fp64: V V^T = H (V upper) outside the aligned 512-blocks, inv(V[G, G]) inside;
-    the diagonal blocks agree with the other form's U to fp32 rounding."""
+    """form = FACTOR_GROUPS against fp64: V V^T = H (V upper) outside the 512-blocks (aligned to the last column; a
+    width that is not a multiple of 512 starts with a short one), inv(V[G, G]) inside; the diagonal blocks agree
+    with the other form's U to fp32 rounding."""
     from llmcompressor_amd import ops
 
     H, _ = _hessian(K, 3 * K, K + 1)
@@ -498,15 +507,15 @@ def test_grouped_factor_is_the_cholesky_factor_outside_the_diagonal_blocks(K, us
     V64 = torch.flip(torch.linalg.cholesky(torch.flip(Hd, (0, 1))), (0, 1))  # upper, V V^T = H
     assert (V64 @ V64.t() - Hd).abs().max() / Hd.abs().max() < 1e-12 and torch.equal(V64, torch.triu(V64))
     want = V64.clone()
-    for g0 in range(0, K, 512):
-        want[g0:g0 + 512, g0:g0 + 512] = torch.linalg.inv(V64[g0:g0 + 512, g0:g0 + 512])
+    for g0, g1 in _groups(K):
+        want[g0:g1, g0:g1] = torch.linalg.inv(V64[g0:g1, g0:g1])
     pg = perm.cuda() if use_perm else None
     M, dead, info = ops.gptq_hinv_(H.clone().cuda(), pg, divisor=n, percdamp=0.01, form=ops.FACTOR_GROUPS)
     U, _, _ = ops.gptq_hinv_(H.clone().cuda(), pg, divisor=n, percdamp=0.01)
     M, U = M.cpu(), U.cpu()
     assert info.item() == 0 and dead.sum().item() == 0 and torch.equal(M, torch.triu(M))
-    for g0 in range(0, K, 512):
-        G_ = slice(g0, g0 + 512)
+    for g0, g1 in _groups(K):
+        G_ = slice(g0, g1)
         blk, ref = M[G_, G_].double(), want[G_, G_]
         assert ((blk - ref).norm() / ref.norm()).item() < 2e-5
         assert ((blk - U[G_, G_].double()).norm() / ref.norm()).item() < 2e-5
@@ -525,6 +534,8 @@ def test_grouped_factor_is_the_cholesky_factor_outside_the_diagonal_blocks(K, us
         (200, 1536, 128, "weight", dict(symmetric=False)),
         (128, 2048, 32, "weight", {}),
         (256, 1024, 128, None, dict(bits=8)),
+        (96, 1152, 128, "weight", {}),                       # a first group of 128 columns, then two of 512
+        (64, 1920, 64, None, dict(symmetric=False)),         # a first group of 384 columns
         # fewer tokens than columns: only the damping keeps H regular, and an fp32 factor is then ~1e-5 from the exact
         # one whoever computes it (the fp32 oracle itself agrees with its fp64 run on 99.81 % of these 8-bit codes,
         # this form on 99.79 %, the other on 99.75 %): the bar of the rank-deficient expert Hessians
@@ -548,7 +559,7 @@ def test_gptq_from_the_grouped_factor_matches_the_oracle(R, K, g, actorder, kw):
     assert abs(loss_g - loss_o) <= 0.01 * abs(loss_o) + 1e-9
 
 
-@pytest.mark.parametrize("R,K", [(8192, 3072), (1024, 4096), (4096, 5120)])
+@pytest.mark.parametrize("R,K", [(8192, 3072), (1024, 4096), (4096, 5120), (2048, 11008)])
 def test_both_factor_forms_give_the_same_weights_at_size(R, K):
     """Sizes at which the contraction over the earlier columns is cut into pieces (8192 rows: four pieces at most,
     so the five groups before the last one of 3072 columns go 2 + 2 + 1, a shorter last piece)."""
@@ -626,6 +637,7 @@ def _grid_values(fmt_name, bits):
         (513, 1024, "int", 8, 1024, True, False, 0, 1),     # per-channel scales, rows one past a tile
         (64, 2048, "fp4", 4, 16, True, False, 5, 2),        # NVFP4 grid with a global scale, two problems in lock-step
         (130, 1536, "fp8", 8, 1536, True, True, 0, 3),      # fp8 codes per channel, three problems
+        (72, 1664, "int", 4, 128, True, True, 2, 2),        # a first group of 128 columns, two problems in lock-step
     ],
 )
 def test_factor_forms_agree_over_shapes_and_formats(R, K, fmt_name, bits, group, sym, actorder, dead_cols, n):

@@ -92,6 +92,7 @@ GROUPED_FACTOR_CASES = [
     dict(R=64, K=1024, kw=dict(sparsity=0.5)),
     dict(R=96, K=1536, kw=dict(sparsity=0.5, prune_n=2, prune_m=4)),
     dict(R=64, K=1024, zero_frac=0.3, kw=dict(sparsity=0.6, preserve_sparsity_mask=True)),
+    dict(R=48, K=1408, zero_frac=0.2, kw=dict(sparsity=0.5, preserve_sparsity_mask=True)),  # a first group of 384 columns
 ]
 
 
