@@ -13,6 +13,7 @@
 from __future__ import annotations
 
 import contextlib
+import logging
 from typing import Dict, List, Optional
 
 import torch
@@ -20,6 +21,8 @@ import torch
 from ..core import LifecycleCallbacks, active_session
 from ..modifiers.utils.hooks import HooksMixin
 from ..quantization import disable_quantization, enable_quantization
+
+logger = logging.getLogger("llmcompressor_amd")
 
 __all__ = ["CalibrationPipeline", "SequentialPipeline", "DataFreePipeline", "BasicPipeline", "IndependentPipeline",
            "calibration_forward_context", "DisableQuantization", "find_decoder_layers"]
@@ -88,8 +91,15 @@ def find_decoder_layers(model: torch.nn.Module, sequential_targets=None) -> List
     if sequential_targets:
         names = [sequential_targets] if isinstance(sequential_targets, str) else list(sequential_targets)
         layers = [m for m in model.modules() if m.__class__.__name__ in names]
-        if layers:
+        if layers and _is_chain(model, layers):
             return layers
+        if layers:
+            # The reference cuts the traced graph at any module class (attention and each expert of one decoder
+            # layer as separate subgraphs, to bound the Hessians held at once); this pipeline feeds each target's
+            # output to the next one, which only whole layers of one list allow.  A decoder layer's Hessians fit
+            # the GPU, so the layer partition is used instead of failing.
+            logger.warning(f"sequential_targets {names} are not the elements of one layer list; calibrating by "
+                           "decoder layer instead")
     no_split = getattr(model, "_no_split_modules", None)
     if no_split:
         layers = [m for m in model.modules() if m.__class__.__name__ in set(no_split)]
@@ -110,6 +120,15 @@ def find_decoder_layers(model: torch.nn.Module, sequential_targets=None) -> List
     if best is None:
         raise ValueError("could not infer sequential targets: the model has no ModuleList of layers")
     return list(best)
+
+
+def _is_chain(model: torch.nn.Module, layers: List[torch.nn.Module]) -> bool:
+    """Are `layers` exactly the elements of one ModuleList (so that each one's output is the next one's input)?"""
+    ids = {id(l) for l in layers}
+    for m in model.modules():
+        if isinstance(m, torch.nn.ModuleList) and len(m) == len(layers) and all(id(x) in ids for x in m):
+            return True
+    return False
 
 
 from .cache import IntermediatesCache  # noqa: E402

@@ -847,3 +847,39 @@ def test_calibration_dataloader_from_an_in_memory_dataset():
     custom = get_calibration_dataloader(ds, data_collator=lambda feats: {"n": len(feats)}, batch_size=3,
                                         shuffle_calibration_samples=False)
     assert [b["n"] for b in custom] == [3, 3]
+
+
+def test_sequential_targets_that_are_not_a_layer_list_fall_back_to_the_layers(caplog):
+    """The reference cuts its traced graph at any module class (``sequential_targets=["Attention", "ExpertMLP"]`` in
+    its MoE examples); here targets that are not the elements of one layer list would not form a chain, so the
+    model's decoder layers are used and a warning says so."""
+    import logging
+
+    from llmcompressor_amd.pipelines import find_decoder_layers
+
+    class Attn(torch.nn.Module):
+        pass
+
+    class Mlp(torch.nn.Module):
+        pass
+
+    class Block(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.attn, self.mlp = Attn(), Mlp()
+
+    class Model(torch.nn.Module):
+        _no_split_modules = ["Block"]
+
+        def __init__(self):
+            super().__init__()
+            self.layers = torch.nn.ModuleList([Block() for _ in range(3)])
+
+    model = Model()
+    assert find_decoder_layers(model, ["Block"]) == list(model.layers)
+    assert find_decoder_layers(model, "Block") == list(model.layers)
+    with caplog.at_level(logging.WARNING, logger="llmcompressor_amd"):
+        got = find_decoder_layers(model, ["Attn", "Mlp"])
+    assert got == list(model.layers)
+    assert "not the elements of one layer list" in caplog.text
+    assert find_decoder_layers(model, ["NoSuchClass"]) == list(model.layers)
