@@ -509,7 +509,9 @@ def test_sequential_partition_prefers_decoder_layers_over_nested_lists():
     assert find_decoder_layers(m, None) == list(m.layers)
     m._no_split_modules = ["Layer"]
     assert find_decoder_layers(m, None) == list(m.layers)
-    assert find_decoder_layers(m, ["Linear"]) == [x for x in m.modules() if isinstance(x, torch.nn.Linear)]
+    # explicit targets that are not the elements of one list cannot be run as a chain: the layers are used
+    assert find_decoder_layers(m, ["Linear"]) == list(m.layers)
+    assert find_decoder_layers(m, ["Layer"]) == list(m.layers)
 
 
 @pytest.mark.parametrize("transposed,bias", [(False, False), (True, False), (False, True)])
