@@ -1667,6 +1667,60 @@ def test_a_model_on_the_host_is_calibrated_on_the_gpu(monkeypatch):
         oneshot(model=make(), recipe=QuantizationModifier(targets="Linear", scheme="FP8_DYNAMIC", ignore=["lm_head"]))
 
 
+def test_the_reference_example_flow_runs_line_for_line(tmp_path):
+    """examples/quantization_w4a16/llama3_example.py with the hub taken out: a checkpoint directory loaded with
+    ``AutoModelForCausalLM.from_pretrained`` (host memory), an in-memory dataset, the reference's import lines,
+    ``oneshot`` without ``output_dir``, ``model.generate`` on the compressed model, ``model.save_pretrained(SAVE_DIR,
+    save_compressed=True)``; the saved checkpoint decodes to the weights the model holds."""
+    transformers = pytest.importorskip("transformers")
+    datasets = pytest.importorskip("datasets")
+    from safetensors.torch import load_file
+
+    from llmcompressor import oneshot
+    from llmcompressor.modifiers.quantization import GPTQModifier
+    from llmcompressor.utils import dispatch_for_generation
+
+    from llmcompressor_amd.compressors import decompress_weight
+
+    torch.manual_seed(0)
+    cfg = transformers.LlamaConfig(hidden_size=128, intermediate_size=256, num_hidden_layers=2,
+                                   num_attention_heads=4, num_key_value_heads=2, vocab_size=256,
+                                   max_position_embeddings=128)
+    src = str(tmp_path / "checkpoint")
+    transformers.LlamaForCausalLM(cfg).to(torch.bfloat16).save_pretrained(src)
+
+    MODEL_ID = src
+    model = transformers.AutoModelForCausalLM.from_pretrained(MODEL_ID, dtype="auto")
+    assert next(model.parameters()).device.type == "cpu" and next(model.parameters()).dtype == torch.bfloat16
+    NUM_CALIBRATION_SAMPLES, MAX_SEQUENCE_LENGTH = 8, 64
+    rows = [torch.randint(0, 256, (int(n),)).tolist() for n in torch.randint(70, 120, (12,))]
+    ds = datasets.Dataset.from_dict({"input_ids": rows, "attention_mask": [[1] * len(r) for r in rows]})
+    ds = ds.shuffle(seed=42)
+
+    recipe = GPTQModifier(targets="Linear", scheme="W4A16", ignore=["lm_head"])
+    oneshot(model=model, dataset=ds, recipe=recipe, max_seq_length=MAX_SEQUENCE_LENGTH,
+            num_calibration_samples=NUM_CALIBRATION_SAMPLES)
+
+    dispatch_for_generation(model)
+    sample = torch.randint(0, 256, (1, 8)).to(model.device)
+    output = model.generate(sample, max_new_tokens=4, do_sample=False)
+    assert output.shape == (1, 12) and model.device.type == "cuda"
+
+    SAVE_DIR = str(tmp_path / "tiny-W4A16-G128")
+    model.save_pretrained(SAVE_DIR, save_compressed=True)
+    sd = load_file(os.path.join(SAVE_DIR, "model.safetensors"))
+    q = json.load(open(os.path.join(SAVE_DIR, "config.json")))["quantization_config"]
+    assert q["format"] == "pack-quantized" and q["quantization_status"] == "compressed" and "lm_head" in q["ignore"]
+    assert os.path.exists(os.path.join(SAVE_DIR, "recipe.yaml"))
+    for name, lin in model.named_modules():
+        if isinstance(lin, torch.nn.Linear) and name != "lm_head":
+            tensors = {k[len(name) + 1:]: v.to(DEV) for k, v in sd.items() if k.startswith(name + ".")}
+            assert tensors["weight_packed"].dtype == torch.int32
+            assert torch.equal(decompress_weight(tensors, lin.quantization_scheme.weights, "pack-quantized"),
+                               lin.weight.data), name
+    assert sd["lm_head.weight"].dtype == torch.bfloat16
+
+
 def test_gptq_beats_round_to_nearest_end_to_end_on_a_transformers_llama():
     """The whole pipeline on a 4-layer transformers Llama with anisotropic activations: W4A16 through
     GPTQModifier (sequential, error feedback from calibration data) gives a clearly smaller logit error on
