@@ -1198,6 +1198,75 @@ def test_gptq_same_width_linears_in_lock_step_match_per_module_path(actorder):
     assert not torch.equal(results[0][1]["layers.0.q.weight"], init["layers.0.q.weight"])
 
 
+def test_gptq_wide_linears_use_the_factor_in_groups_in_both_paths():
+    """Linears of 8192 input features (a 70B model's hidden width): the modifier asks the chain for the factor in
+    groups and the loops take their far updates from it, in the lock-step set (three projections fed one tensor,
+    one of another height) as in the per-module path; the two paths give the same bits, and the factor the set
+    receives is the grouped one."""
+    from llmcompressor_amd import ops
+    from llmcompressor_amd.core import LifecycleCallbacks, active_session
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+
+    W = 8192
+
+    class Block(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            mk = lambda i, o: torch.nn.Linear(i, o, bias=False)
+            self.q, self.k, self.v, self.o = mk(W, 128), mk(W, 64), mk(W, 64), mk(128, W)
+
+        def forward(self, x):
+            return self.o(self.q(x) + torch.cat([self.k(x), self.v(x)], -1))
+
+    class Wrap(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.layers = torch.nn.ModuleList([Block()])
+
+    assert ops.gptq_factor_form(W, 128) == ops.FACTOR_GROUPS
+    torch.manual_seed(3)
+    init = Wrap().to(DEV).to(torch.bfloat16).state_dict()
+    scale = torch.pow(2.0, 2.0 * torch.rand(W, device=DEV))
+    xs = [(torch.randn(4, 1024, W, device=DEV) * scale).bfloat16() for _ in range(3)]
+    results = []
+    for group_min in (0, 2):
+        model = Wrap().to(DEV).to(torch.bfloat16)
+        model.load_state_dict(init)
+        forms = []
+        raw_g, raw_s = ops.gptq_hinv_grouped, ops.gptq_hinv_
+        ops.gptq_hinv_grouped = lambda Hs, *a, **kw: (forms.append(("set", len(Hs), kw.get("form"))),
+                                                      raw_g(Hs, *a, **kw))[1]
+        ops.gptq_hinv_ = lambda H, *a, **kw: (forms.append(("one", H.shape[0], kw.get("form"))), raw_s(H, *a, **kw))[1]
+        try:
+            mod = GPTQModifier(targets="Linear", group_min_modules=group_min, scheme="W4A16")
+            session = active_session()
+            session.reset()
+            session.initialize(model=model, recipe=mod)
+            LifecycleCallbacks.calibration_start()
+            with torch.no_grad():
+                for x in xs:
+                    model.layers[0](x)
+            LifecycleCallbacks.sequential_epoch_end(modules=list(model.modules()))
+            LifecycleCallbacks.calibration_end()
+            session.finalize()
+        finally:
+            ops.gptq_hinv_grouped, ops.gptq_hinv_ = raw_g, raw_s
+        torch.cuda.synchronize()
+        results.append((forms, {n: p.detach().clone() for n, p in model.named_parameters()}))
+    per_module, lock_step = results
+    wide = [f for f in per_module[0] if f[1] == W]
+    assert len(wide) == 3 and all(f == ("one", W, ops.FACTOR_GROUPS) for f in wide)
+    assert ("set", 1, ops.FACTOR_GROUPS) in lock_step[0]      # q / k / v share one Hessian: one factorisation
+    assert ("one", 128, ops.FACTOR_INVERSE) in per_module[0]  # the narrow o projection keeps the full inverse
+    for n in per_module[1]:
+        assert torch.equal(per_module[1][n], lock_step[1][n]), n
+    q = per_module[1]["layers.0.q.weight"]
+    assert not torch.equal(q, init["layers.0.q.weight"])
+    s = per_module[1]["layers.0.q.weight_scale"].float().repeat_interleave(128, dim=1)
+    codes = q.float() / s
+    assert torch.all((codes - codes.round()).abs() <= 0.005 * codes.abs() + 1e-6) and codes.round().abs().max() <= 8
+
+
 def test_oneshot_gptq_on_a_transformers_llama(tmp_path):
     """A random-init transformers LlamaForCausalLM (2 layers, grouped-query attention) through oneshot with the
     W4A16 preset: every decoder Linear ends on its group's int4 grid with the preset's parameters, lm_head is
