@@ -422,3 +422,61 @@ def _check_experts(scheme, R, K, which, Ws, xs, Hs, outs, loss, scales, gss, cou
         if scheme == "nvfp4":
             assert gss[b].item() == exp["weight_global_scale"].float().item() or \
                 gss[b].to(torch.bfloat16).item() == exp["weight_global_scale"].item()
+
+
+def test_sequential_gptq_through_oneshot_at_the_llama3_8b_layer_shapes():
+    """BASELINE's sequential configuration on the real layer (hidden 4096, intermediate 14336, 32 query and 8
+    key / value heads) of a transformers Llama, two layers deep, 8 batches of 2048 tokens, W4A16 g128 with static
+    activation ordering, through ``oneshot`` with the modifier's defaults (staged Hessian launches, shared inputs,
+    lock-step chain for the six 4096-wide Linears, factor in groups for down_proj): every decoder Linear ends on
+    its groups' int4 grid, and on held-out tokens the logits are closer to the dense model's than with
+    round-to-nearest on the same grid."""
+    transformers = pytest.importorskip("transformers")
+
+    from llmcompressor_amd import oneshot
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+    from llmcompressor_amd.modifiers.quantization import QuantizationModifier
+
+    cfg = transformers.LlamaConfig(hidden_size=4096, intermediate_size=14336, num_hidden_layers=2,
+                                   num_attention_heads=32, num_key_value_heads=8, vocab_size=2048,
+                                   max_position_embeddings=2048)
+
+    def make():
+        torch.manual_seed(0)
+        with torch.device(DEV):
+            m = transformers.LlamaForCausalLM(cfg).to(torch.bfloat16)
+        # anisotropic hidden states, as trained models have: a few embedding channels carry most of the energy
+        with torch.no_grad():
+            boost = torch.ones(4096, device=DEV)
+            boost[torch.randperm(4096, device=DEV)[:64]] = 12.0
+            m.model.embed_tokens.weight.mul_(boost.to(torch.bfloat16))
+        return m
+
+    torch.manual_seed(1)
+    data = [{"input_ids": torch.randint(0, 2048, (1, 2048))} for _ in range(8)]
+    held_out = torch.randint(0, 2048, (1, 1024), device=DEV)
+    dense = make()
+    with torch.no_grad():
+        want = dense(held_out).logits.float()
+    del dense
+
+    def err(model):
+        with torch.no_grad():
+            return (model(held_out).logits.float() - want).norm().item() / want.norm().item()
+
+    gptq = make()
+    oneshot(model=gptq, dataset=data, recipe=GPTQModifier(targets="Linear", scheme="W4A16", ignore=["lm_head"]))
+    e_gptq = err(gptq)
+    for name, lin in gptq.named_modules():
+        if isinstance(lin, torch.nn.Linear) and name != "lm_head":
+            s = lin.weight_scale.data.float().repeat_interleave(128, dim=1)
+            codes = lin.weight.data.float() / s
+            assert torch.all((codes - codes.round()).abs() <= 0.005 * codes.abs() + 1e-6), name
+            assert codes.round().min() >= -8 and codes.round().max() <= 7, name
+            assert not hasattr(lin, "weight_g_idx"), name  # static ordering leaves no permutation behind
+    del gptq
+    rtn = make()
+    oneshot(model=rtn, recipe=QuantizationModifier(targets="Linear", scheme="W4A16", ignore=["lm_head"]))
+    e_rtn = err(rtn)
+    print(f"relative logit error on held-out tokens: GPTQ {e_gptq:.4f}, round-to-nearest {e_rtn:.4f}", flush=True)
+    assert e_gptq < 0.9 * e_rtn, (e_gptq, e_rtn)
