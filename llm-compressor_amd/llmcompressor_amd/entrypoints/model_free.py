@@ -188,15 +188,19 @@ def _store_compressed(tensors: Dict[str, torch.Tensor], name: str, module_name: 
 
 
 def process_file(inverse_weight_map: Dict[str, Optional[List[str]]], save_path: str, config: QuantizationConfig,
-                 device) -> Tuple[int, Dict[str, str]]:
+                 device, converter=None) -> Tuple[int, Dict[str, str]]:
     """Quantize and compress the tensors of one output shard.  ``inverse_weight_map`` maps a source
-    file to the tensor names to read from it (None = all)."""
+    file to the tensor names to read from it (None = all).  A ``converter`` rewrites the shard's tensors
+    (``converter.process(tensors) -> tensors``) before anything is matched against the schemes
+    (reference: process.py:111-112)."""
     tensors: Dict[str, torch.Tensor] = {}
     for path, wanted in inverse_weight_map.items():
         with safe_open(path, framework="pt", device="cpu") as f:
             for key in (f.keys() if wanted is None else wanted):
                 tensors[key] = f.get_tensor(key)
     tensors = split_fused_moe_experts(tensors)
+    if converter is not None:
+        tensors = converter.process(tensors)
 
     fused_index: Dict[str, int] = {}
     nfused = 0
@@ -248,7 +252,10 @@ def _checkpoint_files(model_stub) -> Dict[str, str]:
     return {str(p.relative_to(root)): str(p) for p in sorted(root.rglob("*")) if p.is_file()}
 
 
-def _build_jobs(model_files: Dict[str, str], save_directory: str, config: QuantizationConfig):
+def _build_jobs(model_files: Dict[str, str], save_directory: str, config: QuantizationConfig, converter=None):
+    """One job per output shard.  Tensors that must be read together (the partners of a fused global scale, and
+    whatever ``converter.get_dependencies(name)`` names for a tensor) are moved to the shard of the tensor that
+    needs them."""
     shards = {rel: path for rel, path in model_files.items() if rel.endswith(".safetensors")}
     location: Dict[str, str] = {}
     for rel, path in shards.items():
@@ -267,6 +274,11 @@ def _build_jobs(model_files: Dict[str, str], save_directory: str, config: Quanti
                     partner = t.format(**m.groupdict())
                     if partner in location and location[partner] != rel:
                         moved[partner] = rel
+    if converter is not None and hasattr(converter, "get_dependencies"):
+        for name, rel in location.items():
+            for dep in converter.get_dependencies(name) or ():
+                if dep in location and location[dep] != rel and dep not in moved and name not in moved:
+                    moved[dep] = rel
     jobs = []
     for rel, path in shards.items():
         own = [k for k, r in location.items() if r == rel and k not in moved]
@@ -280,14 +292,75 @@ def _build_jobs(model_files: Dict[str, str], save_directory: str, config: Quanti
     return jobs, location
 
 
-def update_config(save_directory: str, config: QuantizationConfig):
-    """Write ``quantization_config`` into ``config.json`` (reference: save_utils.py:24-121)."""
+def _converted_groups(converter) -> Tuple[Dict[str, dict], List[str], Optional[dict]]:
+    """Config groups, ignore list and kv-cache scheme that ``converter.create_config()`` declares for the tensors it
+    rewrote (reference: save_utils.py:79-80); the result may be a config object of this package, any object with
+    the same attributes, a plain dict, or None."""
+    made = converter.create_config() if hasattr(converter, "create_config") else None
+    if made is None:
+        return {}, [], None
+    if hasattr(made, "model_dump"):
+        made = made.model_dump(mode="json")
+    elif not isinstance(made, dict):
+        made = {k: getattr(made, k, None) for k in ("config_groups", "ignore", "kv_cache_scheme", "format")}
+    groups = {}
+    for gname, g in (made.get("config_groups") or {}).items():
+        groups[gname] = g.model_dump(mode="json") if hasattr(g, "model_dump") else dict(g)
+        if not groups[gname].get("format"):  # a group that names no format of its own is stored in the config's
+            groups[gname]["format"] = made.get("format")
+    kv = made.get("kv_cache_scheme")
+    if kv is not None and hasattr(kv, "model_dump"):
+        kv = kv.model_dump(mode="json")
+    return groups, list(made.get("ignore") or []), kv
+
+
+_SAFETENSORS_DTYPES = {"BF16": torch.bfloat16, "F16": torch.float16, "F32": torch.float32, "F64": torch.float64,
+                       "I8": torch.int8, "U8": torch.uint8, "I16": torch.int16, "I32": torch.int32,
+                       "I64": torch.int64, "BOOL": torch.bool, "F8_E4M3": torch.float8_e4m3fn,
+                       "F8_E5M2": torch.float8_e5m2}
+
+
+def _validate_converted(jobs, config: QuantizationConfig, converter) -> None:
+    """The reference's validation pass with a converter (process.py:62-87): every job's tensors as meta tensors
+    go through ``converter.validate``; what the converter would leave behind cannot be known without running it,
+    so the schemes are checked against the tensors as they are in the shard."""
+    for iwm, _ in jobs:
+        tensors: Dict[str, torch.Tensor] = {}
+        for path, wanted in iwm.items():
+            with safe_open(path, framework="pt", device="cpu") as f:
+                for key in (f.keys() if wanted is None else wanted):
+                    sl = f.get_slice(key)
+                    tensors[key] = torch.empty(tuple(sl.get_shape()), device="meta",
+                                               dtype=_SAFETENSORS_DTYPES.get(sl.get_dtype(), torch.float32))
+        if hasattr(converter, "validate"):
+            converter.validate(tensors)
+        for _, name, sch in _match_tensors_to_schemes(list(tensors), config):
+            validate_weight_for_quantization(tuple(tensors[name].shape), tensors[name].dtype, sch, name)
+
+
+def update_config(save_directory: str, config: QuantizationConfig, converter=None):
+    """Write ``quantization_config`` into ``config.json`` (reference: save_utils.py:24-121).
+
+    With a converter, the config it declares for the converted tensors is the starting point and this run's groups
+    are appended to it under names that are still free; the ignore lists are joined and the format is
+    ``mixed-precision`` as soon as two groups store their weights differently.  The reference leaves that merge to
+    ``QuantizationConfig.merge`` of compressed-tensors, which is not part of the reference tree: the rule here is
+    this package's own."""
     groups, formats = {}, set()
+    extra_ignore: List[str] = []
+    kv_converted = None
+    if converter is not None:
+        groups, extra_ignore, kv_converted = _converted_groups(converter)
+        formats.update(g["format"] for g in groups.values() if g.get("format"))
     for gname, scheme in config.config_groups.items():
         fmt = infer_format(scheme)
         formats.add(fmt)
         d = scheme.model_dump(mode="json")
         d["format"] = fmt
+        n = len(groups)
+        while gname in groups:
+            gname = f"config_group_{n}"
+            n += 1
         groups[gname] = d
     fmt = formats.pop() if len(formats) == 1 else ("mixed-precision" if formats else "dense")
     qconfig = {
@@ -295,8 +368,9 @@ def update_config(save_directory: str, config: QuantizationConfig):
         "quant_method": "compressed-tensors",
         "transform_config": {},
         "config_groups": groups,
-        "kv_cache_scheme": None if config.kv_cache_scheme is None else config.kv_cache_scheme.model_dump(mode="json"),
-        "ignore": list(config.ignore or []),
+        "kv_cache_scheme": (kv_converted if config.kv_cache_scheme is None
+                            else config.kv_cache_scheme.model_dump(mode="json")),
+        "ignore": list(dict.fromkeys(list(config.ignore or []) + extra_ignore)),
         "quantization_status": QuantizationStatus.COMPRESSED.value,
         "format": fmt,
         "global_compression_ratio": None,
@@ -325,10 +399,14 @@ def model_free_ptq(model_stub, save_directory, scheme=None, config: Optional[Qua
     :param ignore: modules to ignore; modules ending with "norm" are ignored automatically
     :param max_workers: worker threads; shards are independent jobs on the one device
     :param device: device for quantization (default cuda:0)
-    :param converter: not supported
+    :param converter: optional converter applied to every shard before quantization, e.g. one that rewrites
+        another toolkit's quantized layers into this checkpoint format.  Any object with
+        ``process(tensors) -> tensors``; ``validate(tensors)`` (called with meta tensors before anything is
+        quantized), ``create_config()`` (the quantization config of what it converted, merged into the output's)
+        and ``get_dependencies(name)`` (tensors that must be read with ``name``) are used when present
     """
-    if converter is not None:
-        raise NotImplementedError("checkpoint converters are not part of this build")
+    if converter is not None and not callable(getattr(converter, "process", None)):
+        raise TypeError("converter must have a process(tensors) method")
     model_files = _checkpoint_files(model_stub)
     config = validate_config(config, scheme, ignore)
     if isinstance(device, (list, tuple)):  # the reference spreads shards over several GPUs; one GPU here
@@ -342,11 +420,13 @@ def model_free_ptq(model_stub, save_directory, scheme=None, config: Optional[Qua
             dst.parent.mkdir(parents=True, exist_ok=True)
             shutil.copyfile(path, dst)
 
-    jobs, location = _build_jobs(model_files, save_directory, config)
+    jobs, location = _build_jobs(model_files, save_directory, config, converter)
 
     # validate first (shapes only, nothing is loaded)
+    if converter is not None:
+        _validate_converted(jobs, config, converter)
     for rel, path in model_files.items():
-        if rel.endswith(".safetensors"):
+        if converter is None and rel.endswith(".safetensors"):
             with safe_open(path, framework="pt", device="cpu") as f:
                 keys = list(f.keys())
                 for _, name, sch in _match_tensors_to_schemes(keys, config):
@@ -364,7 +444,7 @@ def model_free_ptq(model_stub, save_directory, scheme=None, config: Optional[Qua
     def run(job):
         iwm, save_path = job
         Path(save_path).parent.mkdir(parents=True, exist_ok=True)
-        return process_file(iwm, save_path, config, device)
+        return process_file(iwm, save_path, config, device, converter)
 
     if max_workers > 1:
         with ThreadPoolExecutor(max_workers=max_workers) as pool:
@@ -375,7 +455,7 @@ def model_free_ptq(model_stub, save_directory, scheme=None, config: Optional[Qua
         total_size += size
         weight_map.update(wm)
 
-    update_config(save_directory, config)
+    update_config(save_directory, config, converter)
     if len(jobs) > 1 or _INDEX_NAME in model_files:
         with open(os.path.join(save_directory, _INDEX_NAME), "w") as f:
             json.dump({"metadata": {"total_size": total_size}, "weight_map": weight_map}, f, indent=2, sort_keys=True)

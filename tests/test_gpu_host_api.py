@@ -1930,3 +1930,93 @@ def test_checkpoint_omits_zero_points_of_symmetric_activations(tmp_path):
         key = "layers.0.q_proj."
         assert key + "input_scale" in sd and key + "weight_scale" in sd and key + "weight_zero_point" not in sd
         assert (key + "input_zero_point" in sd) == (not symmetric)
+
+
+def test_model_free_ptq_with_a_converter_keeps_converted_layers_and_quantizes_the_rest(tmp_path):
+    """``model_free_ptq(converter=…)`` (reference: entrypoints/model_free/__init__.py:53,101,126,
+    process.py:111-112; the flow of examples/model_free_ptq/deepseek_r1_nvfp4_fp8_block.py): the MLP layers of the
+    checkpoint are already NVFP4 in another toolkit's naming, with a second-level scale stored in the other shard;
+    the converter renames them and inverts their global scales, the attention layers are quantized to FP8 by this
+    run, bit-identical to a run on the attention tensors alone, and config.json carries both groups."""
+    import json
+    import os
+
+    from safetensors import safe_open
+    from safetensors.torch import save_file
+    from test_host_api import _ModelOptStyleConverter
+
+    from llmcompressor_amd import model_free_ptq
+
+    g = torch.Generator().manual_seed(11)
+
+    def w(r, c):
+        return (torch.randn(r, c, generator=g) * 0.05).bfloat16()
+
+    attn = {f"model.layers.0.self_attn.{p}_proj.weight": w(64, 64) for p in "qkvo"}
+    mlp_a, mlp_b = {}, {}
+    for p, (r, c) in {"gate": (128, 64), "up": (128, 64), "down": (64, 128)}.items():
+        m = f"model.layers.0.mlp.{p}_proj."
+        mlp_a[m + "weight"] = torch.randint(0, 256, (r, c // 2), generator=g, dtype=torch.uint8)
+        mlp_a[m + "weight_scale"] = (torch.rand(r, c // 16, generator=g) * 4 + 0.5).to(torch.float8_e4m3fn)
+        mlp_b[m + "weight_scale_2"] = torch.rand(1, generator=g) * 1e-3 + 1e-4
+        mlp_b[m + "input_scale"] = torch.rand(1, generator=g) * 1e-2 + 1e-3
+    other = {"model.norm.weight": torch.ones(64, dtype=torch.bfloat16), "lm_head.weight": w(50, 64)}
+    src = str(tmp_path / "src")
+    os.makedirs(src)
+    s0, s1 = {**attn, **mlp_a}, {**mlp_b, **other}
+    save_file(s0, f"{src}/model-00001-of-00002.safetensors")
+    save_file(s1, f"{src}/model-00002-of-00002.safetensors")
+    wm = {k: "model-00001-of-00002.safetensors" for k in s0}
+    wm.update({k: "model-00002-of-00002.safetensors" for k in s1})
+    json.dump({"metadata": {}, "weight_map": wm}, open(f"{src}/model.safetensors.index.json", "w"))
+    json.dump({"model_type": "toy"}, open(f"{src}/config.json", "w"))
+
+    def read(root, wmap):
+        out = {}
+        for fn in sorted(set(wmap.values())):
+            with safe_open(f"{root}/{fn}", framework="pt") as f:
+                for k in f.keys():
+                    assert k not in out, f"{k} written twice"
+                    out[k] = f.get_tensor(k)
+        return out
+
+    from llmcompressor_amd.quantization import preset_name_to_scheme
+
+    scheme = preset_name_to_scheme("FP8_DYNAMIC", ["re:.*self_attn\\.(q|k|v|o)_proj$"])
+    conv = _ModelOptStyleConverter(["re:.*mlp\\.(gate|up|down)_proj$"])
+    dst = str(tmp_path / "dst")
+    total, wmap = model_free_ptq(src, dst, scheme=scheme, ignore=["lm_head"], device="cuda:0", converter=conv)
+    out = read(dst, wmap)
+    assert set(out) == set(wmap) and total == sum(t.numel() * t.element_size() for t in out.values())
+    assert sorted(conv.seen_meta) == sorted(k for k in mlp_a if k.endswith(".weight"))
+    for p in ("gate", "up", "down"):
+        m = f"model.layers.0.mlp.{p}_proj."
+        assert m + "weight" not in out and m + "weight_scale_2" not in out and m + "input_scale" not in out
+        assert torch.equal(out[m + "weight_packed"], mlp_a[m + "weight"])
+        assert torch.equal(out[m + "weight_scale"].view(torch.uint8), mlp_a[m + "weight_scale"].view(torch.uint8))
+        assert torch.equal(out[m + "weight_global_scale"], 1.0 / mlp_b[m + "weight_scale_2"])
+        assert torch.equal(out[m + "input_global_scale"], 1.0 / mlp_b[m + "input_scale"])
+        # read with its weight, written with its weight
+        assert wmap[m + "weight_global_scale"] == wmap[m + "weight_packed"] == "model-00001-of-00002.safetensors"
+    assert torch.equal(out["lm_head.weight"], other["lm_head.weight"])
+
+    # the attention layers are what a run without the converter makes of them
+    plain_src, plain_dst = str(tmp_path / "plain_src"), str(tmp_path / "plain_dst")
+    os.makedirs(plain_src)
+    save_file(attn, f"{plain_src}/model.safetensors")
+    json.dump({"model_type": "toy"}, open(f"{plain_src}/config.json", "w"))
+    _, plain_map = model_free_ptq(plain_src, plain_dst, scheme=scheme, device="cuda:0")
+    plain = read(plain_dst, plain_map)
+    for k, v in plain.items():
+        assert out[k].dtype == v.dtype and torch.equal(out[k].view(torch.uint8), v.view(torch.uint8)), k
+    assert out["model.layers.0.self_attn.q_proj.weight"].dtype == torch.float8_e4m3fn
+
+    q = json.load(open(f"{dst}/config.json"))["quantization_config"]
+    # a scheme object is filed as config_group_0, which the converter's group already is: it moves on by one
+    assert list(q["config_groups"]) == ["config_group_0", "config_group_1"]
+    assert q["config_groups"]["config_group_0"]["format"] == "nvfp4-pack-quantized"
+    assert q["config_groups"]["config_group_1"]["format"] == "float-quantized"
+    assert q["config_groups"]["config_group_1"]["targets"] == ["re:.*self_attn\\.(q|k|v|o)_proj$"]
+    assert q["format"] == "mixed-precision" and q["ignore"] == ["lm_head"]
+    index = json.load(open(f"{dst}/model.safetensors.index.json"))
+    assert index["weight_map"] == wmap

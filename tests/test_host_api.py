@@ -885,3 +885,115 @@ def test_sequential_targets_that_are_not_a_layer_list_fall_back_to_the_layers(ca
     assert got == list(model.layers)
     assert "not the elements of one layer list" in caplog.text
     assert find_decoder_layers(model, ["NoSuchClass"]) == list(model.layers)
+
+
+class _ModelOptStyleConverter:
+    """A user-side converter of the kind the reference's ``converter=`` argument takes: NVFP4 layers stored the
+    ModelOpt way (``weight`` packed, ``weight_scale_2`` and ``input_scale`` as divisors) are renamed to the
+    compressed-tensors names with the global scales inverted (the mapping table of the reference's
+    docs/guides/entrypoints/convert.md)."""
+
+    def __init__(self, targets):
+        import re
+
+        self.patterns = [re.compile(t[3:]) for t in targets]
+        self.seen_meta = []
+
+    def _hit(self, name):
+        module = name.rsplit(".", 1)[0]
+        return any(p.match(module) for p in self.patterns)
+
+    def get_dependencies(self, name):
+        if name.endswith(".weight") and self._hit(name):
+            m = name[: -len("weight")]
+            return [m + "weight_scale", m + "weight_scale_2", m + "input_scale"]
+        return []
+
+    def validate(self, tensors):
+        for name, t in tensors.items():
+            assert t.device.type == "meta"
+            if name.endswith(".weight") and self._hit(name):
+                self.seen_meta.append(name)
+                if t.dtype != torch.uint8:
+                    raise ValueError(f"{name} is not packed fp4")
+                if name[: -len("weight")] + "weight_scale_2" not in tensors:
+                    raise ValueError(f"{name} has no second-level scale beside it")
+
+    def process(self, tensors):
+        out = {}
+        for name, t in tensors.items():
+            module, leaf = name.rsplit(".", 1)
+            if not self._hit(name):
+                out[name] = t
+            elif leaf == "weight":
+                out[module + ".weight_packed"] = t
+            elif leaf == "weight_scale_2":
+                out[module + ".weight_global_scale"] = 1.0 / t
+            elif leaf == "input_scale":
+                out[module + ".input_global_scale"] = 1.0 / t
+            else:
+                out[name] = t
+        return out
+
+    def create_config(self):
+        from llmcompressor_amd.quantization import QuantizationConfig, preset_name_to_scheme
+
+        sch = preset_name_to_scheme("NVFP4", ["re:" + p.pattern for p in self.patterns])
+        return QuantizationConfig(config_groups={"config_group_0": sch}, format="nvfp4-pack-quantized",
+                                  ignore=["lm_head"])
+
+
+def test_model_free_converter_config_merge_and_dependencies(tmp_path):
+    """``converter=`` host logic (reference: entrypoints/model_free/__init__.py:101,126, save_utils.py:64-126):
+    the converter's config is the starting point and this run's groups are appended to it; tensors a converter
+    needs together are planned into one job; validation hands the converter meta tensors."""
+    import json
+
+    from safetensors.torch import save_file
+
+    from llmcompressor_amd.entrypoints.model_free import (_build_jobs, _validate_converted, update_config,
+                                                          validate_config)
+
+    conv = _ModelOptStyleConverter(["re:.*mlp\\.(gate|up|down)_proj$"])
+    cfg = validate_config(None, "FP8_DYNAMIC", ["lm_head"])
+    (tmp_path / "config.json").write_text(json.dumps({"model_type": "toy"}))
+    q = update_config(str(tmp_path), cfg, conv)
+    assert list(q["config_groups"]) == ["config_group_0", "FP8_DYNAMIC"]
+    assert q["config_groups"]["config_group_0"]["weights"]["group_size"] == 16
+    assert q["config_groups"]["FP8_DYNAMIC"]["format"] == "float-quantized"
+    assert q["format"] == "mixed-precision" and q["ignore"] == ["lm_head"]
+    assert json.loads((tmp_path / "config.json").read_text())["quantization_config"] == q
+    # a group name that is taken is not overwritten
+    cfg0 = validate_config(None, "FP8_DYNAMIC", [])
+    cfg0.config_groups = {"config_group_0": cfg0.config_groups["FP8_DYNAMIC"]}
+    q0 = update_config(str(tmp_path), cfg0, conv)
+    assert list(q0["config_groups"]) == ["config_group_0", "config_group_1"]
+    assert q0["config_groups"]["config_group_1"]["weights"]["num_bits"] == 8
+    # without a converter nothing is merged
+    assert list(update_config(str(tmp_path), cfg)["config_groups"]) == ["FP8_DYNAMIC"]
+
+    # the second-level scale of down_proj lives in the other shard: it is planned into the job of its weight
+    src = tmp_path / "src"
+    src.mkdir()
+    a = {"m.mlp.down_proj.weight": torch.zeros(8, 16, dtype=torch.uint8),
+         "m.mlp.down_proj.weight_scale": torch.ones(8, 2).to(torch.float8_e4m3fn),
+         "m.self_attn.o_proj.weight": torch.zeros(8, 8, dtype=torch.bfloat16)}
+    b = {"m.mlp.down_proj.weight_scale_2": torch.ones(1), "m.mlp.down_proj.input_scale": torch.ones(1)}
+    save_file(a, str(src / "a.safetensors"))
+    save_file(b, str(src / "b.safetensors"))
+    files = {"a.safetensors": str(src / "a.safetensors"), "b.safetensors": str(src / "b.safetensors")}
+    jobs, _ = _build_jobs(files, str(tmp_path / "dst"), cfg, conv)
+    by_out = {os.path.basename(p): iwm for iwm, p in jobs}
+    assert sorted(by_out["a.safetensors"][files["b.safetensors"]]) == ["m.mlp.down_proj.input_scale",
+                                                                     "m.mlp.down_proj.weight_scale_2"]
+    assert by_out["b.safetensors"][files["b.safetensors"]] == []
+    _validate_converted(jobs, cfg, conv)
+    assert conv.seen_meta == ["m.mlp.down_proj.weight"]
+    # a converter that refuses a shard stops the run before anything is quantized
+    jobs_split, _ = _build_jobs(files, str(tmp_path / "dst"), cfg, None)
+    with pytest.raises(ValueError, match="no second-level scale"):
+        _validate_converted(jobs_split, cfg, conv)
+    from llmcompressor_amd import model_free_ptq
+
+    with pytest.raises(TypeError, match="process"):
+        model_free_ptq(str(src), str(tmp_path / "dst"), scheme="FP8_DYNAMIC", converter=object())
