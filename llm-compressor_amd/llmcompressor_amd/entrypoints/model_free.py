@@ -296,7 +296,8 @@ def _converted_groups(converter) -> Tuple[Dict[str, dict], List[str], Optional[d
     """Config groups, ignore list and kv-cache scheme that ``converter.create_config()`` declares for the tensors it
     rewrote (reference: save_utils.py:79-80); the result may be a config object of this package, any object with
     the same attributes, a plain dict, or None."""
-    made = converter.create_config() if hasattr(converter, "create_config") else None
+    made = converter if isinstance(converter, dict) else (
+        converter.create_config() if hasattr(converter, "create_config") else None)
     if made is None:
         return {}, [], None
     if hasattr(made, "model_dump"):
@@ -341,16 +342,30 @@ def _validate_converted(jobs, config: QuantizationConfig, converter) -> None:
 def update_config(save_directory: str, config: QuantizationConfig, converter=None):
     """Write ``quantization_config`` into ``config.json`` (reference: save_utils.py:24-121).
 
-    With a converter, the config it declares for the converted tensors is the starting point and this run's groups
-    are appended to it under names that are still free; the ignore lists are joined and the format is
-    ``mixed-precision`` as soon as two groups store their weights differently.  The reference leaves that merge to
+    With a converter, the config it declares for the converted tensors is the starting point; without one, a
+    compressed-tensors ``quantization_config`` that the checkpoint's ``config.json`` already holds is (a checkpoint
+    of which some layers were quantized before).  This run's groups are appended to the starting point under names
+    that are still free; the ignore lists are joined and the format is ``mixed-precision`` as soon as two groups
+    store their weights differently.  The reference leaves that merge to
     ``QuantizationConfig.merge`` of compressed-tensors, which is not part of the reference tree: the rule here is
     this package's own."""
     groups, formats = {}, set()
     extra_ignore: List[str] = []
     kv_converted = None
+    path = os.path.join(save_directory, "config.json")
+    before = None
     if converter is not None:
-        groups, extra_ignore, kv_converted = _converted_groups(converter)
+        before = converter
+    elif os.path.exists(path):
+        with open(path) as f:
+            before = json.load(f).get("quantization_config")
+        if before is not None and not (isinstance(before, dict) and isinstance(before.get("config_groups"), dict)
+                                       and before.get("quant_method", "compressed-tensors") == "compressed-tensors"):
+            logger.warning("Unable to parse the original checkpoint's quantization_config. "
+                           "The quantization_config will be created from scratch")
+            before = None
+    if before is not None:
+        groups, extra_ignore, kv_converted = _converted_groups(before)
         formats.update(g["format"] for g in groups.values() if g.get("format"))
     for gname, scheme in config.config_groups.items():
         fmt = infer_format(scheme)
@@ -375,7 +390,6 @@ def update_config(save_directory: str, config: QuantizationConfig, converter=Non
         "format": fmt,
         "global_compression_ratio": None,
     }
-    path = os.path.join(save_directory, "config.json")
     if os.path.exists(path):
         with open(path) as f:
             data = json.load(f)

@@ -969,7 +969,14 @@ def test_model_free_converter_config_merge_and_dependencies(tmp_path):
     q0 = update_config(str(tmp_path), cfg0, conv)
     assert list(q0["config_groups"]) == ["config_group_0", "config_group_1"]
     assert q0["config_groups"]["config_group_1"]["weights"]["num_bits"] == 8
-    # without a converter nothing is merged
+    # without a converter the checkpoint's own compressed-tensors config is the starting point (what the last call
+    # left in config.json: the converter's group and the FP8 one), and a config of another method is dropped
+    q1 = update_config(str(tmp_path), validate_config(None, "W8A16", []))
+    assert list(q1["config_groups"]) == ["config_group_0", "config_group_1", "W8A16"] and q1["ignore"] == ["lm_head"]
+    assert q1["format"] == "mixed-precision"
+    (tmp_path / "config.json").write_text(json.dumps({"quantization_config": {"quant_method": "fp8"}}))
+    assert list(update_config(str(tmp_path), cfg)["config_groups"]) == ["FP8_DYNAMIC"]
+    (tmp_path / "config.json").write_text(json.dumps({"model_type": "toy"}))
     assert list(update_config(str(tmp_path), cfg)["config_groups"]) == ["FP8_DYNAMIC"]
 
     # the second-level scale of down_proj lives in the other shard: it is planned into the job of its weight
