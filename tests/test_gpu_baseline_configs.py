@@ -13,6 +13,8 @@ q/k/v/o/gate/up/down weights bf16 ~ N(0, 0.02), Linear i drawn from seed i.
   [0.2, 1.0], norm 2.4: (min, max) of every group equal (a group may differ only on a documented rounding tie).
 * MoE layer of the Qwen3-30B-A3B shape (128 experts, 768 x 2048 and 2048 x 768): grouped GPTQ, W4A16 g128 and NVFP4,
   sampled experts against the oracle's quantize_weight at >= 99.9 % identical weights.
+* Sequential GPTQ through ``oneshot`` on two such decoder layers of a transformers Llama: every Linear on its int4
+  grid, and closer to the dense model on held-out tokens than round-to-nearest.
 """
 import math
 
@@ -425,8 +427,8 @@ def _check_experts(scheme, R, K, which, Ws, xs, Hs, outs, loss, scales, gss, cou
 
 
 def test_sequential_gptq_through_oneshot_at_the_llama3_8b_layer_shapes():
-    """BASELINE's sequential configuration on the real layer (hidden 4096, intermediate 14336, 32 query and 8
-    key / value heads) of a transformers Llama, two layers deep, 8 batches of 2048 tokens, W4A16 g128 with static
+    """The benchmark's sequential GPTQ configuration on the real layer (hidden 4096, intermediate 14336, 32 query
+    and 8 key / value heads) of a transformers Llama, two layers deep, 8 batches of 2048 tokens, W4A16 g128 with static
     activation ordering, through ``oneshot`` with the modifier's defaults (staged Hessian launches, shared inputs,
     lock-step chain for the six 4096-wide Linears, factor in groups for down_proj): every decoder Linear ends on
     its groups' int4 grid, and on held-out tokens the logits are closer to the dense model's than with
