@@ -483,6 +483,40 @@ def test_factor_form_choice():
     assert ops.gptq_factor_form(14336, 64) == ops.FACTOR_INVERSE   # narrower column blocks
 
 
+def test_factor_form_is_checked_by_every_entry_point():
+    """A form the width or the column blocks do not allow, or a number that names no form, is refused by the
+    library before anything is launched (the weight and the Hessian stay as they were)."""
+    from llmcompressor_amd import ops
+
+    K = 192  # not a multiple of 128
+    H = _hessian(K, 3 * K, 3)[0].cuda()
+    keep = H.clone()
+    with pytest.raises(ValueError, match="llmc_gptq_hinv: argument 7"):
+        ops.gptq_hinv_(H, form=ops.FACTOR_GROUPS)
+    with pytest.raises(ValueError, match="llmc_gptq_hinv: argument 7"):
+        ops.gptq_hinv_(H, form=5)
+    with pytest.raises(ValueError, match="llmc_gptq_hinv_grouped: argument 8"):
+        ops.gptq_hinv_grouped([H, H.clone()], form=ops.FACTOR_GROUPS)
+    assert torch.equal(H, keep)
+    K = 256
+    H = _hessian(K, 3 * K, 4)[0].cuda()
+    U, dead, _ = ops.gptq_hinv_(H.clone(), form=ops.FACTOR_GROUPS)
+    W = (torch.randn(8, K, device="cuda") * 0.05).bfloat16()
+    Wkeep = W.clone()
+    scale = torch.full((8, K // 128), 0.01, device="cuda", dtype=torch.bfloat16)
+    g_idx = (torch.arange(K, dtype=torch.int32) // 128).cuda()
+    args = (W, U, scale, None, ops.FMT_INT, 4, 1, K // 128, g_idx)
+    with pytest.raises(ValueError, match="llmc_gptq_quantize: argument 20"):
+        ops.gptq_quantize(*args, dead=dead, blocksize=64, form=ops.FACTOR_GROUPS)  # blocks narrower than 128
+    with pytest.raises(ValueError, match="llmc_gptq_quantize: argument 20"):
+        ops.gptq_quantize(*args, dead=dead, form=3)
+    with pytest.raises(ValueError, match="llmc_sparsegpt_sparsify: argument 13"):
+        ops.sparsegpt_sparsify(W, U, 0.5, dead=dead, blocksize=64, form=ops.FACTOR_GROUPS)  # exactly 128 there
+    assert torch.equal(W, Wkeep)
+    out, _ = ops.gptq_quantize(*args, dead=dead, form=ops.FACTOR_GROUPS)
+    assert out.shape == W.shape and torch.isfinite(out.float()).all()
+
+
 def _groups(K):
     """Column ranges of the diagonal blocks: 512 wide, aligned to the last column, the first one what is left."""
     first = K % 512 or 512
