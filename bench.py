@@ -558,6 +558,10 @@ def main():
     ap.add_argument("--vocab", type=int, default=32000, help="--probe-oneshot: vocabulary size (config: 128256)")
     ap.add_argument("--probe-chain", action="store_true",
                     help="time the Cholesky chain, the column loop and their fp32 products alone, print tables")
+    ap.add_argument("--probe-product", type=int, default=0, metavar="N",
+                    help="counter runs: launch only the split fp32 product C -= A B of 8192^3 N times through "
+                    "llmc_sgemm (with --probe-trans-b: C -= A B^T)")
+    ap.add_argument("--probe-trans-b", action="store_true", help="--probe-product: B is stored transposed")
     ap.add_argument("--probe-moe", action="store_true",
                     help="print the timings of one 128-expert MoE layer through GPTQModifier instead of the bench line")
     a = ap.parse_args()
@@ -585,6 +589,15 @@ def main():
         return
     if a.probe_moe:
         probe_moe(a.moe_mode)
+        return
+    if a.probe_product:
+        n = 8192
+        A, Bm = torch.randn(n, n, device=dev), torch.randn(n, n, device=dev)
+        C = torch.zeros(n, n, device=dev)
+        for _ in range(a.probe_product):
+            ops.sgemm_(C, A, Bm, -1.0, 1.0, a.probe_trans_b, 0)
+        torch.cuda.synchronize()
+        print(f"probe: {a.probe_product} x llmc_sgemm {n}^3, B {'transposed' if a.probe_trans_b else 'as stored'}")
         return
     if a.probe_oneshot:
         probe_oneshot(a.batches, a.tokens, a.layers, a.vocab)
