@@ -354,6 +354,58 @@ def probe_chain():
         del A, B, C
 
 
+def probe_vendor_gemm(tokens=65536):
+    """The dominant launch beside the vendor library's bf16 GEMM (through ``torch.matmul``) on the same operands:
+    the full product X^T X in the hook's layout (tokens strided), the same with all-zero data (matrix instructions
+    on constant operands draw less power, so the chip clocks higher), and a product of the same size whose operands
+    are stored with the contraction index contiguous.  Event-timed, mean of 6 launches after 2."""
+    import torch
+
+    from llmcompressor_amd import ops
+
+    def timed(fn, n=6):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n
+
+    T, K = tokens, INTER
+    x = torch.randn(T, K, device="cuda").bfloat16()
+    out = torch.empty(K, K, device="cuda", dtype=torch.bfloat16)
+    H = torch.zeros(K, K, device="cuda")
+    full = 2.0 * T * K * K
+    tiles = (K // 256) * (K // 256 + 1) // 2
+    executed = 2.0 * T * tiles * 256 * 256
+    rows = []
+    for data in ("random", "zero"):
+        if data == "zero":
+            x.zero_()
+        ms = timed(lambda: ops.hessian_accumulate_(H, x))
+        rows.append((f"hessian_syrk_kernel, X [{T} x {K}] {data} data (upper-triangular tiles only)", ms, executed))
+        ms = timed(lambda: torch.matmul(x.t(), x, out=out))
+        rows.append((f"vendor GEMM X^T X on the same tensor, {data} data (all of the product)", ms, full))
+    del x, out, H
+    K2 = 8192
+    xt = torch.randn(K2, T, device="cuda").bfloat16()
+    out = torch.empty(K2, K2, device="cuda", dtype=torch.bfloat16)
+    ms = timed(lambda: torch.matmul(xt, xt.t(), out=out))
+    rows.append((f"vendor GEMM A A^T, A [{K2} x {T}] random data (contraction index contiguous in both operands)",
+                 ms, 2.0 * T * K2 * K2))
+    x2 = xt.t().contiguous()
+    ms = timed(lambda: torch.matmul(x2.t(), x2, out=out))
+    rows.append((f"vendor GEMM X^T X, X [{T} x {K2}] random data (the hook's layout)", ms, 2.0 * T * K2 * K2))
+    print("| launch | ms | executed bf16 matrix TFLOP/s |")
+    print("|---|---|---|")
+    for name, ms, flop in rows:
+        print(f"| {name} | {ms:.2f} | {flop / ms / 1e9:.0f} |")
+
+
 def probe_moe(mode="both"):
     """One MoE expert layer (128 experts, hidden 2048, intermediate 768, top-8 routing of 4096 tokens: 384 expert
     Linears) through GPTQModifier W4A16 and NVFP4A16: time of the calibration forward (grouped Hessian launches from
@@ -558,6 +610,8 @@ def main():
     ap.add_argument("--vocab", type=int, default=32000, help="--probe-oneshot: vocabulary size (config: 128256)")
     ap.add_argument("--probe-chain", action="store_true",
                     help="time the Cholesky chain, the column loop and their fp32 products alone, print tables")
+    ap.add_argument("--probe-vendor-gemm", action="store_true",
+                    help="time the dominant launch beside the vendor library's bf16 GEMM on the same operands")
     ap.add_argument("--probe-product", type=int, default=0, metavar="N",
                     help="counter runs: launch only the split fp32 product C -= A B of 8192^3 N times through "
                     "llmc_sgemm (with --probe-trans-b: C -= A B^T)")
@@ -589,6 +643,9 @@ def main():
         return
     if a.probe_moe:
         probe_moe(a.moe_mode)
+        return
+    if a.probe_vendor_gemm:
+        probe_vendor_gemm(a.stage_tokens or 65536)
         return
     if a.probe_product:
         n = 8192
