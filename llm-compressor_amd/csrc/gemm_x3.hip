@@ -12,8 +12,10 @@
 // planes in the same step and stores them to one of three LDS stages k-contiguous (a row of a plane is 16 bf16
 // = 32 bytes = two 16-byte chunks, the chunk index XOR-ed with bit 2 of the row so that eight consecutive
 // rows of one chunk fall into distinct banks), so that an MFMA operand (8 consecutive k of one row) is one
-// ds_read_b128.  Operand B stored [Kc, N] (not transposed) is transposed on the way: a thread loads two
-// consecutive k rows of 4 columns and writes, per column, its k pair.  The split/store work for a later step
+// ds_read_b128.  Operand B stored [Kc, N] (not transposed) is transposed on the way: a thread loads eight
+// consecutive k rows of one column (a wave: two runs of 32 consecutive columns, one per half of the k-step) and
+// writes that column's half row of every plane, so that a wave's stores cover whole rows of LDS one after the
+// other.  The split/store work for a later step
 // sits between the matrix instructions of the current one, one barrier per k-step.  Sustained rate on
 // MI355X: about 200 TFLOP/s of fp32-equivalent work (1.2 PFLOP/s of bf16 matrix instructions, the rate
 // the chip also sustains in the Hessian kernel) against about 130 TFLOP/s of the fp32 matrix instruction.
@@ -56,8 +58,8 @@ struct X3 {
   static constexpr int PLANE_A = BM * 32, PLANE_B = BN * 32;  // bytes of one plane in one stage
   static constexpr int STAGE = 3 * (PLANE_A + PLANE_B);       // A planes 0..2, then B planes 0..2
   static constexpr int NLD_A = BM * 4 / NTHREADS, NLD_B = BN * 4 / NTHREADS;
-  static constexpr int KP = XK * (BN / 4) / NTHREADS;  // non-transposed B: consecutive k rows held by one thread
-  static_assert(NLD_A == 2 && NLD_B == 2 && KP == 2, "thread mapping below assumes two float4 per operand and thread");
+  static_assert(NLD_A == 2 && NLD_B == 2 && NTHREADS == 2 * BN,
+                "thread mapping below assumes two float4 per operand and thread, and two threads per column of B");
   static constexpr int CHUNKS = NLD_A + NLD_B;  // split/store chunks per k-step (A then B)
 
   struct Slab {
@@ -79,8 +81,9 @@ struct X3 {
       const int f = tid + i * NTHREADS;
       s.b[i] = *(const float4*)(B + (int64_t)(n0 + (f >> 2)) * g.ldb + k + ((f & 3) << 2));
     } else {
-      const int kg = tid / (BN / 4), nq = tid % (BN / 4);
-      s.b[i] = *(const float4*)(B + (int64_t)(k + kg * KP + i) * g.ldb + n0 + (nq << 2));
+      // non-transposed B: thread t holds column t / 2, k rows 8 (t % 2) .. + 7; load i fetches four of them
+      const float* src = B + (int64_t)(k + (tid & 1) * 8 + i * 4) * g.ldb + n0 + (tid >> 1);
+      s.b[i] = make_float4(src[0], src[g.ldb], src[2 * g.ldb], src[3 * g.ldb]);
     }
   }
   static __device__ __forceinline__ void load(const GemmF32& g, const float* A, const float* B, int m0, int n0, int k,
@@ -108,23 +111,16 @@ struct X3 {
 #pragma unroll
       for (int q = 0; q < 3; ++q) *(uint2*)(base + q * plane) = make_uint2(p[q][0], p[q][1]);
     } else {
-      // non-transposed B: this thread holds the rows k = 2 kg and 2 kg + 1 of the columns 4 nq .. 4 nq + 3;
-      // chunk i covers the columns 2 i and 2 i + 1 (two consecutive k of one column = one 4-byte store per plane)
-      const int kg = tid / (BN / 4), nq = tid % (BN / 4);
-      const int k = kg * KP;
+      // non-transposed B: load i holds the k rows 8 (t % 2) + 4 i .. + 3 of column t / 2, i.e. 8 bytes of that
+      // column's row in every plane; the two threads of a column and their neighbours write consecutive bytes
+      const float4 v = s.b[i];
+      const int row = tid >> 1, half = tid & 1;
+      uint32_t p[3][2];
+      split3(v.x, v.y, p[0][0], p[1][0], p[2][0]);
+      split3(v.z, v.w, p[0][1], p[1][1], p[2][1]);
+      unsigned char* base = stage + 3 * PLANE_A + plane_off(row, half) + (i << 3);
 #pragma unroll
-      for (int cc = 0; cc < 2; ++cc) {
-        const int col = i * 2 + cc;
-        const float e0 = col == 0 ? s.b[0].x : col == 1 ? s.b[0].y : col == 2 ? s.b[0].z : s.b[0].w;
-        const float e1 = col == 0 ? s.b[1].x : col == 1 ? s.b[1].y : col == 2 ? s.b[1].z : s.b[1].w;
-        const int row = (nq << 2) + col;
-        unsigned char* base = stage + 3 * PLANE_A + plane_off(row, k >> 3) + ((k & 7) << 1);
-        uint32_t p0, p1, p2;
-        split3(e0, e1, p0, p1, p2);
-        *(uint32_t*)(base) = p0;
-        *(uint32_t*)(base + PLANE_B) = p1;
-        *(uint32_t*)(base + 2 * PLANE_B) = p2;
-      }
+      for (int q = 0; q < 3; ++q) *(uint2*)(base + q * PLANE_B) = make_uint2(p[q][0], p[q][1]);
     }
   }
 };
@@ -204,12 +200,7 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) __attribute__((amdgpu_waves
     auto chunk = [&](auto tag) {
       constexpr int c = decltype(tag)::value;
       C::template split_store<c>(slab, nxt);
-      if (c < C::NLD_A || TRANS_B) {
-        C::template load_chunk<c>(g, A, B, m0, n0, kf, slab);
-      } else if (c == C::CHUNKS - 1) {  // a column of the non-transposed B needs both B registers: refill at the end
-        C::template load_chunk<C::NLD_A>(g, A, B, m0, n0, kf, slab);
-        C::template load_chunk<C::NLD_A + 1>(g, A, B, m0, n0, kf, slab);
-      }
+      C::template load_chunk<c>(g, A, B, m0, n0, kf, slab);
     };
     // four chunks of split/store work per step: one after each column of the wide wave tile, two after each
     // column of the narrow one
