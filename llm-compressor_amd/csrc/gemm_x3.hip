@@ -10,9 +10,10 @@
 // 64 x 64).  A k-step is 16 deep.  Per k-step the workgroup fetches the fp32 slabs of both operands
 // (tile edge x 16 each) into registers two steps ahead of their use, splits them into the three
 // planes in the same step and stores them to one of three LDS stages k-contiguous (a row of a plane is 16 bf16
-// = 32 bytes = two 16-byte chunks, the chunk index XOR-ed with bit 2 of the row so that eight consecutive
-// rows of one chunk fall into distinct banks), so that an MFMA operand (8 consecutive k of one row) is one
-// ds_read_b128.  Operand B stored [Kc, N] (not transposed) is transposed on the way: a thread loads eight
+// = 32 bytes = two 16-byte chunks, the chunk index XOR-ed with bit 3 of the row: a 16-byte read is served
+// sixteen lanes at a time over 64 banks, and the sixteen consecutive rows of one chunk that those lanes ask for
+// then fall into distinct banks -- no conflicts counted), so that an MFMA operand (8 consecutive k of one row) is
+// one ds_read_b128.  Operand B stored [Kc, N] (not transposed) is transposed on the way: a thread loads eight
 // consecutive k rows of one column (a wave: two runs of 32 consecutive columns, one per half of the k-step) and
 // writes that column's half row of every plane, so that a wave's stores cover whole rows of LDS one after the
 // other.  The split/store work for a later step
@@ -29,7 +30,7 @@ namespace {
 
 constexpr int XK = 16;
 
-__device__ __forceinline__ int plane_off(int row, int chunk) { return row * 32 + ((chunk ^ ((row >> 2) & 1)) << 4); }
+__device__ __forceinline__ int plane_off(int row, int chunk) { return row * 32 + ((chunk ^ ((row >> 3) & 1)) << 4); }
 
 // (x, y) -> the packed bf16 pairs of the three planes
 __device__ __forceinline__ void split3(float x, float y, uint32_t& p0, uint32_t& p1, uint32_t& p2) {
