@@ -463,12 +463,16 @@ def probe_moe(mode="both"):
     print("|---|---|---|---|")
     from llmcompressor_amd.modeling.moe import moe_calibration_context
 
-    variants = (("W4A16, lock-step groups (default)", 8, "lockstep", "W4A16", False),
-                ("W4A16, one module at a time, 4 streams", 0, "permodule", "W4A16", False),
-                ("NVFP4A16, lock-step groups (default)", 8, "lockstep", "NVFP4A16", False),
+    variants = (("W4A16, lock-step groups (default)", 8, "lockstep", "W4A16", False, False),
+                ("W4A16, one module at a time, 4 streams", 0, "permodule", "W4A16", False, False),
+                ("NVFP4A16, lock-step groups (default)", 8, "lockstep", "NVFP4A16", False, False),
                 ("W4A16, lock-step groups, every expert calibrated on all tokens (`moe_calibrate_all_experts`, the "
-                 "`oneshot` default)", 8, "lockstep", "W4A16", True))
-    for label, gmin, key, scheme, all_experts in variants:
+                 "`oneshot` default)", 8, "lockstep", "W4A16", True, False),
+                ("W4A16, lock-step groups, grouped launches in the observed pass too (`moe_grouped_calibration`)",
+                 8, "lockstep", "W4A16", False, True),
+                ("W4A16, lock-step groups, every expert on all tokens, grouped launches in the observed pass too",
+                 8, "lockstep", "W4A16", True, True))
+    for label, gmin, key, scheme, all_experts, grouped_cal in variants:
         if mode not in ("both", key):
             continue
         best = None
@@ -481,7 +485,7 @@ def probe_moe(mode="both"):
             s.reset()
             s.initialize(model=model, recipe=mod)
             LifecycleCallbacks.calibration_start()
-            with torch.no_grad(), moe_calibration_context(all_experts):
+            with torch.no_grad(), moe_calibration_context(all_experts, grouped=grouped_cal):
                 model.layers[0](x, idx, w.to(x.dtype))  # first batch: the Hessians are allocated here
                 torch.cuda.synchronize()
                 t0 = time.perf_counter()

@@ -382,10 +382,12 @@ int llmc_sparsegpt_sparsify(const void* weight, int32_t w_dtype, int64_t R, int6
  *   y[r, s*N + n] = sum_k x[r, k] * W_{s,e(r)}[n, k]   for every routed row r, bf16 in, fp32 accumulation,
  * one rounding to bf16.  x [rows, K] (row stride ldx) holds the routed rows expert after expert; `tiles`
  * (device, int32 [ntiles][4], 16-byte aligned) lists runs of at most 128 rows of one expert as
- * {expert, first row, rows, 0}; w (device array of splits * experts pointers, 16-byte aligned each) holds the
+ * {expert, first row, rows, shift}: the results of the tile's rows go to the rows first row + shift .. of y
+ * (0: y has x's row numbering; another value lets several experts read the same rows of x and write apart, the
+ * reference's calibrate_all_experts case, where every expert is called on every token); w (device array of splits * experts pointers, 16-byte aligned each) holds the
  * [N, K] weights (row stride ldw) of split s and expert e at w[s * experts + e]; splits that share their input
  * (gate and up) write side by side into y (row stride ldy >= splits * N).  N % 128 == 0, K % 64 == 0,
- * dtype LLMC_BF16.  Rows no tile names are not written.  The sum over k runs in a different order than a
+ * dtype LLMC_BF16.  Rows no tile names are not written; the caller sizes y for the largest row a tile names.  The sum over k runs in a different order than a
  * library GEMM's, so results agree with F.linear to the last bf16 digit, not bit for bit: use it where hooks do
  * not need the exact inputs of the reference's forward (the propagation pass of a sequential pipeline). */
 int llmc_grouped_linear(const void* x, int32_t dtype, int64_t ldx, const void* const* w, int64_t ldw,

@@ -4,6 +4,8 @@
 // small table names, per tile of up to 128 rows, its expert, first row and row count, so ragged token counts
 // (also zero) cost no empty workgroups.  `splits` projections that read the same rows (gate and up) share a
 // launch: split s takes its weights from w[s * E + e] and writes the columns s * N .. s * N + N - 1 of y.
+// A tile's results go to the rows of y that its fourth table entry names (its input rows' numbers plus that
+// offset), so several experts can read the same rows of x and write apart: every expert on every token.
 //
 // One workgroup of four waves owns a 128 x 128 tile of y (64 x 64 per wave, 2 x 2 accumulator tiles of
 // v_mfma_f32_32x32x16_bf16, fp32 accumulation, one rounding to bf16 at the end as F.linear does).  A k-step is
@@ -29,7 +31,7 @@ struct GroupedLinear {
   int64_t ldw;
   uint16_t* y;
   int64_t ldy;
-  const int32_t* tiles;  // [ntiles][4]: expert, first row, rows (1..128), unused
+  const int32_t* tiles;  // [ntiles][4]: expert, first row, rows (1..128), output row of the first row minus first row
   int ntiles, experts, N, K, ncol;
 };
 
@@ -139,7 +141,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #undef GL_PUT
 
   // element v of an accumulator tile: row (v / 4) * 8 + (lane / 32) * 4 + v % 4, column lane % 32
-  uint16_t* Y = g.y + (int64_t)row0 * g.ldy + col;
+  uint16_t* Y = g.y + ((int64_t)row0 + tile.w) * g.ldy + col;
 #pragma unroll
   for (int a = 0; a < 2; ++a)
 #pragma unroll

@@ -25,6 +25,7 @@ class DatasetArguments:
     pad_to_max_length: bool = True
     dataloader_num_workers: int = 0
     moe_calibrate_all_experts: bool = True
+    moe_grouped_calibration: bool = False  # this build's own: grouped expert launches in observed passes too
     pipeline: Optional[str] = "independent"
     sequential_targets: Optional[List[str]] = None
     sequential_offload_device: Optional[str] = None  # None: activations stay in HBM (the reference defaults to "cpu")

@@ -29,7 +29,7 @@ class _DatasetArgs:
 class Oneshot:
     def __init__(self, model, recipe=None, dataset=None, output_dir: Optional[str] = None, pipeline: str = "independent",
                  sequential_targets=None, stage: Optional[str] = None, save_compressed: bool = True,
-                 moe_calibrate_all_experts: bool = True, **kwargs):
+                 moe_calibrate_all_experts: bool = True, moe_grouped_calibration: bool = False, **kwargs):
         if isinstance(model, str):
             raise ValueError("oneshot: pass an instantiated torch.nn.Module; loading by name is not available offline")
         self.model = model
@@ -41,7 +41,8 @@ class Oneshot:
         self.save_compressed = save_compressed
         self.processor = kwargs.pop("processor", None) or kwargs.pop("tokenizer", None)
         self.dataset_args = _DatasetArgs(sequential_targets=sequential_targets, pipeline=pipeline,
-                                         moe_calibrate_all_experts=moe_calibrate_all_experts, **kwargs)
+                                         moe_calibrate_all_experts=moe_calibrate_all_experts,
+                                         moe_grouped_calibration=moe_grouped_calibration, **kwargs)
 
     def __call__(self):
         from ..modeling.moe import get_non_linearized_moes, linearize_moe
@@ -82,17 +83,25 @@ class Oneshot:
         return self.model
 
     def apply_recipe_modifiers(self, calibration_dataloader):
+        from ..modeling.moe import moe_calibration_context
+
         session = active_session()
         session.reset()
-        session.initialize(model=self.model, recipe=self.recipe, recipe_stage=self.stage,
-                           calib_data=calibration_dataloader)
-        mods = session.get_modifiers()
-        user = self.pipeline
-        pipeline = CalibrationPipeline.from_modifiers(mods, user=user)
-        if calibration_dataloader is None and any(m.requires_calibration_data for m in mods):
-            raise ValueError("the recipe requires calibration data but no `dataset` was given")
-        pipeline(self.model, calibration_dataloader, self.dataset_args)
-        session.finalize()
+        # reference: entrypoints/oneshot.py:247-250 -- the whole calibration runs inside the MoE context when
+        # ``moe_calibrate_all_experts`` is set: every expert is then called on every token while hooks observe it.
+        # ``moe_grouped_calibration`` (this build's own switch, off by default) lets an experts block whose live
+        # hooks only read their inputs take its grouped launches in the observed pass as well.
+        with moe_calibration_context(bool(self.dataset_args.moe_calibrate_all_experts),
+                                     grouped=bool(self.dataset_args.moe_grouped_calibration)):
+            session.initialize(model=self.model, recipe=self.recipe, recipe_stage=self.stage,
+                               calib_data=calibration_dataloader)
+            mods = session.get_modifiers()
+            user = self.pipeline
+            pipeline = CalibrationPipeline.from_modifiers(mods, user=user)
+            if calibration_dataloader is None and any(m.requires_calibration_data for m in mods):
+                raise ValueError("the recipe requires calibration data but no `dataset` was given")
+            pipeline(self.model, calibration_dataloader, self.dataset_args)
+            session.finalize()
 
 
 def oneshot(model, recipe=None, dataset=None, output_dir: Optional[str] = None, pipeline: str = "independent",

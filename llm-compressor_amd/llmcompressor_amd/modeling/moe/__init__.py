@@ -26,17 +26,27 @@ __all__ = ["ExpertMLP", "LinearExperts2D", "Llama4LinearExperts", "moe_calibrati
 _CALIBRATE_ALL_EXPERTS = False
 # replace the per-expert loop by grouped launches when no hook or quantised forward needs the single calls
 GROUPED_FORWARD = True
+# Off by default: take the grouped launches in observed passes too, when every hook that would fire on an
+# expert Linear only reads the module's input (the Hessian hooks of GPTQ and SparseGPT say so about themselves).
+# The hooks are then called with the same rows as in the loop, but what down_proj receives was computed by the
+# grouped product, whose sums run in another order than the library GEMM's: equal to the last bf16 digit, not
+# bit for bit.
+GROUPED_CALIBRATION = False
 
 
 @contextlib.contextmanager
-def moe_calibration_context(calibrate_all_experts: bool = True):
-    global _CALIBRATE_ALL_EXPERTS
-    prev = _CALIBRATE_ALL_EXPERTS
+def moe_calibration_context(calibrate_all_experts: bool = True, grouped: bool | None = None):
+    """``calibrate_all_experts``: every expert is called on every token (reference: modeling/moe/context.py);
+    ``grouped``: value of ``GROUPED_CALIBRATION`` inside the context (None = leave it as it is)."""
+    global _CALIBRATE_ALL_EXPERTS, GROUPED_CALIBRATION
+    prev = _CALIBRATE_ALL_EXPERTS, GROUPED_CALIBRATION
     _CALIBRATE_ALL_EXPERTS = calibrate_all_experts
+    if grouped is not None:
+        GROUPED_CALIBRATION = bool(grouped)
     try:
         yield
     finally:
-        _CALIBRATE_ALL_EXPERTS = prev
+        _CALIBRATE_ALL_EXPERTS, GROUPED_CALIBRATION = prev
 
 
 class ExpertMLP(nn.Module):
@@ -67,6 +77,24 @@ def _hooks_inert(module: nn.Module, hook_is_inert) -> bool:
         if hooks and not all(hook_is_inert(h) for h in hooks.values()):
             return False
     return True
+
+
+def _reads_input_only(hook) -> bool:
+    return bool(getattr(hook, "_llmc_input_only", False)
+                or getattr(getattr(hook, "__wrapped__", None), "_llmc_input_only", False))
+
+
+def _input_hooks(module: nn.Module, hook_is_inert):
+    """The forward hooks of ``module`` that would act now, if all of them only read the module's input and take
+    the plain (module, args, output) call; None if some other hook would act."""
+    d = module.__dict__
+    for hooks in (d["_forward_pre_hooks"], d["_backward_hooks"], d["_backward_pre_hooks"]):
+        if hooks and not all(hook_is_inert(h) for h in hooks.values()):
+            return None
+    if d.get("_forward_hooks_with_kwargs") or d.get("_forward_hooks_always_called"):
+        return None
+    live = [h for h in d["_forward_hooks"].values() if not hook_is_inert(h)]
+    return live if all(_reads_input_only(h) for h in live) else None
 
 
 class LinearExperts2D(nn.ModuleList):
@@ -123,8 +151,11 @@ class LinearExperts2D(nn.ModuleList):
     # per instance switch for the grouped launches (see ``_grouped_plan``)
     grouped_forward = True
 
-    def _grouped_plan(self, hidden_states: torch.Tensor):
-        """The experts' weights as two pointer tables, or None when the per-expert calls must stay: some hook on
+    def _grouped_plan(self, hidden_states: torch.Tensor, observed: bool = False):
+        """(``observed``: hooks on the Linears that only read their input may be live; the plan then lists them
+        under "hooks", per projection and expert, for the caller to call.)
+
+        The experts' weights as two pointer tables, or None when the per-expert calls must stay: some hook on
         an expert or one of its Linears would fire (only hooks registered through ``HooksMixin`` can be told to be
         off), a Linear has a bias, a quantised forward is active, the experts are not plain ``ExpertMLP``s of
         bf16 Linears of one shape, gradients are recorded, or the shapes do not fit the kernel's tiles.  The
@@ -138,6 +169,7 @@ class LinearExperts2D(nn.ModuleList):
                 or nn.modules.module._global_forward_pre_hooks):
             return None
         weights = ([], [], [])
+        live_hooks = ([], [], [])
         first = self[0]
         act_type, gate_fn = type(first._modules["act_fn"]), first._gate_fn
         names = ("gate_proj", "up_proj", "down_proj")
@@ -158,7 +190,12 @@ class LinearExperts2D(nn.ModuleList):
                     return None
                 if (d["_forward_hooks"] or d["_forward_pre_hooks"] or d["_backward_hooks"]
                         or d["_backward_pre_hooks"]) and not _hooks_inert(lin, hook_is_inert):
-                    return None
+                    found = _input_hooks(lin, hook_is_inert) if observed else None
+                    if found is None:
+                        return None
+                    live_hooks[slot].append(found)
+                elif observed:
+                    live_hooks[slot].append(())
                 if "forward" in d and not (
                         d.get("_llmc_forward_wrapped", False)
                         and (d.get("quantization_scheme") is None or not d.get("quantization_enabled", True))):
@@ -169,7 +206,7 @@ class LinearExperts2D(nn.ModuleList):
         key = tuple(w.data_ptr() for group in weights for w in group)
         cached = self.__dict__.get("_grouped_cache")
         if cached is not None and cached[0] == key and cached[1] == hidden_states.device:
-            return cached[2]
+            return dict(cached[2], hooks=live_hooks) if observed else cached[2]
         gate, up, down = weights
         inter, hidden = gate[0].shape
         for group, shape in ((gate, (inter, hidden)), (up, (inter, hidden)), (down, (hidden, inter))):
@@ -187,7 +224,68 @@ class LinearExperts2D(nn.ModuleList):
         except ValueError:  # a weight that is not 16-byte aligned
             return None
         object.__setattr__(self, "_grouped_cache", (key, hidden_states.device, plan))
-        return plan
+        return dict(plan, hooks=live_hooks) if observed else plan
+
+    def _forward_grouped_observed(self, plan, hidden_states, expert_sorted, tok_sorted, counts) -> torch.Tensor:
+        """The grouped launches with live input-reading hooks: every hook is called with the rows its Linear would
+        have received in the loop (all rows of the block's input with ``calibrate_all_experts``, else the expert's
+        routed rows; an expert without rows still gets its call), the output argument being None.  Returns the
+        experts' outputs for the routed rows, sorted by expert."""
+        from ... import ops
+
+        E, inter, hidden = self.num_experts, plan["inter"], plan["hidden"]
+        hooks_gate, hooks_up, hooks_down = plan["hooks"]
+        names = ("gate_proj", "up_proj", "down_proj")
+        lins = [[expert._modules[n] for expert in self._modules.values()] for n in names]
+        tiles, ntiles = ops.grouped_linear_tiles(counts, hidden_states.device)
+        first = self[0]
+
+        def gate(gate_up):
+            if first._gate_fn is not None:
+                return first._gate_fn(gate_up).contiguous()
+            return (first.act_fn(gate_up[:, :inter]) * gate_up[:, inter:]).contiguous()
+
+        def call(found, lin, rows):
+            for hook in found:
+                hook(lin, (rows,), None)
+
+        if _CALIBRATE_ALL_EXPERTS:
+            T = hidden_states.shape[0]
+            x = hidden_states if hidden_states.is_contiguous() else hidden_states.contiguous()
+            key = (E, T, x.device)
+            cached = self.__dict__.get("_all_tiles")
+            if cached is None or cached[0] != key:
+                cached = (key, ops.grouped_linear_tiles_all(E, T, x.device))
+                object.__setattr__(self, "_all_tiles", cached)
+            all_tiles, n_all = cached[1]
+            gate_up = ops.grouped_linear(x, plan["gate_up"], E, 2, inter, plan["ld_gate_up"], all_tiles, n_all,
+                                         out_rows=E * T)
+            for e in range(E):  # the host walks the hooks while the device multiplies
+                call(hooks_gate[e], lins[0][e], hidden_states)
+                call(hooks_up[e], lins[1][e], hidden_states)
+            mid = gate(gate_up)
+            del gate_up
+            for e in range(E):
+                if hooks_down[e]:
+                    call(hooks_down[e], lins[2][e], mid[e * T:(e + 1) * T])
+            routed_mid = mid[expert_sorted * T + tok_sorted]
+        else:
+            routed = hidden_states[tok_sorted]
+            gate_up = ops.grouped_linear(routed, plan["gate_up"], E, 2, inter, plan["ld_gate_up"], tiles, ntiles)
+            at = 0
+            for e in range(E):
+                rows = routed[at:at + counts[e]]
+                call(hooks_gate[e], lins[0][e], rows)
+                call(hooks_up[e], lins[1][e], rows)
+                at += counts[e]
+            routed_mid = gate(gate_up)
+            del gate_up
+            at = 0
+            for e in range(E):
+                if hooks_down[e]:
+                    call(hooks_down[e], lins[2][e], routed_mid[at:at + counts[e]])
+                at += counts[e]
+        return ops.grouped_linear(routed_mid, plan["down"], E, 1, hidden, plan["ld_down"], tiles, ntiles)
 
     def _forward_grouped(self, plan, routed: torch.Tensor, counts) -> torch.Tensor:
         """``expert(rows)`` for every expert's rows of ``routed`` (sorted by expert) in two launches."""
@@ -227,8 +325,13 @@ class LinearExperts2D(nn.ModuleList):
             place[order] = torch.arange(order.numel(), device=order.device)
             place = place.view(k, T).sort(dim=0).values
         plan = self._grouped_plan(hidden_states) if GROUPED_FORWARD and self.grouped_forward else None
+        observed = None
+        if plan is None and GROUPED_CALIBRATION and GROUPED_FORWARD and self.grouped_forward:
+            observed = self._grouped_plan(hidden_states, observed=True)
         if plan is not None:
             expert_out = self._forward_grouped(plan, hidden_states[tok_sorted], counts)
+        elif observed is not None:
+            expert_out = self._forward_grouped_observed(observed, hidden_states, flat[order], tok_sorted, counts)
         else:
             routed = None if _CALIBRATE_ALL_EXPERTS else hidden_states[tok_sorted]
             outs, at = [], 0

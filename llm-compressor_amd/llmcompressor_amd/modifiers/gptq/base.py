@@ -449,3 +449,8 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
         if self.offload_hessians:
             if module in self._hessians:
                 self._hessians[module] = self._hessians[module].to(device="cpu")
+
+
+# the Hessian hook reads the module and its input, never the output: an experts block may then call it with the
+# rows the Linear would have received without running that Linear by itself
+GPTQModifier.calibrate_module._llmc_input_only = True

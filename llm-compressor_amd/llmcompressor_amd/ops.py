@@ -737,18 +737,36 @@ def weight_pointer_table(weights, device) -> torch.Tensor:
     return torch.tensor(ptrs, dtype=torch.int64, device=device)
 
 
+def grouped_linear_tiles_all(experts: int, rows: int, device) -> tuple[torch.Tensor, int]:
+    """Tile table of ``grouped_linear`` for every expert on all ``rows`` rows of one input: expert e reads the
+    rows 0 .. rows - 1 and writes the rows e * rows .. of the output (``out_rows = experts * rows``)."""
+    import numpy as np
+
+    per = (rows + GROUPED_LINEAR_ROWS - 1) // GROUPED_LINEAR_ROWS
+    n = experts * per
+    table = np.zeros((max(n, 1), 4), dtype=np.int32)
+    if n:
+        start = np.tile(np.arange(per) * GROUPED_LINEAR_ROWS, experts)
+        expert = np.repeat(np.arange(experts), per)
+        table[:, 0], table[:, 1] = expert, start
+        table[:, 2] = np.minimum(rows - start, GROUPED_LINEAR_ROWS)
+        table[:, 3] = expert * rows
+    return torch.from_numpy(table).to(device), n
+
+
 def grouped_linear(x: torch.Tensor, pointers: torch.Tensor, experts: int, splits: int, N: int, ldw: int,
-                   tiles: torch.Tensor, ntiles: int) -> torch.Tensor:
+                   tiles: torch.Tensor, ntiles: int, out_rows: int | None = None) -> torch.Tensor:
     """y [rows, splits * N] (bf16): the rows the tile table assigns to expert e times the transposed weights
-    ``pointers[s * experts + e]`` ([N, K] bf16, row stride ldw) for every split s.  Every row of x must belong to
-    a tile (the output is not cleared)."""
+    ``pointers[s * experts + e]`` ([N, K] bf16, row stride ldw) for every split s.  Every row of y must belong to
+    a tile (the output is not cleared).  ``out_rows``: rows of y when the table's fourth entries move the tiles'
+    results to other rows than their inputs' (default: as many as x has)."""
     _require_gpu(x, pointers, tiles)
     assert x.ndim == 2 and x.dtype == torch.bfloat16 and x.stride(1) == 1
     assert pointers.dtype == torch.int64 and pointers.numel() == experts * splits
     assert tiles.dtype == torch.int32 and tiles.ndim == 2 and tiles.shape[1] == 4 and tiles.shape[0] >= ntiles
     K = x.shape[1]
-    y = torch.empty((x.shape[0], splits * N), dtype=x.dtype, device=x.device)
-    if x.shape[0] == 0:
+    y = torch.empty((x.shape[0] if out_rows is None else out_rows, splits * N), dtype=x.dtype, device=x.device)
+    if x.shape[0] == 0 or ntiles == 0:
         return y
     with torch.cuda.device(x.device):
         rc = _lib.lib().llmc_grouped_linear(x.data_ptr(), _dt(x), x.stride(0), pointers.data_ptr(), ldw, experts,

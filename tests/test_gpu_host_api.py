@@ -2020,3 +2020,108 @@ def test_model_free_ptq_with_a_converter_keeps_converted_layers_and_quantizes_th
     assert q["format"] == "mixed-precision" and q["ignore"] == ["lm_head"]
     index = json.load(open(f"{dst}/model.safetensors.index.json"))
     assert index["weight_map"] == wmap
+
+
+def _tiny_qwen3_moe(seed=0):
+    transformers = pytest.importorskip("transformers")
+    from llmcompressor_amd.modeling import linearize_moe
+
+    torch.manual_seed(seed)
+    cfg = transformers.Qwen3MoeConfig(hidden_size=128, intermediate_size=256, moe_intermediate_size=128,
+                                      num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2,
+                                      head_dim=32, vocab_size=256, max_position_embeddings=128, num_experts=8,
+                                      num_experts_per_tok=2)
+    return linearize_moe(transformers.Qwen3MoeForCausalLM(cfg).to(torch.bfloat16).to(DEV))
+
+
+@pytest.mark.parametrize("all_experts", [True, False])
+def test_oneshot_calibrates_every_expert_on_every_token_unless_told_otherwise(all_experts):
+    """``oneshot(moe_calibrate_all_experts=True)`` (the default) runs the calibration inside
+    ``moe_calibration_context`` (reference: entrypoints/oneshot.py:247-250): while the Hessian hooks observe, every
+    expert Linear is called on all tokens of the batch; with ``False`` only on the tokens routed to its expert.
+    The flag is back to its old value afterwards."""
+    from llmcompressor_amd import oneshot
+    from llmcompressor_amd.modeling import moe as moe_module
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+
+    model = _tiny_qwen3_moe()
+    experts = model.model.layers[0].mlp.experts
+    seen = []
+    watch = experts[3].gate_proj.register_forward_hook(lambda m, args, out: seen.append(args[0].shape[0]))
+    data = [{"input_ids": torch.randint(0, 256, (1, 64))} for _ in range(4)]
+    kw = {} if all_experts else {"moe_calibrate_all_experts": False}
+    oneshot(model=model, recipe=GPTQModifier(targets="Linear", scheme="W4A16", ignore=["lm_head", "re:.*mlp.gate$"]),
+            dataset=data, **kw)
+    watch.remove()
+    # per batch one call in the calibration pass and one in the propagation pass (the test's own hook is live
+    # there too, which keeps the block on its per-expert calls)
+    assert len(seen) == 8
+    if all_experts:
+        assert seen == [64] * 8
+    else:
+        assert all(n < 64 for n in seen) and sum(seen) < 8 * 32
+    assert moe_module._CALIBRATE_ALL_EXPERTS is False and moe_module.GROUPED_CALIBRATION is False
+
+
+@pytest.mark.parametrize("all_experts", [True, False])
+def test_grouped_expert_calibration_agrees_with_the_loop(all_experts):
+    """``moe_grouped_calibration`` (off by default): the observed pass of an experts block takes its grouped
+    launches when the live hooks only read their inputs.  The Hessian hooks are called with the same rows as in
+    the loop: gate_proj / up_proj Hessians are bit-identical (their input is the block's input), down_proj's
+    agree to bf16 rounding of the intermediate activations (relative Frobenius error <= 2e-3), the block's output
+    to the last bf16 digits, every tally is the same -- and no expert Linear is called by itself."""
+    from llmcompressor_amd.core import LifecycleCallbacks, active_session
+    from llmcompressor_amd.modeling import LinearExperts2D, moe_calibration_context
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+
+    torch.manual_seed(0)
+    E, H, I, T = 8, 256, 128, 320
+    fused = (torch.randn(E, 2 * I, H) * 0.05, torch.randn(E, H, I) * 0.05)
+    batches = [torch.randn(T, H, device=DEV).bfloat16() for _ in range(3)]
+    idx = torch.stack([torch.arange(T) % 5, (torch.arange(T) * 3 + 1) % E], dim=1).to(DEV)  # expert 7 rarely, 5-6 less
+    idx[:, 0] = torch.where(idx[:, 0] == idx[:, 1], (idx[:, 0] + 1) % E, idx[:, 0])
+    wts = torch.rand(T, 2, device=DEV).bfloat16()
+    got = {}
+    for grouped in (False, True):
+        experts = LinearExperts2D.from_fused(*fused).to(DEV).to(torch.bfloat16)
+
+        class Wrap(torch.nn.Module):
+            def __init__(self):
+                super().__init__()
+                self.layers = torch.nn.ModuleList([experts])
+
+        model = Wrap()
+        mod = GPTQModifier(targets="Linear", config_groups={"g": dict(
+            targets=["Linear"], weights=dict(num_bits=4, strategy="group", group_size=32))})
+        session = active_session()
+        session.reset()
+        session.initialize(model=model, recipe=mod)
+        LifecycleCallbacks.calibration_start()
+        single_calls = []
+        for e, expert in enumerate(experts):
+            for name in ("gate_proj", "up_proj", "down_proj"):
+                lin = getattr(expert, name)
+                raw = lin.forward
+                lin.forward = (lambda raw, tag: lambda x: (single_calls.append(tag), raw(x))[1])(raw, (e, name))
+        outs = []
+        with torch.no_grad(), moe_calibration_context(all_experts, grouped=grouped):
+            for x in batches:
+                outs.append(experts(x, idx, wts))
+        hess = {(e, n): (mod._hessians[mod._leader.get(getattr(ex, n), getattr(ex, n))].clone(),
+                         float(mod._num_samples[getattr(ex, n)]))
+                for e, ex in enumerate(experts) for n in ("gate_proj", "up_proj", "down_proj")}
+        got[grouped] = (outs, hess, list(single_calls))
+        session.reset()
+    assert len(got[False][2]) == 3 * E * 3 and got[True][2] == []  # the loop calls every Linear, the grouped pass none
+    for a, b in zip(got[False][0], got[True][0]):
+        assert (a.float() - b.float()).norm() <= 1e-2 * a.float().norm()
+    for key, (h_loop, n_loop) in got[False][1].items():
+        h_grp, n_grp = got[True][1][key]
+        assert n_loop == n_grp, key
+        if key[1] == "down_proj":
+            if h_loop.norm() == 0:
+                assert h_grp.norm() == 0, key
+            else:
+                assert (h_loop - h_grp).norm() <= 2e-3 * h_loop.norm(), key
+        else:
+            assert torch.equal(h_loop, h_grp), key
