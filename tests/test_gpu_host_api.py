@@ -2125,3 +2125,38 @@ def test_grouped_expert_calibration_agrees_with_the_loop(all_experts):
                 assert (h_loop - h_grp).norm() <= 2e-3 * h_loop.norm(), key
         else:
             assert torch.equal(h_loop, h_grp), key
+
+
+def test_oneshot_with_grouped_expert_calibration_on_a_transformers_qwen3_moe():
+    """``oneshot(moe_grouped_calibration=True)`` end to end: no expert Linear is called by itself in either pass,
+    every expert Linear ends on its int4 grid, and the quantized model's logits are as close to the dense model's
+    as those of the run that calibrates through the per-expert calls."""
+    from llmcompressor_amd import oneshot
+    from llmcompressor_amd.modeling import ExpertMLP
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+
+    probe = torch.randint(0, 256, (2, 32), device=DEV)
+    data = [{"input_ids": torch.randint(0, 256, (1, 64), generator=torch.Generator().manual_seed(i))} for i in range(8)]
+    errs = {}
+    raw = ExpertMLP.forward
+    for grouped in (False, True):
+        model = _tiny_qwen3_moe()
+        with torch.no_grad():
+            dense = model(probe).logits.float()
+        calls = []
+        experts = model.model.layers[1].mlp.experts
+        ExpertMLP.forward = lambda self, x: (calls.append(x.shape[0]), raw(self, x))[1]  # on the class: no instance differs
+        try:
+            oneshot(model=model, dataset=data, moe_grouped_calibration=grouped,
+                    recipe=GPTQModifier(targets="Linear", scheme="W4A16", ignore=["lm_head", "re:.*mlp.gate$"]))
+        finally:
+            ExpertMLP.forward = raw
+        # per-expert calls: 2 layers x 8 experts x 8 batches in the observed pass, none when it is grouped (the
+        # propagation pass is grouped either way)
+        assert calls == ([] if grouped else [64] * (2 * 8 * 8)), (len(calls), calls[:4])
+        for lin in (experts[2].down_proj, experts[5].gate_proj):
+            code = lin.weight.float() / lin.weight_scale.float().repeat_interleave(128, dim=1)
+            assert (code - code.round()).abs().max() <= 8 * 2.0 ** -8 and code.round().abs().max() <= 8
+        with torch.no_grad():
+            errs[grouped] = ((model(probe).logits.float() - dense).norm() / dense.norm()).item()
+    assert errs[True] < 0.4 and abs(errs[True] - errs[False]) < 0.05, errs
