@@ -543,11 +543,13 @@ def probe_oneshot(batches, tokens, layers=2, vocab=32000):
     print("|---|---|---|---|---|")
     print(f"| model forward alone, one pass over the data (embedding included, lm_head on the last token) | {fwd:.2f} | "
           f"{fwd / layers * 1e3:.0f} | | |")
-    variants = [("Hessian launches of 65536 staged tokens (default)", 65536)]
+    variants = [("Hessian launches of 65536 staged tokens (default)", 65536, True),
+                ("the same with `propagate_error=False`: the next layer calibrated on the uncompressed layer's "
+                 "outputs, one pass per layer", 65536, False)]
     if not whole:
-        variants.append(("one Hessian launch per hook call", 0))
+        variants.append(("one Hessian launch per hook call", 0, True))
     raw_end = LifecycleCallbacks.sequential_epoch_end
-    for label, stage in variants:
+    for label, stage, propagate in variants:
         best = None
         for rep in range(1 if whole else 2):
             model = make()
@@ -566,8 +568,9 @@ def probe_oneshot(batches, tokens, layers=2, vocab=32000):
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             try:
-                oneshot(model=model, dataset=data, recipe=GPTQModifier(targets="Linear", scheme="W4A16", ignore=["lm_head"],
-                                                                         hessian_batch_tokens=stage))
+                oneshot(model=model, dataset=data, propagate_error=propagate,
+                        recipe=GPTQModifier(targets="Linear", scheme="W4A16", ignore=["lm_head"],
+                                            hessian_batch_tokens=stage))
             finally:
                 LifecycleCallbacks.sequential_epoch_end = raw_end
             torch.cuda.synchronize()

@@ -27,6 +27,7 @@ class DatasetArguments:
     moe_calibrate_all_experts: bool = True
     moe_grouped_calibration: bool = False  # this build's own: grouped expert launches in observed passes too
     pipeline: Optional[str] = "independent"
+    propagate_error: bool = True  # sequential pipeline: feed the next layer the compressed layer's outputs
     sequential_targets: Optional[List[str]] = None
     sequential_offload_device: Optional[str] = None  # None: activations stay in HBM (the reference defaults to "cpu")
     tracing_ignore: List[str] = field(default_factory=list)

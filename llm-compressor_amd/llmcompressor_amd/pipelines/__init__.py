@@ -194,21 +194,34 @@ class SequentialPipeline(CalibrationPipeline):
                 cache.update(i, {"args": tuple(args), "kwargs": dict(kwargs)})
             del captured
             returns_tuple = False
+            # reference: pipelines/sequential/pipeline.py:155-176 -- with ``propagate_error=False`` the next layer
+            # is fed what the calibration pass produced (the outputs of the layer before it was compressed) and
+            # the second pass is not run: half the forwards
+            propagate = getattr(dataset_args, "propagate_error", True) if dataset_args is not None else True
             for idx, layer in enumerate(layers):
                 if onload is not None:
                     layer.to(onload)
                 # pass 1: calibrate (hooks fire: Hessians / activation observers)
-                for inputs in cache.iter_prefetch():
-                    layer(*inputs["args"], **inputs["kwargs"])
-                LifecycleCallbacks.sequential_epoch_end(modules=list(layer.modules()))
-                # pass 2: propagate through the compressed layer without triggering hooks
-                with HooksMixin.disable_hooks():
+                if propagate:
+                    for inputs in cache.iter_prefetch():
+                        layer(*inputs["args"], **inputs["kwargs"])
+                else:
                     for i in range(len(cache)):
                         inputs = cache.fetch(i)
                         out = layer(*inputs["args"], **inputs["kwargs"])
                         returns_tuple = isinstance(out, (tuple, list))
                         hidden = out[0] if returns_tuple else out
                         cache.update(i, {"args": (hidden,) + tuple(inputs["args"][1:])})
+                LifecycleCallbacks.sequential_epoch_end(modules=list(layer.modules()))
+                # pass 2: propagate through the compressed layer without triggering hooks
+                if propagate:
+                    with HooksMixin.disable_hooks():
+                        for i in range(len(cache)):
+                            inputs = cache.fetch(i)
+                            out = layer(*inputs["args"], **inputs["kwargs"])
+                            returns_tuple = isinstance(out, (tuple, list))
+                            hidden = out[0] if returns_tuple else out
+                            cache.update(i, {"args": (hidden,) + tuple(inputs["args"][1:])})
                 if onload is not None:
                     layer.to(home)
             # what follows the last layer (final norm, lm_head): the reference's last traced subgraph holds it

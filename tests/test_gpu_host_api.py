@@ -2160,3 +2160,59 @@ def test_oneshot_with_grouped_expert_calibration_on_a_transformers_qwen3_moe():
         with torch.no_grad():
             errs[grouped] = ((model(probe).logits.float() - dense).norm() / dense.norm()).item()
     assert errs[True] < 0.4 and abs(errs[True] - errs[False]) < 0.05, errs
+
+
+def test_sequential_pipeline_without_error_propagation():
+    """``oneshot(propagate_error=False)`` (reference: pipelines/sequential/pipeline.py:155-176,
+    args/dataset_arguments.py:266-274): the next layer is calibrated on the outputs of the uncompressed layer
+    before it and the second pass is not run -- every layer's forward runs once per batch instead of twice, the
+    first layer (whose inputs are the same either way) gets the very same weights, and the later ones are GPTQ
+    results on their own grid with a comparable error on held-out tokens."""
+    transformers = pytest.importorskip("transformers")
+
+    from llmcompressor_amd import oneshot
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+
+    def make():
+        torch.manual_seed(0)
+        cfg = transformers.LlamaConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=3,
+                                       num_attention_heads=4, num_key_value_heads=2, vocab_size=512,
+                                       max_position_embeddings=128)
+        m = transformers.LlamaForCausalLM(cfg).to(torch.bfloat16).to(DEV)
+        with torch.no_grad():
+            m.model.embed_tokens.weight[:, :16] *= 8
+        return m
+
+    torch.manual_seed(1)
+    data = [{"input_ids": torch.randint(0, 512, (1, 128))} for _ in range(8)]
+    held = torch.randint(0, 512, (4, 128), device=DEV)
+    with torch.no_grad():
+        dense = make()(held).logits.float()
+    out = {}
+    for propagate in (True, False):
+        m = make()
+        calls = [0, 0]
+        hooks = [m.model.layers[i + 1].register_forward_pre_hook(
+            lambda mod, args, i=i: calls.__setitem__(i, calls[i] + 1)) for i in (0, 1)]
+        kw = {} if propagate else {"propagate_error": False}
+        oneshot(model=m, dataset=data, recipe=GPTQModifier(targets="Linear", scheme="W4A16", ignore=["lm_head"]), **kw)
+        for h in hooks:
+            h.remove()
+        assert calls == ([16, 16] if propagate else [8, 8]), calls
+        with torch.no_grad():
+            err = ((m(held).logits.float() - dense).norm() / dense.norm()).item()
+        out[propagate] = (m, err)
+    a, b = out[True][0], out[False][0]
+    for name in ("self_attn.q_proj", "self_attn.o_proj", "mlp.gate_proj", "mlp.down_proj"):
+        la, lb = a.model.layers[0].get_submodule(name), b.model.layers[0].get_submodule(name)
+        assert torch.equal(la.weight, lb.weight) and torch.equal(la.weight_scale, lb.weight_scale), name
+    differs = False
+    for i in (1, 2):
+        for name in ("self_attn.q_proj", "mlp.down_proj"):
+            la, lb = a.model.layers[i].get_submodule(name), b.model.layers[i].get_submodule(name)
+            assert torch.equal(la.weight_scale, lb.weight_scale)  # min-max scales come from the weight alone
+            code = lb.weight.float() / lb.weight_scale.float().repeat_interleave(128, dim=1)
+            assert (code - code.round()).abs().max() <= 8 * 2.0 ** -8 and code.round().abs().max() <= 8
+            differs |= not torch.equal(la.weight, lb.weight)
+    assert differs  # the later layers were calibrated on other inputs
+    assert out[False][1] < 1.25 * out[True][1] + 0.02, (out[True][1], out[False][1])
