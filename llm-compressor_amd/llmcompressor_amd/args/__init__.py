@@ -29,5 +29,6 @@ class DatasetArguments:
     pipeline: Optional[str] = "independent"
     propagate_error: bool = True  # sequential pipeline: feed the next layer the compressed layer's outputs
     sequential_targets: Optional[List[str]] = None
+    sequential_targets_per_subgraph: int = 1
     sequential_offload_device: Optional[str] = None  # None: activations stay in HBM (the reference defaults to "cpu")
     tracing_ignore: List[str] = field(default_factory=list)

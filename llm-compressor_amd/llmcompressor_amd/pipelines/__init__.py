@@ -198,32 +198,43 @@ class SequentialPipeline(CalibrationPipeline):
             # is fed what the calibration pass produced (the outputs of the layer before it was compressed) and
             # the second pass is not run: half the forwards
             propagate = getattr(dataset_args, "propagate_error", True) if dataset_args is not None else True
-            for idx, layer in enumerate(layers):
+            # reference: ``sequential_targets_per_subgraph`` (pipelines/sequential/helpers.py) -- that many
+            # consecutive layers are calibrated together, each on what the uncompressed layers before it in the
+            # group produce, and compressed by one epoch-end event
+            per = getattr(dataset_args, "sequential_targets_per_subgraph", 1) if dataset_args is not None else 1
+            per = max(1, int(per or 1))
+
+            def through(group, inputs):
+                """The group's layers one after the other on one batch; returns the arguments for what follows."""
+                nonlocal returns_tuple
+                args = tuple(inputs["args"])
+                for member in group:
+                    out = member(*args, **inputs["kwargs"])
+                    returns_tuple = isinstance(out, (tuple, list))
+                    args = ((out[0] if returns_tuple else out),) + args[1:]
+                return args
+
+            for start in range(0, len(layers), per):
+                group = layers[start:start + per]
                 if onload is not None:
-                    layer.to(onload)
+                    for layer in group:
+                        layer.to(onload)
                 # pass 1: calibrate (hooks fire: Hessians / activation observers)
                 if propagate:
                     for inputs in cache.iter_prefetch():
-                        layer(*inputs["args"], **inputs["kwargs"])
+                        through(group, inputs)
                 else:
                     for i in range(len(cache)):
-                        inputs = cache.fetch(i)
-                        out = layer(*inputs["args"], **inputs["kwargs"])
-                        returns_tuple = isinstance(out, (tuple, list))
-                        hidden = out[0] if returns_tuple else out
-                        cache.update(i, {"args": (hidden,) + tuple(inputs["args"][1:])})
-                LifecycleCallbacks.sequential_epoch_end(modules=list(layer.modules()))
-                # pass 2: propagate through the compressed layer without triggering hooks
+                        cache.update(i, {"args": through(group, cache.fetch(i))})
+                LifecycleCallbacks.sequential_epoch_end(modules=[m for layer in group for m in layer.modules()])
+                # pass 2: propagate through the compressed layers without triggering hooks
                 if propagate:
                     with HooksMixin.disable_hooks():
                         for i in range(len(cache)):
-                            inputs = cache.fetch(i)
-                            out = layer(*inputs["args"], **inputs["kwargs"])
-                            returns_tuple = isinstance(out, (tuple, list))
-                            hidden = out[0] if returns_tuple else out
-                            cache.update(i, {"args": (hidden,) + tuple(inputs["args"][1:])})
+                            cache.update(i, {"args": through(group, cache.fetch(i))})
                 if onload is not None:
-                    layer.to(home)
+                    for layer in group:
+                        layer.to(home)
             # what follows the last layer (final norm, lm_head): the reference's last traced subgraph holds it
             # (pipelines/sequential/pipeline.py:136-181), so a module there that a modifier hooked is calibrated too
             tail = [m for m in rest if id(m) not in before and _has_calibration_hooks(m)]

@@ -2216,3 +2216,59 @@ def test_sequential_pipeline_without_error_propagation():
             differs |= not torch.equal(la.weight, lb.weight)
     assert differs  # the later layers were calibrated on other inputs
     assert out[False][1] < 1.25 * out[True][1] + 0.02, (out[True][1], out[False][1])
+
+
+def test_sequential_pipeline_with_several_layers_per_subgraph():
+    """``oneshot(sequential_targets_per_subgraph=2)`` (reference: pipelines/sequential/pipeline.py:103-110): two
+    consecutive layers are calibrated together and compressed by one epoch-end event.  The first layer of a group
+    sees what it would see alone (same weights as the default run), the second is calibrated on the uncompressed
+    first layer's outputs (other weights, own grid); with a group that spans the whole model and no error
+    propagation every layer's forward runs once per batch."""
+    transformers = pytest.importorskip("transformers")
+
+    from llmcompressor_amd import oneshot
+    from llmcompressor_amd.core import LifecycleCallbacks
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+
+    def make():
+        torch.manual_seed(0)
+        cfg = transformers.LlamaConfig(hidden_size=256, intermediate_size=512, num_hidden_layers=3,
+                                       num_attention_heads=4, num_key_value_heads=2, vocab_size=512,
+                                       max_position_embeddings=128)
+        m = transformers.LlamaForCausalLM(cfg).to(torch.bfloat16).to(DEV)
+        with torch.no_grad():
+            m.model.embed_tokens.weight[:, :16] *= 8
+        return m
+
+    torch.manual_seed(1)
+    data = [{"input_ids": torch.randint(0, 512, (1, 128))} for _ in range(8)]
+    recipe = lambda: GPTQModifier(targets="Linear", scheme="W4A16", ignore=["lm_head"])  # noqa: E731
+    base = make()
+    oneshot(model=base, dataset=data, recipe=recipe())
+    raw_end = LifecycleCallbacks.sequential_epoch_end
+    events = []
+    LifecycleCallbacks.sequential_epoch_end = staticmethod(
+        lambda *a, modules=(), **kw: (events.append(sum(isinstance(m, transformers.models.llama.modeling_llama.
+                                                                   LlamaDecoderLayer) for m in modules)),
+                                      raw_end(*a, modules=modules, **kw))[1])
+    try:
+        two = make()
+        oneshot(model=two, dataset=data, recipe=recipe(), sequential_targets_per_subgraph=2)
+        assert [e for e in events if e] == [2, 1]
+        events.clear()
+        whole = make()
+        calls = [0]
+        hook = whole.model.layers[2].register_forward_pre_hook(lambda mod, args: calls.__setitem__(0, calls[0] + 1))
+        oneshot(model=whole, dataset=data, recipe=recipe(), sequential_targets_per_subgraph=8, propagate_error=False)
+        hook.remove()
+        assert [e for e in events if e] == [3] and calls == [8]
+    finally:
+        LifecycleCallbacks.sequential_epoch_end = raw_end
+    for name in ("self_attn.q_proj", "mlp.down_proj"):
+        get = lambda m, i: m.model.layers[i].get_submodule(name).weight  # noqa: E731
+        assert torch.equal(get(base, 0), get(two, 0)) and torch.equal(get(base, 0), get(whole, 0)), name
+        assert not torch.equal(get(base, 1), get(two, 1)), name
+        assert torch.equal(get(two, 1), get(whole, 1)), name  # both calibrated on the uncompressed layer 0
+        lin = whole.model.layers[2].get_submodule(name)
+        code = lin.weight.float() / lin.weight_scale.float().repeat_interleave(128, dim=1)
+        assert (code - code.round()).abs().max() <= 8 * 2.0 ** -8 and code.round().abs().max() <= 8
