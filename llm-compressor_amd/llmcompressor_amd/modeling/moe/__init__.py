@@ -230,7 +230,8 @@ class LinearExperts2D(nn.ModuleList):
         """The grouped launches with live input-reading hooks: every hook is called with the rows its Linear would
         have received in the loop (all rows of the block's input with ``calibrate_all_experts``, else the expert's
         routed rows; an expert without rows still gets its call), the output argument being None.  Returns the
-        experts' outputs for the routed rows, sorted by expert."""
+        experts' outputs for the routed rows, sorted by expert.  With ``calibrate_all_experts`` gate and up of all
+        experts are one library product on the stacked weights, and down_proj runs on the routed rows only."""
         from ... import ops
 
         E, inter, hidden = self.num_experts, plan["inter"], plan["hidden"]
@@ -251,19 +252,16 @@ class LinearExperts2D(nn.ModuleList):
 
         if _CALIBRATE_ALL_EXPERTS:
             T = hidden_states.shape[0]
-            x = hidden_states if hidden_states.is_contiguous() else hidden_states.contiguous()
-            key = (E, T, x.device)
-            cached = self.__dict__.get("_all_tiles")
-            if cached is None or cached[0] != key:
-                cached = (key, ops.grouped_linear_tiles_all(E, T, x.device))
-                object.__setattr__(self, "_all_tiles", cached)
-            all_tiles, n_all = cached[1]
-            gate_up = ops.grouped_linear(x, plan["gate_up"], E, 2, inter, plan["ld_gate_up"], all_tiles, n_all,
-                                         out_rows=E * T)
+            # every expert reads the same rows: one library product with the experts' gate / up weights stacked
+            # into one [E * 2I, H] matrix (a copy per call, so that it is never stale) instead of E tiles' worth of
+            # grouped launches
+            stacked = torch.cat([lin.weight for pair in zip(lins[0], lins[1]) for lin in pair])
+            gate_up = torch.nn.functional.linear(hidden_states, stacked).view(T * E, 2 * inter)
+            del stacked
             for e in range(E):  # the host walks the hooks while the device multiplies
                 call(hooks_gate[e], lins[0][e], hidden_states)
                 call(hooks_up[e], lins[1][e], hidden_states)
-            mid = gate(gate_up)
+            mid = gate(gate_up).view(T, E, inter).permute(1, 0, 2).contiguous().view(E * T, inter)
             del gate_up
             for e in range(E):
                 if hooks_down[e]:

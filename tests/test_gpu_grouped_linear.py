@@ -55,6 +55,28 @@ def test_grouped_linear_against_per_expert_linear(N, K, splits):
         at += c
 
 
+def test_grouped_linear_every_expert_on_the_same_rows():
+    """The tile table's fourth entry moves a tile's results to other rows than its inputs': every expert reads the
+    rows 0 .. T - 1 of one input and writes its own block of T rows (``grouped_linear_tiles_all``), the values a
+    call with the input repeated expert after expert gives, bit for bit."""
+    from llmcompressor_amd import ops
+
+    torch.manual_seed(3)
+    E, T, N, K = 5, 200, 256, 128
+    x = torch.randn(T, K, device=DEV).bfloat16()
+    weights = [[(torch.randn(N, K, device=DEV) * K ** -0.5).bfloat16() for _ in range(E)] for _ in range(2)]
+    table = ops.weight_pointer_table([w for group in weights for w in group], DEV)
+    tiles, ntiles = ops.grouped_linear_tiles_all(E, T, DEV)
+    assert ntiles == E * 2 and tiles[:, 3].tolist() == [e * T for e in range(E) for _ in range(2)]
+    y = ops.grouped_linear(x, table, E, 2, N, K, tiles, ntiles, out_rows=E * T)
+    assert y.shape == (E * T, 2 * N)
+    rep_tiles, rep_n = ops.grouped_linear_tiles([T] * E, DEV)
+    want = ops.grouped_linear(x.repeat(E, 1), table, E, 2, N, K, rep_tiles, rep_n)
+    assert torch.equal(y, want)
+    ref = torch.nn.functional.linear(x, weights[1][3])
+    _assert_same_to_one_ulp(y[3 * T:4 * T, N:], ref, x.double() @ weights[1][3].double().t(), "expert 3, split 1")
+
+
 def test_grouped_linear_reads_strided_rows_and_rejects_what_it_cannot_tile():
     from llmcompressor_amd import _lib, ops
 
