@@ -21,6 +21,7 @@ import torch
 from torch import nn
 
 __all__ = ["ExpertMLP", "LinearExperts2D", "Llama4LinearExperts", "moe_calibration_context",
+           "get_calibrate_all_experts_flag",
            "get_non_linearized_moes", "linearize_moe"]
 
 _CALIBRATE_ALL_EXPERTS = False
@@ -32,6 +33,11 @@ GROUPED_FORWARD = True
 # grouped product, whose sums run in another order than the library GEMM's: equal to the last bf16 digit, not
 # bit for bit.
 GROUPED_CALIBRATION = False
+
+
+def get_calibrate_all_experts_flag() -> bool:
+    """Is every expert called on every token right now (reference: modeling/moe/context.py:6-7)?"""
+    return _CALIBRATE_ALL_EXPERTS
 
 
 @contextlib.contextmanager

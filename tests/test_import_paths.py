@@ -64,7 +64,7 @@ _REFERENCE_IMPORT_LINES = [
     "from llmcompressor.pipelines.registry import CalibrationPipeline",
     "from llmcompressor.modeling.moe.linear_experts import LinearExperts2D",
     "from llmcompressor.modeling.moe.linearize import linearize_moe, load_quantizable_moe",
-    "from llmcompressor.modeling.moe.context import moe_calibration_context",
+    "from llmcompressor.modeling.moe.context import moe_calibration_context, get_calibrate_all_experts_flag",
     "from llmcompressor.entrypoints.model_free import model_free_ptq",
     "from llmcompressor.transformers.compression.compressed_tensors_utils import modify_save_pretrained",
 ]
@@ -87,6 +87,12 @@ def test_helpers_the_examples_wrap_their_loading_in():
     from llmcompressor.modeling.moe.linearize import load_quantizable_moe
     from llmcompressor.utils import dispatch_for_generation, load_context
 
+    from llmcompressor.modeling.moe.context import get_calibrate_all_experts_flag, moe_calibration_context
+
+    assert get_calibrate_all_experts_flag() is False
+    with moe_calibration_context():
+        assert get_calibrate_all_experts_flag() is True
+    assert get_calibrate_all_experts_flag() is False
     with load_context(), load_quantizable_moe():
         model = torch.nn.Linear(4, 4)
     assert dispatch_for_generation(model) is model  # no GPU here: stays on the host
