@@ -1004,3 +1004,98 @@ def test_model_free_converter_config_merge_and_dependencies(tmp_path):
 
     with pytest.raises(TypeError, match="process"):
         model_free_ptq(str(src), str(tmp_path / "dst"), scheme="FP8_DYNAMIC", converter=object())
+
+
+def test_sequential_pipeline_pass_structure_on_the_host():
+    """The sequential pipeline's passes with a recording modifier on a CPU model (no kernel involved; reference:
+    pipelines/sequential/pipeline.py:136-181): by default every layer runs twice per batch (hooks live, then hooks
+    off on the layer the epoch-end event has just changed) and the next layer is fed the second pass's outputs;
+    ``propagate_error=False`` runs the first pass only and feeds its outputs on;
+    ``sequential_targets_per_subgraph=2`` hands two layers to one epoch-end event."""
+    from llmcompressor_amd.core import active_session
+    from llmcompressor_amd.modifiers import Modifier
+    from llmcompressor_amd.pipelines import CalibrationPipeline
+
+    class Layer(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.lin = torch.nn.Linear(4, 4, bias=False)
+            with torch.no_grad():
+                self.lin.weight.copy_(torch.eye(4))
+
+        def forward(self, x):
+            return self.lin(x)
+
+    class Model(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.layers = torch.nn.ModuleList([Layer() for _ in range(3)])
+
+        def forward(self, x):
+            for layer in self.layers:
+                x = layer(x)
+            return x
+
+    class Recorder(Modifier):
+        requires_calibration_data: bool = True
+        log: list = []
+
+        def on_initialize(self, state, **kwargs):
+            self.log.clear()
+            return True
+
+        def on_calibration_start(self, state, event, **kwargs):
+            for i, layer in enumerate(state.model.layers):
+                self.register_hook(layer.lin, lambda m, args, out, i=i: self.log.append(("seen", i, args[0].sum().item())),
+                                   "forward")
+
+        def on_sequential_epoch_end(self, state, event, modules=(), **kwargs):
+            lins = [m for m in modules if isinstance(m, torch.nn.Linear)]
+            if lins:
+                self.log.append(("epoch_end", len(lins)))
+            for lin in lins:  # "compress": the layer doubles its input from now on
+                lin.weight.data.mul_(2.0)
+
+        def on_calibration_end(self, state, event, **kwargs):
+            self.remove_hooks()
+
+        def on_finalize(self, state, **kwargs):
+            return True
+
+    class Args:
+        sequential_targets = None
+
+    data = [torch.ones(1, 4), 2 * torch.ones(1, 4)]
+
+    def run(**kw):
+        model, mod = Model(), Recorder()
+        session = active_session()
+        session.reset()
+        session.initialize(model=model, recipe=mod)
+        args = Args()
+        for k, v in kw.items():
+            setattr(args, k, v)
+        forwards = [0, 0, 0]
+        handles = [l.register_forward_pre_hook(lambda m, a, i=i: forwards.__setitem__(i, forwards[i] + 1))
+                   for i, l in enumerate(model.layers)]
+        CalibrationPipeline.load_from_registry("sequential")(model, data, args)
+        for h in handles:
+            h.remove()
+        session.finalize()
+        session.reset()
+        return list(mod.log), forwards
+
+    log, forwards = run()
+    # layer 0 is also entered once per batch by the pass that captures its inputs
+    assert forwards == [6, 4, 4]
+    # layer 1 sees layer 0's compressed (doubled) outputs, layer 2 the twice-doubled ones
+    assert log == [("seen", 0, 4.0), ("seen", 0, 8.0), ("epoch_end", 1), ("seen", 1, 8.0), ("seen", 1, 16.0),
+                   ("epoch_end", 1), ("seen", 2, 16.0), ("seen", 2, 32.0), ("epoch_end", 1)]
+    log, forwards = run(propagate_error=False)
+    assert forwards == [4, 2, 2]
+    assert log == [("seen", 0, 4.0), ("seen", 0, 8.0), ("epoch_end", 1), ("seen", 1, 4.0), ("seen", 1, 8.0),
+                   ("epoch_end", 1), ("seen", 2, 4.0), ("seen", 2, 8.0), ("epoch_end", 1)]
+    log, forwards = run(sequential_targets_per_subgraph=2)
+    assert forwards == [6, 4, 4]
+    assert log == [("seen", 0, 4.0), ("seen", 1, 4.0), ("seen", 0, 8.0), ("seen", 1, 8.0), ("epoch_end", 2),
+                   ("seen", 2, 16.0), ("seen", 2, 32.0), ("epoch_end", 1)]
