@@ -1099,3 +1099,45 @@ def test_sequential_pipeline_pass_structure_on_the_host():
     assert forwards == [6, 4, 4]
     assert log == [("seen", 0, 4.0), ("seen", 1, 4.0), ("seen", 0, 8.0), ("seen", 1, 8.0), ("epoch_end", 2),
                    ("seen", 2, 16.0), ("seen", 2, 32.0), ("epoch_end", 1)]
+
+
+def test_experts_block_tells_input_reading_hooks_from_the_rest():
+    """What lets an experts block call a Linear's hooks itself instead of the Linear (``moe_grouped_calibration``):
+    every live hook is a plain forward hook that declares it only reads the module's input, as GPTQ's Hessian hook
+    does; anything else (an undeclared hook, a pre-hook, a hook taking keyword arguments) keeps the per-expert
+    calls, and hooks that ``disable_hooks`` has switched off do not count."""
+    from llmcompressor_amd.modeling.moe import _input_hooks
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+    from llmcompressor_amd.modifiers.utils.hooks import HooksMixin, hook_is_inert
+
+    assert GPTQModifier.calibrate_module._llmc_input_only is True
+    lin = torch.nn.Linear(4, 4)
+    assert _input_hooks(lin, hook_is_inert) == []
+    owner = HooksMixin()
+    seen = []
+
+    def reads_input(module, args, output):
+        seen.append(args[0].shape)
+
+    reads_input._llmc_input_only = True
+    handle = owner.register_hook(lin, reads_input, "forward")
+    live = _input_hooks(lin, hook_is_inert)
+    assert len(live) == 1
+    live[0](lin, (torch.zeros(3, 4),), None)  # the call an experts block makes
+    assert seen == [torch.Size([3, 4])]
+    with HooksMixin.disable_hooks():
+        assert _input_hooks(lin, hook_is_inert) == []
+    with HooksMixin.disable_hooks(keep={handle}):
+        assert len(_input_hooks(lin, hook_is_inert)) == 1
+    plain = lin.register_forward_hook(lambda m, a, o: None)  # says nothing about itself
+    assert _input_hooks(lin, hook_is_inert) is None
+    plain.remove()
+    pre = lin.register_forward_pre_hook(lambda m, a: None)
+    assert _input_hooks(lin, hook_is_inert) is None
+    pre.remove()
+    kw = lin.register_forward_hook(lambda m, a, k, o: None, with_kwargs=True)
+    assert _input_hooks(lin, hook_is_inert) is None
+    kw.remove()
+    assert len(_input_hooks(lin, hook_is_inert)) == 1
+    owner.remove_hooks()
+    assert _input_hooks(lin, hook_is_inert) == []
