@@ -504,6 +504,52 @@ def probe_moe(mode="both"):
         print(f"| {label} | {best[0] * 1e3:.1f} | {best[1] * 1e3:.1f} | {best[1] * 1e3 / (3 * E):.2f} |")
 
 
+def probe_oneshot_moe(batches=16, tokens=2048, layers=2):
+    """oneshot() on a transformers Qwen3MoeForCausalLM with `layers` decoder layers of the Qwen3-30B-A3B shape
+    (hidden 2048, 32 query and 4 key / value heads of 128, 128 experts of intermediate size 768, top-8 routing,
+    random weights, fused expert tensors that oneshot replaces by per-expert Linears), GPTQ W4A16 on attention and
+    expert Linears, in the four ways the experts can be calibrated.  Wall time around oneshot."""
+    import torch
+    import transformers
+
+    from llmcompressor_amd import oneshot
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+
+    cfg = transformers.Qwen3MoeConfig(hidden_size=2048, intermediate_size=6144, moe_intermediate_size=768,
+                                      num_hidden_layers=layers, num_attention_heads=32, num_key_value_heads=4,
+                                      head_dim=128, vocab_size=32000, max_position_embeddings=4096, num_experts=128,
+                                      num_experts_per_tok=8, decoder_sparse_step=1, mlp_only_layers=[])
+    data = [{"input_ids": torch.randint(0, 32000, (1, tokens))} for _ in range(batches)]
+    print(f"| oneshot GPTQ W4A16, {layers} Qwen3-30B-A3B-shaped layers, {batches} x {tokens} tokens | s | "
+          "ms per layer and batch | peak GiB |")
+    print("|---|---|---|---|")
+    for label, kw in (
+            ("every expert on every token, per-expert calls (default)", {}),
+            ("every expert on every token, `moe_grouped_calibration=True`", {"moe_grouped_calibration": True}),
+            ("routed tokens only (`moe_calibrate_all_experts=False`), per-expert calls",
+             {"moe_calibrate_all_experts": False}),
+            ("routed tokens only, `moe_grouped_calibration=True`",
+             {"moe_calibrate_all_experts": False, "moe_grouped_calibration": True})):
+        best = None
+        for _ in range(2):
+            torch.manual_seed(0)
+            with torch.device("cuda"):
+                model = transformers.Qwen3MoeForCausalLM(cfg).to(torch.bfloat16)
+            torch.cuda.synchronize()
+            torch.cuda.reset_peak_memory_stats()
+            t0 = time.perf_counter()
+            oneshot(model=model, dataset=data, recipe=GPTQModifier(targets="Linear", scheme="W4A16",
+                                                                   ignore=["lm_head", "re:.*mlp.gate$"]), **kw)
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            peak = torch.cuda.max_memory_allocated() / 2 ** 30
+            del model
+            torch.cuda.empty_cache()
+            if best is None or dt < best[0]:
+                best = (dt, peak)
+        print(f"| {label} | {best[0]:.2f} | {best[0] / layers / batches * 1e3:.1f} | {best[1]:.1f} |")
+
+
 def probe_oneshot(batches, tokens, layers=2, vocab=32000):
     """oneshot() on a transformers LlamaForCausalLM with `layers` Llama-3-8B-shaped decoder layers (random
     weights), GPTQ W4A16 with the modifier's defaults, `batches` x `tokens` calibration tokens: wall time per layer
@@ -617,6 +663,9 @@ def main():
     ap.add_argument("--vocab", type=int, default=32000, help="--probe-oneshot: vocabulary size (config: 128256)")
     ap.add_argument("--probe-chain", action="store_true",
                     help="time the Cholesky chain, the column loop and their fp32 products alone, print tables")
+    ap.add_argument("--probe-oneshot-moe", action="store_true",
+                    help="print end-to-end oneshot timings on a transformers Qwen3-MoE with two 30B-A3B-shaped layers "
+                    "for the four ways of calibrating the experts")
     ap.add_argument("--probe-vendor-gemm", action="store_true",
                     help="time the dominant launch beside the vendor library's bf16 GEMM on the same operands")
     ap.add_argument("--probe-product", type=int, default=0, metavar="N",
@@ -650,6 +699,9 @@ def main():
         return
     if a.probe_moe:
         probe_moe(a.moe_mode)
+        return
+    if a.probe_oneshot_moe:
+        probe_oneshot_moe()
         return
     if a.probe_vendor_gemm:
         probe_vendor_gemm(a.stage_tokens or 65536)

@@ -226,9 +226,11 @@ class GPTQModifier(Modifier, QuantizationMixin, HessianStagingMixin):
         priv = self.__pydantic_private__ if priv is None else priv
         width = module.in_features if isinstance(module, torch.nn.Linear) else None
         recent = priv["_recent_input"].get(width) if width is not None else None
+        # an empty tensor is "the same" only as the very object: the empty row ranges of two neighbouring experts
+        # without tokens start at one address and have one shape, and are still two inputs
         same = (recent is not None and recent[2] is not module and inp.data_ptr() == recent[0].data_ptr()
                 and inp.shape == recent[0].shape and inp.dtype == recent[0].dtype and inp.stride() == recent[0].stride()
-                and inp._version == recent[1])
+                and inp._version == recent[1] and (inp.numel() > 0 or inp is recent[0]))
         leaders, num_samples = priv["_leader"], priv["_num_samples"]
         leader = leaders.get(module)
         if same and (leader is recent[2] or (leader is None and module not in num_samples)):

@@ -1141,3 +1141,34 @@ def test_experts_block_tells_input_reading_hooks_from_the_rest():
     assert len(_input_hooks(lin, hook_is_inert)) == 1
     owner.remove_hooks()
     assert _input_hooks(lin, hook_is_inert) == []
+
+
+def test_shared_inputs_do_not_pair_up_neighbouring_experts_without_tokens():
+    """``share_identical_inputs``: two experts that receive no token in a batch are handed empty row ranges that
+    start at one address and have one shape; they are two inputs all the same (only the very same tensor object
+    counts when it is empty), so neither becomes the other's follower -- and an expert's up_proj, which is handed
+    the very object its gate_proj got, still follows it, empty or not."""
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+
+    mod = GPTQModifier(targets="Linear", scheme="W4A16")
+    gate = [torch.nn.Linear(8, 4, bias=False) for _ in range(2)]
+    up = [torch.nn.Linear(8, 4, bias=False) for _ in range(2)]
+    routed = torch.randn(6, 8)
+
+    def batch(rows_of_expert):
+        followed = []
+        for e, (lo, hi) in enumerate(rows_of_expert):
+            x = routed[lo:hi]
+            for lin in (gate[e], up[e]):
+                follows = mod._follows_recent_input(lin, x)
+                followed.append(follows)
+                if not follows and lin not in mod._num_samples:  # what the hook does for a module of its own
+                    mod._num_samples[lin] = 0
+        return followed
+
+    # both experts without tokens: the ranges routed[3:3] and routed[3:3] are equal in every respect but identity
+    assert batch([(3, 3), (3, 3)]) == [False, True, False, True]
+    assert mod._leader == {up[0]: gate[0], up[1]: gate[1]}
+    # later they get different rows: nobody raises, everybody still follows its own gate_proj
+    assert batch([(0, 2), (2, 6)]) == [False, True, False, True]
+    assert batch([(0, 0), (0, 6)]) == [False, True, False, True]
