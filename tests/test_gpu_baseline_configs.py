@@ -13,6 +13,8 @@ q/k/v/o/gate/up/down weights bf16 ~ N(0, 0.02), Linear i drawn from seed i.
   [0.2, 1.0], norm 2.4: (min, max) of every group equal (a group may differ only on a documented rounding tie).
 * MoE layer of the Qwen3-30B-A3B shape (128 experts, 768 x 2048 and 2048 x 768): grouped GPTQ, W4A16 g128 and NVFP4,
   sampled experts against the oracle's quantize_weight at >= 99.9 % identical weights.
+* The same MoE shape end to end: one transformers Qwen3-MoE decoder layer through ``oneshot`` in the four ways its
+  experts can be calibrated.
 * Sequential GPTQ through ``oneshot`` on two such decoder layers of a transformers Llama: every Linear on its int4
   grid, and closer to the dense model on held-out tokens than round-to-nearest.
 """
@@ -482,3 +484,58 @@ def test_sequential_gptq_through_oneshot_at_the_llama3_8b_layer_shapes():
     e_rtn = err(rtn)
     print(f"relative logit error on held-out tokens: GPTQ {e_gptq:.4f}, round-to-nearest {e_rtn:.4f}", flush=True)
     assert e_gptq < 0.9 * e_rtn, (e_gptq, e_rtn)
+
+
+@pytest.mark.parametrize("mode", ["all_experts", "routed", "all_experts_grouped", "routed_grouped"])
+def test_gptq_through_oneshot_at_the_qwen3_30b_a3b_layer_shape(mode):
+    """The MoE configuration end to end: one transformers Qwen3-MoE decoder layer of the 30B-A3B shape (hidden
+    2048, 128 experts of intermediate size 768, top-8 routing by a random-init router that leaves some experts with
+    no token in a batch), fused expert tensors replaced by per-expert Linears, GPTQ W4A16 through ``oneshot`` in the
+    four ways the experts can be calibrated: all 388 Linears end on their int4 grid, the logits stay finite, and
+    with every expert on every token all gate / up projections of the layer end up on one Hessian."""
+    transformers = pytest.importorskip("transformers")
+
+    from llmcompressor_amd import oneshot
+    from llmcompressor_amd.modeling import LinearExperts2D
+    from llmcompressor_amd.modifiers.gptq import GPTQModifier
+
+    cfg = transformers.Qwen3MoeConfig(hidden_size=2048, intermediate_size=6144, moe_intermediate_size=768,
+                                      num_hidden_layers=1, num_attention_heads=32, num_key_value_heads=4, head_dim=128,
+                                      vocab_size=4096, max_position_embeddings=2048, num_experts=128,
+                                      num_experts_per_tok=8, decoder_sparse_step=1, mlp_only_layers=[])
+    torch.manual_seed(0)
+    with torch.device(DEV):
+        model = transformers.Qwen3MoeForCausalLM(cfg).to(torch.bfloat16)
+    data = [{"input_ids": torch.randint(0, 4096, (1, 1024), generator=torch.Generator().manual_seed(i))}
+            for i in range(6)]
+    kw = {"moe_calibrate_all_experts": mode.startswith("all_experts"), "moe_grouped_calibration": mode.endswith("grouped")}
+    mod = GPTQModifier(targets="Linear", scheme="W4A16", ignore=["lm_head", "re:.*mlp.gate$"])
+    leaders = {}
+    raw = GPTQModifier._begin_compress
+
+    def spy(self, module_list):
+        leaders.update(self._leader)
+        return raw(self, module_list)
+
+    GPTQModifier._begin_compress = spy
+    try:
+        oneshot(model=model, dataset=data, recipe=mod, **kw)
+    finally:
+        GPTQModifier._begin_compress = raw
+    experts = model.model.layers[0].mlp.experts
+    assert isinstance(experts, LinearExperts2D) and len(experts) == 128
+    count = 0
+    for name, lin in model.named_modules():
+        if isinstance(lin, torch.nn.Linear) and hasattr(lin, "weight_scale"):
+            code = lin.weight.float() / lin.weight_scale.float().repeat_interleave(128, dim=1)
+            assert (code - code.round()).abs().max() <= 8 * 2.0 ** -8 and code.round().abs().max() <= 8, name
+            count += 1
+    assert count == 4 + 3 * 128
+    with torch.no_grad():
+        assert torch.isfinite(model(torch.randint(0, 4096, (1, 64), device=DEV)).logits.float()).all()
+    gate_up = [lin for e in experts for lin in (e.gate_proj, e.up_proj)]
+    led = {leaders.get(lin, lin) for lin in gate_up}
+    if mode.startswith("all_experts"):
+        assert len(led) == 1  # the block's input, once
+    else:
+        assert len(led) == 128 and all(leaders.get(e.up_proj) is e.gate_proj for e in experts)
