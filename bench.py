@@ -504,7 +504,7 @@ def probe_moe(mode="both"):
         print(f"| {label} | {best[0] * 1e3:.1f} | {best[1] * 1e3:.1f} | {best[1] * 1e3 / (3 * E):.2f} |")
 
 
-def probe_oneshot_moe(batches=16, tokens=2048, layers=2):
+def probe_oneshot_moe(batches=16, tokens=2048, layers=2, vocab=32000):
     """oneshot() on a transformers Qwen3MoeForCausalLM with `layers` decoder layers of the Qwen3-30B-A3B shape
     (hidden 2048, 32 query and 4 key / value heads of 128, 128 experts of intermediate size 768, top-8 routing,
     random weights, fused expert tensors that oneshot replaces by per-expert Linears), GPTQ W4A16 on attention and
@@ -513,13 +513,14 @@ def probe_oneshot_moe(batches=16, tokens=2048, layers=2):
     import transformers
 
     from llmcompressor_amd import oneshot
+    from llmcompressor_amd.core import active_session
     from llmcompressor_amd.modifiers.gptq import GPTQModifier
 
     cfg = transformers.Qwen3MoeConfig(hidden_size=2048, intermediate_size=6144, moe_intermediate_size=768,
                                       num_hidden_layers=layers, num_attention_heads=32, num_key_value_heads=4,
-                                      head_dim=128, vocab_size=32000, max_position_embeddings=4096, num_experts=128,
+                                      head_dim=128, vocab_size=vocab, max_position_embeddings=4096, num_experts=128,
                                       num_experts_per_tok=8, decoder_sparse_step=1, mlp_only_layers=[])
-    data = [{"input_ids": torch.randint(0, 32000, (1, tokens))} for _ in range(batches)]
+    data = [{"input_ids": torch.randint(0, vocab, (1, tokens))} for _ in range(batches)]
     print(f"| oneshot GPTQ W4A16, {layers} Qwen3-30B-A3B-shaped layers, {batches} x {tokens} tokens | s | "
           "ms per layer and batch | peak GiB |")
     print("|---|---|---|---|")
@@ -531,7 +532,7 @@ def probe_oneshot_moe(batches=16, tokens=2048, layers=2):
             ("routed tokens only, `moe_grouped_calibration=True`",
              {"moe_calibrate_all_experts": False, "moe_grouped_calibration": True})):
         best = None
-        for _ in range(2):
+        for _ in range(2 if layers <= 8 else 1):
             torch.manual_seed(0)
             with torch.device("cuda"):
                 model = transformers.Qwen3MoeForCausalLM(cfg).to(torch.bfloat16)
@@ -544,6 +545,7 @@ def probe_oneshot_moe(batches=16, tokens=2048, layers=2):
             dt = time.perf_counter() - t0
             peak = torch.cuda.max_memory_allocated() / 2 ** 30
             del model
+            active_session().reset()  # the session still refers to the model it compressed
             torch.cuda.empty_cache()
             if best is None or dt < best[0]:
                 best = (dt, peak)
@@ -666,6 +668,7 @@ def main():
     ap.add_argument("--probe-oneshot-moe", action="store_true",
                     help="print end-to-end oneshot timings on a transformers Qwen3-MoE with two 30B-A3B-shaped layers "
                     "for the four ways of calibrating the experts")
+    ap.add_argument("--moe-batches", type=int, default=16, help="--probe-oneshot-moe: calibration batches of --tokens tokens")
     ap.add_argument("--probe-vendor-gemm", action="store_true",
                     help="time the dominant launch beside the vendor library's bf16 GEMM on the same operands")
     ap.add_argument("--probe-product", type=int, default=0, metavar="N",
@@ -701,7 +704,7 @@ def main():
         probe_moe(a.moe_mode)
         return
     if a.probe_oneshot_moe:
-        probe_oneshot_moe()
+        probe_oneshot_moe(a.moe_batches, a.tokens, a.layers, a.vocab)
         return
     if a.probe_vendor_gemm:
         probe_vendor_gemm(a.stage_tokens or 65536)
